@@ -1,0 +1,186 @@
+// Bandwidth-bound pieces of the attention layer: causal mask, softmax over the key
+// axis of the head-interleaved score tensor [nrow, nvec, ncol] (ncol = heads, innermost), and
+// its backward.  Reference: VMath::set_mh_attention_mask (vmath.cu:6833-6860),
+// softmax_direct_on_axis (vmath.cu:6864-6916), softmax_direct_on_axis_backward
+// (vmath.cu:6920-6973).
+//
+// The data of one outer row (nvec*ncol floats) is contiguous.  Three access plans keep every
+// global access coalesced whatever the head count:
+//   ncol == 1        one wave per row, lanes stride the row
+//   2..128 heads     one workgroup per outer row; thread t walks elements t, t+TB, ... with TB a
+//                    multiple of ncol, so a thread always sees the same head; per-head partials
+//                    meet in LDS
+//   > 128 heads      one thread per (row, head); neighbouring threads touch neighbouring heads
+// The row stays in L1/L2 between the max, sum and write passes, so HBM sees one read and one
+// write per element.
+#include <float.h>
+
+#include "elementwise.h"
+
+namespace kai {
+
+constexpr int kTB = 256;
+
+__device__ __forceinline__ float wmax(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float wsum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// ---- mask -------------------------------------------------------------------------------------
+
+__global__ void __launch_bounds__(kTB) attention_mask_kernel(float* __restrict__ pp, int64_t total, int64_t ntimes,
+                                                             int64_t nhead, int forward) {
+    const int64_t stride = (int64_t)gridDim.x * kTB;
+    const float fillv = forward ? -INFINITY : 0.f;
+    for (int64_t n = (int64_t)blockIdx.x * kTB + threadIdx.x; n < total; n += stride) {
+        const int64_t nq = n / (ntimes * nhead) % ntimes;
+        const int64_t nk = n / nhead % ntimes;
+        if (nq < nk) pp[n] = fillv;
+    }
+}
+
+int launch_attention_mask(float* pp, int64_t ndat, int64_t ntimes, int64_t nhead, int forward, hipStream_t stream) {
+    const int64_t total = ndat * ntimes * ntimes * nhead;
+    if (total <= 0) return KAI_OK;
+    int64_t blocks = (total + kTB - 1) / kTB;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    attention_mask_kernel<<<dim3((unsigned)blocks), kTB, 0, stream>>>(pp, total, ntimes, nhead, forward);
+    return check_launch("attention_mask_kernel");
+}
+
+// ---- softmax over the middle axis ---------------------------------------------------------------
+// BACKWARD = false: p <- softmax(p) in place.
+// BACKWARD = true : g <- coef * p * (g - sum_k p*g) in place on g.
+
+template <bool BACKWARD>
+__global__ void __launch_bounds__(kTB) softmax_axis_wave_kernel(float* __restrict__ io, const float* __restrict__ pp,
+                                                                int64_t nrow, int64_t nvec,
+                                                                const float* __restrict__ hcoef) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (kTB / 64) + (threadIdx.x >> 6);
+    if (row >= nrow) return;
+    float* __restrict__ r = io + row * nvec;
+    if (!BACKWARD) {
+        float mx = -FLT_MAX;
+        for (int64_t v = lane; v < nvec; v += 64) mx = fmaxf(mx, r[v]);
+        mx = wmax(mx);
+        float sum = 0.f;
+        for (int64_t v = lane; v < nvec; v += 64) sum += expf(r[v] - mx);
+        sum = wsum(sum);
+        for (int64_t v = lane; v < nvec; v += 64) r[v] = expf(r[v] - mx) / sum;
+    } else {
+        const float coef = hcoef ? *hcoef : 0.f;
+        const float* __restrict__ p = pp + row * nvec;
+        float dot = 0.f;
+        for (int64_t v = lane; v < nvec; v += 64) dot += p[v] * r[v];
+        dot = wsum(dot);
+        for (int64_t v = lane; v < nvec; v += 64) r[v] = coef * p[v] * (r[v] - dot);
+    }
+}
+
+template <bool BACKWARD>
+__global__ void __launch_bounds__(kTB) softmax_axis_block_kernel(float* __restrict__ io,
+                                                                 const float* __restrict__ pp, int64_t nvec,
+                                                                 int ncol, int tb, const float* __restrict__ hcoef) {
+    __shared__ float red[kTB];
+    const int t = threadIdx.x;
+    const int64_t len = nvec * ncol;
+    float* __restrict__ r = io + (int64_t)blockIdx.x * len;
+    const bool active = t < tb;   // tb = ncol * floor(kTB / ncol): a thread keeps one head
+    const int c = t % ncol;
+
+    // folds the per-thread values of all threads that own head c, in thread order
+    auto fold = [&](float mine, bool is_max) -> float {
+        __syncthreads();
+        red[t] = mine;
+        __syncthreads();
+        float a = is_max ? -FLT_MAX : 0.f;
+        for (int u = c; u < tb; u += ncol) a = is_max ? fmaxf(a, red[u]) : a + red[u];
+        return a;
+    };
+
+    if (!BACKWARD) {
+        float mx = -FLT_MAX;
+        if (active)
+            for (int64_t e = t; e < len; e += tb) mx = fmaxf(mx, r[e]);
+        mx = fold(mx, true);
+        float sum = 0.f;
+        if (active)
+            for (int64_t e = t; e < len; e += tb) sum += expf(r[e] - mx);
+        sum = fold(sum, false);
+        if (active)
+            for (int64_t e = t; e < len; e += tb) r[e] = expf(r[e] - mx) / sum;
+    } else {
+        const float coef = hcoef ? *hcoef : 0.f;
+        const float* __restrict__ p = pp + (int64_t)blockIdx.x * len;
+        float dot = 0.f;
+        if (active)
+            for (int64_t e = t; e < len; e += tb) dot += p[e] * r[e];
+        dot = fold(dot, false);
+        if (active)
+            for (int64_t e = t; e < len; e += tb) r[e] = coef * p[e] * (r[e] - dot);
+    }
+}
+
+template <bool BACKWARD>
+__global__ void __launch_bounds__(kTB) softmax_axis_thread_kernel(float* __restrict__ io,
+                                                                  const float* __restrict__ pp, int64_t nrow,
+                                                                  int64_t nvec, int64_t ncol,
+                                                                  const float* __restrict__ hcoef) {
+    const int64_t n = (int64_t)blockIdx.x * kTB + threadIdx.x;
+    if (n >= nrow * ncol) return;
+    const int64_t base = (n / ncol) * nvec * ncol + n % ncol;
+    float* __restrict__ r = io + base;
+    if (!BACKWARD) {
+        float mx = -FLT_MAX;
+        for (int64_t v = 0; v < nvec; v++) mx = fmaxf(mx, r[v * ncol]);
+        float sum = 0.f;
+        for (int64_t v = 0; v < nvec; v++) sum += expf(r[v * ncol] - mx);
+        for (int64_t v = 0; v < nvec; v++) r[v * ncol] = expf(r[v * ncol] - mx) / sum;
+    } else {
+        const float coef = hcoef ? *hcoef : 0.f;
+        const float* __restrict__ p = pp + base;
+        float dot = 0.f;
+        for (int64_t v = 0; v < nvec; v++) dot += p[v * ncol] * r[v * ncol];
+        for (int64_t v = 0; v < nvec; v++) r[v * ncol] = coef * p[v * ncol] * (r[v * ncol] - dot);
+    }
+}
+
+template <bool BACKWARD>
+static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, int64_t nvec, int64_t ncol,
+                                    const float* hcoef, hipStream_t stream) {
+    if (nrow <= 0 || nvec <= 0 || ncol <= 0) return KAI_OK;
+    if (ncol == 1) {
+        const int64_t blocks = (nrow + kTB / 64 - 1) / (kTB / 64);
+        if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "softmax_direct_on_axis: too many rows");
+        softmax_axis_wave_kernel<BACKWARD><<<dim3((unsigned)blocks), kTB, 0, stream>>>(io, pp, nrow, nvec, hcoef);
+    } else if (ncol <= 128) {
+        if (nrow > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "softmax_direct_on_axis: too many rows");
+        const int tb = (int)ncol * (kTB / (int)ncol);
+        softmax_axis_block_kernel<BACKWARD><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol, tb,
+                                                                                     hcoef);
+    } else {
+        const int64_t blocks = (nrow * ncol + kTB - 1) / kTB;
+        if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "softmax_direct_on_axis: too many rows");
+        softmax_axis_thread_kernel<BACKWARD><<<dim3((unsigned)blocks), kTB, 0, stream>>>(io, pp, nrow, nvec, ncol,
+                                                                                        hcoef);
+    }
+    return check_launch("softmax_axis_kernel");
+}
+
+int launch_softmax_axis(float* pp, int64_t nrow, int64_t nvec, int64_t ncol, hipStream_t stream) {
+    return launch_softmax_axis_impl<false>(pp, nullptr, nrow, nvec, ncol, nullptr, stream);
+}
+
+int launch_softmax_axis_backward(float* pgp, const float* pp, int64_t nrow, int64_t nvec, int64_t ncol,
+                                 const float* hcoef, hipStream_t stream) {
+    return launch_softmax_axis_impl<true>(pgp, pp, nrow, nvec, ncol, hcoef, stream);
+}
+
+}  // namespace kai

@@ -1,0 +1,27 @@
+// Launchers of the bandwidth-bound kernels in elementwise.hip and attention_ops.hip.
+#pragma once
+
+#include "kai_common.h"
+
+namespace kai {
+
+int launch_add_bias(float* y, const float* a, const float* b, int64_t nrow, int64_t ncol, hipStream_t stream);
+int launch_colsum(float* gb, const float* gy, int64_t nrow, int64_t ncol, int acc, hipStream_t stream);
+int launch_activate(float* y, const float* x, int64_t total, int act, const float* hleaky, hipStream_t stream);
+int launch_activate_backward(float* gx, const float* gy, const float* x, int64_t total, int act, const float* hleaky,
+                             hipStream_t stream);
+int launch_activate_backward_with_y(float* gx, const float* gy, const float* y, int64_t total, int act,
+                                    const float* hleaky, hipStream_t stream);
+int launch_softmax_rows(float* y, const float* x, int64_t nrow, int64_t ncol, hipStream_t stream);
+int launch_softmax_rows_backward(float* gx, const float* gy, const float* x, int64_t nrow, int64_t ncol,
+                                 hipStream_t stream);
+int launch_fill_float(float* p, int64_t n, float value, hipStream_t stream);
+int launch_fill_int(int* p, int64_t n, int value, hipStream_t stream);
+
+// attention_ops.hip
+int launch_attention_mask(float* pp, int64_t ndat, int64_t ntimes, int64_t nhead, int forward, hipStream_t stream);
+int launch_softmax_axis(float* pp, int64_t nrow, int64_t nvec, int64_t ncol, hipStream_t stream);
+int launch_softmax_axis_backward(float* pgp, const float* pp, int64_t nrow, int64_t nvec, int64_t ncol,
+                                 const float* hcoef, hipStream_t stream);
+
+}  // namespace kai

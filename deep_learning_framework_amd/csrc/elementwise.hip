@@ -1,0 +1,247 @@
+// Bandwidth-bound companions of the dense layer: bias add, bias gradient (column sum),
+// activations and their derivatives, fills.  Reference: VMath::add_bias /
+// add_bias_backward_b (vmath.cu:875-932), activate / activate_backward /
+// activate_backward_with_y (vmath.cu:3097-3486), fill_int / fill_float (vmath.cu:494-530).
+//
+// All kernels are grid-stride streams with 128-bit accesses when the buffers allow it.
+#include "elementwise.h"
+
+#include <float.h>
+
+#include "act_funcs.h"
+
+namespace kai {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kEwThreads = 256;
+constexpr int kMaxBlocks = 256 * 16;   // 16 workgroups per CU keep every CU's queues full
+
+static unsigned blocks_for(int64_t work_items) {
+    int64_t b = (work_items + kEwThreads - 1) / kEwThreads;
+    if (b < 1) b = 1;
+    if (b > kMaxBlocks) b = kMaxBlocks;
+    return (unsigned)b;
+}
+
+// ---- add_bias ---------------------------------------------------------------------------------
+
+template <bool VEC>
+__global__ void __launch_bounds__(kEwThreads) add_bias_kernel(float* y, const float* a,
+                                                              const float* __restrict__ b, int64_t total,
+                                                              int64_t ncol) {
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    if (VEC) {
+        const int64_t nvec = total / 4;   // ncol % 4 == 0, so a chunk never crosses a row
+        for (; i < nvec; i += stride) {
+            const int64_t e = i * 4;
+            const int64_t c = e % ncol;
+            const f32x4 va = *reinterpret_cast<const f32x4*>(a + e);
+            const f32x4 vb = *reinterpret_cast<const f32x4*>(b + c);
+            *reinterpret_cast<f32x4*>(y + e) = va + vb;
+        }
+    } else {
+        for (; i < total; i += stride) y[i] = a[i] + b[i % ncol];
+    }
+}
+
+int launch_add_bias(float* y, const float* a, const float* b, int64_t nrow, int64_t ncol, hipStream_t stream) {
+    const int64_t total = nrow * ncol;
+    if (total <= 0) return KAI_OK;
+    const bool vec = ncol % 4 == 0 && aligned16(y) && aligned16(a) && aligned16(b);
+    if (vec)
+        add_bias_kernel<true><<<blocks_for(total / 4), kEwThreads, 0, stream>>>(y, a, b, total, ncol);
+    else
+        add_bias_kernel<false><<<blocks_for(total), kEwThreads, 0, stream>>>(y, a, b, total, ncol);
+    return check_launch("add_bias_kernel");
+}
+
+// ---- add_bias_backward_b: gb[c] (=|+=) sum_r gy[r,c] -------------------------------------------
+//
+// One workgroup owns a panel of 32 columns (one 128-byte line per row) and all rows: thread
+// (ty, tx) sums rows ty, ty+32, ... of column tx, then the 32 partial sums of a column are
+// folded through LDS in a fixed order, so the result does not depend on scheduling.
+
+constexpr int kColsumCols = 32;
+constexpr int kColsumRows = 32;
+
+__global__ void __launch_bounds__(kColsumCols* kColsumRows)
+    colsum_kernel(float* __restrict__ gb, const float* __restrict__ gy, int64_t nrow, int64_t ncol, int acc) {
+    __shared__ float part[kColsumRows][kColsumCols + 1];
+    const int tx = threadIdx.x % kColsumCols;
+    const int ty = threadIdx.x / kColsumCols;
+    const int64_t c = (int64_t)blockIdx.x * kColsumCols + tx;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    if (c < ncol) {
+        const float* __restrict__ p = gy + c;
+        int64_t r = ty;
+        for (; r + 3 * kColsumRows < nrow; r += 4 * kColsumRows) {
+            s0 += p[r * ncol];
+            s1 += p[(r + kColsumRows) * ncol];
+            s2 += p[(r + 2 * kColsumRows) * ncol];
+            s3 += p[(r + 3 * kColsumRows) * ncol];
+        }
+        for (; r < nrow; r += kColsumRows) s0 += p[r * ncol];
+    }
+    part[ty][tx] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (ty == 0 && c < ncol) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < kColsumRows; i++) s += part[i][tx];
+        if (acc) s += gb[c];
+        gb[c] = s;
+    }
+}
+
+int launch_colsum(float* gb, const float* gy, int64_t nrow, int64_t ncol, int acc, hipStream_t stream) {
+    if (ncol <= 0) return KAI_OK;
+    const int64_t blocks = (ncol + kColsumCols - 1) / kColsumCols;
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "add_bias_backward_b: too many columns");
+    colsum_kernel<<<dim3((unsigned)blocks), dim3(kColsumCols * kColsumRows), 0, stream>>>(gb, gy, nrow, ncol, acc);
+    return check_launch("colsum_kernel");
+}
+
+// ---- element-wise activations -------------------------------------------------------------------
+
+// MODE 0: y = f(x);  MODE 1: gx = f'(x) * gy;  MODE 2: gx = f'(y) * gy (derivative from the output)
+template <int MODE, bool VEC>
+__global__ void __launch_bounds__(kEwThreads) act_kernel(float* out, const float* g,
+                                                         const float* in, int64_t total, int act,
+                                                         const float* __restrict__ hleaky) {
+    const float leaky = hleaky ? *hleaky : 0.f;
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+    auto f = [&](float x, float gy) -> float {
+        if (MODE == 0) return apply_act(x, act, leaky);
+        if (MODE == 1) return act_derivative(x, act, leaky) * gy;
+        return act_derivative_from_y(x, act, leaky) * gy;
+    };
+    if (VEC) {
+        const int64_t nvec = total / 4;
+        for (; i < nvec; i += stride) {
+            const f32x4 x = *reinterpret_cast<const f32x4*>(in + i * 4);
+            f32x4 gy = {0.f, 0.f, 0.f, 0.f};
+            if (MODE != 0) gy = *reinterpret_cast<const f32x4*>(g + i * 4);
+            f32x4 o;
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[j] = f(x[j], gy[j]);
+            *reinterpret_cast<f32x4*>(out + i * 4) = o;
+        }
+        // tail (total % 4 elements)
+        const int64_t t = nvec * 4 + (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+        if (t < total) out[t] = f(in[t], MODE != 0 ? g[t] : 0.f);
+    } else {
+        for (; i < total; i += stride) out[i] = f(in[i], MODE != 0 ? g[i] : 0.f);
+    }
+}
+
+template <int MODE>
+static int launch_act_mode(float* out, const float* g, const float* in, int64_t total, int act, const float* hleaky,
+                           hipStream_t stream) {
+    if (total <= 0) return KAI_OK;
+    const bool vec = aligned16(out) && aligned16(in) && (MODE == 0 || aligned16(g)) && total >= 4;
+    if (vec)
+        act_kernel<MODE, true><<<blocks_for(total / 4), kEwThreads, 0, stream>>>(out, g, in, total, act, hleaky);
+    else
+        act_kernel<MODE, false><<<blocks_for(total), kEwThreads, 0, stream>>>(out, g, in, total, act, hleaky);
+    return check_launch("act_kernel");
+}
+
+int launch_activate(float* y, const float* x, int64_t total, int act, const float* hleaky, hipStream_t stream) {
+    return launch_act_mode<0>(y, nullptr, x, total, act, hleaky, stream);
+}
+int launch_activate_backward(float* gx, const float* gy, const float* x, int64_t total, int act, const float* hleaky,
+                             hipStream_t stream) {
+    return launch_act_mode<1>(gx, gy, x, total, act, hleaky, stream);
+}
+int launch_activate_backward_with_y(float* gx, const float* gy, const float* y, int64_t total, int act,
+                                    const float* hleaky, hipStream_t stream) {
+    return launch_act_mode<2>(gx, gy, y, total, act, hleaky, stream);
+}
+
+// ---- softmax as an activation (row of ncol contiguous elements) ---------------------------------
+//
+// One wave per row.  Forward: y = exp(x - max) / sum.  Backward (device twin of the reference,
+// vmath.cu:3363-3394): gx_i = y_i * (gy_i - sum_j y_j gy_j), written there as
+// sum_j (delta_ij y_i - y_i y_j) gy_j.
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_add(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+template <bool BACKWARD>
+__global__ void __launch_bounds__(kEwThreads) softmax_rows_kernel(float* __restrict__ out,
+                                                                  const float* __restrict__ gy,
+                                                                  const float* __restrict__ x, int64_t nrow,
+                                                                  int64_t ncol) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
+    if (row >= nrow) return;
+    const float* __restrict__ xr = x + row * ncol;
+    float mx = -FLT_MAX;
+    for (int64_t c = lane; c < ncol; c += 64) mx = fmaxf(mx, xr[c]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int64_t c = lane; c < ncol; c += 64) sum += expf(xr[c] - mx);
+    sum = wave_add(sum);
+    if (!BACKWARD) {
+        for (int64_t c = lane; c < ncol; c += 64) out[row * ncol + c] = expf(xr[c] - mx) / sum;
+    } else {
+        const float* __restrict__ gr = gy + row * ncol;
+        float dot = 0.f;
+        for (int64_t c = lane; c < ncol; c += 64) dot += (expf(xr[c] - mx) / sum) * gr[c];
+        dot = wave_add(dot);
+        for (int64_t c = lane; c < ncol; c += 64) {
+            const float yi = expf(xr[c] - mx) / sum;
+            out[row * ncol + c] = yi * gr[c] - yi * dot;
+        }
+    }
+}
+
+int launch_softmax_rows(float* y, const float* x, int64_t nrow, int64_t ncol, hipStream_t stream) {
+    if (nrow <= 0 || ncol <= 0) return KAI_OK;
+    const int64_t blocks = (nrow + kEwThreads / 64 - 1) / (kEwThreads / 64);
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "activate(softmax): too many rows");
+    softmax_rows_kernel<false><<<dim3((unsigned)blocks), kEwThreads, 0, stream>>>(y, nullptr, x, nrow, ncol);
+    return check_launch("softmax_rows_kernel");
+}
+
+int launch_softmax_rows_backward(float* gx, const float* gy, const float* x, int64_t nrow, int64_t ncol,
+                                 hipStream_t stream) {
+    if (nrow <= 0 || ncol <= 0) return KAI_OK;
+    const int64_t blocks = (nrow + kEwThreads / 64 - 1) / (kEwThreads / 64);
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "activate_backward(softmax): too many rows");
+    softmax_rows_kernel<true><<<dim3((unsigned)blocks), kEwThreads, 0, stream>>>(gx, gy, x, nrow, ncol);
+    return check_launch("softmax_rows_kernel");
+}
+
+// ---- fills ----------------------------------------------------------------------------------------
+
+template <typename T>
+__global__ void __launch_bounds__(kEwThreads) fill_kernel(T* __restrict__ p, int64_t n, T value) {
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) p[i] = value;
+}
+
+int launch_fill_float(float* p, int64_t n, float value, hipStream_t stream) {
+    if (n <= 0) return KAI_OK;
+    fill_kernel<float><<<blocks_for(n), kEwThreads, 0, stream>>>(p, n, value);
+    return check_launch("fill_kernel");
+}
+
+int launch_fill_int(int* p, int64_t n, int value, hipStream_t stream) {
+    if (n <= 0) return KAI_OK;
+    fill_kernel<int><<<blocks_for(n), kEwThreads, 0, stream>>>(p, n, value);
+    return check_launch("fill_kernel");
+}
+
+}  // namespace kai

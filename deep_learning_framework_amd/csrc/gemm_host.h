@@ -1,0 +1,84 @@
+// Host-side description of one (batched) GEMM and the launcher of one kernel
+// configuration.  Used by gemm_dispatch.hip, which picks the configuration.
+#pragma once
+
+#include "gemm_mfma.h"
+#include "kai_common.h"
+
+namespace kai {
+
+// C(m,n) (=|+=) act(alpha * sum_k A(m,k)*B(n,k) + bias[n]) with arbitrary element strides.
+struct GemmDesc {
+    const float* A = nullptr;
+    const float* B = nullptr;
+    float* C = nullptr;
+    float* C2 = nullptr;
+    const float* bias = nullptr;
+    const float* alpha = nullptr;
+    const float* leaky = nullptr;
+    int64_t M = 0, N = 0, K = 0;
+    int64_t a_rs = 0, a_ks = 1, b_rs = 0, b_ks = 1, c_rs = 0, c_cs = 1;
+    int64_t nbatch = 1, bdiv = 1;
+    int64_t a_bs0 = 0, a_bs1 = 0, b_bs0 = 0, b_bs1 = 0, c_bs0 = 0, c_bs1 = 0;
+    int act = 0;
+    int acc = 0;
+    int has_alpha = 0;
+};
+
+// LDS orientation of an operand: reduction index contiguous (KC) or output index contiguous (MC).
+// A strided operand (neither stride is 1) goes to the orientation of its smaller stride.
+inline bool operand_is_kc(int64_t rs, int64_t ks) { return ks == 1 || (rs != 1 && ks <= rs); }
+
+inline GemmParams make_params(const GemmDesc& d, bool a_kc, bool b_kc) {
+    GemmParams p{};
+    p.A = d.A; p.B = d.B; p.C = d.C; p.C2 = d.C2; p.bias = d.bias; p.alpha = d.alpha; p.leaky = d.leaky;
+    p.M = (int)d.M; p.N = (int)d.N; p.K = (int)d.K;
+    p.a_rs = d.a_rs; p.a_ks = d.a_ks; p.b_rs = d.b_rs; p.b_ks = d.b_ks; p.c_rs = d.c_rs; p.c_cs = d.c_cs;
+    p.a_bs0 = d.a_bs0; p.a_bs1 = d.a_bs1; p.b_bs0 = d.b_bs0; p.b_bs1 = d.b_bs1; p.c_bs0 = d.c_bs0; p.c_bs1 = d.c_bs1;
+    p.bdiv = (int)d.bdiv;
+    // 128-bit loads need: unit stride along the LDS-contiguous index, the other stride and every
+    // batch stride a multiple of 4 elements, and a 16-byte aligned base
+    const int64_t a_cont = a_kc ? d.a_ks : d.a_rs, a_ld = a_kc ? d.a_rs : d.a_ks;
+    const int64_t b_cont = b_kc ? d.b_ks : d.b_rs, b_ld = b_kc ? d.b_rs : d.b_ks;
+    p.a_vec = a_cont == 1 && a_ld % 4 == 0 && d.a_bs0 % 4 == 0 && d.a_bs1 % 4 == 0 && aligned16(d.A);
+    p.b_vec = b_cont == 1 && b_ld % 4 == 0 && d.b_bs0 % 4 == 0 && d.b_bs1 % 4 == 0 && aligned16(d.B);
+    p.c_vec = d.c_cs == 1 && d.c_rs % 4 == 0 && d.N % 4 == 0 && d.c_bs0 % 4 == 0 && d.c_bs1 % 4 == 0 &&
+              aligned16(d.C) && (d.C2 == nullptr || aligned16(d.C2));
+    p.act = d.act;
+    p.accflag = d.acc;
+    p.has_alpha = d.has_alpha;
+    return p;
+}
+
+// true when the predicate-free kernel variant may run this problem with tile BM x BN x BK
+inline bool fits_without_edges(const GemmParams& p, bool a_kc, bool b_kc, int BM, int BN, int BK) {
+    const int64_t a_ld = a_kc ? p.a_rs : p.a_ks, b_ld = b_kc ? p.b_rs : p.b_ks;
+    return p.a_vec && p.b_vec && p.M % BM == 0 && p.N % BN == 0 && p.K % BK == 0 && p.K > 0 &&
+           a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30);
+}
+
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE>
+int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t stream) {
+    constexpr int BM = WM * NBM * 32, BN = WN * NBN * 32;
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    p.group_m = group_m < 1 ? 1 : group_m;
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    if (tiles <= 0 || nbatch <= 0) return KAI_OK;
+    if (tiles > kMaxDim || nbatch > 65535) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
+    dim3 grid((unsigned)tiles, 1, (unsigned)nbatch);
+    gemm_mfma_kernel<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE><<<grid, dim3(64 * WM * WN), 0, stream>>>(p);
+    return check_launch("gemm_mfma_kernel");
+}
+
+// picks kernel family, tile and variant; defined in gemm_dispatch.hip
+int launch_gemm(const GemmDesc& d, hipStream_t stream);
+
+// per-layout entry points (one translation unit each, to compile in parallel)
+enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2 };
+int launch_gemm_kc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
+int launch_gemm_kc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
+int launch_gemm_mc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
+int launch_gemm_mc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
+
+}  // namespace kai

@@ -1,0 +1,366 @@
+// fp32 MFMA GEMM for gfx950 (MI355X): C[M,N] (=|+=) act(alpha * A.B + bias)
+//
+// One kernel template covers the three operand forms of the engine's dense layer
+// (VMath::matmul / matmul_backward_x / matmul_backward_w, vmath.cu:2961-3093 of the
+// reference) and the strided, batched products of its attention layer
+// (mult_on_heads / mix_values and their backward twins, vmath.cu:6729-7129)
+// without ever materialising a transpose:
+//
+//  * Each operand tile is staged in LDS in the orientation in which it is
+//    contiguous in global memory: "KC" = [rows][BK+4] when the reduction index is
+//    contiguous, "MC" = [BK][rows+4] when the output index is.  Both orientations
+//    are read back with 128-bit LDS loads.  A KC read hands a lane four
+//    consecutive k of one row (used by four successive MFMAs); an MC read hands a
+//    lane one k of four consecutive rows (used by the four 32-row MFMA blocks of
+//    the wave).  The k-slot a lane feeds is the same for both operands:
+//        k = 8*group + 4*(lane/32) + step,    step = 0..3
+//    so products always pair equal k, whatever the orientation mix.
+//  * v_mfma_f32_32x32x2_f32: every wave owns NBM x NBN blocks of 32x32 outputs held
+//    in accumulator registers (16 per lane per block).
+//  * Global -> register -> LDS staging, double buffered: the loads of tile t+1 are
+//    in flight while the MFMAs of tile t run; one barrier per K-tile.
+//  * Interior blocks with 16-byte aligned operands take a predicate-free 128-bit
+//    load path; edge blocks, ragged K and unaligned or strided operands take a
+//    predicated path (vector where a whole chunk is valid and aligned, scalar
+//    otherwise) that writes zeros into LDS outside the matrix.
+//  * Workgroup ids are remapped so that the workgroups that share one XCD (and its
+//    L2) cover a compact patch of C.
+//  * Epilogue in registers: alpha, C += (acc), bias add, optional store of the
+//    pre-activation, activation, store (128-bit stores when the B operand is MC).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "act_funcs.h"
+
+namespace kai {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct GemmParams {
+    const float* A;
+    const float* B;
+    float* C;
+    float* C2;            // optional second output: value before the activation
+    const float* bias;    // optional, indexed by output column
+    const float* alpha;   // optional device scalar multiplied into the product (null pointer semantics in has_alpha)
+    const float* leaky;   // optional device scalar for leaky relu
+    int M, N, K;
+    int64_t a_rs, a_ks;   // A(m,k) = A[m*a_rs + k*a_ks]
+    int64_t b_rs, b_ks;   // B(n,k) = B[n*b_rs + k*b_ks]
+    int64_t c_rs, c_cs;   // C(m,n) = C[m*c_rs + n*c_cs]
+    // batch z = blockIdx.z is split as (z / bdiv, z % bdiv); offset = q*bs0 + r*bs1
+    int64_t a_bs0, a_bs1, b_bs0, b_bs1, c_bs0, c_bs1;
+    int bdiv;
+    int a_vec, b_vec, c_vec;  // 128-bit access along the contiguous index is legal
+    int act;
+    int accflag;
+    int has_alpha;        // 1: multiply by (*alpha, or 0 if alpha is null)
+    int tiles_m, tiles_n;
+    int group_m;          // tile rows per column sweep of the XCD-local ordering
+};
+
+constexpr int kLdsPad = 4;
+
+template <bool KC, int ROWS, int BK>
+struct TileShape {
+    // KC: [ROWS][BK+pad], MC: [BK][ROWS+pad]
+    static constexpr int kStride = KC ? (BK + kLdsPad) : (ROWS + kLdsPad);
+    static constexpr int kFloats = KC ? ROWS * (BK + kLdsPad) : BK * (ROWS + kLdsPad);
+    static constexpr int kChunks = ROWS * BK / 4;
+    // chunk c -> (row, k) of its first element
+    static constexpr int kChunksPerLine = KC ? BK / 4 : ROWS / 4;
+};
+
+// Predicate-free load of one operand tile: every chunk is a 16-byte aligned float4 inside the matrix.
+// `base` (wave-uniform) points at element (row0, k0); `ld` is the stride of the non-contiguous index;
+// `toff` is the calling thread's element offset of its first chunk, line0*ld + off0, which does not
+// change along K.  Chunk i of a thread lies a uniform i*(NT/chunks-per-line)*ld further on, so the
+// address is a scalar base plus one 32-bit vector offset.
+template <bool KC, int ROWS, int BK, int NT>
+__device__ __forceinline__ void load_tile_fast(f32x4 (&reg)[ROWS * BK / 4 / NT], const float* __restrict__ base,
+                                               int64_t ld, uint32_t toff) {
+    using TS = TileShape<KC, ROWS, BK>;
+    constexpr int NCH = TS::kChunks / NT;
+    static_assert(NT % TS::kChunksPerLine == 0, "threads must cover whole lines");
+    constexpr int kLinesPerPass = NT / TS::kChunksPerLine;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const float* bi = base + (int64_t)(i * kLinesPerPass) * ld;
+        reg[i] = *reinterpret_cast<const f32x4*>(bi + toff);
+    }
+}
+
+// Predicated load: rows_left / k_left are the numbers of valid rows / k from the tile origin.
+// rs / ks are the element strides of the row index and the reduction index.
+template <bool KC, int ROWS, int BK, int NT>
+__device__ __forceinline__ void load_tile_edge(f32x4 (&reg)[ROWS * BK / 4 / NT], const float* __restrict__ base,
+                                               int64_t rs, int64_t ks, int rows_left, int k_left, int vec_ok,
+                                               int tid) {
+    using TS = TileShape<KC, ROWS, BK>;
+    constexpr int NCH = TS::kChunks / NT;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * NT;
+        const int line = c / TS::kChunksPerLine;
+        const int off = (c % TS::kChunksPerLine) * 4;
+        const int r = KC ? line : off;   // first row of the chunk
+        const int k = KC ? off : line;   // first k of the chunk
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (KC) {
+            if (r < rows_left) {
+                const float* p = base + (int64_t)r * rs + (int64_t)k * ks;
+                if (vec_ok && k + 3 < k_left) {
+                    v = *reinterpret_cast<const f32x4*>(p);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (k + j < k_left) v[j] = p[(int64_t)j * ks];
+                }
+            }
+        } else {
+            if (k < k_left) {
+                const float* p = base + (int64_t)r * rs + (int64_t)k * ks;
+                if (vec_ok && r + 3 < rows_left) {
+                    v = *reinterpret_cast<const f32x4*>(p);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (r + j < rows_left) v[j] = p[(int64_t)j * rs];
+                }
+            }
+        }
+        reg[i] = v;
+    }
+}
+
+template <bool KC, int ROWS, int BK, int NT>
+__device__ __forceinline__ void store_tile_lds(float* __restrict__ lds, const f32x4 (&reg)[ROWS * BK / 4 / NT],
+                                               int tid) {
+    using TS = TileShape<KC, ROWS, BK>;
+    constexpr int NCH = TS::kChunks / NT;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * NT;
+        const int line = c / TS::kChunksPerLine;
+        const int off = (c % TS::kChunksPerLine) * 4;
+        *reinterpret_cast<f32x4*>(lds + line * TS::kStride + off) = reg[i];
+    }
+}
+
+// Fragments of one operand for one group of 8 k (4 MFMA steps), NB 32-row blocks.
+template <bool KC, int NB>
+struct Frag {
+    // KC: v[b] holds k-steps 0..3 of block b.  MC: v[t][b] holds block b of step t.
+    f32x4 v[KC ? NB : 4];
+    __device__ __forceinline__ float get(int b, int t) const { return KC ? v[b][t] : v[t][b]; }
+};
+
+template <bool KC, int NB, int ROWS, int BK>
+__device__ __forceinline__ void read_frag(Frag<KC, NB>& f, const float* __restrict__ lds, int w_r0, int kg, int l32,
+                                          int half) {
+    using TS = TileShape<KC, ROWS, BK>;
+    if (KC) {
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+            f.v[b] = *reinterpret_cast<const f32x4*>(lds + (w_r0 + 32 * b + l32) * TS::kStride + kg * 8 + 4 * half);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const float* p = lds + (kg * 8 + 4 * half + t) * TS::kStride + w_r0 + NB * l32;
+            if (NB == 4) {
+                f.v[t] = *reinterpret_cast<const f32x4*>(p);
+            } else if (NB == 2) {
+                const f32x2 q = *reinterpret_cast<const f32x2*>(p);
+                f.v[t][0] = q[0];
+                f.v[t][1] = q[1];
+            } else {
+                f.v[t][0] = p[0];
+            }
+        }
+    }
+}
+
+// Workgroup id -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin over
+// the 8 XCDs; ids congruent mod 8 therefore share an L2.  They are renumbered so that each XCD
+// walks a contiguous run of tiles, and the run is ordered in column sweeps of `group_m` tile rows
+// so that tiles that are live together share A row panels and B column panels.
+__device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    int id = bid;
+    if ((total & 7) == 0) id = (bid & 7) * (total >> 3) + (bid >> 3);
+    const int per_group = group_m * tiles_n;
+    const int g = id / per_group;
+    const int first_m = g * group_m;
+    const int rows = min(group_m, tiles_m - first_m);
+    const int in_g = id - g * per_group;
+    tm = first_m + in_g % rows;
+    tn = in_g / rows;
+}
+
+// EDGE = false: the host has checked that M, N, K are multiples of the tile, that both operands
+// allow aligned 128-bit loads and that a tile's offsets fit 32 bits; the kernel then holds no
+// predicated load code at all (fewer registers).  EDGE = true: general shapes.
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE>
+__global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const GemmParams p) {
+    constexpr int NT = 64 * WM * WN;
+    constexpr int BM = WM * NBM * 32;
+    constexpr int BN = WN * NBN * 32;
+    using TA = TileShape<A_KC, BM, BK>;
+    using TB = TileShape<B_KC, BN, BK>;
+    constexpr int NCHA = TA::kChunks / NT;
+    constexpr int NCHB = TB::kChunks / NT;
+    static_assert(TA::kChunks % NT == 0 && TB::kChunks % NT == 0, "tile must divide over the threads");
+    static_assert(BK % 8 == 0, "BK must hold whole groups of 8 k");
+
+    __shared__ __attribute__((aligned(16))) float lds_a[2][TA::kFloats];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][TB::kFloats];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    const int wm0 = (wave / WN) * (NBM * 32);
+    const int wn0 = (wave % WN) * (NBN * 32);
+
+    int tm, tn;
+    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    const int m0 = tm * BM;
+    const int n0 = tn * BN;
+
+    const int z = blockIdx.z;
+    const int zq = z / p.bdiv, zr = z % p.bdiv;
+    const float* __restrict__ Ab = p.A + zq * p.a_bs0 + zr * p.a_bs1 + (int64_t)m0 * p.a_rs;
+    const float* __restrict__ Bb = p.B + zq * p.b_bs0 + zr * p.b_bs1 + (int64_t)n0 * p.b_rs;
+    const int64_t c_off = zq * p.c_bs0 + zr * p.c_bs1;
+
+    const int rows_a = p.M - m0;
+    const int rows_b = p.N - n0;
+    const int64_t a_ld = A_KC ? p.a_rs : p.a_ks;
+    const int64_t b_ld = B_KC ? p.b_rs : p.b_ks;
+    // fast path: whole tile inside the matrix, aligned, and 32-bit thread offsets
+    const bool interior = !EDGE || ((rows_a >= BM) && (rows_b >= BN) && p.a_vec && p.b_vec &&
+                                    a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30));
+    const uint32_t toff_a =
+        (uint32_t)(tid / TA::kChunksPerLine) * (uint32_t)a_ld + (uint32_t)(tid % TA::kChunksPerLine) * 4u;
+    const uint32_t toff_b =
+        (uint32_t)(tid / TB::kChunksPerLine) * (uint32_t)b_ld + (uint32_t)(tid % TB::kChunksPerLine) * 4u;
+
+    f32x16 acc[NBM][NBN];
+#pragma unroll
+    for (int i = 0; i < NBM; i++)
+#pragma unroll
+        for (int j = 0; j < NBN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    f32x4 ra[NCHA], rb[NCHB];
+    const int nkt = (p.K + BK - 1) / BK;
+
+    auto load_global = [&](int kt) {
+        const int k0 = kt * BK;
+        const int k_left = p.K - k0;
+        const float* ap = Ab + (int64_t)k0 * p.a_ks;
+        const float* bp = Bb + (int64_t)k0 * p.b_ks;
+        if (!EDGE || (interior && k_left >= BK)) {
+            load_tile_fast<A_KC, BM, BK, NT>(ra, ap, a_ld, toff_a);
+            load_tile_fast<B_KC, BN, BK, NT>(rb, bp, b_ld, toff_b);
+        } else {
+            load_tile_edge<A_KC, BM, BK, NT>(ra, ap, p.a_rs, p.a_ks, rows_a, k_left, p.a_vec, tid);
+            load_tile_edge<B_KC, BN, BK, NT>(rb, bp, p.b_rs, p.b_ks, rows_b, k_left, p.b_vec, tid);
+        }
+    };
+
+    if (nkt > 0) {
+        load_global(0);
+        store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
+        store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < nkt; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < nkt) load_global(kt + 1);
+
+        const float* la = lds_a[cur];
+        const float* lb = lds_b[cur];
+#pragma unroll
+        for (int kg = 0; kg < BK / 8; kg++) {
+            Frag<A_KC, NBM> fa;
+            Frag<B_KC, NBN> fb;
+            read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
+            read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int i = 0; i < NBM; i++)
+#pragma unroll
+                    for (int j = 0; j < NBN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(i, t), fb.get(j, t), acc[i][j], 0, 0, 0);
+        }
+
+        if (kt + 1 < nkt) {
+            store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], ra, tid);
+            store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rb, tid);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue ------------------------------------------------------------------------------
+    const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
+    const float leaky = p.leaky ? *p.leaky : 0.f;
+    float* __restrict__ C = p.C + c_off;
+    float* __restrict__ C2 = p.C2 ? p.C2 + c_off : nullptr;
+
+    auto finish = [&](float v, int col, int64_t idx) -> float {
+        if (p.has_alpha) v *= alpha;
+        if (p.accflag) v += C[idx];
+        if (p.bias) v += p.bias[col];
+        if (C2) C2[idx] = v;
+        return apply_act(v, p.act, leaky);
+    };
+
+#pragma unroll
+    for (int i = 0; i < NBM; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int mi = 8 * (r >> 2) + 4 * half + (r & 3);   // row inside the 32x32 block
+            const int row = m0 + (A_KC ? wm0 + 32 * i + mi : wm0 + NBM * mi + i);
+            if (row >= p.M) continue;
+            if (!B_KC && NBN == 4 && p.c_vec) {
+                const int col = n0 + wn0 + 4 * l32;
+                if (col < p.N) {   // N % 4 == 0 under c_vec, so the whole chunk is inside
+                    const int64_t idx = (int64_t)row * p.c_rs + col;
+                    f32x4 o;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float v = acc[i][j][r];
+                        if (p.has_alpha) v *= alpha;
+                        if (p.accflag) v += C[idx + j];
+                        if (p.bias) v += p.bias[col + j];
+                        o[j] = v;
+                    }
+                    if (C2) *reinterpret_cast<f32x4*>(C2 + idx) = o;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) o[j] = apply_act(o[j], p.act, leaky);
+                    *reinterpret_cast<f32x4*>(C + idx) = o;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NBN; j++) {
+                    const int col = n0 + (B_KC ? wn0 + 32 * j + l32 : wn0 + NBN * l32 + j);
+                    if (col < p.N) {
+                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
+                        C[idx] = finish(acc[i][j][r], col, idx);
+                    }
+                }
+            }
+        }
+    }
+}
+
+}  // namespace kai

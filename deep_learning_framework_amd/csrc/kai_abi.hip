@@ -1,0 +1,474 @@
+// extern "C" surface of libkai_hip.so (declared in include/kai_hip.h): argument checks, mapping
+// of the engine's VMath argument lists onto GEMM descriptors, library state.
+//
+// The mapping of (yvec, ndat, xvec) follows the call sites in the reference:
+// VTensor::matmul (api_objects/vtensor.cpp:1282-1335), matmul_backprop (:1337-1375),
+// mh_attention (:2978-3052) and multihead_attention_backprop (:3054-3227).
+#include <cstring>
+#include <cstdlib>
+
+#include "elementwise.h"
+#include "gemm_host.h"
+#include "kai_common.h"
+
+namespace kai {
+
+static thread_local std::string tl_error;
+static thread_local hipStream_t tl_stream = nullptr;
+
+int fail(int code, const std::string& msg) {
+    tl_error = msg;
+    return code;
+}
+void clear_error() { tl_error.clear(); }
+hipStream_t current_stream() { return tl_stream; }
+
+int check_hip(hipError_t st, const char* what) {
+    if (st == hipSuccess) return KAI_OK;
+    return fail(KAI_ERR_GPU, std::string("hip:") + what + ": " + hipGetErrorString(st));
+}
+
+int check_launch(const char* kernel_name) { return check_hip(hipGetLastError(), kernel_name); }
+
+static bool act_is_elementwise(int act) { return act >= KAI_ACT_NONE && act <= KAI_ACT_SWISH; }
+
+}  // namespace kai
+
+using namespace kai;
+
+#define KAI_REQUIRE_PTR(p) KAI_REQUIRE((p) != nullptr, KAI_ERR_INVALID_POINTER, "null pointer: " #p)
+#define KAI_REQUIRE_DIM(v) \
+    KAI_REQUIRE((v) >= 0 && (v) <= kMaxDim, KAI_ERR_INVALID_ARGUMENT, "dimension out of range: " #v)
+
+extern "C" {
+
+// ---- library state -----------------------------------------------------------------------------
+
+const char* kai_last_error(void) { return tl_error.c_str(); }
+
+int kai_device_count(int* count) {
+    KAI_REQUIRE_PTR(count);
+    return check_hip(hipGetDeviceCount(count), "hipGetDeviceCount");
+}
+
+int kai_set_device(int device) { return check_hip(hipSetDevice(device), "hipSetDevice"); }
+
+int kai_device_synchronize(void) { return check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
+
+int kai_set_stream(void* hip_stream) {
+    tl_stream = reinterpret_cast<hipStream_t>(hip_stream);
+    return KAI_OK;
+}
+
+int kai_arch_info(char* built_for, char* device_arch, int buflen) {
+    KAI_REQUIRE(buflen > 0, KAI_ERR_INVALID_ARGUMENT, "buflen <= 0");
+    if (built_for) {
+        std::strncpy(built_for, "gfx950", buflen - 1);
+        built_for[buflen - 1] = 0;
+    }
+    if (device_arch) {
+        int dev = 0;
+        KAI_TRY(check_hip(hipGetDevice(&dev), "hipGetDevice"));
+        hipDeviceProp_t prop;
+        KAI_TRY(check_hip(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties"));
+        std::strncpy(device_arch, prop.gcnArchName, buflen - 1);
+        device_arch[buflen - 1] = 0;
+    }
+    return KAI_OK;
+}
+
+// ---- memory ------------------------------------------------------------------------------------
+
+int kai_mem_alloc(int device, int64_t size, void** out_ptr) {
+    KAI_REQUIRE_PTR(out_ptr);
+    *out_ptr = nullptr;
+    KAI_REQUIRE(size >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (device < 0) {
+        void* p = std::malloc((size_t)(size > 0 ? size : 1));
+        if (!p) return fail(KAI_ERR_HOSTMEM_ALLOC_FAILURE, "kai_mem_alloc: host allocation failed");
+        *out_ptr = p;
+        return KAI_OK;
+    }
+    if (size % 16 != 0) size += 16 - size % 16;
+    if (size == 0) size = 16;
+    int old_device = 0;
+    KAI_TRY(check_hip(hipGetDevice(&old_device), "hipGetDevice"));
+    KAI_TRY(check_hip(hipSetDevice(device), "hipSetDevice"));
+    void* p = nullptr;
+    const hipError_t st = hipMalloc(&p, (size_t)size);
+    const hipError_t st2 = hipSetDevice(old_device);
+    KAI_TRY(check_hip(st, "hipMalloc"));
+    KAI_TRY(check_hip(st2, "hipSetDevice"));
+    if (!p) return fail(KAI_ERR_INVALID_POINTER, "kai_mem_alloc: hipMalloc returned null");
+    *out_ptr = p;
+    return KAI_OK;
+}
+
+int kai_mem_free(int device, void* ptr) {
+    if (device < 0) {
+        std::free(ptr);
+        return KAI_OK;
+    }
+    return check_hip(hipFree(ptr), "hipFree");
+}
+
+static int copy_blocking(void* d, const void* s, int64_t size, hipMemcpyKind kind, const char* what) {
+    KAI_REQUIRE(size >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (size == 0) return KAI_OK;
+    KAI_REQUIRE(d != nullptr && s != nullptr, KAI_ERR_INVALID_POINTER, "null pointer");
+    if (kind == hipMemcpyHostToHost) {
+        std::memcpy(d, s, (size_t)size);
+        return KAI_OK;
+    }
+    // ordered after the work already enqueued on this thread's stream, then blocks, like the
+    // reference's cudaMemcpy on the legacy stream
+    hipStream_t st = current_stream();
+    KAI_TRY(check_hip(hipMemcpyAsync(d, s, (size_t)size, kind, st), what));
+    return check_hip(hipStreamSynchronize(st), what);
+}
+
+int kai_memcpy_host_to_host(void* d, const void* s, int64_t size) {
+    return copy_blocking(d, s, size, hipMemcpyHostToHost, "memcpy_host_to_host");
+}
+int kai_memcpy_host_to_device(void* d, const void* s, int64_t size) {
+    return copy_blocking(d, s, size, hipMemcpyHostToDevice, "memcpy_host_to_device");
+}
+int kai_memcpy_device_to_host(void* d, const void* s, int64_t size) {
+    return copy_blocking(d, s, size, hipMemcpyDeviceToHost, "memcpy_device_to_host");
+}
+int kai_memcpy_device_to_device(void* d, const void* s, int64_t size) {
+    return copy_blocking(d, s, size, hipMemcpyDeviceToDevice, "memcpy_device_to_device");
+}
+
+int kai_copy_data(int dest_device, int src_device, void* py, const void* px, int64_t nbytes) {
+    if (dest_device < 0)
+        return src_device < 0 ? kai_memcpy_host_to_host(py, px, nbytes) : kai_memcpy_device_to_host(py, px, nbytes);
+    return src_device < 0 ? kai_memcpy_host_to_device(py, px, nbytes) : kai_memcpy_device_to_device(py, px, nbytes);
+}
+
+int kai_fill_int(int device, int* ptr, int64_t size, int value) {
+    KAI_REQUIRE(size >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (size == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(ptr);
+    if (device < 0) {
+        for (int64_t i = 0; i < size; i++) ptr[i] = value;
+        return KAI_OK;
+    }
+    return launch_fill_int(ptr, size, value, current_stream());
+}
+
+int kai_fill_float(int device, float* ptr, int64_t size, float value) {
+    KAI_REQUIRE(size >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (size == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(ptr);
+    if (device < 0) {
+        for (int64_t i = 0; i < size; i++) ptr[i] = value;
+        return KAI_OK;
+    }
+    return launch_fill_float(ptr, size, value, current_stream());
+}
+
+int kai_set_zero(int device, void* ptr, int64_t size) {
+    KAI_REQUIRE(size >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (size == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(ptr);
+    if (device < 0) {
+        std::memset(ptr, 0, (size_t)size);
+        return KAI_OK;
+    }
+    // a fill kernel rather than hipMemsetAsync, so that callers may capture the call in a graph
+    if (size % 4 == 0 && (reinterpret_cast<uintptr_t>(ptr) & 3u) == 0)
+        return launch_fill_int(static_cast<int*>(ptr), size / 4, 0, current_stream());
+    return check_hip(hipMemsetAsync(ptr, 0, (size_t)size, current_stream()), "hipMemsetAsync");
+}
+
+int kai_memcpy_from_host(int device, void* py, const void* px, int64_t size) {
+    return device < 0 ? kai_memcpy_host_to_host(py, px, size) : kai_memcpy_host_to_device(py, px, size);
+}
+int kai_memcpy_to_host(int device, void* py, const void* px, int64_t size) {
+    return device < 0 ? kai_memcpy_host_to_host(py, px, size) : kai_memcpy_device_to_host(py, px, size);
+}
+int kai_memcpy_to_device(int device, void* py, const void* px, int64_t size) {
+    return device < 0 ? kai_memcpy_host_to_device(py, px, size) : kai_memcpy_device_to_device(py, px, size);
+}
+int kai_get_slice(int device, void* py, const void* px, int64_t nbytes) {
+    return device < 0 ? kai_memcpy_host_to_device(py, px, nbytes) : kai_memcpy_device_to_device(py, px, nbytes);
+}
+
+// ---- dense layer -------------------------------------------------------------------------------
+
+int kai_gemm_f32(int device, int transA, int transB, int64_t M, int64_t N, int64_t K, const float* A, int64_t lda,
+                 const float* B, int64_t ldb, float* C, int64_t ldc, const float* bias, int actFunc,
+                 const float* hLeakyAlpha, int acc) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE_DIM(M); KAI_REQUIRE_DIM(N); KAI_REQUIRE_DIM(K);
+    KAI_REQUIRE(act_is_elementwise(actFunc), KAI_ERR_CONDITIONAL_STATEMENT, "activation code must be 0..8");
+    if (M == 0 || N == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(C);
+    if (K > 0) { KAI_REQUIRE_PTR(A); KAI_REQUIRE_PTR(B); }
+    KAI_REQUIRE(lda >= (transA ? M : K) && ldb >= (transB ? K : N) && ldc >= N, KAI_ERR_INVALID_ARGUMENT,
+                "leading dimension smaller than the row length");
+    KAI_REQUIRE(lda <= kMaxDim && ldb <= kMaxDim && ldc <= kMaxDim, KAI_ERR_INVALID_ARGUMENT,
+                "leading dimension out of range");
+    GemmDesc d;
+    d.A = A; d.B = B; d.C = C; d.bias = bias; d.leaky = hLeakyAlpha;
+    d.M = M; d.N = N; d.K = K;
+    if (transA) { d.a_rs = 1; d.a_ks = lda; } else { d.a_rs = lda; d.a_ks = 1; }
+    if (transB) { d.b_rs = ldb; d.b_ks = 1; } else { d.b_rs = 1; d.b_ks = ldb; }
+    d.c_rs = ldc; d.c_cs = 1;
+    d.act = actFunc; d.acc = acc != 0;
+    return launch_gemm(d, current_stream());
+}
+
+int kai_matmul(int device, float* py, const float* pw, const float* px, int64_t yvec, int64_t ndat, int64_t xvec,
+               int acc) {
+    // y[ndat,yvec] = x[ndat,xvec] . w[yvec,xvec]^T : A = x (K-contiguous), B = w stored [N,K]
+    return kai_gemm_f32(device, 0, 1, ndat, yvec, xvec, px, xvec, pw, xvec, py, yvec, nullptr, KAI_ACT_NONE, nullptr,
+                        acc);
+}
+
+int kai_matmul_backward_x(int device, float* pgx, const float* pgy, const float* pw, int64_t yvec, int64_t ndat,
+                          int64_t xvec, int acc) {
+    // gx[ndat,xvec] = gy[ndat,yvec] . w[yvec,xvec] : reduction over yvec, B = w stored [K,N]
+    return kai_gemm_f32(device, 0, 0, ndat, xvec, yvec, pgy, yvec, pw, xvec, pgx, xvec, nullptr, KAI_ACT_NONE,
+                        nullptr, acc);
+}
+
+int kai_matmul_backward_w(int device, float* pgw, const float* pgy, const float* px, int64_t yvec, int64_t ndat,
+                          int64_t xvec, int acc) {
+    // gw[yvec,xvec] = gy[ndat,yvec]^T . x[ndat,xvec] : reduction over ndat, A stored [K,M], B stored [K,N]
+    return kai_gemm_f32(device, 1, 0, yvec, xvec, ndat, pgy, yvec, px, xvec, pgw, xvec, nullptr, KAI_ACT_NONE,
+                        nullptr, acc);
+}
+
+int kai_add_bias(int device, float* py, const float* pa, const float* pb, int64_t nrow, int64_t ncol) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (nrow == 0 || ncol == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pa); KAI_REQUIRE_PTR(pb);
+    return launch_add_bias(py, pa, pb, nrow, ncol, current_stream());
+}
+
+int kai_add_bias_backward_b(int device, float* pgb, const float* pgy, int64_t nrow, int64_t ncol, int acc) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (ncol == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgb);
+    if (nrow > 0) KAI_REQUIRE_PTR(pgy);
+    return launch_colsum(pgb, pgy, nrow, ncol, acc != 0, current_stream());
+}
+
+int kai_activate(int device, float* py, const float* px, int64_t nrow, int64_t ncol, int actFunc,
+                 const float* hLeakyAlpha) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    KAI_REQUIRE(actFunc >= KAI_ACT_NONE && actFunc <= KAI_ACT_SOFTMAX, KAI_ERR_CONDITIONAL_STATEMENT,
+                "unknown activation code");
+    if (nrow == 0 || ncol == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(px);
+    if (actFunc == KAI_ACT_SOFTMAX) return launch_softmax_rows(py, px, nrow, ncol, current_stream());
+    return launch_activate(py, px, nrow * ncol, actFunc, hLeakyAlpha, current_stream());
+}
+
+int kai_activate_backward(int device, float* pgx, const float* pgy, const float* px, int64_t nrow, int64_t ncol,
+                          int actFunc, const float* hLeakyAlpha) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    KAI_REQUIRE(actFunc >= KAI_ACT_NONE && actFunc <= KAI_ACT_SOFTMAX, KAI_ERR_CONDITIONAL_STATEMENT,
+                "unknown activation code");
+    if (nrow == 0 || ncol == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgx); KAI_REQUIRE_PTR(pgy); KAI_REQUIRE_PTR(px);
+    if (actFunc == KAI_ACT_SOFTMAX) return launch_softmax_rows_backward(pgx, pgy, px, nrow, ncol, current_stream());
+    return launch_activate_backward(pgx, pgy, px, nrow * ncol, actFunc, hLeakyAlpha, current_stream());
+}
+
+int kai_activate_backward_with_y(int device, float* pgx, const float* pgy, const float* py, int64_t nrow,
+                                 int64_t ncol, int actFunc, const float* hLeakyAlpha) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    KAI_REQUIRE(actFunc >= KAI_ACT_NONE && actFunc <= KAI_ACT_TANH, KAI_ERR_CONDITIONAL_STATEMENT,
+                "activation code must be 0..4");
+    if (nrow == 0 || ncol == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgx); KAI_REQUIRE_PTR(pgy); KAI_REQUIRE_PTR(py);
+    return launch_activate_backward_with_y(pgx, pgy, py, nrow * ncol, actFunc, hLeakyAlpha, current_stream());
+}
+
+// ---- attention ---------------------------------------------------------------------------------
+
+static int check_heads(const char* fn, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece) {
+    if (nbat < 0 || ntimes < 0 || nvec < 0 || nhead < 0 || npiece < 0)
+        return fail(KAI_ERR_INVALID_ARGUMENT, std::string(fn) + ": negative dimension");
+    if (nhead * npiece > nvec) return fail(KAI_ERR_INVALID_ARGUMENT, std::string(fn) + ": nhead*npiece > nvec");
+    if (ntimes > kMaxDim || nvec > kMaxDim || nbat * nhead > 65535)
+        return fail(KAI_ERR_INVALID_ARGUMENT, std::string(fn) + ": dimension out of range");
+    return KAI_OK;
+}
+
+int kai_mult_on_heads(int device, float* pp, const float* pK, const float* pQ, int64_t nbat, int64_t ntimes,
+                      int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pp); KAI_REQUIRE_PTR(pK); KAI_REQUIRE_PTR(pQ);
+    // per (b,h): S[q,k] = coef * Q_h[q,:] . K_h[k,:] ; both K-contiguous; S element stride nhead
+    GemmDesc d;
+    d.A = pQ; d.B = pK; d.C = pp; d.alpha = hCoef; d.has_alpha = 1;
+    d.M = ntimes; d.N = ntimes; d.K = npiece;
+    d.a_rs = nvec; d.a_ks = 1; d.b_rs = nvec; d.b_ks = 1;
+    d.c_rs = ntimes * nhead; d.c_cs = nhead;
+    d.nbatch = nbat * nhead; d.bdiv = nhead;
+    d.a_bs0 = ntimes * nvec; d.a_bs1 = npiece;
+    d.b_bs0 = ntimes * nvec; d.b_bs1 = npiece;
+    d.c_bs0 = ntimes * ntimes * nhead; d.c_bs1 = 1;
+    return launch_gemm(d, current_stream());
+}
+
+int kai_mult_on_heads_backward(int device, float* pgQKV, const float* pgp, const float* pQKV, int64_t nbat,
+                               int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgQKV); KAI_REQUIRE_PTR(pgp); KAI_REQUIRE_PTR(pQKV);
+    // per (b,h): G[t,p] = sum_k gp[b,t,k,h] * KQ[b,k,h*npiece+p]
+    GemmDesc d;
+    d.A = pgp; d.B = pQKV; d.C = pgQKV;
+    d.M = ntimes; d.N = npiece; d.K = ntimes;
+    d.a_rs = ntimes * nhead; d.a_ks = nhead;
+    d.b_rs = 1; d.b_ks = nvec;
+    d.c_rs = nvec; d.c_cs = 1;
+    d.nbatch = nbat * nhead; d.bdiv = nhead;
+    d.a_bs0 = ntimes * ntimes * nhead; d.a_bs1 = 1;
+    d.b_bs0 = ntimes * nvec; d.b_bs1 = npiece;
+    d.c_bs0 = ntimes * nvec; d.c_bs1 = npiece;
+    return launch_gemm(d, current_stream());
+}
+
+int kai_set_mh_attention_mask(int device, float* pp, int64_t ndat, int64_t ntimes, int64_t nhead, int forward) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0 && ntimes >= 0 && nhead >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (ndat == 0 || ntimes == 0 || nhead == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pp);
+    return launch_attention_mask(pp, ndat, ntimes, nhead, forward != 0, current_stream());
+}
+
+int kai_softmax_direct_on_axis(int device, float* pp, int64_t nrow, int64_t nvec, int64_t ncol) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0 && nvec >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (nrow == 0 || nvec == 0 || ncol == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pp);
+    return launch_softmax_axis(pp, nrow, nvec, ncol, current_stream());
+}
+
+int kai_softmax_direct_on_axis_backward(int device, float* pgp, const float* pp, int64_t nbat, int64_t ntimes,
+                                        int64_t nhead, const float* hCoef) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nbat >= 0 && ntimes >= 0 && nhead >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (nbat == 0 || ntimes == 0 || nhead == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgp); KAI_REQUIRE_PTR(pp);
+    return launch_softmax_axis_backward(pgp, pp, nbat * ntimes, ntimes, nhead, hCoef, current_stream());
+}
+
+int kai_mix_values(int device, float* py, const float* pp, const float* pV, int64_t nbat, int64_t ntimes,
+                   int64_t nvec, int64_t nhead, int64_t npiece) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pp); KAI_REQUIRE_PTR(pV);
+    // per (b,h): Y[q,p] = sum_k P[b,q,k,h] * V[b,k,h*npiece+p]; Y is [nbat, ntimes, nhead, npiece]
+    GemmDesc d;
+    d.A = pp; d.B = pV; d.C = py;
+    d.M = ntimes; d.N = npiece; d.K = ntimes;
+    d.a_rs = ntimes * nhead; d.a_ks = nhead;
+    d.b_rs = 1; d.b_ks = nvec;
+    d.c_rs = nhead * npiece; d.c_cs = 1;
+    d.nbatch = nbat * nhead; d.bdiv = nhead;
+    d.a_bs0 = ntimes * ntimes * nhead; d.a_bs1 = 1;
+    d.b_bs0 = ntimes * nvec; d.b_bs1 = npiece;
+    d.c_bs0 = ntimes * nhead * npiece; d.c_bs1 = npiece;
+    return launch_gemm(d, current_stream());
+}
+
+int kai_mix_values_backward_prop(int device, float* pgp, const float* pgy, const float* pV, int64_t nbat,
+                                 int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgp); KAI_REQUIRE_PTR(pgy); KAI_REQUIRE_PTR(pV);
+    // per (b,h): gP[q,k] = sum_p gY[b,q,h,p] * V[b,k,h*npiece+p]
+    GemmDesc d;
+    d.A = pgy; d.B = pV; d.C = pgp;
+    d.M = ntimes; d.N = ntimes; d.K = npiece;
+    d.a_rs = nhead * npiece; d.a_ks = 1;
+    d.b_rs = nvec; d.b_ks = 1;
+    d.c_rs = ntimes * nhead; d.c_cs = nhead;
+    d.nbatch = nbat * nhead; d.bdiv = nhead;
+    d.a_bs0 = ntimes * nhead * npiece; d.a_bs1 = npiece;
+    d.b_bs0 = ntimes * nvec; d.b_bs1 = npiece;
+    d.c_bs0 = ntimes * ntimes * nhead; d.c_bs1 = 1;
+    return launch_gemm(d, current_stream());
+}
+
+int kai_mix_values_backward_value(int device, float* pgV, const float* pgy, const float* pp, int64_t nbat,
+                                  int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgV); KAI_REQUIRE_PTR(pgy); KAI_REQUIRE_PTR(pp);
+    // per (b,h): gV[k,p] = sum_q P[b,q,k,h] * gY[b,q,h,p] : rows of the product are k, reduction over q
+    GemmDesc d;
+    d.A = pp; d.B = pgy; d.C = pgV;
+    d.M = ntimes; d.N = npiece; d.K = ntimes;
+    d.a_rs = nhead; d.a_ks = ntimes * nhead;
+    d.b_rs = 1; d.b_ks = nhead * npiece;
+    d.c_rs = nvec; d.c_cs = 1;
+    d.nbatch = nbat * nhead; d.bdiv = nhead;
+    d.a_bs0 = ntimes * ntimes * nhead; d.a_bs1 = 1;
+    d.b_bs0 = ntimes * nhead * npiece; d.b_bs1 = npiece;
+    d.c_bs0 = ntimes * nvec; d.c_bs1 = npiece;
+    return launch_gemm(d, current_stream());
+}
+
+// ---- fused dense layer -------------------------------------------------------------------------
+
+int kai_dense_forward(int device, float* py, float* ppre, const float* pw, const float* pb, const float* px,
+                      int64_t yvec, int64_t ndat, int64_t xvec, int actFunc, const float* hLeakyAlpha) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE_DIM(yvec); KAI_REQUIRE_DIM(ndat); KAI_REQUIRE_DIM(xvec);
+    KAI_REQUIRE(act_is_elementwise(actFunc), KAI_ERR_CONDITIONAL_STATEMENT, "activation code must be 0..8");
+    if (ndat == 0 || yvec == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py);
+    if (xvec > 0) { KAI_REQUIRE_PTR(pw); KAI_REQUIRE_PTR(px); }
+    GemmDesc d;
+    d.A = px; d.B = pw; d.C = py; d.C2 = ppre; d.bias = pb; d.leaky = hLeakyAlpha;
+    d.M = ndat; d.N = yvec; d.K = xvec;
+    d.a_rs = xvec; d.a_ks = 1; d.b_rs = xvec; d.b_ks = 1; d.c_rs = yvec; d.c_cs = 1;
+    d.act = actFunc;
+    return launch_gemm(d, current_stream());
+}
+
+int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pga_work, const float* pgy,
+                       const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
+                       int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE_DIM(yvec); KAI_REQUIRE_DIM(ndat); KAI_REQUIRE_DIM(xvec);
+    KAI_REQUIRE(act_is_elementwise(actFunc), KAI_ERR_CONDITIONAL_STATEMENT, "activation code must be 0..8");
+    KAI_REQUIRE_PTR(pgy);
+    const float* ga = pgy;
+    if (actFunc != KAI_ACT_NONE && ppre != nullptr) {
+        KAI_REQUIRE(pga_work != nullptr, KAI_ERR_INVALID_POINTER, "pga_work is required when an activation is applied");
+        KAI_TRY(launch_activate_backward(pga_work, pgy, ppre, ndat * yvec, actFunc, hLeakyAlpha, current_stream()));
+        ga = pga_work;
+    }
+    if (pgb) KAI_TRY(kai_add_bias_backward_b(device, pgb, ga, ndat, yvec, acc));
+    if (pgx) {
+        KAI_REQUIRE_PTR(pw);
+        KAI_TRY(kai_matmul_backward_x(device, pgx, ga, pw, yvec, ndat, xvec, acc));
+    }
+    if (pgw) {
+        KAI_REQUIRE_PTR(px);
+        KAI_TRY(kai_matmul_backward_w(device, pgw, ga, px, yvec, ndat, xvec, acc));
+    }
+    return KAI_OK;
+}
+
+}  // extern "C"

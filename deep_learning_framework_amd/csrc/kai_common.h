@@ -1,0 +1,44 @@
+// Internal helpers shared by the host-side translation units of libkai_hip.so:
+// error reporting (numeric codes of the reference, thread-local message), the
+// calling thread's stream, and argument checks.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/kai_hip.h"
+
+namespace kai {
+
+// thread-local last error text; returns `code` so that callers can `return fail(...)`
+int fail(int code, const std::string& msg);
+void clear_error();
+// stream of the calling thread (null stream unless kai_set_stream was called on this thread)
+hipStream_t current_stream();
+
+// turns a HIP status into KAI_ERR_GPU with the runtime's message
+int check_hip(hipError_t st, const char* what);
+// status of the launch that was just enqueued
+int check_launch(const char* kernel_name);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr int64_t kMaxDim = (1ll << 31) - 1;
+
+}  // namespace kai
+
+#define KAI_REQUIRE(cond, code, msg)                                   \
+    do {                                                               \
+        if (!(cond)) return ::kai::fail((code), std::string(__func__) + ": " + (msg)); \
+    } while (0)
+
+#define KAI_REQUIRE_DEVICE(device) \
+    KAI_REQUIRE((device) >= 0, KAI_ERR_INVALID_ARGUMENT, "device < 0 selects the engine's host loop, which this GPU library does not contain")
+
+#define KAI_TRY(expr)               \
+    do {                            \
+        int kai_rc_ = (expr);       \
+        if (kai_rc_ != KAI_OK) return kai_rc_; \
+    } while (0)

@@ -1,0 +1,236 @@
+"""Host-side mirror of the engine's tensor operators that call the matmul path.
+
+``Tensor`` is a shape plus a device buffer; its methods derive the raw-pointer argument
+lists exactly as the reference's ``VTensor`` methods do and issue the same sequence of
+``VMath`` calls:
+
+* ``matmul`` / ``matmul_backprop``   -- api_objects/vtensor.cpp:1282-1375
+* ``add`` / ``add_backprop``         -- api_objects/vtensor.cpp:3395-3485
+* ``activate`` / ``activate_backprop`` -- api_objects/vtensor.cpp:5674-5718
+* ``mh_attention`` / ``mh_attention_backprop`` -- api_objects/vtensor.cpp:2978-3227
+
+Shape errors raise ``KaiError`` with the reference's codes (VERR_BAD_SHAPE_TENSOR = 10003).
+The graph, autograd queue and tracer of the engine are not rebuilt: backprop methods
+return the gradients instead of registering them in a queue.
+"""
+import numpy as np
+
+from . import kai
+from .kai import ACT, DeviceBuffer, KaiError, VMath
+
+VERR_BAD_SHAPE_TENSOR = 10003
+VERR_UNDEFINED = 2
+
+
+def _total(shape):
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+class Tensor:
+    """A float32 device tensor: ``shape`` and a ``DeviceBuffer`` (reference: VTensor + VTensorData)."""
+
+    def __init__(self, shape, device=0, buf=None):
+        self.shape = tuple(int(s) for s in shape)
+        self.device = device
+        self.buf = buf if buf is not None else DeviceBuffer(max(_total(self.shape), 1) * 4, device)
+        self.saved = {}
+
+    @classmethod
+    def from_numpy(cls, a, device=0):
+        a = np.ascontiguousarray(a, dtype=np.float32)
+        return cls(a.shape, device, DeviceBuffer.from_numpy(a, device))
+
+    def numpy(self):
+        return self.buf.to_numpy(self.shape, np.float32)
+
+    @property
+    def ptr(self):
+        return self.buf.ptr
+
+    def total_size(self):
+        return _total(self.shape)
+
+    # ---- matmul: vtensor.cpp:1282-1335 ------------------------------------------------------------
+    def matmul(self, w):
+        x = self
+        if len(x.shape) < 2:
+            raise KaiError(VERR_BAD_SHAPE_TENSOR, "matmul")
+        if len(w.shape) != 2:
+            raise KaiError(VERR_BAD_SHAPE_TENSOR, "matmul")
+        yvec, xvec = w.shape
+        ndat = x.total_size() // xvec
+        yshape = list(x.shape)
+        while True:
+            yshape = yshape[:-1]
+            t = _total(yshape)
+            if t == ndat:
+                break
+            if t < ndat:
+                raise KaiError(VERR_UNDEFINED, "matmul: input cannot be split into rows of the weight's width")
+        yshape.append(yvec)
+        y = Tensor(yshape, x.device)
+        VMath.matmul(x.device, y.ptr, w.ptr, x.ptr, yvec, ndat, xvec, False)
+        y.saved = {"op": "matmul", "x": x, "w": w}
+        return y
+
+    # vtensor.cpp:1337-1375
+    def matmul_backprop(self, ygrad, need_x=True, need_w=True):
+        x, w = self.saved["x"], self.saved["w"]
+        yvec, xvec = w.shape
+        ndat = x.total_size() // xvec
+        xgrad = wgrad = None
+        if need_x:
+            xgrad = Tensor(x.shape, x.device)
+            VMath.matmul_backward_x(x.device, xgrad.ptr, ygrad.ptr, w.ptr, yvec, ndat, xvec, False)
+        if need_w:
+            wgrad = Tensor(w.shape, x.device)
+            VMath.matmul_backward_w(x.device, wgrad.ptr, ygrad.ptr, x.ptr, yvec, ndat, xvec, False)
+        return xgrad, wgrad
+
+    # ---- add (bias form): vtensor.cpp:3395-3436 -----------------------------------------------------
+    def add(self, b):
+        a = self
+        if a.shape != b.shape and a.total_size() % b.total_size() != 0:
+            raise KaiError(VERR_BAD_SHAPE_TENSOR, "add")
+        if a.shape == b.shape:
+            raise NotImplementedError("same-shape add is VMath::add, outside the matmul path")
+        ndat = a.total_size()
+        ncol = b.total_size()
+        nrow = ndat // ncol
+        y = Tensor(a.shape, a.device)
+        VMath.add_bias(a.device, y.ptr, a.ptr, b.ptr, nrow, ncol)
+        y.saved = {"op": "add", "a": a, "b": b}
+        return y
+
+    # vtensor.cpp:3438-3485 (bias branch): the gradient of `a` is ygrad itself
+    def add_backprop(self, ygrad):
+        a, b = self.saved["a"], self.saved["b"]
+        ndat = a.total_size()
+        ncol = b.shape[-1]
+        nrow = ndat // ncol
+        bgrad = Tensor(b.shape, a.device)
+        VMath.add_bias_backward_b(a.device, bgrad.ptr, ygrad.ptr, nrow, ncol, False)
+        return ygrad, bgrad
+
+    # ---- activate: vtensor.cpp:5674-5695 ---------------------------------------------------------------
+    def activate(self, actfunc, leaky_alpha=None):
+        x = self
+        ncol = x.shape[-1]
+        nrow = x.total_size() // ncol
+        code = ACT[actfunc] if isinstance(actfunc, str) else int(actfunc)
+        h = kai.hyper(leaky_alpha, x.device)
+        y = Tensor(x.shape, x.device)
+        VMath.activate(x.device, y.ptr, x.ptr, nrow, ncol, code, h)
+        y.saved = {"op": "activate", "x": x, "actfunc": code, "leaky_alpha": h}
+        return y
+
+    # vtensor.cpp:5697-5718
+    def activate_backprop(self, ygrad):
+        x = self.saved["x"]
+        ncol = self.shape[-1]
+        nrow = self.total_size() // ncol
+        xgrad = Tensor(x.shape, x.device)
+        VMath.activate_backward(x.device, xgrad.ptr, ygrad.ptr, x.ptr, nrow, ncol, self.saved["actfunc"],
+                                self.saved["leaky_alpha"])
+        return xgrad
+
+    # ---- mh_attention: vtensor.cpp:2978-3052 ----------------------------------------------------------
+    def mh_attention(self, key, query, value, Kw, Kb, Qw, Qb, Vw, Vb, Ow, Ob, head_cnt, mask=False, coef=None):
+        x = self
+        if len(x.shape) != 3 or x.shape[2] % head_cnt != 0:
+            raise KaiError(VERR_BAD_SHAPE_TENSOR, "mh_attention")
+        if x.shape != key.shape or x.shape != query.shape or x.shape != value.shape:
+            raise KaiError(VERR_BAD_SHAPE_TENSOR, "mh_attention")
+        nbat, ntimes, nvec = x.shape
+        nhead = head_cnt
+        npiece = nvec // nhead
+        for w in (Kw, Qw, Vw):
+            if w.shape != (nvec, nvec):
+                raise KaiError(VERR_BAD_SHAPE_TENSOR, "mh_attention")
+        if coef is None:
+            coef = 1.0 / np.sqrt(nvec / nhead)   # api_objects/vmodule.cpp:1805
+        hcoef = kai.hyper(coef, x.device)
+        dev = x.device
+        y = Tensor(x.shape, dev)
+        K = Tensor((nbat, ntimes, nvec), dev)
+        Q = Tensor((nbat, ntimes, nvec), dev)
+        V = Tensor((nbat, ntimes, nvec), dev)
+        probs = Tensor((nbat, ntimes, ntimes, nhead), dev)
+        mixed = Tensor(x.shape, dev)
+        n = nbat * ntimes
+        VMath.matmul(dev, K.ptr, Kw.ptr, key.ptr, nvec, n, nvec, False)
+        VMath.matmul(dev, Q.ptr, Qw.ptr, query.ptr, nvec, n, nvec, False)
+        VMath.matmul(dev, V.ptr, Vw.ptr, value.ptr, nvec, n, nvec, False)
+        VMath.add_bias(dev, K.ptr, K.ptr, Kb.ptr, n, nvec)
+        VMath.add_bias(dev, Q.ptr, Q.ptr, Qb.ptr, n, nvec)
+        VMath.add_bias(dev, V.ptr, V.ptr, Vb.ptr, n, nvec)
+        VMath.mult_on_heads(dev, probs.ptr, K.ptr, Q.ptr, nbat, ntimes, nvec, nhead, npiece, hcoef)
+        if mask:
+            VMath.set_mh_attention_mask(dev, probs.ptr, nbat, ntimes, nhead, True)
+        VMath.softmax_direct_on_axis(dev, probs.ptr, nbat * ntimes, ntimes, nhead)
+        VMath.mix_values(dev, mixed.ptr, probs.ptr, V.ptr, nbat, ntimes, nvec, nhead, npiece)
+        VMath.matmul(dev, y.ptr, Ow.ptr, mixed.ptr, nvec, n, nvec, False)
+        VMath.add_bias(dev, y.ptr, y.ptr, Ob.ptr, n, nvec)
+        y.saved = {"op": "mh_attention", "key": key, "query": query, "value": value, "Kw": Kw, "Qw": Qw, "Vw": Vw,
+                   "Ow": Ow, "K": K, "Q": Q, "V": V, "probs": probs, "mixed": mixed, "head_cnt": nhead,
+                   "mask": mask, "coef": hcoef}
+        return y
+
+    # vtensor.cpp:3054-3166 (the math calls; gradient registration is the engine's business)
+    def mh_attention_backprop(self, ygrad):
+        s = self.saved
+        nbat, ntimes, nvec = self.shape
+        nhead = s["head_cnt"]
+        npiece = nvec // nhead
+        dev = self.device
+        n = nbat * ntimes
+        T = lambda shape: Tensor(shape, dev)
+        g = {name: T((nvec, nvec)) for name in ("Kw", "Qw", "Vw", "Ow")}
+        g.update({name: T((nvec,)) for name in ("Kb", "Qb", "Vb", "Ob")})
+        g.update({name: T(self.shape) for name in ("key", "query", "value", "mixed", "K", "Q", "V")})
+        g["probs"] = T((nbat, ntimes, ntimes, nhead))
+        gy = ygrad.ptr
+        VMath.add_bias_backward_b(dev, g["Ob"].ptr, gy, n, nvec, False)
+        VMath.matmul_backward_w(dev, g["Ow"].ptr, gy, s["mixed"].ptr, nvec, n, nvec, False)
+        VMath.matmul_backward_x(dev, g["mixed"].ptr, gy, s["Ow"].ptr, nvec, n, nvec, False)
+        VMath.mix_values_backward_prop(dev, g["probs"].ptr, g["mixed"].ptr, s["V"].ptr, nbat, ntimes, nvec, nhead,
+                                       npiece)
+        VMath.mix_values_backward_value(dev, g["V"].ptr, g["mixed"].ptr, s["probs"].ptr, nbat, ntimes, nvec, nhead,
+                                        npiece)
+        VMath.softmax_direct_on_axis_backward(dev, g["probs"].ptr, s["probs"].ptr, nbat, ntimes, nhead, s["coef"])
+        if s["mask"]:
+            VMath.set_mh_attention_mask(dev, g["probs"].ptr, nbat, ntimes, nhead, False)
+        VMath.mult_on_heads_backward(dev, g["K"].ptr, g["probs"].ptr, s["Q"].ptr, nbat, ntimes, nvec, nhead, npiece)
+        VMath.mult_on_heads_backward(dev, g["Q"].ptr, g["probs"].ptr, s["K"].ptr, nbat, ntimes, nvec, nhead, npiece)
+        VMath.add_bias_backward_b(dev, g["Kb"].ptr, g["K"].ptr, n, nvec, False)
+        VMath.add_bias_backward_b(dev, g["Qb"].ptr, g["Q"].ptr, n, nvec, False)
+        VMath.add_bias_backward_b(dev, g["Vb"].ptr, g["V"].ptr, n, nvec, False)
+        VMath.matmul_backward_w(dev, g["Kw"].ptr, g["K"].ptr, s["key"].ptr, nvec, n, nvec, False)
+        VMath.matmul_backward_w(dev, g["Qw"].ptr, g["Q"].ptr, s["query"].ptr, nvec, n, nvec, False)
+        VMath.matmul_backward_w(dev, g["Vw"].ptr, g["V"].ptr, s["value"].ptr, nvec, n, nvec, False)
+        VMath.matmul_backward_x(dev, g["key"].ptr, g["K"].ptr, s["Kw"].ptr, nvec, n, nvec, False)
+        VMath.matmul_backward_x(dev, g["query"].ptr, g["Q"].ptr, s["Qw"].ptr, nvec, n, nvec, False)
+        VMath.matmul_backward_x(dev, g["value"].ptr, g["V"].ptr, s["Vw"].ptr, nvec, n, nvec, False)
+        return g
+
+
+def dense(x, w, b, actfunc="relu", leaky_alpha=None, fused=True, keep_pre=False):
+    """The engine's ``dense`` layer formula activate(add(matmul(x, w), b)) (api/vconst.cpp:11).
+
+    ``fused=False`` issues the three reference calls; ``fused=True`` the single-launch
+    kai_dense_forward.  Returns (y, pre_activation or None)."""
+    if not fused:
+        pre = x.matmul(w).add(b)
+        return pre.activate(actfunc, leaky_alpha), pre
+    yvec, xvec = w.shape
+    ndat = x.total_size() // xvec
+    code = ACT[actfunc] if isinstance(actfunc, str) else int(actfunc)
+    y = Tensor(x.shape[:-1] + (yvec,), x.device)
+    pre = Tensor(y.shape, x.device) if keep_pre else None
+    h = kai.hyper(leaky_alpha, x.device)
+    VMath.dense_forward(x.device, y.ptr, pre.ptr if pre else None, w.ptr, b.ptr if b is not None else None, x.ptr,
+                        yvec, ndat, xvec, code, h)
+    return y, pre

@@ -1,0 +1,196 @@
+/*
+ * kai_hip.h -- C-ABI of libkai_hip.so: the fp32 matrix-multiplication path of
+ * the KONAN AI engine (class VMath, source/engine/support/vmath.h of the
+ * reference) as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions (they hold for every entry point below)
+ *  - Return value: 0 (KAI_OK) or one of the reference's numeric error codes
+ *    (source/engine/include/verrors.h).  Nothing is thrown across this boundary;
+ *    kai_last_error() returns the calling thread's last message.
+ *  - `device`: the reference selects the host loop with device < 0 and the GPU
+ *    kernel with device >= 0 (CUDA_CALL, vmath.cu:46-55).  This library is the GPU
+ *    side only.  device < 0 returns KAI_ERR_INVALID_ARGUMENT for compute entry
+ *    points: the host loops stay in the engine.  For device >= 0 the kernel is
+ *    enqueued on the calling thread's CURRENT device, which the caller has already
+ *    selected (the engine does it in VDeviceManager::setCurDevice,
+ *    local_objects/vdevicemanager.cpp:110-122); kai_set_device() is exported for
+ *    that.  Only kai_mem_alloc switches devices itself, as the reference does
+ *    (vmath.cu:170-204).
+ *  - Pointers are raw device pointers owned by the caller; the library never
+ *    allocates, frees or caches them.  Whole buffers from kai_mem_alloc are
+ *    16-byte aligned; sub-buffer pointers of any 4-byte alignment are accepted
+ *    (slower loads are chosen automatically).  In-place aliasing is legal where the
+ *    reference uses it: add_bias (py == pa), activate (py == px), the softmax and
+ *    mask ops.  A GEMM output must not alias its inputs.
+ *  - Hyper-parameters (`hLeakyAlpha`, `hCoef`) are DEVICE pointers to one float,
+ *    read inside the kernel; null reads as 0 (HYPER_ACCESS,
+ *    local_objects/vhypermanager.h:9).
+ *  - Work is enqueued asynchronously on the stream set by kai_set_stream (the null
+ *    stream by default, matching the reference's use of the legacy default
+ *    stream); results are ordered by stream order and by the blocking copies.
+ *  - `acc` != 0 adds the product to the existing output instead of overwriting it.
+ *  - All matrices are dense row-major fp32.  Sizes are int64_t as in the reference
+ *    (include/vtypes.h:18-22); each dimension and each leading dimension must be
+ *    below 2^31.
+ */
+#ifndef KAI_HIP_H
+#define KAI_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* error codes: the reference's numbers (source/engine/include/verrors.h:4,12,39,52,149,164) */
+#define KAI_OK 0
+#define KAI_ERR_CONDITIONAL_STATEMENT 8   /* unknown activation code (vmath.cu:3159-3161) */
+#define KAI_ERR_INVALID_ARGUMENT 510
+#define KAI_ERR_INVALID_POINTER 523
+#define KAI_ERR_HOSTMEM_ALLOC_FAILURE 10012
+#define KAI_ERR_GPU 50002                 /* VERR_CUDA_ERROR: any HIP runtime or launch error */
+
+/* activation codes, enum class ActFunc (source/engine/include/vtypes.h:37-39) */
+#define KAI_ACT_NONE 0
+#define KAI_ACT_RELU 1
+#define KAI_ACT_LEAKY 2
+#define KAI_ACT_SIGMOID 3
+#define KAI_ACT_TANH 4
+#define KAI_ACT_GELU 5
+#define KAI_ACT_SELU 6
+#define KAI_ACT_MISH 7
+#define KAI_ACT_SWISH 8
+#define KAI_ACT_SOFTMAX 9
+
+/* ---- library state --------------------------------------------------------------------------- */
+
+/* Message of the calling thread's last failing call ("" if none).  Replaces the text the
+ * reference passes to VP_THROW1(VERR_CUDA_ERROR, "cuda:"+msg) in VMath::cudaCheck (vmath.cu:64-87). */
+const char* kai_last_error(void);
+/* Number of visible GPUs (reference: cudaGetDeviceCount, local_objects/vdevicemanager.cpp:59-63). */
+int kai_device_count(int* count);
+/* hipSetDevice for the calling thread (reference: VDeviceManager::setCurDevice, vdevicemanager.cpp:110-122). */
+int kai_set_device(int device);
+/* Blocks until the current device is idle.  The reference's live path has no such call (it relies
+ * on blocking cudaMemcpy); exported for harnesses that time kernels. */
+int kai_device_synchronize(void);
+/* Stream (a hipStream_t, or null for the null stream) that this THREAD's later calls enqueue on.
+ * No counterpart in the reference, which only uses the legacy default stream. */
+int kai_set_stream(void* hip_stream);
+/* Name of the code object's target ("gfx950") and of the current device's architecture. */
+int kai_arch_info(char* built_for, char* device_arch, int buflen);
+
+/* ---- memory (VMath::mem_alloc ... get_slice, vmath.h:18-24,40-46,56) ---------------------------- */
+
+/* vmath.cu:170-210: device >= 0 allocates `size` bytes rounded up to a multiple of 16 on that
+ * device (saving and restoring the current device); device < 0 allocates host memory. */
+int kai_mem_alloc(int device, int64_t size, void** out_ptr);
+/* vmath.cu:232-265 */
+int kai_mem_free(int device, void* ptr);
+/* vmath.cu:278-293: blocking copies */
+int kai_memcpy_host_to_host(void* dptr, const void* sptr, int64_t size);
+int kai_memcpy_host_to_device(void* dptr, const void* sptr, int64_t size);
+int kai_memcpy_device_to_host(void* dptr, const void* sptr, int64_t size);
+int kai_memcpy_device_to_device(void* dptr, const void* sptr, int64_t size);
+/* vmath.cu:351-360 */
+int kai_copy_data(int dest_device, int src_device, void* py, const void* px, int64_t nbytes);
+/* vmath.cu:494-530 (`size` counts elements) */
+int kai_fill_int(int device, int* ptr, int64_t size, int value);
+int kai_fill_float(int device, float* ptr, int64_t size, float value);
+/* vmath.cu:534-541 (`size` counts bytes) */
+int kai_set_zero(int device, void* ptr, int64_t size);
+/* vmath.cu:545-578: py on `device` (host if < 0) <- host px / py host <- px on device / device<-device */
+int kai_memcpy_from_host(int device, void* py, const void* px, int64_t size);
+int kai_memcpy_to_host(int device, void* py, const void* px, int64_t size);
+int kai_memcpy_to_device(int device, void* py, const void* px, int64_t size);
+/* vmath.cu:708-715 */
+int kai_get_slice(int device, void* py, const void* px, int64_t nbytes);
+
+/* ---- dense layer: VMath::matmul family (vmath.h:137-139) ------------------------------------- */
+
+/* VMath::matmul, vmath.cu:2961-3003.  y[ndat,yvec] (=|+=) x[ndat,xvec] . w[yvec,xvec]^T */
+int kai_matmul(int device, float* py, const float* pw, const float* px, int64_t yvec, int64_t ndat, int64_t xvec,
+               int acc);
+/* VMath::matmul_backward_x, vmath.cu:3007-3047.  gx[ndat,xvec] (=|+=) gy[ndat,yvec] . w[yvec,xvec] */
+int kai_matmul_backward_x(int device, float* pgx, const float* pgy, const float* pw, int64_t yvec, int64_t ndat,
+                          int64_t xvec, int acc);
+/* VMath::matmul_backward_w, vmath.cu:3051-3093.  gw[yvec,xvec] (=|+=) gy[ndat,yvec]^T . x[ndat,xvec] */
+int kai_matmul_backward_w(int device, float* pgw, const float* pgy, const float* px, int64_t yvec, int64_t ndat,
+                          int64_t xvec, int acc);
+
+/* VMath::add_bias, vmath.cu:875-897.  y[r,c] = a[r,c] + b[c]; py may equal pa */
+int kai_add_bias(int device, float* py, const float* pa, const float* pb, int64_t nrow, int64_t ncol);
+/* VMath::add_bias_backward_b, vmath.cu:901-932.  gb[c] (=|+=) sum_r gy[r,c] */
+int kai_add_bias_backward_b(int device, float* pgb, const float* pgy, int64_t nrow, int64_t ncol, int acc);
+
+/* VMath::activate, vmath.cu:3097-3243; py may equal px (except for softmax).  The softmax case
+ * normalises each row of ncol elements (the reference's row pointer arithmetic at vmath.cu:3146
+ * reads outside the buffer; the row-wise meaning is implemented). */
+int kai_activate(int device, float* py, const float* px, int64_t nrow, int64_t ncol, int actFunc,
+                 const float* hLeakyAlpha);
+/* VMath::activate_backward, vmath.cu:3247-3407; px is the pre-activation input.  Codes 0..8 as on the
+ * reference's host path plus softmax (9) as on its device path (vmath.cu:3363-3394). */
+int kai_activate_backward(int device, float* pgx, const float* pgy, const float* px, int64_t nrow, int64_t ncol,
+                          int actFunc, const float* hLeakyAlpha);
+/* VMath::activate_backward_with_y, vmath.cu:3411-3486; codes 0..4 only */
+int kai_activate_backward_with_y(int device, float* pgx, const float* pgy, const float* py, int64_t nrow,
+                                 int64_t ncol, int actFunc, const float* hLeakyAlpha);
+
+/* ---- attention: VMath::mult_on_heads family (vmath.h:234-241) --------------------------------- */
+
+/* VMath::mult_on_heads, vmath.cu:6729-6779.  pp[b,q,k,h] = coef * sum_p K[b,k,h*npiece+p]*Q[b,q,h*npiece+p];
+ * K, Q are [nbat, ntimes, nvec]; pp is [nbat, ntimes, ntimes, nhead] (head index innermost). */
+int kai_mult_on_heads(int device, float* pp, const float* pK, const float* pQ, int64_t nbat, int64_t ntimes,
+                      int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef);
+/* VMath::mult_on_heads_backward, vmath.cu:6783-6829.  g[b,t,h*npiece+p] = sum_k gp[b,t,k,h]*KQ[b,k,h*npiece+p] */
+int kai_mult_on_heads_backward(int device, float* pgQKV, const float* pgp, const float* pQKV, int64_t nbat,
+                               int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece);
+/* VMath::set_mh_attention_mask, vmath.cu:6833-6860.  pp[b,q,k,h] = forward ? -inf : 0 for k > q */
+int kai_set_mh_attention_mask(int device, float* pp, int64_t ndat, int64_t ntimes, int64_t nhead, int forward);
+/* VMath::softmax_direct_on_axis, vmath.cu:6864-6916.  In place, softmax over the middle axis of
+ * [nrow, nvec, ncol]. */
+int kai_softmax_direct_on_axis(int device, float* pp, int64_t nrow, int64_t nvec, int64_t ncol);
+/* VMath::softmax_direct_on_axis_backward, vmath.cu:6920-6973.  In place on pgp:
+ * gp = coef * p * (gp - sum_k p*gp) */
+int kai_softmax_direct_on_axis_backward(int device, float* pgp, const float* pp, int64_t nbat, int64_t ntimes,
+                                        int64_t nhead, const float* hCoef);
+/* VMath::mix_values, vmath.cu:6977-7025.  y[b,q,h,p] = sum_k pp[b,q,k,h] * V[b,k,h*npiece+p] */
+int kai_mix_values(int device, float* py, const float* pp, const float* pV, int64_t nbat, int64_t ntimes,
+                   int64_t nvec, int64_t nhead, int64_t npiece);
+/* VMath::mix_values_backward_prop, vmath.cu:7029-7077.  gp[b,q,k,h] = sum_p gy[b,q,h,p] * V[b,k,h*npiece+p] */
+int kai_mix_values_backward_prop(int device, float* pgp, const float* pgy, const float* pV, int64_t nbat,
+                                 int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece);
+/* VMath::mix_values_backward_value, vmath.cu:7081-7129.  gV[b,k,h*npiece+p] = sum_q pp[b,q,k,h] * gy[b,q,h,p] */
+int kai_mix_values_backward_value(int device, float* pgV, const float* pgy, const float* pp, int64_t nbat,
+                                  int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece);
+
+/* ---- fused entry points (additive: each equals a fixed sequence of the calls above) ------------ */
+
+/* C[M,N] (=|+=) act( op(A) . op(B) + bias ), row-major.
+ *   transA == 0: A is [M,K] with row stride lda;  transA != 0: A is stored [K,M] (lda = its row stride)
+ *   transB == 0: B is [K,N] with row stride ldb;  transB != 0: B is stored [N,K]
+ * bias (length N) may be null; actFunc is an element-wise code 0..8.  With acc != 0 the order is
+ * C = act(C + A.B + bias).  Equals matmul / matmul_backward_x / matmul_backward_w for the operand
+ * forms (0,1) / (0,0) / (1,0), followed by add_bias and activate. */
+int kai_gemm_f32(int device, int transA, int transB, int64_t M, int64_t N, int64_t K, const float* A, int64_t lda,
+                 const float* B, int64_t ldb, float* C, int64_t ldc, const float* bias, int actFunc,
+                 const float* hLeakyAlpha, int acc);
+
+/* The engine's `dense` layer formula activate(add(matmul(x,w),b)) (api/vconst.cpp:11) in one launch:
+ * py = act(x . w^T + b).  ppre, if not null, receives the pre-activation x . w^T + b that
+ * VTensor::activate_backprop needs (vtensor.cpp:5697-5718).  pb may be null (no bias). */
+int kai_dense_forward(int device, float* py, float* ppre, const float* pw, const float* pb, const float* px,
+                      int64_t yvec, int64_t ndat, int64_t xvec, int actFunc, const float* hLeakyAlpha);
+
+/* Backward of the same layer: ga = activate_backward(gy, ppre) (skipped when ppre is null or
+ * actFunc == 0), then gb = colsum(ga), gx = ga . w, gw = ga^T . x.  Any of pgx, pgw, pgb may be
+ * null.  pga_work is a caller buffer of ndat*yvec floats for ga (required when an activation is
+ * applied; may equal pgy to overwrite it). */
+int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pga_work, const float* pgy,
+                       const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
+                       int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,101 @@
+/*
+ * kai_oracle.h -- CPU restatement of the KONAN AI engine's host math loops for
+ * the matrix-multiplication path.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only the test-suite, the
+ * smoke check and the cpu_baseline leg of the benchmark may link or load it.
+ * The shipped library never calls into it and has no CPU fallback.
+ *
+ * Every function follows, loop for loop, one `*_host` function of the
+ * reference engine (file source/engine/support/vmath.cu, cited per function):
+ * the same index order, a `float` accumulator that starts at 0.0f, a separately
+ * rounded multiply and add (build with -ffp-contract=off, no fast-math), and the
+ * `acc` flag applied after the dot product.  Argument order and meaning are
+ * those of the reference's VMath methods (source/engine/support/vmath.h:65-66,
+ * 137-143, 234-241) minus the leading `device` argument.
+ *
+ * Hyper-parameters (`hLeakyAlpha`, `hCoef`) are pointers to one float; a null
+ * pointer reads as 0, as the reference's HYPER_ACCESS does
+ * (source/engine/local_objects/vhypermanager.h:9).
+ *
+ * Return value: 0 on success, KO_ERR_CONDITIONAL_STATEMENT (8) where the
+ * reference throws VERR_CONDITIONAL_STATEMENT (unknown activation code).
+ *
+ * Parity status: every function here is pinned by tests/test_oracle_pins.py
+ * (closed forms in float64, exact small-integer cases, brute force on tiny
+ * shapes, adjoint identities and special values).  The reference holds no golden
+ * vectors and cannot be compiled in this image (it needs the CUDA toolkit,
+ * curand and OpenCV), so those checks are the whole pin; nothing is left
+ * "parity unpinned" except the libm-level rounding of expf/erff/logf, which the
+ * tolerance covers.
+ */
+#ifndef KAI_ORACLE_H
+#define KAI_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KO_OK 0
+#define KO_ERR_CONDITIONAL_STATEMENT 8
+
+/* activation codes: source/engine/include/vtypes.h:37-39 */
+enum {
+    KO_ACT_NONE = 0, KO_ACT_RELU = 1, KO_ACT_LEAKY = 2, KO_ACT_SIGMOID = 3, KO_ACT_TANH = 4,
+    KO_ACT_GELU = 5, KO_ACT_SELU = 6, KO_ACT_MISH = 7, KO_ACT_SWISH = 8, KO_ACT_SOFTMAX = 9
+};
+
+/* vmath.cu:2961-2977  y[nd,ny] (=|+=) sum_nx w[ny,nx]*x[nd,nx] */
+int ko_matmul(float* py, const float* pw, const float* px, int64_t yvec, int64_t ndat, int64_t xvec, int acc);
+/* same loop restricted to rows nd in [nd_begin, nd_end): lets callers sample rows of a
+ * large product or spread rows over threads; each element's sum order is unchanged. */
+int ko_matmul_rows(float* py, const float* pw, const float* px, int64_t yvec, int64_t nd_begin, int64_t nd_end,
+                   int64_t xvec, int acc);
+/* vmath.cu:3007-3022  gx[nd,nx] (=|+=) sum_ny w[ny,nx]*gy[nd,ny] */
+int ko_matmul_backward_x(float* pgx, const float* pgy, const float* pw, int64_t yvec, int64_t ndat, int64_t xvec, int acc);
+/* vmath.cu:3051-3067  gw[ny,nx] (=|+=) sum_nd x[nd,nx]*gy[nd,ny] */
+int ko_matmul_backward_w(float* pgw, const float* pgy, const float* px, int64_t yvec, int64_t ndat, int64_t xvec, int acc);
+
+/* vmath.cu:875-881 */
+int ko_add_bias(float* py, const float* pa, const float* pb, int64_t nrow, int64_t ncol);
+/* vmath.cu:901-911 */
+int ko_add_bias_backward_b(float* pgb, const float* pgy, int64_t nrow, int64_t ncol, int acc);
+
+/* vmath.cu:3097-3167 (helpers :297-307) */
+int ko_activate(float* py, const float* px, int64_t nrow, int64_t ncol, int actFunc, const float* hLeakyAlpha);
+/* vmath.cu:3247-3308 */
+int ko_activate_backward(float* pgx, const float* pgy, const float* px, int64_t nrow, int64_t ncol, int actFunc,
+                         const float* hLeakyAlpha);
+/* vmath.cu:3411-3444 */
+int ko_activate_backward_with_y(float* pgx, const float* pgy, const float* py, int64_t nrow, int64_t ncol, int actFunc,
+                                const float* hLeakyAlpha);
+
+/* vmath.cu:6729-6750 */
+int ko_mult_on_heads(float* pp, const float* pK, const float* pQ, int64_t nbat, int64_t ntimes, int64_t nvec,
+                     int64_t nhead, int64_t npiece, const float* hCoef);
+/* vmath.cu:6783-6802 */
+int ko_mult_on_heads_backward(float* pgQK, const float* pgp, const float* pKQ, int64_t nbat, int64_t ntimes,
+                              int64_t nvec, int64_t nhead, int64_t npiece);
+/* vmath.cu:6833-6844 */
+int ko_set_mh_attention_mask(float* pp, int64_t ndat, int64_t ntimes, int64_t nhead, int forward);
+/* vmath.cu:6864-6885 */
+int ko_softmax_direct_on_axis(float* pp, int64_t nrow, int64_t nvec, int64_t ncol);
+/* vmath.cu:6920-6942 */
+int ko_softmax_direct_on_axis_backward(float* pgp, const float* pp, int64_t nbat, int64_t ntimes, int64_t nhead,
+                                       const float* hCoef);
+/* vmath.cu:6977-6997 */
+int ko_mix_values(float* py, const float* pp, const float* pV, int64_t nbat, int64_t ntimes, int64_t nvec,
+                  int64_t nhead, int64_t npiece);
+/* vmath.cu:7029-7049 */
+int ko_mix_values_backward_prop(float* pgp, const float* pgy, const float* pV, int64_t nbat, int64_t ntimes,
+                                int64_t nvec, int64_t nhead, int64_t npiece);
+/* vmath.cu:7081-7101 */
+int ko_mix_values_backward_value(float* pgV, const float* pgy, const float* pp, int64_t nbat, int64_t ntimes,
+                                 int64_t nvec, int64_t nhead, int64_t npiece);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,258 @@
+"""ctypes binding of the CPU oracle (oracle/kai_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by ``__graft_entry__.smoke()`` and by
+the ``cpu_baseline`` leg of ``bench.py``.  The product package never imports it.
+
+Each wrapper takes and returns C-contiguous float32 numpy arrays and keeps the
+argument order of the reference's ``VMath`` methods
+(source/engine/support/vmath.h:65-66, 137-143, 234-241) without ``device``.
+"""
+import ctypes
+import os
+import subprocess
+import threading
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libkai_oracle.so")
+_lib = None
+
+_F = ctypes.POINTER(ctypes.c_float)
+_I64 = ctypes.c_int64
+_INT = ctypes.c_int
+
+ACT = {"none": 0, "relu": 1, "leaky": 2, "sigmoid": 3, "tanh": 4, "gelu": 5, "selu": 6, "mish": 7, "swish": 8,
+       "softmax": 9}
+
+
+def build(force=False):
+    """Compile the C restatement with the reference's strict-FP flags."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "libkai_oracle.so"])
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_LIB_PATH)
+        sig = {
+            "ko_matmul": [_F, _F, _F, _I64, _I64, _I64, _INT],
+            "ko_matmul_rows": [_F, _F, _F, _I64, _I64, _I64, _I64, _INT],
+            "ko_matmul_backward_x": [_F, _F, _F, _I64, _I64, _I64, _INT],
+            "ko_matmul_backward_w": [_F, _F, _F, _I64, _I64, _I64, _INT],
+            "ko_add_bias": [_F, _F, _F, _I64, _I64],
+            "ko_add_bias_backward_b": [_F, _F, _I64, _I64, _INT],
+            "ko_activate": [_F, _F, _I64, _I64, _INT, _F],
+            "ko_activate_backward": [_F, _F, _F, _I64, _I64, _INT, _F],
+            "ko_activate_backward_with_y": [_F, _F, _F, _I64, _I64, _INT, _F],
+            "ko_mult_on_heads": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F],
+            "ko_mult_on_heads_backward": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
+            "ko_set_mh_attention_mask": [_F, _I64, _I64, _I64, _INT],
+            "ko_softmax_direct_on_axis": [_F, _I64, _I64, _I64],
+            "ko_softmax_direct_on_axis_backward": [_F, _F, _I64, _I64, _I64, _F],
+            "ko_mix_values": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
+            "ko_mix_values_backward_prop": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
+            "ko_mix_values_backward_value": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
+        }
+        for name, args in sig.items():
+            fn = getattr(L, name)
+            fn.argtypes = args
+            fn.restype = _INT
+        _lib = L
+    return _lib
+
+
+class OracleError(RuntimeError):
+    def __init__(self, code):
+        super().__init__("oracle returned error code %d" % code)
+        self.code = code
+
+
+def _p(a):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_F)
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _hyper(v):
+    """float or None -> (keepalive, pointer); None is the reference's null HYPER (reads as 0)."""
+    if v is None:
+        return None, None
+    c = ctypes.c_float(v)
+    return c, ctypes.pointer(c)
+
+
+def _check(rc):
+    if rc != 0:
+        raise OracleError(rc)
+
+
+def matmul(w, x, acc_into=None):
+    """y[ndat,yvec] (+)= x[ndat,xvec] . w[yvec,xvec]^T"""
+    w, x = _f32(w), _f32(x)
+    yvec, xvec = w.shape
+    ndat = x.size // xvec
+    y = np.zeros((ndat, yvec), np.float32) if acc_into is None else _f32(acc_into).copy().reshape(ndat, yvec)
+    _check(lib().ko_matmul(_p(y), _p(w), _p(x), yvec, ndat, xvec, int(acc_into is not None)))
+    return y
+
+
+def matmul_rows(w, x, rows):
+    """Oracle rows ``rows`` (a list of row indices) of matmul(w, x); used to sample a big product."""
+    w, x = _f32(w), _f32(x)
+    yvec, xvec = w.shape
+    xs = np.ascontiguousarray(x.reshape(-1, xvec)[rows])
+    y = np.zeros((xs.shape[0], yvec), np.float32)
+    _check(lib().ko_matmul(_p(y), _p(w), _p(xs), yvec, xs.shape[0], xvec, 0))
+    return y
+
+
+def matmul_parallel(w, x, threads):
+    """matmul(w, x) with the rows spread over ``threads`` host threads (ctypes drops the GIL);
+    each element's summation order is unchanged, so the result is bit-identical."""
+    w, x = _f32(w), _f32(x)
+    yvec, xvec = w.shape
+    ndat = x.size // xvec
+    y = np.zeros((ndat, yvec), np.float32)
+    bounds = np.linspace(0, ndat, threads + 1).astype(np.int64)
+    L = lib()
+
+    def work(i):
+        L.ko_matmul_rows(_p(y), _p(w), _p(x), yvec, int(bounds[i]), int(bounds[i + 1]), xvec, 0)
+
+    ts = [threading.Thread(target=work, args=(i,)) for i in range(threads)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    return y
+
+
+def matmul_backward_x(gy, w, acc_into=None):
+    gy, w = _f32(gy), _f32(w)
+    yvec, xvec = w.shape
+    ndat = gy.size // yvec
+    gx = np.zeros((ndat, xvec), np.float32) if acc_into is None else _f32(acc_into).copy().reshape(ndat, xvec)
+    _check(lib().ko_matmul_backward_x(_p(gx), _p(gy), _p(w), yvec, ndat, xvec, int(acc_into is not None)))
+    return gx
+
+
+def matmul_backward_w(gy, x, yvec, xvec, acc_into=None):
+    gy, x = _f32(gy), _f32(x)
+    ndat = x.size // xvec
+    gw = np.zeros((yvec, xvec), np.float32) if acc_into is None else _f32(acc_into).copy().reshape(yvec, xvec)
+    _check(lib().ko_matmul_backward_w(_p(gw), _p(gy), _p(x), yvec, ndat, xvec, int(acc_into is not None)))
+    return gw
+
+
+def add_bias(a, b):
+    a, b = _f32(a), _f32(b)
+    ncol = b.size
+    y = np.empty_like(a)
+    _check(lib().ko_add_bias(_p(y), _p(a), _p(b), a.size // ncol, ncol))
+    return y
+
+
+def add_bias_backward_b(gy, ncol, acc_into=None):
+    gy = _f32(gy)
+    gb = np.zeros(ncol, np.float32) if acc_into is None else _f32(acc_into).copy()
+    _check(lib().ko_add_bias_backward_b(_p(gb), _p(gy), gy.size // ncol, ncol, int(acc_into is not None)))
+    return gb
+
+
+def activate(x, act, leaky_alpha=None):
+    x = _f32(x)
+    ncol = x.shape[-1]
+    y = np.empty_like(x)
+    keep, h = _hyper(leaky_alpha)
+    _check(lib().ko_activate(_p(y), _p(x), x.size // ncol, ncol, ACT[act] if isinstance(act, str) else act, h))
+    return y
+
+
+def activate_backward(gy, x, act, leaky_alpha=None):
+    gy, x = _f32(gy), _f32(x)
+    ncol = x.shape[-1]
+    gx = np.empty_like(x)
+    keep, h = _hyper(leaky_alpha)
+    _check(lib().ko_activate_backward(_p(gx), _p(gy), _p(x), x.size // ncol, ncol,
+                                      ACT[act] if isinstance(act, str) else act, h))
+    return gx
+
+
+def activate_backward_with_y(gy, y, act, leaky_alpha=None):
+    gy, y = _f32(gy), _f32(y)
+    ncol = y.shape[-1]
+    gx = np.empty_like(y)
+    keep, h = _hyper(leaky_alpha)
+    _check(lib().ko_activate_backward_with_y(_p(gx), _p(gy), _p(y), y.size // ncol, ncol,
+                                             ACT[act] if isinstance(act, str) else act, h))
+    return gx
+
+
+def mult_on_heads(K, Q, nhead, coef):
+    """K, Q: [nbat, ntimes, nvec] -> scores [nbat, ntimes, ntimes, nhead]"""
+    K, Q = _f32(K), _f32(Q)
+    nbat, ntimes, nvec = K.shape
+    p = np.empty((nbat, ntimes, ntimes, nhead), np.float32)
+    keep, h = _hyper(coef)
+    _check(lib().ko_mult_on_heads(_p(p), _p(K), _p(Q), nbat, ntimes, nvec, nhead, nvec // nhead, h))
+    return p
+
+
+def mult_on_heads_backward(gp, KQ, nhead):
+    gp, KQ = _f32(gp), _f32(KQ)
+    nbat, ntimes, nvec = KQ.shape
+    g = np.empty_like(KQ)
+    _check(lib().ko_mult_on_heads_backward(_p(g), _p(gp), _p(KQ), nbat, ntimes, nvec, nhead, nvec // nhead))
+    return g
+
+
+def set_mh_attention_mask(p, forward=True):
+    p = _f32(p).copy()
+    nbat, ntimes, _, nhead = p.shape
+    _check(lib().ko_set_mh_attention_mask(_p(p), nbat, ntimes, nhead, int(forward)))
+    return p
+
+
+def softmax_direct_on_axis(p, nrow, nvec, ncol):
+    p = _f32(p).copy()
+    _check(lib().ko_softmax_direct_on_axis(_p(p), nrow, nvec, ncol))
+    return p
+
+
+def softmax_direct_on_axis_backward(gp, p, coef):
+    gp, p = _f32(gp).copy(), _f32(p)
+    nbat, ntimes, _, nhead = p.shape
+    keep, h = _hyper(coef)
+    _check(lib().ko_softmax_direct_on_axis_backward(_p(gp), _p(p), nbat, ntimes, nhead, h))
+    return gp
+
+
+def mix_values(p, V, nhead):
+    p, V = _f32(p), _f32(V)
+    nbat, ntimes, nvec = V.shape
+    y = np.empty((nbat, ntimes, nvec), np.float32)
+    _check(lib().ko_mix_values(_p(y), _p(p), _p(V), nbat, ntimes, nvec, nhead, nvec // nhead))
+    return y
+
+
+def mix_values_backward_prop(gy, V, nhead):
+    gy, V = _f32(gy), _f32(V)
+    nbat, ntimes, nvec = V.shape
+    gp = np.empty((nbat, ntimes, ntimes, nhead), np.float32)
+    _check(lib().ko_mix_values_backward_prop(_p(gp), _p(gy), _p(V), nbat, ntimes, nvec, nhead, nvec // nhead))
+    return gp
+
+
+def mix_values_backward_value(gy, p, nhead):
+    gy, p = _f32(gy), _f32(p)
+    nbat, ntimes, nvec = gy.shape
+    gV = np.empty((nbat, ntimes, nvec), np.float32)
+    _check(lib().ko_mix_values_backward_value(_p(gV), _p(gy), _p(p), nbat, ntimes, nvec, nhead, nvec // nhead))
+    return gV

@@ -1,0 +1,462 @@
+"""Parity of the HIP path with the CPU oracle, through the C-ABI, on the five benchmark
+configurations and on the edge cases of the path.  Bar: relative Frobenius error <= 1e-5
+(fp32, differences of summation order only); exact where no arithmetic is involved."""
+import numpy as np
+import pytest
+
+from util import REL_FRO_TOL, cfg1, cfg2, cfg3, cfg4, cfg5, ko, rel_fro
+
+pytestmark = pytest.mark.gpu
+
+kai = None
+VMath = None
+DB = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _lib():
+    global kai, VMath, DB
+    from deep_learning_framework_amd import kai as _kai
+    kai = _kai
+    VMath = _kai.VMath
+    DB = _kai.DeviceBuffer
+    kai.load()
+    kai.set_device(0)
+    yield
+    kai.synchronize()
+
+
+def dev(a):
+    return DB.from_numpy(np.ascontiguousarray(a, np.float32))
+
+
+def check(got, ref, tol=REL_FRO_TOL, what=""):
+    err = rel_fro(got, ref)
+    assert np.isfinite(got).all(), what + ": non-finite output"
+    assert err <= tol, "%s: rel Frobenius error %.3e > %.1e" % (what, err, tol)
+
+
+# ---- configuration 1: dense forward 64 x 784 -> 512, ReLU ------------------------------------------
+
+def test_cfg1_dense_forward_unfused_and_fused():
+    x, w, b = cfg1()
+    ref_pre = ko.add_bias(ko.matmul(w, x), b)
+    ref = ko.activate(ref_pre, "relu")
+    dx, dw, db = dev(x), dev(w), dev(b)
+    # the engine's three calls: matmul -> add_bias -> activate (api/vconst.cpp:11)
+    y = DB(64 * 512 * 4)
+    VMath.matmul(0, y, dw, dx, 512, 64, 784, False)
+    VMath.add_bias(0, y, y, db, 64, 512)
+    VMath.activate(0, y, y, 64, 512, kai.ACT["relu"], None)
+    check(y.to_numpy((64, 512)), ref, what="cfg1 unfused")
+    # one launch
+    y2, pre = DB(64 * 512 * 4), DB(64 * 512 * 4)
+    VMath.dense_forward(0, y2, pre, dw, db, dx, 512, 64, 784, kai.ACT["relu"], None)
+    check(y2.to_numpy((64, 512)), ref, what="cfg1 fused")
+    check(pre.to_numpy((64, 512)), ref_pre, what="cfg1 fused pre-activation")
+    # BASELINE layout W'[784,512] = w.T as a row-major [K,N] operand
+    wt = dev(np.ascontiguousarray(w.T))
+    y3 = DB(64 * 512 * 4)
+    VMath.gemm_f32(0, 0, 0, 64, 512, 784, dx, 784, wt, 512, y3, 512, db, kai.ACT["relu"], None, False)
+    check(y3.to_numpy((64, 512)), ref, what="cfg1 [K,N] weight layout")
+
+
+# ---- configuration 2: dense forward + backward 256 x 1024 -> 1024 ---------------------------------------
+
+def test_cfg2_dense_forward_backward():
+    x, w, b, gy = cfg2()
+    ref_y = ko.add_bias(ko.matmul(w, x), b)
+    ref_gx = ko.matmul_backward_x(gy, w)
+    ref_gw = ko.matmul_backward_w(gy, x, 1024, 1024)
+    ref_gb = ko.add_bias_backward_b(gy, 1024)
+    dx, dw, db, dgy = dev(x), dev(w), dev(b), dev(gy)
+    y = DB(256 * 1024 * 4)
+    VMath.matmul(0, y, dw, dx, 1024, 256, 1024, False)
+    VMath.add_bias(0, y, y, db, 256, 1024)
+    check(y.to_numpy((256, 1024)), ref_y, what="cfg2 Y")
+    gx, gw, gb = DB(256 * 1024 * 4), DB(1024 * 1024 * 4), DB(1024 * 4)
+    VMath.matmul_backward_x(0, gx, dgy, dw, 1024, 256, 1024, False)
+    VMath.matmul_backward_w(0, gw, dgy, dx, 1024, 256, 1024, False)
+    VMath.add_bias_backward_b(0, gb, dgy, 256, 1024, False)
+    check(gx.to_numpy((256, 1024)), ref_gx, what="cfg2 dX")
+    check(gw.to_numpy((1024, 1024)), ref_gw, what="cfg2 dW")
+    check(gb.to_numpy((1024,)), ref_gb, what="cfg2 db")
+    # fused backward entry point, no activation
+    gx2, gw2, gb2 = DB(256 * 1024 * 4), DB(1024 * 1024 * 4), DB(1024 * 4)
+    VMath.dense_backward(0, gx2, gw2, gb2, None, dgy, dw, dx, None, 1024, 256, 1024, kai.ACT["none"], None, False)
+    check(gx2.to_numpy((256, 1024)), ref_gx, what="cfg2 fused dX")
+    check(gw2.to_numpy((1024, 1024)), ref_gw, what="cfg2 fused dW")
+    check(gb2.to_numpy((1024,)), ref_gb, what="cfg2 fused db")
+
+
+def test_cfg2_relu_backward_chain():
+    x, w, b, gy = cfg2()
+    pre = ko.add_bias(ko.matmul(w, x), b)
+    ga = ko.activate_backward(gy, pre, "relu")
+    ref_gx = ko.matmul_backward_x(ga, w)
+    ref_gw = ko.matmul_backward_w(ga, x, 1024, 1024)
+    ref_gb = ko.add_bias_backward_b(ga, 1024)
+    dx, dw, dgy, dpre = dev(x), dev(w), dev(gy), dev(pre)
+    gx, gw, gb, work = DB(256 * 1024 * 4), DB(1024 * 1024 * 4), DB(1024 * 4), DB(256 * 1024 * 4)
+    VMath.dense_backward(0, gx, gw, gb, work, dgy, dw, dx, dpre, 1024, 256, 1024, kai.ACT["relu"], None, False)
+    check(gx.to_numpy((256, 1024)), ref_gx, what="relu chain dX")
+    check(gw.to_numpy((1024, 1024)), ref_gw, what="relu chain dW")
+    check(gb.to_numpy((1024,)), ref_gb, what="relu chain db")
+
+
+# ---- configuration 3: 8192^3 GEMM + bias + ReLU -------------------------------------------------------------
+
+def test_cfg3_large_gemm_bias_relu_row_sample():
+    n = 8192
+    a, b, bias = cfg3(n)
+    da, dbm, dbias = dev(a), dev(b), dev(bias)
+    c = DB(n * n * 4)
+    # row-major A.B: B is a [K,N] operand
+    VMath.gemm_f32(0, 0, 0, n, n, n, da, n, dbm, n, c, n, dbias, kai.ACT["relu"], None, False)
+    got = c.to_numpy((n, n))
+    rows = np.sort(np.random.default_rng(33).choice(n, 48, replace=False))
+    bt = np.ascontiguousarray(b.T)
+    ref = ko.activate(ko.add_bias(ko.matmul_rows(bt, a, rows), bias), "relu")
+    check(got[rows], ref, what="cfg3 NN sampled rows")
+    # engine layout: the same product with B pre-stored [N,K], fused dense entry point
+    dbt = dev(bt)
+    c2 = DB(n * n * 4)
+    VMath.dense_forward(0, c2, None, dbt, dbias, da, n, n, n, kai.ACT["relu"], None)
+    got2 = c2.to_numpy((n, n))
+    check(got2[rows], ref, what="cfg3 NT sampled rows")
+    # whole matrix: the two operand forms must agree with each other far inside the tolerance
+    check(got2, got, tol=2e-6, what="cfg3 NN vs NT full matrix")
+    # linearity over the full size: relu(A.B + bias) has no negative entry and the share of
+    # positive entries of a symmetric product is one half
+    assert (got >= 0).all()
+    assert abs((got > 0).mean() - 0.5) < 0.01
+
+
+# ---- configuration 4: attention batched matmul ---------------------------------------------------------------
+
+@pytest.mark.parametrize("nbat,nhead,nvec", [(32, 1, 64), (4, 8, 512)])
+def test_cfg4_attention_forward(nbat, nhead, nvec):
+    ntimes = 512
+    npiece = nvec // nhead
+    q, k, v = cfg4(nbat, ntimes, nvec)
+    coef = 1.0 / np.sqrt(npiece)
+    ref_s = ko.mult_on_heads(k, q, nhead, coef)
+    ref_p = ko.softmax_direct_on_axis(ref_s, nbat * ntimes, ntimes, nhead)
+    ref_o = ko.mix_values(ref_p, v, nhead)
+    dq, dk, dv = dev(q), dev(k), dev(v)
+    hcoef = kai.hyper(coef)
+    p = DB(nbat * ntimes * ntimes * nhead * 4)
+    VMath.mult_on_heads(0, p, dk, dq, nbat, ntimes, nvec, nhead, npiece, hcoef)
+    check(p.to_numpy(ref_s.shape), ref_s, what="cfg4 scores")
+    VMath.softmax_direct_on_axis(0, p, nbat * ntimes, ntimes, nhead)
+    got_p = p.to_numpy(ref_p.shape)
+    check(got_p, ref_p, what="cfg4 softmax")
+    np.testing.assert_allclose(got_p.sum(axis=2), 1.0, atol=1e-5)
+    o = DB(nbat * ntimes * nvec * 4)
+    VMath.mix_values(0, o, p, dv, nbat, ntimes, nvec, nhead, npiece)
+    check(o.to_numpy((nbat, ntimes, nvec)), ref_o, what="cfg4 output")
+
+
+# ---- configuration 5: skinny and ragged ------------------------------------------------------------------------
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_cfg5_skinny(m):
+    w, x = cfg5(m)
+    ref = ko.matmul(w, x)
+    dw, dx = dev(w), dev(x)
+    y = DB(m * 4096 * 4)
+    VMath.matmul(0, y, dw, dx, 4096, m, 4096, False)
+    check(y.to_numpy((m, 4096)), ref, what="cfg5 M=%d" % m)
+    # [K,N] weight layout of the same product
+    wt = dev(np.ascontiguousarray(w.T))
+    y2 = DB(m * 4096 * 4)
+    VMath.gemm_f32(0, 0, 0, m, 4096, 4096, dx, 4096, wt, 4096, y2, 4096, None, kai.ACT["none"], None, False)
+    check(y2.to_numpy((m, 4096)), ref, what="cfg5 M=%d [K,N] layout" % m)
+
+
+def test_cfg5_ragged():
+    m, k, n = 1000, 777, 333
+    w, x = cfg5(m, k, n)
+    gy = (0.01 * np.random.default_rng(55).standard_normal((m, n))).astype(np.float32)
+    dw, dx, dgy = dev(w), dev(x), dev(gy)
+    y, gx, gw = DB(m * n * 4), DB(m * k * 4), DB(n * k * 4)
+    VMath.matmul(0, y, dw, dx, n, m, k, False)
+    VMath.matmul_backward_x(0, gx, dgy, dw, n, m, k, False)
+    VMath.matmul_backward_w(0, gw, dgy, dx, n, m, k, False)
+    check(y.to_numpy((m, n)), ko.matmul(w, x), what="ragged Y")
+    check(gx.to_numpy((m, k)), ko.matmul_backward_x(gy, w), what="ragged dX")
+    check(gw.to_numpy((n, k)), ko.matmul_backward_w(gy, x, n, k), what="ragged dW")
+
+
+# ---- shapes around the tile edges, every operand form, acc, unaligned pointers ---------------------------------
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 9), (64, 64, 64), (65, 63, 66), (100, 300, 50), (128, 128, 32),
+          (129, 257, 40), (256, 256, 16), (300, 520, 128), (31, 1000, 4), (513, 64, 260), (40, 24, 1000)]
+
+
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemm_all_operand_forms(m, n, k):
+    rng = np.random.default_rng(m * 1000003 + n * 1009 + k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    bt = np.ascontiguousarray(b.T)
+    at = np.ascontiguousarray(a.T)
+    ref = ko.matmul(bt, a)                       # a . b
+    ref_acc = ko.matmul(bt, a, acc_into=c0)
+    ref_full = ko.activate(ko.add_bias(ref_acc, bias), "leaky", 0.1)
+    da, dat, dbm, dbt, dbias = dev(a), dev(at), dev(b), dev(bt), dev(bias)
+    alpha = kai.hyper(0.1)
+    for ta, tb, A, lda, B, ldb in [(0, 1, da, k, dbt, k), (0, 0, da, k, dbm, n), (1, 0, dat, m, dbm, n),
+                                   (1, 1, dat, m, dbt, k)]:
+        c = DB(m * n * 4)
+        VMath.gemm_f32(0, ta, tb, m, n, k, A, lda, B, ldb, c, n, None, 0, None, False)
+        check(c.to_numpy((m, n)), ref, what="gemm form (%d,%d) %dx%dx%d" % (ta, tb, m, n, k))
+        c = dev(c0)
+        VMath.gemm_f32(0, ta, tb, m, n, k, A, lda, B, ldb, c, n, dbias, kai.ACT["leaky"], alpha, True)
+        check(c.to_numpy((m, n)), ref_full, what="gemm form (%d,%d) acc+bias+leaky" % (ta, tb))
+
+
+def test_engine_calls_with_acc_and_unaligned_subbuffers():
+    # the RNN driver passes base + t*size pointers and acc = true (vtensor.cpp:2462-2474)
+    rng = np.random.default_rng(7)
+    ndat, xvec, yvec = 37, 53, 29
+    x = rng.standard_normal((ndat, xvec)).astype(np.float32)
+    w = rng.standard_normal((yvec, xvec)).astype(np.float32)
+    y0 = rng.standard_normal((ndat, yvec)).astype(np.float32)
+    pad = 3   # floats: shifts every pointer off 16-byte alignment
+    bx = dev(np.concatenate([np.zeros(pad, np.float32), x.ravel()]))
+    bw = dev(np.concatenate([np.zeros(pad, np.float32), w.ravel()]))
+    by = dev(np.concatenate([np.zeros(pad, np.float32), y0.ravel()]))
+    VMath.matmul(0, by.offset(4 * pad), bw.offset(4 * pad), bx.offset(4 * pad), yvec, ndat, xvec, True)
+    got = by.to_numpy((pad + ndat * yvec,))[pad:].reshape(ndat, yvec)
+    check(got, ko.matmul(w, x, acc_into=y0), what="acc + unaligned matmul")
+    gy = rng.standard_normal((ndat, yvec)).astype(np.float32)
+    bgy = dev(np.concatenate([np.zeros(pad, np.float32), gy.ravel()]))
+    gx0 = rng.standard_normal((ndat, xvec)).astype(np.float32)
+    gw0 = rng.standard_normal((yvec, xvec)).astype(np.float32)
+    bgx = dev(np.concatenate([np.zeros(pad, np.float32), gx0.ravel()]))
+    bgw = dev(np.concatenate([np.zeros(pad, np.float32), gw0.ravel()]))
+    VMath.matmul_backward_x(0, bgx.offset(4 * pad), bgy.offset(4 * pad), bw.offset(4 * pad), yvec, ndat, xvec, True)
+    VMath.matmul_backward_w(0, bgw.offset(4 * pad), bgy.offset(4 * pad), bx.offset(4 * pad), yvec, ndat, xvec, True)
+    check(bgx.to_numpy((pad + ndat * xvec,))[pad:].reshape(ndat, xvec), ko.matmul_backward_x(gy, w, acc_into=gx0),
+          what="acc + unaligned backward_x")
+    check(bgw.to_numpy((pad + yvec * xvec,))[pad:].reshape(yvec, xvec),
+          ko.matmul_backward_w(gy, x, yvec, xvec, acc_into=gw0), what="acc + unaligned backward_w")
+
+
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 4096), (2, 1000, 300), (7, 130, 1024), (16, 4100, 257), (16, 3, 5),
+                                   (5, 8192, 256)])
+def test_skinny_shapes_bias_act_acc(m, k, n):
+    rng = np.random.default_rng(m + k + n)
+    w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    y0 = rng.standard_normal((m, n)).astype(np.float32)
+    dw, dx, db = dev(w), dev(x), dev(b)
+    y, pre = DB(m * n * 4), DB(m * n * 4)
+    VMath.dense_forward(0, y, pre, dw, db, dx, n, m, k, kai.ACT["relu"], None)
+    ref_pre = ko.add_bias(ko.matmul(w, x), b)
+    check(pre.to_numpy((m, n)), ref_pre, what="skinny pre")
+    check(y.to_numpy((m, n)), ko.activate(ref_pre, "relu"), what="skinny relu")
+    ya = dev(y0)
+    VMath.matmul(0, ya, dw, dx, n, m, k, True)
+    check(ya.to_numpy((m, n)), ko.matmul(w, x, acc_into=y0), what="skinny acc")
+
+
+def test_empty_and_degenerate_sizes():
+    d = dev(np.ones(16, np.float32))
+    out = dev(np.full(16, 7.0, np.float32))
+    VMath.matmul(0, out, d, d, 4, 0, 4, False)          # no rows: nothing written
+    VMath.matmul(0, out, d, d, 0, 4, 4, False)
+    np.testing.assert_array_equal(out.to_numpy((16,)), 7.0)
+    VMath.matmul(0, out, d, d, 4, 4, 0, False)          # empty reduction: zeros
+    np.testing.assert_array_equal(out.to_numpy((16,)), 0.0)
+    VMath.add_bias(0, out, d, d, 0, 4)
+    VMath.add_bias_backward_b(0, out, d, 0, 4, False)   # column sum over no rows: zeros
+    np.testing.assert_array_equal(out.to_numpy((16,))[:4], 0.0)
+    VMath.softmax_direct_on_axis(0, out, 0, 4, 1)
+    VMath.activate(0, out, d, 0, 0, 1, None)
+
+
+# ---- bias, activations ----------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("nrow,ncol", [(1, 1), (7, 13), (256, 1024), (33, 4), (1000, 333), (5000, 64)])
+def test_add_bias_and_column_sum(nrow, ncol):
+    rng = np.random.default_rng(nrow * 31 + ncol)
+    a = rng.standard_normal((nrow, ncol)).astype(np.float32)
+    b = rng.standard_normal(ncol).astype(np.float32)
+    da, db = dev(a), dev(b)
+    y = DB(nrow * ncol * 4)
+    VMath.add_bias(0, y, da, db, nrow, ncol)
+    np.testing.assert_array_equal(y.to_numpy((nrow, ncol)), ko.add_bias(a, b))
+    VMath.add_bias(0, da, da, db, nrow, ncol)   # in place, as the attention layer calls it
+    np.testing.assert_array_equal(da.to_numpy((nrow, ncol)), ko.add_bias(a, b))
+    gb0 = rng.standard_normal(ncol).astype(np.float32)
+    gb = dev(gb0)
+    dgy = dev(a)
+    VMath.add_bias_backward_b(0, gb, dgy, nrow, ncol, False)
+    check(gb.to_numpy((ncol,)), ko.add_bias_backward_b(a, ncol), what="colsum")
+    gb = dev(gb0)
+    VMath.add_bias_backward_b(0, gb, dgy, nrow, ncol, True)
+    check(gb.to_numpy((ncol,)), ko.add_bias_backward_b(a, ncol, acc_into=gb0), what="colsum acc")
+
+
+ACT_NAMES = ["none", "relu", "leaky", "sigmoid", "tanh", "gelu", "selu", "mish", "swish"]
+
+
+@pytest.mark.parametrize("act", ACT_NAMES)
+def test_activate_and_backward(act):
+    rng = np.random.default_rng(11)
+    x = (3 * rng.standard_normal((37, 101))).astype(np.float32)
+    x[0, :6] = [0.0, -0.0, np.inf, -np.inf, 1e-30, -1e-30]
+    gy = rng.standard_normal(x.shape).astype(np.float32)
+    alpha = 0.1 if act == "leaky" else None
+    h = kai.hyper(alpha)
+    dx, dgy = dev(x), dev(gy)
+    y, gx = DB(x.nbytes), DB(x.nbytes)
+    VMath.activate(0, y, dx, 37, 101, kai.ACT[act], h)
+    ref = ko.activate(x, act, alpha)
+    got = y.to_numpy(x.shape)
+    finite = np.isfinite(ref)
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(ref))
+    np.testing.assert_allclose(got[finite], ref[finite], rtol=2e-6, atol=1e-7)
+    xs = x.copy()
+    xs[0, :6] = [0.0, -0.0, 50.0, -50.0, 1e-30, -1e-30]
+    dxs = dev(xs)
+    VMath.activate_backward(0, gx, dgy, dxs, 37, 101, kai.ACT[act], h)
+    np.testing.assert_allclose(gx.to_numpy(x.shape), ko.activate_backward(gy, xs, act, alpha), rtol=1e-5, atol=1e-6)
+    if act in ("none", "relu", "leaky", "sigmoid", "tanh"):
+        yv = ko.activate(xs, act, alpha)
+        dy = dev(yv)
+        VMath.activate_backward_with_y(0, gx, dgy, dy, 37, 101, kai.ACT[act], h)
+        np.testing.assert_allclose(gx.to_numpy(x.shape), ko.activate_backward_with_y(gy, yv, act, alpha), rtol=1e-5,
+                                   atol=1e-6)
+    # in place (vtensor.cpp:2480)
+    VMath.activate(0, dx, dx, 37, 101, kai.ACT[act], h)
+    np.testing.assert_array_equal(dx.to_numpy(x.shape), got)
+
+
+def test_relu_special_values_and_null_leaky_alpha():
+    x = np.array([[-0.0, 0.0, np.nan, np.inf, -np.inf, -1.5, 2.5, 1e-45]], np.float32)
+    dx = dev(x)
+    y = DB(x.nbytes)
+    VMath.activate(0, y, dx, 1, 8, kai.ACT["relu"], None)
+    got = y.to_numpy(x.shape)
+    np.testing.assert_array_equal(got, ko.activate(x, "relu"))
+    assert not np.signbit(got[0, 0]) and got[0, 2] == 0.0   # -0 -> +0, NaN -> 0
+    VMath.activate(0, y, dx, 1, 8, kai.ACT["leaky"], None)   # null HYPER reads as alpha = 0
+    ref = ko.activate(x, "leaky", None)
+    got = y.to_numpy(x.shape)
+    np.testing.assert_array_equal(np.isnan(got), np.isnan(ref))
+    np.testing.assert_array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)])
+
+
+def test_softmax_activation_rows():
+    rng = np.random.default_rng(5)
+    x = (4 * rng.standard_normal((50, 77))).astype(np.float32)
+    gy = rng.standard_normal(x.shape).astype(np.float32)
+    dx, dgy = dev(x), dev(gy)
+    y, gx = DB(x.nbytes), DB(x.nbytes)
+    VMath.activate(0, y, dx, 50, 77, kai.ACT["softmax"], None)
+    ref = ko.activate(x, "softmax")
+    check(y.to_numpy(x.shape), ref, what="softmax activation")
+    VMath.activate_backward(0, gx, dgy, dx, 50, 77, kai.ACT["softmax"], None)
+    p = ref.astype(np.float64)
+    ref_g = p * (gy - (p * gy).sum(axis=1, keepdims=True))
+    check(gx.to_numpy(x.shape), ref_g, what="softmax activation backward")
+
+
+# ---- attention ops at small sizes, masks, backward --------------------------------------------------------------------
+
+@pytest.mark.parametrize("nbat,ntimes,nhead,npiece", [(2, 5, 1, 3), (3, 17, 4, 8), (1, 64, 2, 64), (2, 33, 3, 5),
+                                                      (1, 130, 1, 64), (1, 7, 200, 2)])
+def test_attention_ops_small(nbat, ntimes, nhead, npiece):
+    nvec = nhead * npiece
+    rng = np.random.default_rng(nbat * 100 + ntimes * 10 + nhead)
+    q = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    k = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    v = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    gy = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    coef = 1.0 / np.sqrt(npiece)
+    hcoef = kai.hyper(coef)
+    dq, dk, dv, dgy = dev(q), dev(k), dev(v), dev(gy)
+    pshape = (nbat, ntimes, ntimes, nhead)
+    p = DB(int(np.prod(pshape)) * 4)
+    VMath.mult_on_heads(0, p, dk, dq, nbat, ntimes, nvec, nhead, npiece, hcoef)
+    ref_s = ko.mult_on_heads(k, q, nhead, coef)
+    check(p.to_numpy(pshape), ref_s, what="scores")
+    VMath.set_mh_attention_mask(0, p, nbat, ntimes, nhead, True)
+    ref_m = ko.set_mh_attention_mask(ref_s, True)
+    np.testing.assert_array_equal(np.isinf(p.to_numpy(pshape)), np.isinf(ref_m))
+    VMath.softmax_direct_on_axis(0, p, nbat * ntimes, ntimes, nhead)
+    ref_p = ko.softmax_direct_on_axis(ref_m, nbat * ntimes, ntimes, nhead)
+    got_p = p.to_numpy(pshape)
+    check(got_p, ref_p, what="masked softmax")
+    assert (got_p[np.isinf(ref_m)] == 0).all()          # masked entries are exactly 0
+    o = DB(nbat * ntimes * nvec * 4)
+    dp = dev(ref_p)
+    VMath.mix_values(0, o, dp, dv, nbat, ntimes, nvec, nhead, npiece)
+    check(o.to_numpy((nbat, ntimes, nvec)), ko.mix_values(ref_p, v, nhead), what="mix_values")
+    # backward ops, fed with oracle intermediates so that each op is compared on equal inputs
+    gp = DB(int(np.prod(pshape)) * 4)
+    VMath.mix_values_backward_prop(0, gp, dgy, dv, nbat, ntimes, nvec, nhead, npiece)
+    ref_gp = ko.mix_values_backward_prop(gy, v, nhead)
+    check(gp.to_numpy(pshape), ref_gp, what="mix_values_backward_prop")
+    gv = DB(nbat * ntimes * nvec * 4)
+    VMath.mix_values_backward_value(0, gv, dgy, dp, nbat, ntimes, nvec, nhead, npiece)
+    check(gv.to_numpy((nbat, ntimes, nvec)), ko.mix_values_backward_value(gy, ref_p, nhead),
+          what="mix_values_backward_value")
+    dgp = dev(ref_gp)
+    VMath.softmax_direct_on_axis_backward(0, dgp, dp, nbat, ntimes, nhead, hcoef)
+    ref_gs = ko.softmax_direct_on_axis_backward(ref_gp, ref_p, coef)
+    check(dgp.to_numpy(pshape), ref_gs, what="softmax backward")
+    VMath.set_mh_attention_mask(0, dgp, nbat, ntimes, nhead, False)
+    ref_gs = ko.set_mh_attention_mask(ref_gs, False)
+    dgs = dev(ref_gs)
+    gk = DB(nbat * ntimes * nvec * 4)
+    VMath.mult_on_heads_backward(0, gk, dgs, dq, nbat, ntimes, nvec, nhead, npiece)
+    check(gk.to_numpy((nbat, ntimes, nvec)), ko.mult_on_heads_backward(ref_gs, q, nhead), what="mult_on_heads_backward")
+
+
+@pytest.mark.parametrize("nrow,nvec,ncol", [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8),
+                                            (3, 20, 128), (2, 9, 129), (2, 5, 300)])
+def test_softmax_axis_layouts(nrow, nvec, ncol):
+    rng = np.random.default_rng(nrow + nvec + ncol)
+    s = (5 * rng.standard_normal((nrow, nvec, ncol))).astype(np.float32)
+    d = dev(s)
+    VMath.softmax_direct_on_axis(0, d, nrow, nvec, ncol)
+    check(d.to_numpy(s.shape), ko.softmax_direct_on_axis(s, nrow, nvec, ncol), what="softmax axis")
+
+
+# ---- memory helpers and errors ----------------------------------------------------------------------------------------
+
+def test_memory_helpers():
+    a = np.arange(1000, dtype=np.float32)
+    d = dev(a)
+    e = DB(a.nbytes)
+    VMath.copy_data(0, 0, e, d, a.nbytes)
+    np.testing.assert_array_equal(e.to_numpy(a.shape), a)
+    VMath.set_zero(0, e, 400)
+    got = e.to_numpy(a.shape)
+    assert (got[:100] == 0).all() and (got[100:] == a[100:]).all()
+    VMath.fill_float(0, e, 10, 2.5)
+    assert (e.to_numpy(a.shape)[:10] == 2.5).all()
+    VMath.fill_int(0, e, 3, 7)
+    assert (e.to_numpy(a.shape, np.int32)[:3] == 7).all()
+    VMath.get_slice(0, e, d.offset(400), 400)
+    np.testing.assert_array_equal(e.to_numpy(a.shape)[:100], a[100:200])
+    assert kai.arch_info()[0] == "gfx950" and "gfx950" in kai.arch_info()[1]
+
+
+def test_errors_do_not_poison_the_stream():
+    d = dev(np.ones(4, np.float32))
+    with pytest.raises(kai.KaiError) as e:
+        VMath.activate(0, d, d, 1, 4, 42, None)
+    assert e.value.code == 8
+    with pytest.raises(kai.KaiError) as e:
+        VMath.matmul(-1, d, d, d, 1, 1, 1, False)
+    assert e.value.code == 510
+    VMath.activate(0, d, d, 1, 4, 1, None)   # the library still works afterwards
+    np.testing.assert_array_equal(d.to_numpy((4,)), 1.0)
