@@ -1,0 +1,74 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/matmul_path_small.npz: inputs and expected outputs of every operator of
+the matmul path at small shapes.
+
+The reference ships no golden vectors, known-answer tests or fixtures for this path and cannot be
+built or run here, so the expected outputs are produced by the CPU oracle (oracle/kai_oracle.c),
+which tests/test_oracle_pins.py pins against closed forms.  The fixture freezes those outputs so
+that a later change of the oracle, of its compiler flags or of the host libm shows up as a diff,
+and gives the GPU tests a fixed data set.  Run from the repository root:
+
+    python tests/golden/make_golden.py
+"""
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+import oracle as ko  # noqa: E402
+
+
+def main():
+    rng = np.random.default_rng(20240607)
+    f = {}
+    # dense layer: ndat 19, xvec 23, yvec 11 (all distinct, none a multiple of 4)
+    ndat, xvec, yvec = 19, 23, 11
+    x = rng.standard_normal((ndat, xvec)).astype(np.float32)
+    w = rng.uniform(-0.2, 0.2, (yvec, xvec)).astype(np.float32)
+    b = rng.standard_normal(yvec).astype(np.float32)
+    gy = rng.standard_normal((ndat, yvec)).astype(np.float32)
+    f.update(dense_x=x, dense_w=w, dense_b=b, dense_gy=gy)
+    f["dense_matmul"] = ko.matmul(w, x)
+    f["dense_pre"] = ko.add_bias(f["dense_matmul"], b)
+    f["dense_gx"] = ko.matmul_backward_x(gy, w)
+    f["dense_gw"] = ko.matmul_backward_w(gy, x, yvec, xvec)
+    f["dense_gb"] = ko.add_bias_backward_b(gy, yvec)
+    f["dense_matmul_acc"] = ko.matmul(w, x, acc_into=f["dense_pre"])
+    for name in ["none", "relu", "leaky", "sigmoid", "tanh", "gelu", "selu", "mish", "swish", "softmax"]:
+        alpha = 0.1 if name == "leaky" else None
+        f["act_" + name] = ko.activate(f["dense_pre"], name, alpha)
+        if name != "softmax":
+            f["actbwd_" + name] = ko.activate_backward(gy, f["dense_pre"], name, alpha)
+        if name in ("none", "relu", "leaky", "sigmoid", "tanh"):
+            f["actbwdy_" + name] = ko.activate_backward_with_y(gy, f["act_" + name], name, alpha)
+    # attention: nbat 2, ntimes 9, nhead 3, npiece 5
+    nbat, ntimes, nhead, npiece = 2, 9, 3, 5
+    nvec = nhead * npiece
+    q = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    k = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    v = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    go = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    coef = np.float32(1.0 / np.sqrt(npiece))
+    f.update(att_q=q, att_k=k, att_v=v, att_go=go, att_coef=np.array([coef], np.float32),
+             att_dims=np.array([nbat, ntimes, nhead, npiece], np.int64))
+    s = ko.mult_on_heads(k, q, nhead, float(coef))
+    f["att_scores"] = s
+    f["att_masked"] = ko.set_mh_attention_mask(s, True)
+    f["att_probs"] = ko.softmax_direct_on_axis(s, nbat * ntimes, ntimes, nhead)
+    f["att_probs_masked"] = ko.softmax_direct_on_axis(f["att_masked"], nbat * ntimes, ntimes, nhead)
+    f["att_out"] = ko.mix_values(f["att_probs"], v, nhead)
+    f["att_gprobs"] = ko.mix_values_backward_prop(go, v, nhead)
+    f["att_gv"] = ko.mix_values_backward_value(go, f["att_probs"], nhead)
+    f["att_gscores"] = ko.softmax_direct_on_axis_backward(f["att_gprobs"], f["att_probs"], float(coef))
+    f["att_gk"] = ko.mult_on_heads_backward(f["att_gscores"], q, nhead)
+    f["att_gq"] = ko.mult_on_heads_backward(f["att_gscores"], k, nhead)
+    out = os.path.join(HERE, "matmul_path_small.npz")
+    np.savez_compressed(out, **f)
+    print("wrote", out, os.path.getsize(out), "bytes,", len(f), "arrays")
+
+
+if __name__ == "__main__":
+    main()

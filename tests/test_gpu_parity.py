@@ -321,7 +321,10 @@ def test_activate_and_backward(act):
     got = y.to_numpy(x.shape)
     finite = np.isfinite(ref)
     np.testing.assert_array_equal(np.isnan(got), np.isnan(ref))
-    np.testing.assert_allclose(got[finite], ref[finite], rtol=2e-6, atol=1e-7)
+    # device expf/logf/erff differ from the host libm in the last ulp; cancellation in the
+    # exp-based forms magnifies that for small outputs, hence the absolute term
+    np.testing.assert_allclose(got[finite], ref[finite], rtol=1e-5, atol=1e-6)
+    check(got[finite], ref[finite], what="activate " + act)
     xs = x.copy()
     xs[0, :6] = [0.0, -0.0, 50.0, -50.0, 1e-30, -1e-30]
     dxs = dev(xs)
