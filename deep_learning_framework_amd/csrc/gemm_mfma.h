@@ -204,7 +204,16 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // EDGE = false: the host has checked that M, N, K are multiples of the tile, that both operands
 // allow aligned 128-bit loads and that a tile's offsets fit 32 bits; the kernel then holds no
 // predicated load code at all (fewer registers).  EDGE = true: general shapes.
-template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE>
+//
+// PIPE selects the schedule of the main loop:
+//   0  per K-tile: all fragment reads of a group, then its MFMAs; LDS stores and the barrier at the
+//      end of the tile.
+//   1  fragments double buffered: the reads of group g+1 are issued with the MFMAs of group g and
+//      spread between them, so the waves of a workgroup do not hit LDS in one burst and no MFMA
+//      waits for an LDS round trip.  The next tile is stored to LDS while the second-to-last group
+//      computes; the barrier sits before the last group, whose MFMAs (operands already in
+//      registers) cover the first fragment reads of the next tile.
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0>
 __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const GemmParams p) {
     constexpr int NT = 64 * WM * WN;
     constexpr int BM = WM * NBM * 32;
@@ -282,32 +291,96 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const GemmParam
     }
     __syncthreads();
 
-    for (int kt = 0; kt < nkt; kt++) {
-        const int cur = kt & 1;
-        if (kt + 1 < nkt) load_global(kt + 1);
+    constexpr int NKG = BK / 8;
+    auto mfma_group = [&](const Frag<A_KC, NBM>& fa, const Frag<B_KC, NBN>& fb) {
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int i = 0; i < NBM; i++)
+#pragma unroll
+                for (int j = 0; j < NBN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(i, t), fb.get(j, t), acc[i][j], 0, 0, 0);
+    };
 
-        const float* la = lds_a[cur];
-        const float* lb = lds_b[cur];
+    if (PIPE == 0) {
+        for (int kt = 0; kt < nkt; kt++) {
+            const int cur = kt & 1;
+            if (kt + 1 < nkt) load_global(kt + 1);
+            const float* la = lds_a[cur];
+            const float* lb = lds_b[cur];
 #pragma unroll
-        for (int kg = 0; kg < BK / 8; kg++) {
-            Frag<A_KC, NBM> fa;
-            Frag<B_KC, NBN> fb;
-            read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
-            read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
-#pragma unroll
-            for (int t = 0; t < 4; t++)
-#pragma unroll
-                for (int i = 0; i < NBM; i++)
-#pragma unroll
-                    for (int j = 0; j < NBN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(i, t), fb.get(j, t), acc[i][j], 0, 0, 0);
+            for (int kg = 0; kg < NKG; kg++) {
+                Frag<A_KC, NBM> fa;
+                Frag<B_KC, NBN> fb;
+                read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
+                read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
+                mfma_group(fa, fb);
+            }
+            if (kt + 1 < nkt) {
+                store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], ra, tid);
+                store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rb, tid);
+            }
+            __syncthreads();
         }
-
-        if (kt + 1 < nkt) {
-            store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], ra, tid);
-            store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rb, tid);
+    } else {
+        static_assert(PIPE == 0 || NKG % 2 == 0, "the pipelined schedule needs an even number of groups per tile");
+        constexpr int kReads = (A_KC ? NBM : 4) + (B_KC ? NBN : 4);   // LDS reads per group
+        constexpr int kMfma = 4 * NBM * NBN;                          // MFMAs per group
+        constexpr int kPer = kMfma / kReads;
+        // one LDS read, then kPer MFMAs, and so on: the hint below pins that interleaving
+        auto spread_reads = [&]() {
+#pragma unroll
+            for (int i = 0; i < kReads; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kPer * kReads, 0);
+        };
+        Frag<A_KC, NBM> fa[2];
+        Frag<B_KC, NBN> fb[2];
+        if (nkt > 0) {
+            read_frag<A_KC, NBM, BM, BK>(fa[0], lds_a[0], wm0, 0, l32, half);
+            read_frag<B_KC, NBN, BN, BK>(fb[0], lds_b[0], wn0, 0, l32, half);
         }
-        __syncthreads();
+        for (int kt = 0; kt + 1 < nkt; kt++) {
+            const int cur = kt & 1;
+            load_global(kt + 1);
+            // keep the global loads at the head of the tile: they need the whole tile to land
+            __builtin_amdgcn_sched_barrier(0);
+            const float* la = lds_a[cur];
+            const float* lb = lds_b[cur];
+#pragma unroll
+            for (int kg = 0; kg < NKG; kg++) {
+                const int nb = (kg + 1) & 1;
+                if (kg + 1 < NKG) {
+                    read_frag<A_KC, NBM, BM, BK>(fa[nb], la, wm0, kg + 1, l32, half);
+                    read_frag<B_KC, NBN, BN, BK>(fb[nb], lb, wn0, kg + 1, l32, half);
+                    if (kg == NKG - 2) {
+                        store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], ra, tid);
+                        store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rb, tid);
+                    }
+                } else {
+                    __syncthreads();
+                    read_frag<A_KC, NBM, BM, BK>(fa[nb], lds_a[cur ^ 1], wm0, 0, l32, half);
+                    read_frag<B_KC, NBN, BN, BK>(fb[nb], lds_b[cur ^ 1], wn0, 0, l32, half);
+                }
+                mfma_group(fa[kg & 1], fb[kg & 1]);
+                spread_reads();
+            }
+        }
+        if (nkt > 0) {
+            const int cur = (nkt - 1) & 1;
+#pragma unroll
+            for (int kg = 0; kg < NKG; kg++) {
+                const int nb = (kg + 1) & 1;
+                if (kg + 1 < NKG) {
+                    read_frag<A_KC, NBM, BM, BK>(fa[nb], lds_a[cur], wm0, kg + 1, l32, half);
+                    read_frag<B_KC, NBN, BN, BK>(fb[nb], lds_b[cur], wn0, kg + 1, l32, half);
+                }
+                mfma_group(fa[kg & 1], fb[kg & 1]);
+                if (kg + 1 < NKG) spread_reads();
+            }
+        }
     }
 
     // ---- epilogue ------------------------------------------------------------------------------

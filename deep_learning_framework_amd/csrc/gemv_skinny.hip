@@ -3,12 +3,14 @@
 //   y[m,n] (=|+=) act( sum_k x[m,k] * w[n,k] + bias[n] ),   m < M <= 16
 //
 // This is VMath::matmul (vmath.cu:2961-3003 of the reference) at batch sizes where
-// the weight matrix is read once and everything else is noise: the kernel is a
-// stream over W.  Each wave owns R rows of W and walks them with 128-bit loads, 64
-// lanes wide (1 KiB per row per step, fully coalesced); the M rows of X for the
-// current K chunk sit in LDS ([m][k], conflict-free 128-bit reads); every lane keeps
-// M*R partial sums that are folded across the wave at the end.  No MFMA: at
-// M <= 16 the matrix cores would idle behind HBM anyway.
+// the weight matrix is read once and everything else is noise: every kernel here is a
+// stream over W with 128-bit loads, 64 lanes wide (1 KiB per wave load, fully
+// coalesced), per-lane partial sums and a fold across the wave at the end.  No MFMA: at
+// these sizes the matrix cores would idle behind HBM anyway.  Three plans:
+//   M == 1      gemv_rows_kernel: a wave owns whole rows, x lives in registers
+//   M == 2..4   skinny_slice_kernel: a wave owns a K slice of a few rows, X slice in registers
+//   otherwise   skinny_nt_kernel: X staged in LDS chunk by chunk (also the scalar-load
+//               plan for unaligned or ragged operands)
 #include "gemv_skinny.h"
 
 #include "act_funcs.h"
@@ -118,6 +120,180 @@ __global__ void __launch_bounds__(kSkinnyThreads) skinny_nt_kernel(const SkinnyP
     }
 }
 
+// ---- batch 1: the weight matrix streamed once, x in registers ------------------------------------
+//
+// One wave owns R whole rows of W.  K is walked in chunks of 4096: a lane issues the 16 128-bit
+// loads of each of its rows for the chunk back to back (R*16 KiB in flight per wave), then loads
+// its 16 float4 of x (they hit in L2), then multiplies.  W is read with the non-temporal hint: it
+// is used once and should not displace x from the caches.  No LDS, no barrier.
+
+template <int R>
+__global__ void __launch_bounds__(kSkinnyThreads) gemv_rows_kernel(const SkinnyParams p) {
+    constexpr int CH = 16;   // float4 per lane per chunk of 4096 k
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t n0 = ((int64_t)blockIdx.x * (kSkinnyThreads / 64) + wave) * R;
+    if (n0 >= p.N) return;
+    const float* __restrict__ wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) wrow[r] = p.W + ((n0 + r < p.N) ? (n0 + r) : n0) * p.ldw;
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+
+    for (int kc = 0; kc < p.K; kc += 256 * CH) {
+        const int kbase = kc + 4 * lane;
+        f32x4 w[R][CH];
+        if (kc + 256 * CH <= p.K) {
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int j = 0; j < CH; j++)
+                    w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + kbase + 256 * j));
+            f32x4 x[CH];
+#pragma unroll
+            for (int j = 0; j < CH; j++) x[j] = *reinterpret_cast<const f32x4*>(p.X + kbase + 256 * j);
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int j = 0; j < CH; j++)
+                    acc[r] += w[r][j][0] * x[j][0] + w[r][j][1] * x[j][1] + w[r][j][2] * x[j][2] + w[r][j][3] * x[j][3];
+        } else {
+            // last, partial chunk: K % 4 == 0, so a float4 is entirely inside or outside
+#pragma unroll
+            for (int j = 0; j < CH; j++) {
+                const int k = kbase + 256 * j;
+                if (k < p.K) {
+                    const f32x4 x = *reinterpret_cast<const f32x4*>(p.X + k);
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const f32x4 wv = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + k));
+                        acc[r] += wv[0] * x[0] + wv[1] * x[1] + wv[2] * x[2] + wv[3] * x[3];
+                    }
+                }
+            }
+        }
+    }
+
+    const float leaky = p.leaky ? *p.leaky : 0.f;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        float v = wave_sum(acc[r]);
+        if (lane == r && n0 + r < p.N) {
+            const int64_t n = n0 + r;
+            if (p.accflag) v += p.Y[n];
+            if (p.bias) v += p.bias[n];
+            if (p.Y2) p.Y2[n] = v;
+            p.Y[n] = apply_act(v, p.act, leaky);
+        }
+    }
+}
+
+static int launch_gemv_rows(const SkinnyParams& p, hipStream_t stream) {
+    constexpr int R = 2;
+    const int64_t rows_per_block = (kSkinnyThreads / 64) * R;
+    const int64_t blocks = (p.N + rows_per_block - 1) / rows_per_block;
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
+    gemv_rows_kernel<R><<<dim3((unsigned)blocks), dim3(kSkinnyThreads), 0, stream>>>(p);
+    return check_launch("gemv_rows_kernel");
+}
+
+// ---- 2 to 4 rows of X: a workgroup owns RB rows of W, each wave one 1024-wide slice of K ----------
+//
+// The slice of X a wave needs (MT x 1024 floats) stays in its registers for all RB rows; the RB*4
+// loads of W per lane are issued back to back; the per-wave partial sums meet in LDS once, at the
+// end.  K beyond waves*1024 is covered by further passes of the same wave.
+
+constexpr int kSliceK = 1024;
+constexpr int kSliceMaxWaves = 4;   // 256 threads: leaves each wave 256 registers
+
+template <int MT, int RB>
+__global__ void __launch_bounds__(64 * kSliceMaxWaves) skinny_slice_kernel(const SkinnyParams p, int waves) {
+    __shared__ float part[MT * RB][kSliceMaxWaves];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int64_t n0 = (int64_t)blockIdx.x * RB;
+    const float* __restrict__ wrow[RB];
+#pragma unroll
+    for (int r = 0; r < RB; r++) wrow[r] = p.W + ((n0 + r < p.N) ? (n0 + r) : n0) * p.ldw;
+
+    float acc[MT][RB];
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int r = 0; r < RB; r++) acc[m][r] = 0.f;
+
+    for (int ks = wave * kSliceK; ks < p.K; ks += waves * kSliceK) {
+        f32x4 w[RB][4];
+        f32x4 x[MT][4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int k = ks + 4 * lane + 256 * j;
+            const bool in = k < p.K;
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+                w[r][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (in) w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + k));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int k = ks + 4 * lane + 256 * j;
+            const bool in = k < p.K;
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                x[m][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (in && m < p.M) x[m][j] = *reinterpret_cast<const f32x4*>(p.X + (int64_t)m * p.ldx + k);
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int r = 0; r < RB; r++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[m][r] += w[r][j][0] * x[m][j][0] + w[r][j][1] * x[m][j][1] + w[r][j][2] * x[m][j][2] +
+                                 w[r][j][3] * x[m][j][3];
+    }
+
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            const float v = wave_sum(acc[m][r]);
+            if (lane == 0) part[m * RB + r][wave] = v;
+        }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < MT * RB) {
+        const int m = t / RB, r = t % RB;
+        if (m < p.M && n0 + r < p.N) {
+            float v = 0.f;
+            for (int i = 0; i < waves; i++) v += part[t][i];
+            const float leaky = p.leaky ? *p.leaky : 0.f;
+            const int64_t n = n0 + r;
+            const int64_t idx = (int64_t)m * p.ldy + n;
+            if (p.accflag) v += p.Y[idx];
+            if (p.bias) v += p.bias[n];
+            if (p.Y2) p.Y2[idx] = v;
+            p.Y[idx] = apply_act(v, p.act, leaky);
+        }
+    }
+}
+
+template <int MT>
+static int launch_slice(const SkinnyParams& p, hipStream_t stream) {
+    constexpr int RB = 4;
+    int waves = (p.K + kSliceK - 1) / kSliceK;
+    if (waves < 1) waves = 1;
+    if (waves > kSliceMaxWaves) waves = kSliceMaxWaves;
+    const int64_t blocks = (p.N + RB - 1) / RB;
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
+    skinny_slice_kernel<MT, RB><<<dim3((unsigned)blocks), dim3(64 * waves), 0, stream>>>(p, waves);
+    return check_launch("skinny_slice_kernel");
+}
+
 template <int MT, bool VEC>
 static int launch_mt(const SkinnyParams& p, hipStream_t stream) {
     constexpr int R = 2;
@@ -141,6 +317,11 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0) return KAI_OK;
     if (p.M > kSkinnyMaxRows) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
     const bool vec = p.K % 4 == 0 && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X);
+    if (vec && p.K >= 256) {
+        if (p.M == 1) return launch_gemv_rows(p, stream);
+        if (p.M == 2) return launch_slice<2>(p, stream);
+        if (p.M <= 4) return launch_slice<4>(p, stream);
+    }
     return vec ? launch_vec<true>(p, stream) : launch_vec<false>(p, stream);
 }
 
