@@ -43,7 +43,7 @@ inline GemmParams make_params(const GemmDesc& d, bool a_kc, bool b_kc) {
     p.a_vec = a_cont == 1 && a_ld % 4 == 0 && d.a_bs0 % 4 == 0 && d.a_bs1 % 4 == 0 && aligned16(d.A);
     p.b_vec = b_cont == 1 && b_ld % 4 == 0 && d.b_bs0 % 4 == 0 && d.b_bs1 % 4 == 0 && aligned16(d.B);
     p.c_vec = d.c_cs == 1 && d.c_rs % 4 == 0 && d.N % 4 == 0 && d.c_bs0 % 4 == 0 && d.c_bs1 % 4 == 0 &&
-              aligned16(d.C) && (d.C2 == nullptr || aligned16(d.C2));
+              aligned16(d.C) && (d.C2 == nullptr || aligned16(d.C2)) && (d.bias == nullptr || aligned16(d.bias));
     p.act = d.act;
     p.accflag = d.acc;
     p.has_alpha = d.has_alpha;
@@ -57,7 +57,7 @@ inline bool fits_without_edges(const GemmParams& p, bool a_kc, bool b_kc, int BM
            a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30);
 }
 
-template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE>
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1>
 int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t stream) {
     constexpr int BM = WM * NBM * 32, BN = WN * NBN * 32;
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -67,7 +67,7 @@ int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t st
     if (tiles <= 0 || nbatch <= 0) return KAI_OK;
     if (tiles > kMaxDim || nbatch > 65535) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
     dim3 grid((unsigned)tiles, 1, (unsigned)nbatch);
-    gemm_mfma_kernel<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE><<<grid, dim3(64 * WM * WN), 0, stream>>>(p);
+    gemm_mfma_kernel<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE, PIPE, MINW><<<grid, dim3(64 * WM * WN), 0, stream>>>(p);
     return check_launch("gemm_mfma_kernel");
 }
 

@@ -3,8 +3,10 @@
 // parallel.
 //
 //   large  256x256 tile, 8 waves of 128x64 (2 waves per SIMD)  -- big, compute-bound products
-//   medium 128x128 tile, 4 waves of 64x64                      -- fills the chip at mid sizes
+//   medium 128x128 tile, 4 waves of 64x64, 2 workgroups per CU -- fills the chip at mid sizes
 //   small   64x64  tile, 4 waves of 32x32                      -- small or very ragged products
+// Shapes that are whole multiples of the tile with aligned operands run the pipelined,
+// predicate-free kernel; everything else the general one.
 #pragma once
 
 #include "gemm_host.h"
@@ -17,12 +19,12 @@ template <bool A_KC, bool B_KC>
 int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream) {
     switch (tile) {
     case kTileLarge:
-        if (fits_without_edges(p, A_KC, B_KC, 256, 256, 32))
-            return launch_gemm_config<2, 4, 4, 2, 32, A_KC, B_KC, false>(p, nbatch, kGroupM, stream);
+        if (fits_without_edges(p, A_KC, B_KC, 256, 256, 16))
+            return launch_gemm_config<2, 4, 4, 2, 16, A_KC, B_KC, false, 1>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<2, 4, 4, 2, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);
     case kTileMedium:
         if (fits_without_edges(p, A_KC, B_KC, 128, 128, 32))
-            return launch_gemm_config<2, 2, 2, 2, 32, A_KC, B_KC, false>(p, nbatch, kGroupM, stream);
+            return launch_gemm_config<2, 2, 2, 2, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<2, 2, 2, 2, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);
     default:
         return launch_gemm_config<2, 2, 1, 1, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);

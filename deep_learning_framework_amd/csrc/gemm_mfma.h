@@ -32,9 +32,21 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "act_funcs.h"
 
 namespace kai {
+
+// Loop with compile-time indices: f(std::integral_constant<int, B>), ..., f(<E-1>).  Used where a
+// register array must never be indexed by a run-time value, whatever the unroller decides.
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -92,6 +104,16 @@ __device__ __forceinline__ void load_tile_fast(f32x4 (&reg)[ROWS * BK / 4 / NT],
         const float* bi = base + (int64_t)(i * kLinesPerPass) * ld;
         reg[i] = *reinterpret_cast<const f32x4*>(bi + toff);
     }
+}
+
+// One chunk of the predicate-free load (chunk i of the calling thread).
+template <bool KC, int ROWS, int BK, int NT>
+__device__ __forceinline__ void load_tile_chunk(f32x4 (&reg)[ROWS * BK / 4 / NT], const float* __restrict__ base,
+                                                int64_t ld, uint32_t toff, int i) {
+    using TS = TileShape<KC, ROWS, BK>;
+    constexpr int kLinesPerPass = NT / TS::kChunksPerLine;
+    const float* bi = base + (int64_t)(i * kLinesPerPass) * ld;
+    reg[i] = *reinterpret_cast<const f32x4*>(bi + toff);
 }
 
 // Predicated load: rows_left / k_left are the numbers of valid rows / k from the tile origin.
@@ -184,6 +206,39 @@ __device__ __forceinline__ void read_frag(Frag<KC, NB>& f, const float* __restri
     }
 }
 
+// One LDS read of a fragment: piece < (KC ? NB : 4).
+template <bool KC, int NB, int ROWS, int BK>
+__device__ __forceinline__ void read_frag_piece(Frag<KC, NB>& f, const float* __restrict__ lds, int w_r0, int kg,
+                                                int l32, int half, int piece) {
+    using TS = TileShape<KC, ROWS, BK>;
+    if (KC) {
+        f.v[piece] =
+            *reinterpret_cast<const f32x4*>(lds + (w_r0 + 32 * piece + l32) * TS::kStride + kg * 8 + 4 * half);
+    } else {
+        const float* p = lds + (kg * 8 + 4 * half + piece) * TS::kStride + w_r0 + NB * l32;
+        if (NB == 4) {
+            f.v[piece] = *reinterpret_cast<const f32x4*>(p);
+        } else if (NB == 2) {
+            const f32x2 q = *reinterpret_cast<const f32x2*>(p);
+            f.v[piece][0] = q[0];
+            f.v[piece][1] = q[1];
+        } else {
+            f.v[piece][0] = p[0];
+        }
+    }
+}
+
+// One 128-bit LDS store of a staged tile: chunk i of the calling thread.
+template <bool KC, int ROWS, int BK, int NT>
+__device__ __forceinline__ void store_tile_chunk(float* __restrict__ lds, const f32x4 (&reg)[ROWS * BK / 4 / NT],
+                                                 int tid, int i) {
+    using TS = TileShape<KC, ROWS, BK>;
+    const int c = tid + i * NT;
+    const int line = c / TS::kChunksPerLine;
+    const int off = (c % TS::kChunksPerLine) * 4;
+    *reinterpret_cast<f32x4*>(lds + line * TS::kStride + off) = reg[i];
+}
+
 // Workgroup id -> (tile_m, tile_n).  Hardware deals consecutive workgroup ids round-robin over
 // the 8 XCDs; ids congruent mod 8 therefore share an L2.  They are renumbered so that each XCD
 // walks a contiguous run of tiles, and the run is ordered in column sweeps of `group_m` tile rows
@@ -213,8 +268,12 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 //      waits for an LDS round trip.  The next tile is stored to LDS while the second-to-last group
 //      computes; the barrier sits before the last group, whose MFMAs (operands already in
 //      registers) cover the first fragment reads of the next tile.
-template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0>
-__global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const GemmParams p) {
+//
+// MINW is the number of waves per SIMD the register allocation must leave room for (2 lets two
+// independent workgroups of four waves share a compute unit, so that one computes while the other
+// waits at its barrier).
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1>
+__global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const GemmParams p) {
     constexpr int NT = 64 * WM * WN;
     constexpr int BM = WM * NBM * 32;
     constexpr int BN = WN * NBN * 32;
@@ -324,111 +383,179 @@ __global__ void __launch_bounds__(64 * WM * WN) gemm_mfma_kernel(const GemmParam
         }
     } else {
         static_assert(PIPE == 0 || NKG % 2 == 0, "the pipelined schedule needs an even number of groups per tile");
-        constexpr int kReads = (A_KC ? NBM : 4) + (B_KC ? NBN : 4);   // LDS reads per group
-        constexpr int kMfma = 4 * NBM * NBN;                          // MFMAs per group
-        constexpr int kPer = kMfma / kReads;
-        // one LDS read, then kPer MFMAs, and so on: the hint below pins that interleaving
-        auto spread_reads = [&]() {
-#pragma unroll
-            for (int i = 0; i < kReads; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, kMfma - kPer * kReads, 0);
-        };
+        static_assert(PIPE == 0 || !EDGE, "the pipelined schedule uses the predicate-free loads only");
+        constexpr int kReadsA = A_KC ? NBM : 4;
+        constexpr int kReads = kReadsA + (B_KC ? NBN : 4);   // LDS reads per group
+        constexpr int kWrites = NCHA + NCHB;                  // LDS stores per tile and thread
+        constexpr int kMfma = 4 * NBM * NBN;                  // MFMAs per group
         Frag<A_KC, NBM> fa[2];
         Frag<B_KC, NBN> fb[2];
+
+        // One group of the schedule: the MFMAs of the fragments in `use`, cut into slots; slot s is
+        // preceded by the s-th LDS read of the fragments for the next group (into `fill`, from
+        // tile buffer `rbuf`, group `rkg`) and, when `store` is set, by the s-th LDS store of the
+        // staged next tile (into buffer `wbuf`).  Scheduling fences pin that interleaving, so the
+        // waves of a workgroup never hit LDS in one burst and no MFMA waits for an LDS round trip.
+        auto group = [&](int use, int fill, bool read, int rbuf, int rkg, bool store, int wbuf, bool gload, int gkt) {
+            const int memops = (store || gload) ? kWrites : 0;
+            const int slots = (read ? kReads : 0) > memops ? (read ? kReads : 0) : memops;
+            const float* gap = Ab + (int64_t)gkt * BK * p.a_ks;
+            const float* gbp = Bb + (int64_t)gkt * BK * p.b_ks;
+            const int per = slots > 0 ? kMfma / slots : kMfma;
+            int q = 0;
+#pragma unroll
+            for (int sl = 0; sl < (kReads > kWrites ? kReads : kWrites); sl++) {
+                if (sl < slots) {
+                    if (read && sl < kReads) {
+                        if (sl < kReadsA)
+                            read_frag_piece<A_KC, NBM, BM, BK>(fa[fill], lds_a[rbuf], wm0, rkg, l32, half, sl);
+                        else
+                            read_frag_piece<B_KC, NBN, BN, BK>(fb[fill], lds_b[rbuf], wn0, rkg, l32, half, sl - kReadsA);
+                    }
+                    if (store && sl < kWrites) {
+                        if (sl < NCHA) store_tile_chunk<A_KC, BM, BK, NT>(lds_a[wbuf], ra, tid, sl);
+                        else store_tile_chunk<B_KC, BN, BK, NT>(lds_b[wbuf], rb, tid, sl - NCHA);
+                    }
+                    if (gload && sl < kWrites) {
+                        if (sl < NCHA) load_tile_chunk<A_KC, BM, BK, NT>(ra, gap, a_ld, toff_a, sl);
+                        else load_tile_chunk<B_KC, BN, BK, NT>(rb, gbp, b_ld, toff_b, sl - NCHA);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int u = 0; u < kMfma; u++) {
+                        if (u < per) {
+                            const int t = q / (NBM * NBN), i = (q / NBN) % NBM, j = q % NBN;
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[use].get(i, t), fb[use].get(j, t),
+                                                                            acc[i][j], 0, 0, 0);
+                            q++;
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kMfma; u++) {
+                if (q < kMfma) {
+                    const int t = q / (NBM * NBN), i = (q / NBN) % NBM, j = q % NBN;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[use].get(i, t), fb[use].get(j, t), acc[i][j],
+                                                                    0, 0, 0);
+                    q++;
+                }
+            }
+        };
+
+        // The staging registers run one tile ahead of LDS: at the top of tile kt they hold tile
+        // kt+1 (loaded during the last group of tile kt-1, or by the prologue).  Group NKG-2 moves
+        // them into the free LDS buffer, one store per slot; the last group refills them with tile
+        // kt+2, one global load per slot, so that the waves of a workgroup never queue all their
+        // loads on the address unit at once and every load has most of a tile to land.
+        if (nkt > 1) load_global(1);
         if (nkt > 0) {
             read_frag<A_KC, NBM, BM, BK>(fa[0], lds_a[0], wm0, 0, l32, half);
             read_frag<B_KC, NBN, BN, BK>(fb[0], lds_b[0], wn0, 0, l32, half);
         }
         for (int kt = 0; kt + 1 < nkt; kt++) {
             const int cur = kt & 1;
-            load_global(kt + 1);
-            // keep the global loads at the head of the tile: they need the whole tile to land
-            __builtin_amdgcn_sched_barrier(0);
-            const float* la = lds_a[cur];
-            const float* lb = lds_b[cur];
+            const int gkt = min(kt + 2, nkt - 1);   // clamped: the surplus load of the last round is never stored
 #pragma unroll
             for (int kg = 0; kg < NKG; kg++) {
-                const int nb = (kg + 1) & 1;
                 if (kg + 1 < NKG) {
-                    read_frag<A_KC, NBM, BM, BK>(fa[nb], la, wm0, kg + 1, l32, half);
-                    read_frag<B_KC, NBN, BN, BK>(fb[nb], lb, wn0, kg + 1, l32, half);
-                    if (kg == NKG - 2) {
-                        store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], ra, tid);
-                        store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rb, tid);
-                    }
+                    group(kg & 1, (kg + 1) & 1, true, cur, kg + 1, kg == NKG - 2, cur ^ 1, false, 0);
                 } else {
+                    // last group: everyone's stores are in LDS after the barrier; its MFMAs (operands
+                    // already in registers) cover the first fragment reads of the next tile
                     __syncthreads();
-                    read_frag<A_KC, NBM, BM, BK>(fa[nb], lds_a[cur ^ 1], wm0, 0, l32, half);
-                    read_frag<B_KC, NBN, BN, BK>(fb[nb], lds_b[cur ^ 1], wn0, 0, l32, half);
+                    group(kg & 1, (kg + 1) & 1, true, cur ^ 1, 0, false, 0, true, gkt);
                 }
-                mfma_group(fa[kg & 1], fb[kg & 1]);
-                spread_reads();
             }
         }
         if (nkt > 0) {
             const int cur = (nkt - 1) & 1;
 #pragma unroll
-            for (int kg = 0; kg < NKG; kg++) {
-                const int nb = (kg + 1) & 1;
-                if (kg + 1 < NKG) {
-                    read_frag<A_KC, NBM, BM, BK>(fa[nb], lds_a[cur], wm0, kg + 1, l32, half);
-                    read_frag<B_KC, NBN, BN, BK>(fb[nb], lds_b[cur], wn0, kg + 1, l32, half);
-                }
-                mfma_group(fa[kg & 1], fb[kg & 1]);
-                if (kg + 1 < NKG) spread_reads();
-            }
+            for (int kg = 0; kg < NKG; kg++) group(kg & 1, (kg + 1) & 1, kg + 1 < NKG, cur, kg + 1, false, 0, false, 0);
         }
     }
 
     // ---- epilogue ------------------------------------------------------------------------------
+    // In registers: alpha, += C (acc), bias, optional store of the pre-activation, then none / relu /
+    // leaky relu.  The transcendental activations are applied in a second, rolled pass in which
+    // each thread re-reads the values it has just stored: that keeps the unrolled part small enough
+    // for the accumulators to stay in registers for the whole kernel.
     const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
     const float leaky = p.leaky ? *p.leaky : 0.f;
-    float* __restrict__ C = p.C + c_off;
-    float* __restrict__ C2 = p.C2 ? p.C2 + c_off : nullptr;
+    float* C = p.C + c_off;
+    float* C2 = p.C2 ? p.C2 + c_off : nullptr;
+    const int act = p.act;
+    const bool slow_act = act > kActLeaky;
 
-    auto finish = [&](float v, int col, int64_t idx) -> float {
-        if (p.has_alpha) v *= alpha;
-        if (p.accflag) v += C[idx];
-        if (p.bias) v += p.bias[col];
-        if (C2) C2[idx] = v;
-        return apply_act(v, p.act, leaky);
+    auto row_of = [&](int i, int r) -> int {
+        const int mi = 8 * (r >> 2) + 4 * half + (r & 3);   // row inside the 32x32 block
+        return m0 + (A_KC ? wm0 + 32 * i + mi : wm0 + NBM * mi + i);
     };
+    auto col_of = [&](int j) -> int { return n0 + (B_KC ? wn0 + 32 * j + l32 : wn0 + NBN * l32 + j); };
+    auto cheap_act = [&](float v) -> float {
+        if (act == kActRelu) return (v > 0) ? v : 0.0f;
+        if (act == kActLeaky) return (v > 0) ? v : v * leaky;
+        return v;
+    };
+    const bool vec_store = !B_KC && NBN == 4 && p.c_vec;
 
-#pragma unroll
-    for (int i = 0; i < NBM; i++) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int mi = 8 * (r >> 2) + 4 * half + (r & 3);   // row inside the 32x32 block
-            const int row = m0 + (A_KC ? wm0 + 32 * i + mi : wm0 + NBM * mi + i);
-            if (row >= p.M) continue;
-            if (!B_KC && NBN == 4 && p.c_vec) {
-                const int col = n0 + wn0 + 4 * l32;
-                if (col < p.N) {   // N % 4 == 0 under c_vec, so the whole chunk is inside
+    static_for<0, NBM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            const int row = row_of(i, r);
+            const bool row_ok = row < p.M;
+            if (vec_store) {
+                const int col = col_of(0);
+                if (row_ok && col < p.N) {   // N % 4 == 0 under c_vec, so the whole chunk is inside
                     const int64_t idx = (int64_t)row * p.c_rs + col;
                     f32x4 o;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        float v = acc[i][j][r];
-                        if (p.has_alpha) v *= alpha;
-                        if (p.accflag) v += C[idx + j];
-                        if (p.bias) v += p.bias[col + j];
-                        o[j] = v;
-                    }
+                    static_for<0, 4>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        o[j] = acc[i][j % NBN][r];
+                    });
+                    if (p.has_alpha) o *= alpha;
+                    if (p.accflag) o += *reinterpret_cast<const f32x4*>(C + idx);
+                    if (p.bias) o += *reinterpret_cast<const f32x4*>(p.bias + col);
                     if (C2) *reinterpret_cast<f32x4*>(C2 + idx) = o;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) o[j] = apply_act(o[j], p.act, leaky);
+                    static_for<0, 4>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        o[j] = cheap_act(o[j]);
+                    });
                     *reinterpret_cast<f32x4*>(C + idx) = o;
                 }
             } else {
-#pragma unroll
+                static_for<0, NBN>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    const int col = col_of(j);
+                    if (row_ok && col < p.N) {
+                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
+                        float v = acc[i][j][r];
+                        if (p.has_alpha) v *= alpha;
+                        if (p.accflag) v += C[idx];
+                        if (p.bias) v += p.bias[col];
+                        if (C2) C2[idx] = v;
+                        C[idx] = cheap_act(v);
+                    }
+                });
+            }
+        });
+    });
+
+    if (slow_act) {
+#pragma nounroll
+        for (int i = 0; i < NBM; i++) {
+#pragma nounroll
+            for (int r = 0; r < 16; r++) {
+                const int row = row_of(i, r);
+                if (row >= p.M) continue;
+#pragma nounroll
                 for (int j = 0; j < NBN; j++) {
-                    const int col = n0 + (B_KC ? wn0 + 32 * j + l32 : wn0 + NBN * l32 + j);
+                    const int col = col_of(j);
                     if (col < p.N) {
                         const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
-                        C[idx] = finish(acc[i][j][r], col, idx);
+                        C[idx] = apply_act(C[idx], act, leaky);
                     }
                 }
             }

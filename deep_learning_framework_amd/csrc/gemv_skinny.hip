@@ -22,10 +22,20 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kSkinnyLdsFloats = 16384;   // 64 KiB of X per block
 constexpr int kSkinnyThreads = 256;
 
+// Sum over the 64 lanes of a wave, returned to every lane.  Cross-lane moves go through the DPP
+// data path (a few cycles each) instead of LDS permutes: the fold sits on the critical path at the
+// end of a kernel whose whole run time is ~10 us.
+//   quad_perm [1,0,3,2] and [2,3,0,1]   -> every lane of a quad holds the quad sum
+//   row_half_mirror, row_mirror        -> every lane of a row of 16 holds the row sum
+//   row_bcast:15 (rows 1,3), row_bcast:31 (rows 2,3) -> lane 63 holds the wave sum
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 template <int MT, int R, bool VEC>
@@ -127,40 +137,53 @@ __global__ void __launch_bounds__(kSkinnyThreads) skinny_nt_kernel(const SkinnyP
 // its 16 float4 of x (they hit in L2), then multiplies.  W is read with the non-temporal hint: it
 // is used once and should not displace x from the caches.  No LDS, no barrier.
 
+// amdgpu_waves_per_eu(1, 2): two waves per SIMD are all the grid ever gives a CU, so the register
+// allocator is told not to trade loads in flight for an occupancy it cannot use.
 template <int R>
-__global__ void __launch_bounds__(kSkinnyThreads) gemv_rows_kernel(const SkinnyParams p) {
+__global__ void __launch_bounds__(kSkinnyThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
+gemv_rows_kernel(const SkinnyParams p) {
     constexpr int CH = 16;   // float4 per lane per chunk of 4096 k
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int64_t n0 = ((int64_t)blockIdx.x * (kSkinnyThreads / 64) + wave) * R;
-    if (n0 >= p.N) return;
+    // rows past the end are clamped to the last row (loaded, never stored): no early exit, so the
+    // kernel arguments are fetched in one round trip and the first loads go out at once
     const float* __restrict__ wrow[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) wrow[r] = p.W + ((n0 + r < p.N) ? (n0 + r) : n0) * p.ldw;
+    for (int r = 0; r < R; r++) wrow[r] = p.W + ((n0 + r < p.N) ? (n0 + r) : (p.N - 1)) * p.ldw;
 
     float acc[R];
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
 
-    for (int kc = 0; kc < p.K; kc += 256 * CH) {
+    // one whole chunk of 4096 k: all loads of W, then x, then the multiplies (straight-line code;
+    // the compiler overlaps the second row's loads with the first row's arithmetic)
+    auto full_chunk = [&](int kc) {
         const int kbase = kc + 4 * lane;
         f32x4 w[R][CH];
-        if (kc + 256 * CH <= p.K) {
 #pragma unroll
-            for (int r = 0; r < R; r++)
+        for (int r = 0; r < R; r++)
 #pragma unroll
-                for (int j = 0; j < CH; j++)
-                    w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + kbase + 256 * j));
-            f32x4 x[CH];
+            for (int j = 0; j < CH; j++)
+                w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + kbase + 256 * j));
+        f32x4 x[CH];
 #pragma unroll
-            for (int j = 0; j < CH; j++) x[j] = *reinterpret_cast<const f32x4*>(p.X + kbase + 256 * j);
+        for (int j = 0; j < CH; j++) x[j] = *reinterpret_cast<const f32x4*>(p.X + kbase + 256 * j);
 #pragma unroll
-            for (int r = 0; r < R; r++)
+        for (int r = 0; r < R; r++)
 #pragma unroll
-                for (int j = 0; j < CH; j++)
-                    acc[r] += w[r][j][0] * x[j][0] + w[r][j][1] * x[j][1] + w[r][j][2] * x[j][2] + w[r][j][3] * x[j][3];
-        } else {
+            for (int j = 0; j < CH; j++)
+                acc[r] += w[r][j][0] * x[j][0] + w[r][j][1] * x[j][1] + w[r][j][2] * x[j][2] + w[r][j][3] * x[j][3];
+    };
+
+    if (p.K == 256 * CH) {
+        full_chunk(0);   // the common inference width gets loop-free code
+    } else {
+        int kc = 0;
+        for (; kc + 256 * CH <= p.K; kc += 256 * CH) full_chunk(kc);
+        if (kc < p.K) {
             // last, partial chunk: K % 4 == 0, so a float4 is entirely inside or outside
+            const int kbase = kc + 4 * lane;
 #pragma unroll
             for (int j = 0; j < CH; j++) {
                 const int k = kbase + 256 * j;
@@ -247,6 +270,7 @@ __global__ void __launch_bounds__(64 * kSliceMaxWaves) skinny_slice_kernel(const
                 if (in && m < p.M) x[m][j] = *reinterpret_cast<const f32x4*>(p.X + (int64_t)m * p.ldx + k);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);   // all loads of the pass are in flight before the first multiply
 #pragma unroll
         for (int m = 0; m < MT; m++)
 #pragma unroll
