@@ -25,14 +25,16 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 
 
-def hbm_traffic_from_profile(kernel_key):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), as recorded in
-    profiles/hbm_traffic.json next to the profile summaries; None if not recorded."""
-    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+def hbm_traffic_from_profile(summary_name):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE, scaled by what the
+    same counters read for a plain copy of known size), as recorded in the kernel's summary under
+    profiles/; None if no summary holds the figure."""
+    import re
     try:
-        with open(path) as f:
-            return json.load(f).get(kernel_key, {}).get("bytes_per_launch")
-    except (OSError, ValueError):
+        with open(os.path.join(ROOT, "profiles", summary_name)) as f:
+            m = re.search(r"HBM_TRAFFIC_BYTES_PER_LAUNCH\s*=\s*([0-9.eE+]+)", f.read())
+        return float(m.group(1)) if m else None
+    except OSError:
         return None
 
 
@@ -169,14 +171,14 @@ def main():
         "pct_of_fp32_mfma_peak": 100.0 * tflops / PEAK_FP32_MFMA_TFLOPS,
         "rel_fro_err_vs_f64_rows": err,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": hbm_traffic_from_profile("gemm_8192"),
+                     "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": hbm_traffic_from_profile("gemm_mfma_kernel_8192_gemm_bias_relu.md"),
                      "kernel": "gemm_mfma_kernel", "kernel_ms": kernel_ms, "flops_per_launch": flops},
         "gemv": {"workload": "batch-1 y = x . W^T, W[4096,4096] fp32 (BASELINE configs[4], M=1), kai_matmul",
                  "value": gemv_gbs, "unit": "GB/s", "us_per_call_cold": cold_ms * 1e3,
                  "us_per_call_warm": warm_ms * 1e3, "warm_gbs": gemv_bytes / (warm_ms * 1e-3) * 1e-9,
                  "rel_fro_err_vs_f64": gemv_err,
                  "roofline": {"bound": "hbm", "achieved": gemv_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                              "frac": gemv_gbs / PEAK_HBM_GBS, "traffic": hbm_traffic_from_profile("gemv_4096"),
+                              "frac": gemv_gbs / PEAK_HBM_GBS, "traffic": hbm_traffic_from_profile("gemv_rows_kernel_4096x4096_batch1.md"),
                               "kernel": "gemv_rows_kernel", "bytes_per_launch": gemv_bytes}},
     }
 
