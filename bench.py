@@ -62,12 +62,146 @@ def cpu_baseline(a_rows, bt, bias, seconds_hint=15.0):
     }, y, rows
 
 
+def per_config_table(torch, kai, stream, dev, with_cpu):
+    """The other BASELINE configurations (they are parity cases; reported here for completeness): GPU time
+    per call from HIP events over back-to-back launches, achieved rate, and the oracle's single-thread time."""
+    import ctypes
+    L = kai.load()
+    g = torch.Generator(device=dev)
+    g.manual_seed(11)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    I = ctypes.c_int64
+    if with_cpu:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle as ko
+
+    def gpu_us(fn, iters=50, prep=None):
+        for _ in range(3):
+            if prep:
+                prep()
+            fn()
+        torch.cuda.synchronize()
+        if prep is None:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(iters):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / iters
+        tot = 0.0   # in-place ops: restore the input outside the timed span
+        for _ in range(iters):
+            prep()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            tot += e0.elapsed_time(e1) * 1e3
+        return tot / iters
+
+    def cpu_us(f):
+        if not with_cpu:
+            return None
+        t0 = time.perf_counter()
+        f()
+        return (time.perf_counter() - t0) * 1e6
+
+    rows = []
+
+    def row(name, us, flops=None, nbytes=None, cpu=None):
+        r = {"case": name, "gpu_us": round(us, 2)}
+        if flops:
+            r["tflops"] = round(flops / us * 1e-6, 2)
+            r["frac_fp32_mfma_peak"] = round(flops / us * 1e-6 / PEAK_FP32_MFMA_TFLOPS, 4)
+        if nbytes:
+            r["gbs"] = round(nbytes / us * 1e-3, 1)
+            r["frac_hbm_peak"] = round(nbytes / us * 1e-3 / PEAK_HBM_GBS, 4)
+        if cpu is not None:
+            r["cpu_us_1_thread"] = round(cpu, 1)
+        rows.append(r)
+
+    relu = kai.ACT["relu"]
+    # cfg1: dense forward 64 x 784 -> 512, fused
+    x = torch.randn((64, 784), device=dev, generator=g)
+    w = (torch.rand((512, 784), device=dev, generator=g) * 2 - 1) / 28.0
+    b = torch.zeros(512, device=dev)
+    y = torch.empty((64, 512), device=dev)
+    us = gpu_us(lambda: L.kai_dense_forward(0, P(y), None, P(w), P(b), P(x), I(512), I(64), I(784), relu, None))
+    xc, wc, bc = x.cpu().numpy(), w.cpu().numpy(), b.cpu().numpy()
+    row("cfg1 dense fwd 64x784->512 +bias+relu (1 launch)", us, flops=2.0 * 64 * 784 * 512,
+        cpu=cpu_us(lambda: ko.activate(ko.add_bias(ko.matmul(wc, xc), bc), "relu")))
+    # cfg2: batch 256, 1024 -> 1024
+    x = torch.randn((256, 1024), device=dev, generator=g)
+    w = (torch.rand((1024, 1024), device=dev, generator=g) * 2 - 1) / 32.0
+    b = torch.randn(1024, device=dev, generator=g)
+    gy = torch.randn((256, 1024), device=dev, generator=g) * 0.01
+    y, gx, gw, gb = (torch.empty_like(x), torch.empty_like(x), torch.empty_like(w), torch.empty_like(b))
+    f = 2.0 * 256 * 1024 * 1024
+    xc, wc, bc, gyc = x.cpu().numpy(), w.cpu().numpy(), b.cpu().numpy(), gy.cpu().numpy()
+    row("cfg2 Y = X.W^T + b (fused)", gpu_us(lambda: L.kai_dense_forward(0, P(y), None, P(w), P(b), P(x), I(1024), I(256), I(1024), 0, None)),
+        flops=f, cpu=cpu_us(lambda: ko.add_bias(ko.matmul(wc, xc), bc)))
+    row("cfg2 dX = dY.W", gpu_us(lambda: L.kai_matmul_backward_x(0, P(gx), P(gy), P(w), I(1024), I(256), I(1024), 0)),
+        flops=f, cpu=cpu_us(lambda: ko.matmul_backward_x(gyc, wc)))
+    row("cfg2 dW = dY^T.X", gpu_us(lambda: L.kai_matmul_backward_w(0, P(gw), P(gy), P(x), I(1024), I(256), I(1024), 0)),
+        flops=f, cpu=cpu_us(lambda: ko.matmul_backward_w(gyc, xc, 1024, 1024)))
+    row("cfg2 db = colsum(dY)", gpu_us(lambda: L.kai_add_bias_backward_b(0, P(gb), P(gy), I(256), I(1024), 0)),
+        nbytes=4.0 * 256 * 1024, cpu=cpu_us(lambda: ko.add_bias_backward_b(gyc, 1024)))
+    # cfg4: attention, both mappings of 32 batch x heads, seq 512, head dim 64
+    for nbat, nhead, nvec in ((32, 1, 64), (4, 8, 512)):
+        T, D = 512, 64
+        q, k, v = (torch.randn((nbat, T, nvec), device=dev, generator=g) for _ in range(3))
+        s0 = torch.empty((nbat, T, T, nhead), device=dev)
+        pbuf = torch.empty_like(s0)
+        o = torch.empty((nbat, T, nvec), device=dev)
+        coef = torch.tensor([0.125], device=dev)
+        tag = "cfg4 nbat=%d nhead=%d " % (nbat, nhead)
+        fl = 2.0 * 32 * T * T * D
+        qc, kc, vc = q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy()
+        row(tag + "S = Q.K^T/8 (mult_on_heads)",
+            gpu_us(lambda: L.kai_mult_on_heads(0, P(s0), P(k), P(q), I(nbat), I(T), I(nvec), I(nhead), I(D), P(coef))),
+            flops=fl, cpu=cpu_us(lambda: ko.mult_on_heads(kc, qc, nhead, 0.125)))
+        row(tag + "softmax_direct_on_axis (in place)",
+            gpu_us(lambda: L.kai_softmax_direct_on_axis(0, P(pbuf), I(nbat * T), I(T), I(nhead)), iters=20,
+                   prep=lambda: pbuf.copy_(s0)),
+            nbytes=8.0 * 32 * T * T, cpu=cpu_us(lambda: ko.softmax_direct_on_axis(s0.cpu().numpy(), nbat * T, T, nhead)))
+        row(tag + "O = P.V (mix_values)",
+            gpu_us(lambda: L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))),
+            flops=fl, cpu=cpu_us(lambda: ko.mix_values(pbuf.cpu().numpy(), vc, nhead)))
+    # cfg5: skinny (cold: six rotating weight buffers) and ragged
+    K = N = 4096
+    ws = [torch.rand((N, K), device=dev, generator=g) * 0.1 - 0.05 for _ in range(6)]
+    for m in (1, 4, 16):
+        x = torch.randn((m, K), device=dev, generator=g)
+        y = torch.empty((m, N), device=dev)
+        it = [0]
+
+        def call():
+            it[0] += 1
+            L.kai_matmul(0, P(y), P(ws[it[0] % 6]), P(x), I(N), I(m), I(K), 0)
+
+        wc = ws[0].cpu().numpy() if with_cpu else None
+        xc = x.cpu().numpy()
+        row("cfg5 M=%d x 4096 x 4096 (cold)" % m, gpu_us(call, iters=120), flops=2.0 * m * N * K,
+            nbytes=4.0 * (K * N + m * K + m * N), cpu=cpu_us(lambda: ko.matmul(wc, xc)))
+    del ws
+    m, k, n = 1000, 777, 333
+    x = torch.randn((m, k), device=dev, generator=g)
+    w = torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05
+    y = torch.empty((m, n), device=dev)
+    xc, wc = x.cpu().numpy(), w.cpu().numpy()
+    row("cfg5 ragged 1000x777x333", gpu_us(lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0)),
+        flops=2.0 * m * n * k, cpu=cpu_us(lambda: ko.matmul(wc, xc)))
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true", help="skip the table of the other configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path is built and measured on a single MI355X "
@@ -193,6 +327,8 @@ def main():
         out["cpu_baseline"] = base
     else:
         out["cpu_baseline"] = None
+    if not args.headline_only:
+        out["per_config"] = per_config_table(torch, kai, stream, dev, not args.no_cpu_baseline)
     print(json.dumps(out))
 
 

@@ -6,11 +6,13 @@
 // the weight matrix is read once and everything else is noise: every kernel here is a
 // stream over W with 128-bit loads, 64 lanes wide (1 KiB per wave load, fully
 // coalesced), per-lane partial sums and a fold across the wave at the end.  No MFMA: at
-// these sizes the matrix cores would idle behind HBM anyway.  Three plans:
+// these sizes the matrix cores would idle behind HBM anyway.  Plans:
 //   M == 1      gemv_rows_kernel: a wave owns whole rows, x lives in registers
 //   M == 2..4   skinny_slice_kernel: a wave owns a K slice of a few rows, X slice in registers
-//   otherwise   skinny_nt_kernel: X staged in LDS chunk by chunk (also the scalar-load
-//               plan for unaligned or ragged operands)
+//   M == 5..16  skinny_mfma_kernel: the same stream, multiplied on the matrix core because the
+//               vector ALU would need 8 LDS bytes of X per byte of W (also the plan for
+//               unaligned or ragged skinny operands, with scalar loads)
+//   K < 256     skinny_nt_kernel: X staged in LDS
 #include "gemv_skinny.h"
 
 #include "act_funcs.h"
@@ -318,6 +320,110 @@ static int launch_slice(const SkinnyParams& p, hipStream_t stream) {
     return check_launch("skinny_slice_kernel");
 }
 
+// ---- up to 16 rows of X through the matrix core, still as a stream over W ---------------------------
+//
+// A workgroup of 8 waves owns 16 rows of W; wave w owns the w-th eighth of K.  Per step of 16 k a lane
+// loads one float4 of W (row lane%16, k offset 4*(lane/16)) and the float4 of X at the same (row, k):
+// exactly the operand layout of v_mfma_f32_16x16x4_f32 when element t of both float4 feeds step t,
+// so four MFMAs consume the step with no shuffles, no LDS and no per-row scalar work.  X rows beyond
+// M read as zeros.  The eight partial 16x16 results meet in LDS once, at the end.  The multiply
+// itself is 3 % of what the matrix core could do at this byte rate: the kernel is bound by HBM like
+// the other skinny kernels; with the vector ALU the same product needs 8 LDS bytes per byte of W at
+// 16 rows and is LDS-bound at a quarter of the bandwidth.
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+constexpr int kMmWaves = 8;
+constexpr int kMmUnroll = 16;  // steps of 16 k (1 KiB of W and of X each) in flight per wave
+
+template <bool VEC>
+__global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const SkinnyParams p) {
+    __shared__ float part[kMmWaves][256];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15;    // row of W inside the block's 16 / row of X
+    const int g = lane >> 4;    // k group
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const bool wvalid = n0 + r < p.N;
+    const bool xvalid = r < p.M;
+    const float* __restrict__ wp = p.W + (wvalid ? (n0 + r) : 0) * p.ldw + 4 * g;
+    const float* __restrict__ xp = p.X + (int64_t)(xvalid ? r : 0) * p.ldx + 4 * g;
+
+    // K split into 8 contiguous slices of whole 16-k steps
+    const int steps = (p.K + 15) / 16;
+    const int per = (steps + kMmWaves - 1) / kMmWaves;
+    const int s_begin = wave * per;
+    const int s_end = min(steps, s_begin + per);
+
+    f32x4v acc = {0.f, 0.f, 0.f, 0.f};
+    auto load4 = [&](const float* base, int k, bool valid) -> f32x4v {
+        f32x4v v = {0.f, 0.f, 0.f, 0.f};
+        if (VEC) {
+            // K % 4 == 0: the float4 at k is entirely inside or outside
+            if (valid && k + 4 * g < p.K) v = *reinterpret_cast<const f32x4v*>(base + k);
+        } else {
+            if (valid) {
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (k + 4 * g + j < p.K) v[j] = base[k + j];
+            }
+        }
+        return v;
+    };
+
+    // register ring of kMmUnroll steps: a slot is refilled with the step one ring-length ahead right
+    // after its MFMAs are issued, so kMmUnroll loads of W and of X stay in flight until the slice ends
+    f32x4v w[kMmUnroll], x[kMmUnroll];
+#pragma unroll
+    for (int u = 0; u < kMmUnroll; u++) {
+        const bool in = s_begin + u < s_end;
+        w[u] = load4(wp, (s_begin + u) * 16, wvalid && in);
+        x[u] = load4(xp, (s_begin + u) * 16, xvalid && in);
+    }
+    for (int base = s_begin; base < s_end; base += kMmUnroll) {
+#pragma unroll
+        for (int u = 0; u < kMmUnroll; u++) {
+            // steps past the end of the slice hold zeros and add nothing
+#pragma unroll
+            for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x[u][t], w[u][t], acc, 0, 0, 0);
+            const int nxt = base + kMmUnroll + u;
+            const bool in = nxt < s_end;
+            w[u] = load4(wp, nxt * 16, wvalid && in);
+            x[u] = load4(xp, nxt * 16, xvalid && in);
+        }
+    }
+
+    // acc[v] = D[m = 4*(lane/16) + v][n = lane%16]
+#pragma unroll
+    for (int v = 0; v < 4; v++) part[wave][(4 * g + v) * 16 + r] = acc[v];
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < 256) {
+        const int m = t >> 4, j = t & 15;
+        if (m < p.M && n0 + j < p.N) {
+            float v = 0.f;
+#pragma unroll
+            for (int i = 0; i < kMmWaves; i++) v += part[i][t];
+            const float leaky = p.leaky ? *p.leaky : 0.f;
+            const int64_t n = n0 + j;
+            const int64_t idx = (int64_t)m * p.ldy + n;
+            if (p.accflag) v += p.Y[idx];
+            if (p.bias) v += p.bias[n];
+            if (p.Y2) p.Y2[idx] = v;
+            p.Y[idx] = apply_act(v, p.act, leaky);
+        }
+    }
+}
+
+static int launch_skinny_mfma(const SkinnyParams& p, bool vec, hipStream_t stream) {
+    const int64_t blocks = (p.N + 15) / 16;
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
+    if (vec)
+        skinny_mfma_kernel<true><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
+    else
+        skinny_mfma_kernel<false><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
+    return check_launch("skinny_mfma_kernel");
+}
+
 template <int MT, bool VEC>
 static int launch_mt(const SkinnyParams& p, hipStream_t stream) {
     constexpr int R = 2;
@@ -346,6 +452,7 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
         if (p.M == 2) return launch_slice<2>(p, stream);
         if (p.M <= 4) return launch_slice<4>(p, stream);
     }
+    if (p.M > 4 || !vec) return launch_skinny_mfma(p, vec, stream);
     return vec ? launch_vec<true>(p, stream) : launch_vec<false>(p, stream);
 }
 
