@@ -34,10 +34,11 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
     const bool b_kc = operand_is_kc(d.b_rs, d.b_ks);
     const GemmParams p = make_params(d, a_kc, b_kc);
 
-    // largest tile that still yields about one workgroup per compute unit
+    // largest tile that still yields about one workgroup per compute unit and is not mostly padding
+    const int64_t short_side = d.M < d.N ? d.M : d.N;
     int tile = kTileSmall;
-    if (tiles_of(d.M, d.N, d.nbatch, 256) >= 192) tile = kTileLarge;
-    else if (tiles_of(d.M, d.N, d.nbatch, 128) >= 128) tile = kTileMedium;
+    if (short_side > 128 && tiles_of(d.M, d.N, d.nbatch, 256) >= 192) tile = kTileLarge;
+    else if (short_side > 64 && tiles_of(d.M, d.N, d.nbatch, 128) >= 128) tile = kTileMedium;
 
     if (a_kc && b_kc) return launch_gemm_kc_kc(p, d.nbatch, tile, stream);
     if (a_kc && !b_kc) return launch_gemm_kc_mc(p, d.nbatch, tile, stream);

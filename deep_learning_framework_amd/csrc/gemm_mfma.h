@@ -272,7 +272,11 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 // MINW is the number of waves per SIMD the register allocation must leave room for (2 lets two
 // independent workgroups of four waves share a compute unit, so that one computes while the other
 // waits at its barrier).
-template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1>
+//
+// DEPTH (PIPE 0 only) is the number of K-tiles kept in flight in staging registers: small tiles
+// compute for far less time than a global load takes to return, so they run several tiles ahead.
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
+          int DEPTH = 1>
 __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const GemmParams p) {
     constexpr int NT = 64 * WM * WN;
     constexpr int BM = WM * NBM * 32;
@@ -326,27 +330,36 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    f32x4 ra[NCHA], rb[NCHB];
+    static_assert(DEPTH >= 1 && (PIPE == 0 || DEPTH == 1), "deep register staging belongs to the PIPE 0 schedule");
+    f32x4 rax[DEPTH][NCHA], rbx[DEPTH][NCHB];
+    f32x4(&ra)[NCHA] = rax[0];
+    f32x4(&rb)[NCHB] = rbx[0];
     const int nkt = (p.K + BK - 1) / BK;
 
-    auto load_global = [&](int kt) {
+    auto load_global_into = [&](int kt, f32x4(&da)[NCHA], f32x4(&db)[NCHB]) {
         const int k0 = kt * BK;
         const int k_left = p.K - k0;
         const float* ap = Ab + (int64_t)k0 * p.a_ks;
         const float* bp = Bb + (int64_t)k0 * p.b_ks;
         if (!EDGE || (interior && k_left >= BK)) {
-            load_tile_fast<A_KC, BM, BK, NT>(ra, ap, a_ld, toff_a);
-            load_tile_fast<B_KC, BN, BK, NT>(rb, bp, b_ld, toff_b);
+            load_tile_fast<A_KC, BM, BK, NT>(da, ap, a_ld, toff_a);
+            load_tile_fast<B_KC, BN, BK, NT>(db, bp, b_ld, toff_b);
         } else {
-            load_tile_edge<A_KC, BM, BK, NT>(ra, ap, p.a_rs, p.a_ks, rows_a, k_left, p.a_vec, tid);
-            load_tile_edge<B_KC, BN, BK, NT>(rb, bp, p.b_rs, p.b_ks, rows_b, k_left, p.b_vec, tid);
+            load_tile_edge<A_KC, BM, BK, NT>(da, ap, p.a_rs, p.a_ks, rows_a, k_left, p.a_vec, tid);
+            load_tile_edge<B_KC, BN, BK, NT>(db, bp, p.b_rs, p.b_ks, rows_b, k_left, p.b_vec, tid);
         }
     };
+    auto load_global = [&](int kt) { load_global_into(kt, ra, rb); };
 
+    // prologue: tiles 0 .. DEPTH-1 go to the staging slots, tile 0 on to LDS, and its slot is refilled
     if (nkt > 0) {
-        load_global(0);
+        static_for<0, DEPTH>([&](auto dc) {
+            constexpr int d = decltype(dc)::value;
+            if (d < nkt) load_global_into(d, rax[d], rbx[d]);
+        });
         store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
         store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
+        if (PIPE == 0 && DEPTH > 1 && DEPTH < nkt) load_global_into(DEPTH, ra, rb);
     }
     __syncthreads();
 
@@ -362,24 +375,35 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     };
 
     if (PIPE == 0) {
-        for (int kt = 0; kt < nkt; kt++) {
-            const int cur = kt & 1;
-            if (kt + 1 < nkt) load_global(kt + 1);
-            const float* la = lds_a[cur];
-            const float* lb = lds_b[cur];
+        // At the top of tile kt: LDS[kt & 1] holds tile kt; slot (kt + j) % DEPTH holds tile kt + j for
+        // j = 1 .. DEPTH (slot kt % DEPTH was refilled with tile kt + DEPTH when tile kt left it).
+        // With DEPTH == 1 the single slot is refilled before the MFMAs of the tile instead.
+        for (int kt0 = 0; kt0 < nkt; kt0 += DEPTH) {
+            static_for<0, DEPTH>([&](auto dc) {
+                constexpr int d = decltype(dc)::value;
+                constexpr int nslot = (d + 1) % DEPTH;
+                const int kt = kt0 + d;
+                if (kt < nkt) {
+                    const int cur = kt & 1;
+                    if (DEPTH == 1 && kt + 1 < nkt) load_global(kt + 1);
+                    const float* la = lds_a[cur];
+                    const float* lb = lds_b[cur];
 #pragma unroll
-            for (int kg = 0; kg < NKG; kg++) {
-                Frag<A_KC, NBM> fa;
-                Frag<B_KC, NBN> fb;
-                read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
-                read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
-                mfma_group(fa, fb);
-            }
-            if (kt + 1 < nkt) {
-                store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], ra, tid);
-                store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rb, tid);
-            }
-            __syncthreads();
+                    for (int kg = 0; kg < NKG; kg++) {
+                        Frag<A_KC, NBM> fa;
+                        Frag<B_KC, NBN> fb;
+                        read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
+                        read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
+                        mfma_group(fa, fb);
+                    }
+                    if (kt + 1 < nkt) {
+                        store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], rax[nslot], tid);
+                        store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rbx[nslot], tid);
+                        if (DEPTH > 1 && kt + 1 + DEPTH < nkt) load_global_into(kt + 1 + DEPTH, rax[nslot], rbx[nslot]);
+                    }
+                    __syncthreads();
+                }
+            });
         }
     } else {
         static_assert(PIPE == 0 || NKG % 2 == 0, "the pipelined schedule needs an even number of groups per tile");
