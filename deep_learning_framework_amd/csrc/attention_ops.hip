@@ -21,15 +21,28 @@ namespace kai {
 
 constexpr int kTB = 256;
 
+// Wave-wide reductions through the DPP data path (result in every lane); see gemv_skinny.hip for
+// the sequence.  For the maximum, lanes that a row-masked broadcast step does not write keep their
+// own value (old = v), which leaves the maximum unchanged.
+#define KAI_DPP(old, v, ctrl, rmask) \
+    __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, (old)), __builtin_bit_cast(int, (v)), (ctrl), (rmask), 0xf, false))
 __device__ __forceinline__ float wmax(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+    v = fmaxf(v, KAI_DPP(v, v, 0xB1, 0xf));
+    v = fmaxf(v, KAI_DPP(v, v, 0x4E, 0xf));
+    v = fmaxf(v, KAI_DPP(v, v, 0x141, 0xf));
+    v = fmaxf(v, KAI_DPP(v, v, 0x140, 0xf));
+    v = fmaxf(v, KAI_DPP(v, v, 0x142, 0xa));
+    v = fmaxf(v, KAI_DPP(v, v, 0x143, 0xc));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wsum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    v += KAI_DPP(0.f, v, 0xB1, 0xf);
+    v += KAI_DPP(0.f, v, 0x4E, 0xf);
+    v += KAI_DPP(0.f, v, 0x141, 0xf);
+    v += KAI_DPP(0.f, v, 0x140, 0xf);
+    v += KAI_DPP(0.f, v, 0x142, 0xa);
+    v += KAI_DPP(0.f, v, 0x143, 0xc);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // ---- mask -------------------------------------------------------------------------------------
@@ -128,6 +141,133 @@ __global__ void __launch_bounds__(kTB) softmax_axis_block_kernel(float* __restri
     }
 }
 
+// ncol == 1, row length a multiple of 4 and at most 64*4*NV4: the whole row lives in registers
+// (NV4 float4 per lane), so HBM sees exactly one 128-bit read and one 128-bit write per element.
+typedef float f32x4s __attribute__((ext_vector_type(4)));
+
+template <bool BACKWARD, int NV4>
+__global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __restrict__ io,
+                                                                    const float* __restrict__ pp, int64_t nrow,
+                                                                    int nvec, const float* __restrict__ hcoef) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kTB / 64) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (kTB / 64);
+    const float coef = (BACKWARD && hcoef) ? *hcoef : 0.f;
+    for (int64_t row = wave; row < nrow; row += nwaves) {
+        float* __restrict__ r = io + row * nvec;
+        f32x4s v[NV4];
+#pragma unroll
+        for (int i = 0; i < NV4; i++) {
+            const int k = 4 * lane + 256 * i;
+            v[i] = f32x4s{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            if (k < nvec) v[i] = *reinterpret_cast<const f32x4s*>(r + k);
+        }
+        if (!BACKWARD) {
+            float mx = -FLT_MAX;
+#pragma unroll
+            for (int i = 0; i < NV4; i++) mx = fmaxf(mx, fmaxf(fmaxf(v[i][0], v[i][1]), fmaxf(v[i][2], v[i][3])));
+            mx = wmax(mx);
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < NV4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    v[i][j] = expf(v[i][j] - mx);   // padding lanes hold -inf: exp gives 0
+                    sum += v[i][j];
+                }
+            sum = wsum(sum);
+#pragma unroll
+            for (int i = 0; i < NV4; i++) {
+                const int k = 4 * lane + 256 * i;
+                if (k < nvec) *reinterpret_cast<f32x4s*>(r + k) = v[i] / sum;
+            }
+        } else {
+            const float* __restrict__ pr = pp + row * nvec;
+            f32x4s q[NV4];
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < NV4; i++) {
+                const int k = 4 * lane + 256 * i;
+                q[i] = f32x4s{0.f, 0.f, 0.f, 0.f};
+                if (k < nvec) {
+                    q[i] = *reinterpret_cast<const f32x4s*>(pr + k);
+                    dot += q[i][0] * v[i][0] + q[i][1] * v[i][1] + q[i][2] * v[i][2] + q[i][3] * v[i][3];
+                }
+            }
+            dot = wsum(dot);
+#pragma unroll
+            for (int i = 0; i < NV4; i++) {
+                const int k = 4 * lane + 256 * i;
+                if (k < nvec) *reinterpret_cast<f32x4s*>(r + k) = coef * q[i] * (v[i] - dot);
+            }
+        }
+    }
+}
+
+// 2..128 heads, outer row (nvec*ncol floats) at most kTB*EMAX long: each thread keeps its EMAX
+// elements (all of one head) in registers between the passes.
+template <bool BACKWARD, int EMAX>
+__global__ void __launch_bounds__(kTB) softmax_axis_block_reg_kernel(float* __restrict__ io,
+                                                                     const float* __restrict__ pp, int64_t nvec,
+                                                                     int ncol, int tb,
+                                                                     const float* __restrict__ hcoef) {
+    __shared__ float red[kTB];
+    const int t = threadIdx.x;
+    const int len = (int)(nvec * ncol);
+    float* __restrict__ r = io + (int64_t)blockIdx.x * len;
+    const bool active = t < tb;
+    const int c = t % ncol;
+    auto fold = [&](float mine, bool is_max) -> float {
+        __syncthreads();
+        red[t] = mine;
+        __syncthreads();
+        float a = is_max ? -FLT_MAX : 0.f;
+        for (int u = c; u < tb; u += ncol) a = is_max ? fmaxf(a, red[u]) : a + red[u];
+        return a;
+    };
+    float v[EMAX];
+#pragma unroll
+    for (int i = 0; i < EMAX; i++) {
+        const int e = t + i * tb;
+        v[i] = (active && e < len) ? r[e] : -INFINITY;
+    }
+    if (!BACKWARD) {
+        float mx = -FLT_MAX;
+#pragma unroll
+        for (int i = 0; i < EMAX; i++) mx = fmaxf(mx, v[i]);
+        mx = fold(mx, true);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < EMAX; i++) {
+            v[i] = expf(v[i] - mx);
+            sum += v[i];
+        }
+        sum = fold(sum, false);
+#pragma unroll
+        for (int i = 0; i < EMAX; i++) {
+            const int e = t + i * tb;
+            if (active && e < len) r[e] = v[i] / sum;
+        }
+    } else {
+        const float coef = hcoef ? *hcoef : 0.f;
+        const float* __restrict__ p = pp + (int64_t)blockIdx.x * len;
+        float q[EMAX];
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < EMAX; i++) {
+            const int e = t + i * tb;
+            q[i] = (active && e < len) ? p[e] : 0.f;
+            if (active && e < len) dot += q[i] * v[i];
+        }
+        dot = fold(dot, false);
+#pragma unroll
+        for (int i = 0; i < EMAX; i++) {
+            const int e = t + i * tb;
+            if (active && e < len) r[e] = coef * q[i] * (v[i] - dot);
+        }
+    }
+}
+
 template <bool BACKWARD>
 __global__ void __launch_bounds__(kTB) softmax_axis_thread_kernel(float* __restrict__ io,
                                                                   const float* __restrict__ pp, int64_t nrow,
@@ -159,12 +299,30 @@ static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, in
     if (ncol == 1) {
         const int64_t blocks = (nrow + kTB / 64 - 1) / (kTB / 64);
         if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "softmax_direct_on_axis: too many rows");
-        softmax_axis_wave_kernel<BACKWARD><<<dim3((unsigned)blocks), kTB, 0, stream>>>(io, pp, nrow, nvec, hcoef);
+        const bool vec = nvec % 4 == 0 && nvec <= 2048 && aligned16(io) && (!BACKWARD || aligned16(pp));
+        if (vec) {
+            const unsigned g = (unsigned)(blocks < 256 * 8 ? blocks : 256 * 8);   // grid-stride over rows
+            const int nv = (int)nvec;
+            if (nvec <= 256) softmax_axis_wave_reg_kernel<BACKWARD, 1><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+            else if (nvec <= 512) softmax_axis_wave_reg_kernel<BACKWARD, 2><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+            else if (nvec <= 1024) softmax_axis_wave_reg_kernel<BACKWARD, 4><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+            else softmax_axis_wave_reg_kernel<BACKWARD, 8><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+        } else {
+            softmax_axis_wave_kernel<BACKWARD><<<dim3((unsigned)blocks), kTB, 0, stream>>>(io, pp, nrow, nvec, hcoef);
+        }
     } else if (ncol <= 128) {
         if (nrow > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "softmax_direct_on_axis: too many rows");
         const int tb = (int)ncol * (kTB / (int)ncol);
-        softmax_axis_block_kernel<BACKWARD><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol, tb,
-                                                                                     hcoef);
+        const int64_t len = nvec * ncol;
+        if (len <= (int64_t)tb * 16)
+            softmax_axis_block_reg_kernel<BACKWARD, 16><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol,
+                                                                                                 tb, hcoef);
+        else if (len <= (int64_t)tb * 32)
+            softmax_axis_block_reg_kernel<BACKWARD, 32><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol,
+                                                                                                 tb, hcoef);
+        else
+            softmax_axis_block_kernel<BACKWARD><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol, tb,
+                                                                                         hcoef);
     } else {
         const int64_t blocks = (nrow * ncol + kTB - 1) / kTB;
         if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "softmax_direct_on_axis: too many rows");
