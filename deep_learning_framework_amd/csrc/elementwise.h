@@ -18,6 +18,20 @@ int launch_softmax_rows_backward(float* gx, const float* gy, const float* x, int
 int launch_fill_float(float* p, int64_t n, float value, hipStream_t stream);
 int launch_fill_int(int* p, int64_t n, int value, hipStream_t stream);
 
+// Final pass of a split-K product: C(m,n) (=|+=) act(alpha * sum_s part[s][m][n] + bias[n]), the
+// pre-activation value also to C2 when given.  `part` holds nsplit dense [M,N] matrices.
+struct SplitReduceParams {
+    const float* part;
+    float* C;
+    float* C2;
+    const float* bias;
+    const float* alpha;   // device scalar or null
+    const float* leaky;   // device scalar or null
+    int64_t M, N, c_rs, c_cs;
+    int nsplit, act, accflag;
+};
+int launch_splitk_reduce(const SplitReduceParams& p, hipStream_t stream);
+
 // attention_ops.hip
 int launch_attention_mask(float* pp, int64_t ndat, int64_t ntimes, int64_t nhead, int forward, hipStream_t stream);
 int launch_softmax_axis(float* pp, int64_t nrow, int64_t nvec, int64_t ncol, hipStream_t stream);

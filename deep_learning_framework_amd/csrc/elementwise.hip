@@ -244,4 +244,58 @@ int launch_fill_int(int* p, int64_t n, int value, hipStream_t stream) {
     return check_launch("fill_kernel");
 }
 
+// ---- split-K final pass ---------------------------------------------------------------------
+//
+// Sums the partial products in split order (fixed, so the result does not depend on scheduling)
+// and applies the GEMM epilogue.  VEC: four consecutive columns per thread with 128-bit accesses.
+
+template <bool VEC>
+__global__ void __launch_bounds__(kEwThreads) splitk_reduce_kernel(SplitReduceParams p) {
+    constexpr int W = VEC ? 4 : 1;
+    const int64_t total = p.M * p.N;
+    const int64_t e = ((int64_t)blockIdx.x * kEwThreads + threadIdx.x) * W;
+    if (e >= total) return;
+    const float alpha = p.alpha ? *p.alpha : 1.0f;
+    const float leaky = p.leaky ? *p.leaky : 0.0f;
+    const int64_t m = e / p.N, n = e - m * p.N;
+    float v[W];
+    if (VEC) {
+        f32x4 s = *reinterpret_cast<const f32x4*>(p.part + e);
+        for (int k = 1; k < p.nsplit; k++) s += *reinterpret_cast<const f32x4*>(p.part + k * total + e);
+        for (int j = 0; j < W; j++) v[j] = s[j];
+    } else {
+        float s = p.part[e];
+        for (int k = 1; k < p.nsplit; k++) s += p.part[k * total + e];
+        v[0] = s;
+    }
+    const int64_t idx = m * p.c_rs + n * p.c_cs;
+    for (int j = 0; j < W; j++) {
+        float o = v[j] * alpha;
+        if (p.accflag) o += p.C[idx + j * p.c_cs];
+        if (p.bias) o += p.bias[n + j];
+        v[j] = o;
+    }
+    if (VEC) {
+        f32x4 o = {v[0], v[1], v[2], v[3]};
+        if (p.C2) *reinterpret_cast<f32x4*>(p.C2 + idx) = o;
+        for (int j = 0; j < W; j++) o[j] = apply_act(o[j], p.act, leaky);
+        *reinterpret_cast<f32x4*>(p.C + idx) = o;
+    } else {
+        if (p.C2) p.C2[idx] = v[0];
+        p.C[idx] = apply_act(v[0], p.act, leaky);
+    }
+}
+
+int launch_splitk_reduce(const SplitReduceParams& p, hipStream_t stream) {
+    const int64_t total = p.M * p.N;
+    if (total <= 0) return KAI_OK;
+    const bool vec = p.c_cs == 1 && p.N % 4 == 0 && p.c_rs % 4 == 0 && aligned16(p.part) && aligned16(p.C) &&
+                     (!p.C2 || aligned16(p.C2)) && (!p.bias || aligned16(p.bias));
+    if (vec)
+        splitk_reduce_kernel<true><<<blocks_for(total / 4), kEwThreads, 0, stream>>>(p);
+    else
+        splitk_reduce_kernel<false><<<blocks_for(total), kEwThreads, 0, stream>>>(p);
+    return check_launch("splitk_reduce_kernel");
+}
+
 }  // namespace kai

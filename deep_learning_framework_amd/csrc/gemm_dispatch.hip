@@ -30,9 +30,13 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
         return launch_skinny_nt(s, stream);
     }
 
-    const bool a_kc = operand_is_kc(d.a_rs, d.a_ks);
-    const bool b_kc = operand_is_kc(d.b_rs, d.b_ks);
-    const GemmParams p = make_params(d, a_kc, b_kc);
+    // batch strides that are never multiplied by a non-zero index must not spoil the alignment checks
+    GemmDesc dn = d;
+    if (dn.bdiv <= 1) { dn.bdiv = 1; dn.a_bs1 = dn.b_bs1 = dn.c_bs1 = 0; }
+    if (dn.nbatch <= dn.bdiv) dn.a_bs0 = dn.b_bs0 = dn.c_bs0 = 0;
+    const bool a_kc = operand_is_kc(dn.a_rs, dn.a_ks);
+    const bool b_kc = operand_is_kc(dn.b_rs, dn.b_ks);
+    const GemmParams p = make_params(dn, a_kc, b_kc);
 
     // largest tile that still yields about one workgroup per compute unit and is not mostly padding
     const int64_t short_side = d.M < d.N ? d.M : d.N;

@@ -256,6 +256,94 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     tn = in_g / rows;
 }
 
+// Epilogue of one output tile.  In registers: alpha, += C (acc), bias, optional store of the
+// pre-activation, then none / relu / leaky relu.  The transcendental activations are applied in a
+// second, rolled pass in which each thread re-reads the values it has just stored: that keeps the
+// unrolled part small enough for the accumulators to stay in registers for the whole kernel.
+template <int NBM, int NBN, bool A_KC, bool B_KC>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[NBM][NBN], int m0, int n0,
+                                              int64_t c_off, int wm0, int wn0, int l32, int half, float alpha,
+                                              float leaky) {
+    float* C = p.C + c_off;
+    float* C2 = p.C2 ? p.C2 + c_off : nullptr;
+    const int act = p.act;
+    const bool slow_act = act > kActLeaky;
+
+    auto row_of = [&](int i, int r) -> int {
+        const int mi = 8 * (r >> 2) + 4 * half + (r & 3);   // row inside the 32x32 block
+        return m0 + (A_KC ? wm0 + 32 * i + mi : wm0 + NBM * mi + i);
+    };
+    auto col_of = [&](int j) -> int { return n0 + (B_KC ? wn0 + 32 * j + l32 : wn0 + NBN * l32 + j); };
+    auto cheap_act = [&](float v) -> float {
+        if (act == kActRelu) return (v > 0) ? v : 0.0f;
+        if (act == kActLeaky) return (v > 0) ? v : v * leaky;
+        return v;
+    };
+    const bool vec_store = !B_KC && NBN == 4 && p.c_vec;
+
+    static_for<0, NBM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        static_for<0, 16>([&](auto rc) {
+            constexpr int r = decltype(rc)::value;
+            const int row = row_of(i, r);
+            const bool row_ok = row < p.M;
+            if (vec_store) {
+                const int col = col_of(0);
+                if (row_ok && col < p.N) {   // N % 4 == 0 under c_vec, so the whole chunk is inside
+                    const int64_t idx = (int64_t)row * p.c_rs + col;
+                    f32x4 o;
+                    static_for<0, 4>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        o[j] = acc[i][j % NBN][r];
+                    });
+                    if (p.has_alpha) o *= alpha;
+                    if (p.accflag) o += *reinterpret_cast<const f32x4*>(C + idx);
+                    if (p.bias) o += *reinterpret_cast<const f32x4*>(p.bias + col);
+                    if (C2) *reinterpret_cast<f32x4*>(C2 + idx) = o;
+                    static_for<0, 4>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        o[j] = cheap_act(o[j]);
+                    });
+                    *reinterpret_cast<f32x4*>(C + idx) = o;
+                }
+            } else {
+                static_for<0, NBN>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    const int col = col_of(j);
+                    if (row_ok && col < p.N) {
+                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
+                        float v = acc[i][j][r];
+                        if (p.has_alpha) v *= alpha;
+                        if (p.accflag) v += C[idx];
+                        if (p.bias) v += p.bias[col];
+                        if (C2) C2[idx] = v;
+                        C[idx] = cheap_act(v);
+                    }
+                });
+            }
+        });
+    });
+
+    if (slow_act) {
+#pragma nounroll
+        for (int i = 0; i < NBM; i++) {
+#pragma nounroll
+            for (int r = 0; r < 16; r++) {
+                const int row = row_of(i, r);
+                if (row >= p.M) continue;
+#pragma nounroll
+                for (int j = 0; j < NBN; j++) {
+                    const int col = col_of(j);
+                    if (col < p.N) {
+                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
+                        C[idx] = apply_act(C[idx], act, leaky);
+                    }
+                }
+            }
+        }
+    }
+}
+
 // EDGE = false: the host has checked that M, N, K are multiples of the tile, that both operands
 // allow aligned 128-bit loads and that a tile's offsets fit 32 bits; the kernel then holds no
 // predicated load code at all (fewer registers).  EDGE = true: general shapes.
@@ -500,91 +588,9 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         }
     }
 
-    // ---- epilogue ------------------------------------------------------------------------------
-    // In registers: alpha, += C (acc), bias, optional store of the pre-activation, then none / relu /
-    // leaky relu.  The transcendental activations are applied in a second, rolled pass in which
-    // each thread re-reads the values it has just stored: that keeps the unrolled part small enough
-    // for the accumulators to stay in registers for the whole kernel.
     const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
     const float leaky = p.leaky ? *p.leaky : 0.f;
-    float* C = p.C + c_off;
-    float* C2 = p.C2 ? p.C2 + c_off : nullptr;
-    const int act = p.act;
-    const bool slow_act = act > kActLeaky;
-
-    auto row_of = [&](int i, int r) -> int {
-        const int mi = 8 * (r >> 2) + 4 * half + (r & 3);   // row inside the 32x32 block
-        return m0 + (A_KC ? wm0 + 32 * i + mi : wm0 + NBM * mi + i);
-    };
-    auto col_of = [&](int j) -> int { return n0 + (B_KC ? wn0 + 32 * j + l32 : wn0 + NBN * l32 + j); };
-    auto cheap_act = [&](float v) -> float {
-        if (act == kActRelu) return (v > 0) ? v : 0.0f;
-        if (act == kActLeaky) return (v > 0) ? v : v * leaky;
-        return v;
-    };
-    const bool vec_store = !B_KC && NBN == 4 && p.c_vec;
-
-    static_for<0, NBM>([&](auto ic) {
-        constexpr int i = decltype(ic)::value;
-        static_for<0, 16>([&](auto rc) {
-            constexpr int r = decltype(rc)::value;
-            const int row = row_of(i, r);
-            const bool row_ok = row < p.M;
-            if (vec_store) {
-                const int col = col_of(0);
-                if (row_ok && col < p.N) {   // N % 4 == 0 under c_vec, so the whole chunk is inside
-                    const int64_t idx = (int64_t)row * p.c_rs + col;
-                    f32x4 o;
-                    static_for<0, 4>([&](auto jc) {
-                        constexpr int j = decltype(jc)::value;
-                        o[j] = acc[i][j % NBN][r];
-                    });
-                    if (p.has_alpha) o *= alpha;
-                    if (p.accflag) o += *reinterpret_cast<const f32x4*>(C + idx);
-                    if (p.bias) o += *reinterpret_cast<const f32x4*>(p.bias + col);
-                    if (C2) *reinterpret_cast<f32x4*>(C2 + idx) = o;
-                    static_for<0, 4>([&](auto jc) {
-                        constexpr int j = decltype(jc)::value;
-                        o[j] = cheap_act(o[j]);
-                    });
-                    *reinterpret_cast<f32x4*>(C + idx) = o;
-                }
-            } else {
-                static_for<0, NBN>([&](auto jc) {
-                    constexpr int j = decltype(jc)::value;
-                    const int col = col_of(j);
-                    if (row_ok && col < p.N) {
-                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
-                        float v = acc[i][j][r];
-                        if (p.has_alpha) v *= alpha;
-                        if (p.accflag) v += C[idx];
-                        if (p.bias) v += p.bias[col];
-                        if (C2) C2[idx] = v;
-                        C[idx] = cheap_act(v);
-                    }
-                });
-            }
-        });
-    });
-
-    if (slow_act) {
-#pragma nounroll
-        for (int i = 0; i < NBM; i++) {
-#pragma nounroll
-            for (int r = 0; r < 16; r++) {
-                const int row = row_of(i, r);
-                if (row >= p.M) continue;
-#pragma nounroll
-                for (int j = 0; j < NBN; j++) {
-                    const int col = col_of(j);
-                    if (col < p.N) {
-                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
-                        C[idx] = apply_act(C[idx], act, leaky);
-                    }
-                }
-            }
-        }
-    }
+    gemm_epilogue<NBM, NBN, A_KC, B_KC>(p, acc, m0, n0, c_off, wm0, wn0, l32, half, alpha, leaky);
 }
 
 }  // namespace kai

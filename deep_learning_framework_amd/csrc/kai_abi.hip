@@ -6,6 +6,7 @@
 // mh_attention (:2978-3052) and multihead_attention_backprop (:3054-3227).
 #include <cstring>
 #include <cstdlib>
+#include <mutex>
 
 #include "elementwise.h"
 #include "gemm_host.h"
@@ -29,6 +30,64 @@ int check_hip(hipError_t st, const char* what) {
 }
 
 int check_launch(const char* kernel_name) { return check_hip(hipGetLastError(), kernel_name); }
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_ws_mutex;
+void* g_ws_ptr[kMaxDevices] = {};
+int64_t g_ws_bytes[kMaxDevices] = {};
+int g_cu_count[kMaxDevices] = {};
+}  // namespace
+
+int workspace(int64_t bytes, float** out) {
+    int dev = 0;
+    KAI_TRY(check_hip(hipGetDevice(&dev), "hipGetDevice"));
+    if (dev < 0 || dev >= kMaxDevices) return fail(KAI_ERR_INVALID_ARGUMENT, "workspace: device index out of range");
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (g_ws_bytes[dev] < bytes) {
+        // earlier users of the smaller buffer are ordered before the free by the device-wide wait
+        if (g_ws_ptr[dev]) {
+            KAI_TRY(check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize"));
+            KAI_TRY(check_hip(hipFree(g_ws_ptr[dev]), "hipFree"));
+            g_ws_ptr[dev] = nullptr;
+            g_ws_bytes[dev] = 0;
+        }
+        const int64_t want = bytes < (16ll << 20) ? (16ll << 20) : bytes;
+        KAI_TRY(check_hip(hipMalloc(&g_ws_ptr[dev], (size_t)want), "hipMalloc(workspace)"));
+        g_ws_bytes[dev] = want;
+    }
+    *out = static_cast<float*>(g_ws_ptr[dev]);
+    return KAI_OK;
+}
+
+int compute_units() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    if (g_cu_count[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        g_cu_count[dev] = n;
+    }
+    return g_cu_count[dev];
+}
+
+static int release_workspaces() {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    int old = 0;
+    if (hipGetDevice(&old) != hipSuccess) old = 0;
+    int rc = KAI_OK;
+    for (int d = 0; d < kMaxDevices; d++) {
+        if (!g_ws_ptr[d]) continue;
+        if (hipSetDevice(d) == hipSuccess) {
+            hipDeviceSynchronize();
+            if (hipFree(g_ws_ptr[d]) != hipSuccess) rc = KAI_ERR_GPU;
+        }
+        g_ws_ptr[d] = nullptr;
+        g_ws_bytes[d] = 0;
+    }
+    hipSetDevice(old);
+    return rc;
+}
 
 static bool act_is_elementwise(int act) { return act >= KAI_ACT_NONE && act <= KAI_ACT_SWISH; }
 
@@ -57,6 +116,12 @@ int kai_device_synchronize(void) { return check_hip(hipDeviceSynchronize(), "hip
 
 int kai_set_stream(void* hip_stream) {
     tl_stream = reinterpret_cast<hipStream_t>(hip_stream);
+    return KAI_OK;
+}
+
+int kai_shutdown(void) {
+    const int rc = release_workspaces();
+    if (rc != KAI_OK) return fail(rc, "kai_shutdown: hipFree failed");
     return KAI_OK;
 }
 

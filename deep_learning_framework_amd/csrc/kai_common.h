@@ -23,6 +23,13 @@ int check_hip(hipError_t st, const char* what);
 // status of the launch that was just enqueued
 int check_launch(const char* kernel_name);
 
+// Library-owned scratch memory on the CURRENT device (split-K partial sums).  Allocated on first use,
+// grown when a call needs more, released by kai_shutdown.  Calls that use it must be ordered on one
+// stream per device: the engine runs one thread (and the null stream) per device.
+int workspace(int64_t bytes, float** out);
+// number of compute units of the current device (cached)
+int compute_units();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 constexpr int64_t kMaxDim = (1ll << 31) - 1;

@@ -28,6 +28,7 @@ SIGNATURES = {
     "kai_device_synchronize": [],
     "kai_set_stream": [ctypes.c_void_p],
     "kai_arch_info": [ctypes.c_char_p, ctypes.c_char_p, _INT],
+    "kai_shutdown": [],
     "kai_mem_alloc": [_INT, _I64, ctypes.POINTER(ctypes.c_void_p)],
     "kai_mem_free": [_INT, ctypes.c_void_p],
     "kai_memcpy_host_to_host": [ctypes.c_void_p, ctypes.c_void_p, _I64],
@@ -176,6 +177,11 @@ def synchronize():
 
 def set_stream(stream_handle):
     _ck(load().kai_set_stream(stream_handle))
+
+
+def shutdown():
+    """Release the library's own scratch memory (it is re-created on demand)."""
+    _ck(load().kai_shutdown())
 
 
 def arch_info():

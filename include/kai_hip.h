@@ -77,6 +77,10 @@ int kai_device_synchronize(void);
 /* Stream (a hipStream_t, or null for the null stream) that this THREAD's later calls enqueue on.
  * No counterpart in the reference, which only uses the legacy default stream. */
 int kai_set_stream(void* hip_stream);
+/* Releases the scratch memory the library allocated for itself (split-K partial sums; one buffer per
+ * device, created on first need).  The library stays usable: the buffer is created again on demand.
+ * No counterpart in the reference, whose kernels need no scratch. */
+int kai_shutdown(void);
 /* Name of the code object's target ("gfx950") and of the current device's architecture. */
 int kai_arch_info(char* built_for, char* device_arch, int buflen);
 
