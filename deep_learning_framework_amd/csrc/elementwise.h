@@ -28,7 +28,7 @@ struct SplitReduceParams {
     const float* alpha;   // device scalar or null
     const float* leaky;   // device scalar or null
     int64_t M, N, c_rs, c_cs;
-    int nsplit, act, accflag;
+    int nsplit, act, accflag, has_alpha;   // has_alpha with a null alpha multiplies by 0
 };
 int launch_splitk_reduce(const SplitReduceParams& p, hipStream_t stream);
 

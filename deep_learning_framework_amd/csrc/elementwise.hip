@@ -255,7 +255,7 @@ __global__ void __launch_bounds__(kEwThreads) splitk_reduce_kernel(SplitReducePa
     const int64_t total = p.M * p.N;
     const int64_t e = ((int64_t)blockIdx.x * kEwThreads + threadIdx.x) * W;
     if (e >= total) return;
-    const float alpha = p.alpha ? *p.alpha : 1.0f;
+    const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.0f) : 1.0f;
     const float leaky = p.leaky ? *p.leaky : 0.0f;
     const int64_t m = e / p.N, n = e - m * p.N;
     float v[W];
@@ -270,7 +270,7 @@ __global__ void __launch_bounds__(kEwThreads) splitk_reduce_kernel(SplitReducePa
     }
     const int64_t idx = m * p.c_rs + n * p.c_cs;
     for (int j = 0; j < W; j++) {
-        float o = v[j] * alpha;
+        float o = p.has_alpha ? v[j] * alpha : v[j];
         if (p.accflag) o += p.C[idx + j * p.c_cs];
         if (p.bias) o += p.bias[n + j];
         v[j] = o;

@@ -2,6 +2,7 @@
 // most 16 rows against a K-contiguous weight matrix, otherwise the MFMA kernel in the LDS
 // orientation pair that matches how the operands lie in memory, with the largest tile that still
 // fills the 256 compute units.
+#include "elementwise.h"
 #include "gemm_host.h"
 #include "gemv_skinny.h"
 
@@ -9,6 +10,80 @@ namespace kai {
 
 static int64_t tiles_of(int64_t M, int64_t N, int64_t nbatch, int64_t t) {
     return ((M + t - 1) / t) * ((N + t - 1) / t) * nbatch;
+}
+
+// Only reductions of at least kSplitFromK steps are cut (a shorter one does not repay the second
+// launch), into at most kSplitMax parts of at least kSplitMinK steps each.
+constexpr int64_t kSplitFromK = 512;
+constexpr int64_t kSplitMinK = 64;
+constexpr int64_t kSplitMax = 16;
+
+static int launch_layout(const GemmParams& p, bool a_kc, bool b_kc, int64_t nbatch, int tile, hipStream_t stream) {
+    if (a_kc && b_kc) return launch_gemm_kc_kc(p, nbatch, tile, stream);
+    if (a_kc && !b_kc) return launch_gemm_kc_mc(p, nbatch, tile, stream);
+    if (!a_kc && !b_kc) return launch_gemm_mc_mc(p, nbatch, tile, stream);
+    return launch_gemm_mc_kc(p, nbatch, tile, stream);
+}
+
+namespace {
+
+struct GemmPlan {
+    bool skinny = false;
+    bool a_kc = false, b_kc = false;
+    int tile = kTileSmall;
+    int64_t split = 1;
+    GemmDesc dn;   // the product with batch strides normalised
+};
+
+GemmPlan plan_gemm(const GemmDesc& d) {
+    GemmPlan plan;
+    // skinny: y = x . w^T with both operands K-contiguous, a contiguous output row, no scaling
+    plan.skinny = d.M <= kSkinnyMaxRows && d.nbatch == 1 && d.a_ks == 1 && d.b_ks == 1 && d.c_cs == 1 &&
+                  !d.has_alpha && d.K > 0 && d.N >= 256;
+    // batch strides that are never multiplied by a non-zero index must not spoil the alignment checks
+    GemmDesc& dn = plan.dn;
+    dn = d;
+    if (dn.bdiv <= 1) { dn.bdiv = 1; dn.a_bs1 = dn.b_bs1 = dn.c_bs1 = 0; }
+    if (dn.nbatch <= dn.bdiv) dn.a_bs0 = dn.b_bs0 = dn.c_bs0 = 0;
+    plan.a_kc = operand_is_kc(dn.a_rs, dn.a_ks);
+    plan.b_kc = operand_is_kc(dn.b_rs, dn.b_ks);
+
+    // largest tile that still yields about one workgroup per compute unit and is not mostly padding
+    const int64_t short_side = d.M < d.N ? d.M : d.N;
+    if (short_side > 128 && tiles_of(d.M, d.N, d.nbatch, 256) >= 192) plan.tile = kTileLarge;
+    else if (short_side > 64 && tiles_of(d.M, d.N, d.nbatch, 128) >= 128) plan.tile = kTileMedium;
+
+    // Split-K: a single product whose output tiles leave most compute units idle is cut along K
+    // into `split` equal parts that run as the batch dimension of the same kernel and write raw
+    // partial products to the library's scratch; a second launch sums them in a fixed order and
+    // applies the epilogue.
+    if (!plan.skinny && d.nbatch == 1 && d.K >= kSplitFromK) {
+        const int64_t edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
+        const int64_t tiles = tiles_of(d.M, d.N, 1, edge);
+        int64_t split = compute_units() / tiles;
+        if (split > d.K / kSplitMinK) split = d.K / kSplitMinK;
+        if (split > kSplitMax) split = kSplitMax;
+        // equal parts of whole 16-step tiles if some part count allows it, else parts that at least keep
+        // the operands' 16-byte alignment
+        int64_t whole = split;
+        while (whole >= 2 && d.K % (whole * 16) != 0) whole--;
+        if (whole >= 2) split = whole;
+        else while (split >= 2 && d.K % (split * 4) != 0) split--;
+        if (split >= 2) plan.split = split;
+    }
+    return plan;
+}
+
+bool valid_dims(const GemmDesc& d) {
+    return d.M >= 0 && d.N >= 0 && d.K >= 0 && d.nbatch >= 0 && d.M <= kMaxDim && d.N <= kMaxDim && d.K <= kMaxDim;
+}
+
+}  // namespace
+
+bool gemm_fuses_rowsum(const GemmDesc& d) {
+    if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
+    const GemmPlan plan = plan_gemm(d);
+    return !plan.skinny && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge && plan.split == 1;
 }
 
 int launch_gemm(const GemmDesc& d, hipStream_t stream) {
@@ -19,9 +94,11 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
     if (d.M == 0 || d.N == 0 || d.nbatch == 0) return KAI_OK;
     if (!d.C || (d.K > 0 && (!d.A || !d.B))) return fail(KAI_ERR_INVALID_POINTER, "gemm: null operand");
 
-    // skinny: y = x . w^T with both operands K-contiguous, a contiguous output row, no scaling
-    if (d.M <= kSkinnyMaxRows && d.nbatch == 1 && d.a_ks == 1 && d.b_ks == 1 && d.c_cs == 1 && !d.has_alpha &&
-        d.K > 0 && d.N >= 256) {
+    const GemmPlan plan = plan_gemm(d);
+    if (d.rowsum && !gemm_fuses_rowsum(d))
+        return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: this product cannot carry the fused row sum");
+
+    if (plan.skinny) {
         SkinnyParams s{};
         s.W = d.B; s.X = d.A; s.Y = d.C; s.Y2 = d.C2; s.bias = d.bias; s.leaky = d.leaky;
         s.ldw = d.b_rs; s.ldx = d.a_rs; s.ldy = d.c_rs;
@@ -30,24 +107,27 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
         return launch_skinny_nt(s, stream);
     }
 
-    // batch strides that are never multiplied by a non-zero index must not spoil the alignment checks
-    GemmDesc dn = d;
-    if (dn.bdiv <= 1) { dn.bdiv = 1; dn.a_bs1 = dn.b_bs1 = dn.c_bs1 = 0; }
-    if (dn.nbatch <= dn.bdiv) dn.a_bs0 = dn.b_bs0 = dn.c_bs0 = 0;
-    const bool a_kc = operand_is_kc(dn.a_rs, dn.a_ks);
-    const bool b_kc = operand_is_kc(dn.b_rs, dn.b_ks);
-    const GemmParams p = make_params(dn, a_kc, b_kc);
-
-    // largest tile that still yields about one workgroup per compute unit and is not mostly padding
-    const int64_t short_side = d.M < d.N ? d.M : d.N;
-    int tile = kTileSmall;
-    if (short_side > 128 && tiles_of(d.M, d.N, d.nbatch, 256) >= 192) tile = kTileLarge;
-    else if (short_side > 64 && tiles_of(d.M, d.N, d.nbatch, 128) >= 128) tile = kTileMedium;
-
-    if (a_kc && b_kc) return launch_gemm_kc_kc(p, d.nbatch, tile, stream);
-    if (a_kc && !b_kc) return launch_gemm_kc_mc(p, d.nbatch, tile, stream);
-    if (!a_kc && !b_kc) return launch_gemm_mc_mc(p, d.nbatch, tile, stream);
-    return launch_gemm_mc_kc(p, d.nbatch, tile, stream);
+    const bool a_kc = plan.a_kc, b_kc = plan.b_kc;
+    if (plan.split >= 2) {
+        const int64_t split = plan.split;
+        float* part = nullptr;
+        KAI_TRY(workspace(split * d.M * d.N * (int64_t)sizeof(float), &part));
+        GemmDesc ds = plan.dn;
+        ds.K = d.K / split;
+        ds.nbatch = split; ds.bdiv = 1;
+        ds.a_bs0 = ds.K * d.a_ks; ds.b_bs0 = ds.K * d.b_ks; ds.c_bs0 = d.M * d.N;
+        ds.a_bs1 = ds.b_bs1 = ds.c_bs1 = 0;
+        ds.C = part; ds.c_rs = d.N; ds.c_cs = 1;
+        ds.C2 = nullptr; ds.bias = nullptr; ds.alpha = nullptr; ds.leaky = nullptr;
+        ds.act = 0; ds.acc = 0; ds.has_alpha = 0;
+        KAI_TRY(launch_layout(make_params(ds, a_kc, b_kc), a_kc, b_kc, split, plan.tile, stream));
+        SplitReduceParams r{};
+        r.part = part; r.C = d.C; r.C2 = d.C2; r.bias = d.bias; r.alpha = d.alpha; r.leaky = d.leaky;
+        r.M = d.M; r.N = d.N; r.c_rs = d.c_rs; r.c_cs = d.c_cs;
+        r.nsplit = (int)split; r.act = d.act; r.accflag = d.acc; r.has_alpha = d.has_alpha;
+        return launch_splitk_reduce(r, stream);
+    }
+    return launch_layout(make_params(plan.dn, a_kc, b_kc), a_kc, b_kc, d.nbatch, plan.tile, stream);
 }
 
 }  // namespace kai

@@ -23,6 +23,10 @@ struct GemmDesc {
     int act = 0;
     int acc = 0;
     int has_alpha = 0;
+    // optional: rowsum[m] (=|+=) sum_k A(m,k) computed by the same launch; only products for which
+    // gemm_fuses_rowsum() holds may set it
+    float* rowsum = nullptr;
+    int rowsum_acc = 0;
 };
 
 // LDS orientation of an operand: reduction index contiguous (KC) or output index contiguous (MC).
@@ -47,6 +51,8 @@ inline GemmParams make_params(const GemmDesc& d, bool a_kc, bool b_kc) {
     p.act = d.act;
     p.accflag = d.acc;
     p.has_alpha = d.has_alpha;
+    p.rowsum = d.rowsum;
+    p.rowsum_acc = d.rowsum_acc;
     return p;
 }
 
@@ -58,7 +64,7 @@ inline bool fits_without_edges(const GemmParams& p, bool a_kc, bool b_kc, int BM
 }
 
 template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
-          int DEPTH = 1>
+          int DEPTH = 1, bool ROWSUM = false>
 int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t stream) {
     constexpr int BM = WM * NBM * 32, BN = WN * NBN * 32;
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -68,12 +74,15 @@ int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t st
     if (tiles <= 0 || nbatch <= 0) return KAI_OK;
     if (tiles > kMaxDim || nbatch > 65535) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
     dim3 grid((unsigned)tiles, 1, (unsigned)nbatch);
-    gemm_mfma_kernel<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE, PIPE, MINW, DEPTH><<<grid, dim3(64 * WM * WN), 0, stream>>>(p);
+    gemm_mfma_kernel<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE, PIPE, MINW, DEPTH, ROWSUM><<<grid, dim3(64 * WM * WN), 0, stream>>>(p);
     return check_launch("gemm_mfma_kernel");
 }
 
 // picks kernel family, tile and variant; defined in gemm_dispatch.hip
 int launch_gemm(const GemmDesc& d, hipStream_t stream);
+// true when launch_gemm would compute GemmDesc::rowsum inside the product's own launch (d.rowsum is
+// not looked at); otherwise the caller runs a separate column-sum kernel and leaves rowsum null
+bool gemm_fuses_rowsum(const GemmDesc& d);
 
 // per-layout entry points (one translation unit each, to compile in parallel)
 enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2 };

@@ -15,6 +15,16 @@ namespace kai {
 
 constexpr int kGroupM = 4;
 
+// the variants that also sum the rows of A (medium and small tiles, simple schedule)
+template <bool A_KC, bool B_KC>
+int launch_gemm_layout_rowsum(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream) {
+    if (tile == kTileMedium)
+        return launch_gemm_config<2, 2, 2, 2, 16, A_KC, B_KC, true, 0, 1, 1, true>(p, nbatch, kGroupM, stream);
+    if (fits_without_edges(p, A_KC, B_KC, 64, 64, 16))
+        return launch_gemm_config<2, 2, 1, 1, 16, A_KC, B_KC, false, 0, 2, 8, true>(p, nbatch, kGroupM, stream);
+    return launch_gemm_config<2, 2, 1, 1, 16, A_KC, B_KC, true, 0, 1, 1, true>(p, nbatch, kGroupM, stream);
+}
+
 template <bool A_KC, bool B_KC>
 int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream) {
     switch (tile) {

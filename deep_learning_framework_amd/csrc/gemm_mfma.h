@@ -73,6 +73,10 @@ struct GemmParams {
     int has_alpha;        // 1: multiply by (*alpha, or 0 if alpha is null)
     int tiles_m, tiles_n;
     int group_m;          // tile rows per column sweep of the XCD-local ordering
+    // ROWSUM kernels only: rowsum[m] (=|+=) sum_k A(m,k), summed in ascending k (the bias gradient
+    // when A is the transposed output gradient of a dense layer); null switches it off
+    float* rowsum;
+    int rowsum_acc;
 };
 
 constexpr int kLdsPad = 4;
@@ -363,8 +367,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 //
 // DEPTH (PIPE 0 only) is the number of K-tiles kept in flight in staging registers: small tiles
 // compute for far less time than a global load takes to return, so they run several tiles ahead.
+//
+// ROWSUM (PIPE 0 only): the workgroups of the first tile column also sum every row of their A tile
+// over K, one thread per row reading the tile from LDS, k ascending across tiles: a fixed order
+// that is the order of a sequential loop.
 template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
-          int DEPTH = 1>
+          int DEPTH = 1, bool ROWSUM = false>
 __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const GemmParams p) {
     constexpr int NT = 64 * WM * WN;
     constexpr int BM = WM * NBM * 32;
@@ -419,6 +427,9 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     static_assert(DEPTH >= 1 && (PIPE == 0 || DEPTH == 1), "deep register staging belongs to the PIPE 0 schedule");
+    static_assert(!ROWSUM || (PIPE == 0 && BM <= NT), "row sums: PIPE 0 schedule, one thread per tile row");
+    const bool do_rowsum = ROWSUM && p.rowsum != nullptr && tn == 0 && z == 0 && tid < BM;
+    float rowsum = 0.f;
     f32x4 rax[DEPTH][NCHA], rbx[DEPTH][NCHB];
     f32x4(&ra)[NCHA] = rax[0];
     f32x4(&rb)[NCHB] = rbx[0];
@@ -476,6 +487,10 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
                     if (DEPTH == 1 && kt + 1 < nkt) load_global(kt + 1);
                     const float* la = lds_a[cur];
                     const float* lb = lds_b[cur];
+                    if (ROWSUM && do_rowsum) {   // rows and k beyond the matrix were stored as zeros
+#pragma unroll
+                        for (int kk = 0; kk < BK; kk++) rowsum += la[A_KC ? tid * TA::kStride + kk : kk * TA::kStride + tid];
+                    }
 #pragma unroll
                     for (int kg = 0; kg < NKG; kg++) {
                         Frag<A_KC, NBM> fa;
@@ -588,6 +603,10 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         }
     }
 
+    if (ROWSUM && do_rowsum && m0 + tid < p.M) {
+        float* g = p.rowsum + m0 + tid;
+        *g = p.rowsum_acc ? *g + rowsum : rowsum;
+    }
     const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
     const float leaky = p.leaky ? *p.leaky : 0.f;
     gemm_epilogue<NBM, NBN, A_KC, B_KC>(p, acc, m0, n0, c_off, wm0, wn0, l32, half, alpha, leaky);

@@ -52,7 +52,7 @@ int workspace(int64_t bytes, float** out) {
             g_ws_ptr[dev] = nullptr;
             g_ws_bytes[dev] = 0;
         }
-        const int64_t want = bytes < (16ll << 20) ? (16ll << 20) : bytes;
+        const int64_t want = bytes < (4ll << 20) ? (4ll << 20) : bytes;
         KAI_TRY(check_hip(hipMalloc(&g_ws_ptr[dev], (size_t)want), "hipMalloc(workspace)"));
         g_ws_bytes[dev] = want;
     }
@@ -79,13 +79,13 @@ static int release_workspaces() {
     for (int d = 0; d < kMaxDevices; d++) {
         if (!g_ws_ptr[d]) continue;
         if (hipSetDevice(d) == hipSuccess) {
-            hipDeviceSynchronize();
+            (void)hipDeviceSynchronize();
             if (hipFree(g_ws_ptr[d]) != hipSuccess) rc = KAI_ERR_GPU;
         }
         g_ws_ptr[d] = nullptr;
         g_ws_bytes[d] = 0;
     }
-    hipSetDevice(old);
+    (void)hipSetDevice(old);
     return rc;
 }
 
@@ -524,15 +524,28 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
         KAI_TRY(launch_activate_backward(pga_work, pgy, ppre, ndat * yvec, actFunc, hLeakyAlpha, current_stream()));
         ga = pga_work;
     }
-    if (pgb) KAI_TRY(kai_add_bias_backward_b(device, pgb, ga, ndat, yvec, acc));
+    // gw[yvec,xvec] = ga^T . x reads every element of ga; where that product runs on the medium or small
+    // tile its first tile column also produces gb = column sums of ga, in the order of a sequential loop
+    GemmDesc dw;
+    bool fused_gb = false;
+    if (pgw && yvec > 0 && xvec > 0) {
+        KAI_REQUIRE_PTR(px);
+        dw.A = ga; dw.B = px; dw.C = pgw;
+        dw.M = yvec; dw.N = xvec; dw.K = ndat;
+        dw.a_rs = 1; dw.a_ks = yvec; dw.b_rs = 1; dw.b_ks = xvec; dw.c_rs = xvec; dw.c_cs = 1;
+        dw.acc = acc != 0;
+        if (pgb && ndat > 0 && gemm_fuses_rowsum(dw)) {
+            dw.rowsum = pgb;
+            dw.rowsum_acc = acc != 0;
+            fused_gb = true;
+        }
+    }
+    if (pgb && !fused_gb) KAI_TRY(kai_add_bias_backward_b(device, pgb, ga, ndat, yvec, acc));
     if (pgx) {
         KAI_REQUIRE_PTR(pw);
         KAI_TRY(kai_matmul_backward_x(device, pgx, ga, pw, yvec, ndat, xvec, acc));
     }
-    if (pgw) {
-        KAI_REQUIRE_PTR(px);
-        KAI_TRY(kai_matmul_backward_w(device, pgw, ga, px, yvec, ndat, xvec, acc));
-    }
+    if (pgw && yvec > 0 && xvec > 0) KAI_TRY(launch_gemm(dw, current_stream()));
     return KAI_OK;
 }
 

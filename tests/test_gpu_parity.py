@@ -104,6 +104,31 @@ def test_cfg2_relu_backward_chain():
     check(gb.to_numpy((1024,)), ref_gb, what="relu chain db")
 
 
+# the bias gradient rides on the weight-gradient product where that runs on the small or medium tile (whole
+# tiles, edges in every dimension, a tile column count above one) and is a separate kernel elsewhere (reduction
+# long enough to be split, 256-wide tiles)
+@pytest.mark.parametrize("ndat,yvec,xvec,acc", [(256, 1024, 1024, True), (100, 130, 70, False), (37, 200, 333, True),
+                                                (64, 2048, 1024, False), (1024, 64, 64, False),
+                                                (160, 2304, 2560, True), (5, 64, 64, False), (16, 4096, 4096, False)])
+def test_dense_backward_bias_gradient_fused_or_not(ndat, yvec, xvec, acc):
+    rng = np.random.default_rng(ndat + 3 * yvec + 7 * xvec)
+    x = rng.standard_normal((ndat, xvec)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (yvec, xvec)).astype(np.float32)
+    gy = rng.standard_normal((ndat, yvec)).astype(np.float32)
+    gx0 = rng.standard_normal((ndat, xvec)).astype(np.float32)
+    gw0 = rng.standard_normal((yvec, xvec)).astype(np.float32)
+    gb0 = rng.standard_normal(yvec).astype(np.float32)
+    gx, gw, gb = dev(gx0), dev(gw0), dev(gb0)
+    VMath.dense_backward(0, gx, gw, gb, None, dev(gy), dev(w), dev(x), None, yvec, ndat, xvec, kai.ACT["none"], None,
+                         acc)
+    a = dict(acc_into=gx0) if acc else {}
+    check(gx.to_numpy((ndat, xvec)), ko.matmul_backward_x(gy, w, **a), what="dX")
+    a = dict(acc_into=gw0) if acc else {}
+    check(gw.to_numpy((yvec, xvec)), ko.matmul_backward_w(gy, x, yvec, xvec, **a), what="dW")
+    a = dict(acc_into=gb0) if acc else {}
+    check(gb.to_numpy((yvec,)), ko.add_bias_backward_b(gy, yvec, **a), what="db")
+
+
 # ---- configuration 3: 8192^3 GEMM + bias + ReLU -------------------------------------------------------------
 
 def test_cfg3_large_gemm_bias_relu_row_sample():
@@ -191,7 +216,13 @@ def test_cfg5_ragged():
 # ---- shapes around the tile edges, every operand form, acc, unaligned pointers ---------------------------------
 
 SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 9), (64, 64, 64), (65, 63, 66), (100, 300, 50), (128, 128, 32),
-          (129, 257, 40), (256, 256, 16), (300, 520, 128), (31, 1000, 4), (513, 64, 260), (40, 24, 1000)]
+          (129, 257, 40), (256, 256, 16), (300, 520, 128), (31, 1000, 4), (513, 64, 260), (40, 24, 1000),
+          # split along K (few output tiles, long reduction), with and without whole tiles
+          (64, 64, 1024), (100, 300, 4096), (256, 512, 2048), (20, 130, 4000),
+          # 128-wide tiles: pipelined whole-tile kernel, then its edge variant
+          (1024, 2048, 256), (1000, 2000, 130),
+          # 256-wide tiles with edges in every dimension
+          (1500, 3000, 100)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -423,14 +454,50 @@ def test_attention_ops_small(nbat, ntimes, nhead, npiece):
     check(gk.to_numpy((nbat, ntimes, nvec)), ko.mult_on_heads_backward(ref_gs, q, nhead), what="mult_on_heads_backward")
 
 
-@pytest.mark.parametrize("nrow,nvec,ncol", [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8),
-                                            (3, 20, 128), (2, 9, 129), (2, 5, 300)])
+# one case per kernel variant: rows in registers (1 head; 2..128 heads, short and long axis), rows through
+# LDS (long axis, odd lengths), one thread per head (more than 128 heads)
+SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8), (3, 20, 128), (2, 9, 129),
+                       (2, 5, 300), (300, 512, 1), (3, 2048, 1), (2, 2052, 1), (2, 700, 8), (1, 2000, 8),
+                       (2, 1030, 2), (40, 64, 16)]
+
+
+@pytest.mark.parametrize("nrow,nvec,ncol", SOFTMAX_AXIS_SHAPES)
 def test_softmax_axis_layouts(nrow, nvec, ncol):
     rng = np.random.default_rng(nrow + nvec + ncol)
     s = (5 * rng.standard_normal((nrow, nvec, ncol))).astype(np.float32)
     d = dev(s)
     VMath.softmax_direct_on_axis(0, d, nrow, nvec, ncol)
     check(d.to_numpy(s.shape), ko.softmax_direct_on_axis(s, nrow, nvec, ncol), what="softmax axis")
+
+
+@pytest.mark.parametrize("nbat,ntimes,nhead", [(3, 512, 1), (1, 512, 8), (2, 700, 8), (1, 2000, 4), (1, 300, 130),
+                                               (2, 2052, 1)])
+def test_softmax_axis_backward_layouts(nbat, ntimes, nhead):
+    rng = np.random.default_rng(nbat + ntimes + nhead)
+    shape = (nbat, ntimes, ntimes, nhead)
+    logits = (3 * rng.standard_normal(shape)).astype(np.float32)
+    probs = ko.softmax_direct_on_axis(logits, nbat * ntimes, ntimes, nhead).reshape(shape)
+    gp = rng.standard_normal(shape).astype(np.float32)
+    coef = 0.125
+    dgp, dp, hcoef = dev(gp), dev(probs), kai.hyper(coef)
+    VMath.softmax_direct_on_axis_backward(0, dgp, dp, nbat, ntimes, nhead, hcoef)
+    check(dgp.to_numpy(shape), ko.softmax_direct_on_axis_backward(gp, probs, coef), what="softmax axis backward")
+
+
+def test_split_k_scratch_survives_shutdown_and_growth():
+    # a product cut along K uses scratch memory of the library: small first, then a larger one (the buffer
+    # grows), then released and created again
+    rng = np.random.default_rng(99)
+    for (m, n, k), release in [((64, 64, 2048), False), ((1024, 2048, 1024), False), ((64, 128, 2048), True),
+                               ((64, 128, 2048), False)]:
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+        y = DB(m * n * 4)
+        if release:
+            kai.shutdown()
+        VMath.matmul(0, y, dev(w), dev(x), n, m, k, False)
+        rows = list(range(0, m, max(1, m // 64)))
+        check(y.to_numpy((m, n))[rows], ko.matmul_rows(w, x, rows), what="split-K %dx%dx%d" % (m, n, k))
 
 
 # ---- memory helpers and errors ----------------------------------------------------------------------------------------
