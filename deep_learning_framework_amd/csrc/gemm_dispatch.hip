@@ -31,7 +31,9 @@ struct GemmPlan {
     bool skinny = false;
     bool a_kc = false, b_kc = false;
     int tile = kTileSmall;
-    int64_t split = 1;
+    int64_t split = 1;      // >= 2: cut the reduction into this many parts of k_part steps
+    int64_t k_part = 0;
+    bool ragged_parts = false;   // the last part is shorter than k_part
     GemmDesc dn;   // the product with batch strides normalised
 };
 
@@ -65,11 +67,21 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         if (split > kSplitMax) split = kSplitMax;
         // equal parts of whole 16-step tiles if some part count allows it, else parts that at least keep
         // the operands' 16-byte alignment
+        // equal parts of whole 16-step tiles if some part count allows it; else parts of whole tiles with a
+        // shorter last one, which the general kernel variant handles
         int64_t whole = split;
         while (whole >= 2 && d.K % (whole * 16) != 0) whole--;
-        if (whole >= 2) split = whole;
-        else while (split >= 2 && d.K % (split * 4) != 0) split--;
-        if (split >= 2) plan.split = split;
+        if (whole >= 2) {
+            plan.split = whole;
+            plan.k_part = d.K / whole;
+            plan.ragged_parts = false;
+        } else if (split >= 2) {
+            const int64_t per = ((d.K + split - 1) / split + 15) / 16 * 16;
+            plan.split = (d.K + per - 1) / per;
+            plan.k_part = per;
+            plan.ragged_parts = true;
+            if (plan.split < 2) plan.split = 1;
+        }
     }
     return plan;
 }
@@ -113,9 +125,10 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
         float* part = nullptr;
         KAI_TRY(workspace(split * d.M * d.N * (int64_t)sizeof(float), &part));
         GemmDesc ds = plan.dn;
-        ds.K = d.K / split;
+        if (plan.ragged_parts) ds.k_part = plan.k_part;   // K stays the whole length
+        else ds.K = plan.k_part;
         ds.nbatch = split; ds.bdiv = 1;
-        ds.a_bs0 = ds.K * d.a_ks; ds.b_bs0 = ds.K * d.b_ks; ds.c_bs0 = d.M * d.N;
+        ds.a_bs0 = plan.k_part * d.a_ks; ds.b_bs0 = plan.k_part * d.b_ks; ds.c_bs0 = d.M * d.N;
         ds.a_bs1 = ds.b_bs1 = ds.c_bs1 = 0;
         ds.C = part; ds.c_rs = d.N; ds.c_cs = 1;
         ds.C2 = nullptr; ds.bias = nullptr; ds.alpha = nullptr; ds.leaky = nullptr;

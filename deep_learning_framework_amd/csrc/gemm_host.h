@@ -27,6 +27,9 @@ struct GemmDesc {
     // gemm_fuses_rowsum() holds may set it
     float* rowsum = nullptr;
     int rowsum_acc = 0;
+    // > 0: the nbatch batches are consecutive parts of k_part reduction steps of ONE product of length K
+    // (the last part may be shorter); the batch strides of A and B must then be k_part steps
+    int64_t k_part = 0;
 };
 
 // LDS orientation of an operand: reduction index contiguous (KC) or output index contiguous (MC).
@@ -53,13 +56,14 @@ inline GemmParams make_params(const GemmDesc& d, bool a_kc, bool b_kc) {
     p.has_alpha = d.has_alpha;
     p.rowsum = d.rowsum;
     p.rowsum_acc = d.rowsum_acc;
+    p.k_part = (int)d.k_part;
     return p;
 }
 
 // true when the predicate-free kernel variant may run this problem with tile BM x BN x BK
 inline bool fits_without_edges(const GemmParams& p, bool a_kc, bool b_kc, int BM, int BN, int BK) {
     const int64_t a_ld = a_kc ? p.a_rs : p.a_ks, b_ld = b_kc ? p.b_rs : p.b_ks;
-    return p.a_vec && p.b_vec && p.M % BM == 0 && p.N % BN == 0 && p.K % BK == 0 && p.K > 0 &&
+    return p.k_part == 0 && p.a_vec && p.b_vec && p.M % BM == 0 && p.N % BN == 0 && p.K % BK == 0 && p.K > 0 &&
            a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30);
 }
 

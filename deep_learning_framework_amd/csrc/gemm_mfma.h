@@ -77,6 +77,9 @@ struct GemmParams {
     // when A is the transposed output gradient of a dense layer); null switches it off
     float* rowsum;
     int rowsum_acc;
+    // EDGE kernels only: when > 0 the batch index also cuts the reduction: batch z covers the
+    // k_part steps from z*k_part on (fewer in the last batch), K being the whole length
+    int k_part;
 };
 
 constexpr int kLdsPad = 4;
@@ -433,11 +436,13 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     f32x4 rax[DEPTH][NCHA], rbx[DEPTH][NCHB];
     f32x4(&ra)[NCHA] = rax[0];
     f32x4(&rb)[NCHB] = rbx[0];
-    const int nkt = (p.K + BK - 1) / BK;
+    // reduction length of this workgroup
+    const int Kz = (EDGE && p.k_part > 0) ? min(p.k_part, p.K - z * p.k_part) : p.K;
+    const int nkt = (Kz + BK - 1) / BK;
 
     auto load_global_into = [&](int kt, f32x4(&da)[NCHA], f32x4(&db)[NCHB]) {
         const int k0 = kt * BK;
-        const int k_left = p.K - k0;
+        const int k_left = Kz - k0;
         const float* ap = Ab + (int64_t)k0 * p.a_ks;
         const float* bp = Bb + (int64_t)k0 * p.b_ks;
         if (!EDGE || (interior && k_left >= BK)) {

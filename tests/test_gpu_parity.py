@@ -218,7 +218,7 @@ def test_cfg5_ragged():
 SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 9), (64, 64, 64), (65, 63, 66), (100, 300, 50), (128, 128, 32),
           (129, 257, 40), (256, 256, 16), (300, 520, 128), (31, 1000, 4), (513, 64, 260), (40, 24, 1000),
           # split along K (few output tiles, long reduction), with and without whole tiles
-          (64, 64, 1024), (100, 300, 4096), (256, 512, 2048), (20, 130, 4000),
+          (64, 64, 1024), (100, 300, 4096), (256, 512, 2048), (20, 130, 4000), (20, 130, 4100), (3, 5, 1000),
           # 128-wide tiles: pipelined whole-tile kernel, then its edge variant
           (1024, 2048, 256), (1000, 2000, 130),
           # 256-wide tiles with edges in every dimension
