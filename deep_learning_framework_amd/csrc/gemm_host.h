@@ -88,6 +88,10 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream);
 // not looked at); otherwise the caller runs a separate column-sum kernel and leaves rowsum null
 bool gemm_fuses_rowsum(const GemmDesc& d);
 
+// short reductions (K <= 64) with both operands K-contiguous and a contiguous output row: gemm_shortk.hip
+bool shortk_nt_applies(const GemmDesc& d);
+int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream);
+
 // per-layout entry points (one translation unit each, to compile in parallel)
 enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2 };
 int launch_gemm_kc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);

@@ -1,0 +1,245 @@
+// Products with a short reduction (K <= 64) and both operands K-contiguous:
+// C[M,N] = A[M,K] . B[N,K]^T, the shape of attention scores (K = head size) and of the gradient
+// of attention probabilities.
+//
+// Such a product writes 4 bytes for every 2K <= 128 flops: it is bound by how fast C streams
+// out, not by the matrix cores, and a tiled kernel that loads, computes and then stores runs its
+// three phases one after the other.  Here a workgroup keeps a panel of 128 rows of B in LDS for its
+// whole life and streams row tiles of A (128 rows, all of K) past it through two LDS buffers:
+// while the matrix cores work on tile t the loads of tile t+1 are in flight, and the stores of
+// tile t drain under the work on tile t+1.  The host picks the run of tiles per workgroup so that
+// the grid still covers the compute units.
+//
+// B is held column-contiguous in LDS (transposed on the way in) so that one 128-bit read yields the
+// same row of four interleaved 32-column blocks; a lane then owns four consecutive columns of C
+// and stores them as one 128-bit word, 512 contiguous bytes per row and half wave.
+#include "gemm_host.h"
+
+namespace kai {
+
+namespace {
+
+constexpr int kSkWaves = 4;
+constexpr int kSkThreads = 64 * kSkWaves;
+constexpr int kSkBM = 32 * kSkWaves;   // rows of A per tile: one 32-row block per wave
+constexpr int kSkBN = 128;             // 4 interleaved blocks of 32 columns
+constexpr int kSkK = 64;               // longest reduction
+constexpr int kSkMaxRun = 8;           // most row tiles one workgroup walks
+
+using TileA = TileShape<true, kSkBM, kSkK>;    // [128][68]
+using TileB = TileShape<false, kSkBN, kSkK>;   // [64][132]
+
+// Loads a panel of `ROWS` rows x K (K-contiguous in memory, row stride ld) into registers: chunk c
+// of a thread covers row c / 16, k = 4 * (c % 16) .. +3.  Every address is clamped into the matrix,
+// so the loads carry no branches and all of them are in flight together; mask_panel() then zeroes
+// what lies beyond the matrix.
+template <int ROWS, bool VEC>
+__device__ __forceinline__ void load_panel(f32x4 (&reg)[ROWS * kSkK / 4 / kSkThreads], const float* __restrict__ base,
+                                           int64_t ld, int rows_left, int K, int tid) {
+    constexpr int NCH = ROWS * kSkK / 4 / kSkThreads;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * kSkThreads;
+        const int r = c >> 4;
+        const int k = (c & 15) * 4;
+        const float* row = base + (int64_t)min(r, rows_left - 1) * ld;
+        if (VEC) {   // K % 4 == 0: a chunk is inside or outside as a whole
+            reg[i] = *reinterpret_cast<const f32x4*>(row + (k < K ? k : 0));
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) reg[i][j] = row[min(k + j, K - 1)];
+        }
+    }
+}
+
+template <int ROWS>
+__device__ __forceinline__ void mask_panel(f32x4 (&reg)[ROWS * kSkK / 4 / kSkThreads], int rows_left, int K, int tid) {
+    constexpr int NCH = ROWS * kSkK / 4 / kSkThreads;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * kSkThreads;
+        const int r = c >> 4;
+        const int k = (c & 15) * 4;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            // bitwise, so that the compiler keeps the loads unconditional
+            const int keep = (r < rows_left && k + j < K) ? -1 : 0;
+            const float x = reg[i][j];
+            reg[i][j] = __int_as_float(__float_as_int(x) & keep);
+        }
+    }
+}
+
+// NG: groups of 8 reduction steps that are computed (K <= 8 * NG; the panels are zero beyond K).
+// FULL = false: the epilogue only scales and stores (no accumulation into C, bias, second output
+// or activation), so nothing in the loop waits on a load issued after a store.
+// Grid: one dimension over (batch, column panel, run), where a run is p.group_m consecutive row
+// tiles.  Hardware deals consecutive workgroup ids round-robin over the 8 XCDs; ids are renumbered
+// so that each XCD walks a contiguous range, which keeps the workgroups of one batch entry (they
+// share its A and B) behind one L2.
+template <int NG, bool FULL>
+__global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) float lds_a[2][TileA::kFloats];
+    __shared__ __attribute__((aligned(16))) float lds_b[TileB::kFloats];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    const int wm0 = wave * 32;
+
+    const int run_len = p.group_m;
+    const int runs = (p.tiles_m + run_len - 1) / run_len;
+    const int per_batch = runs * p.tiles_n;
+    const int total = gridDim.x;
+    int id = blockIdx.x;
+    if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    const int z = id / per_batch;
+    const int in_batch = id - z * per_batch;
+    const int tn = in_batch / runs;
+    const int tm_first = (in_batch - tn * runs) * run_len;
+    const int ntile = min(run_len, p.tiles_m - tm_first);
+    const int n0 = tn * kSkBN;
+    const int zq = z / p.bdiv, zr = z % p.bdiv;
+    const float* __restrict__ Az = p.A + zq * p.a_bs0 + zr * p.a_bs1;
+    const float* __restrict__ Bb = p.B + zq * p.b_bs0 + zr * p.b_bs1 + (int64_t)n0 * p.b_rs;
+    const int64_t c_off = zq * p.c_bs0 + zr * p.c_bs1;
+
+    // the two scalars of the epilogue are fetched before any store is in flight
+    float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
+    float leaky = p.leaky ? *p.leaky : 0.f;
+
+    constexpr int NCHA = kSkBM * kSkK / 4 / kSkThreads;
+    constexpr int NCHB = kSkBN * kSkK / 4 / kSkThreads;
+    const bool vec = p.a_vec && p.b_vec && (p.K & 3) == 0;
+    f32x4 ra[NCHA];
+
+    auto load_a = [&](int tm) {
+        const int m0 = tm * kSkBM;
+        const float* ab = Az + (int64_t)m0 * p.a_rs;
+        if (vec) load_panel<kSkBM, true>(ra, ab, p.a_rs, p.M - m0, p.K, tid);
+        else load_panel<kSkBM, false>(ra, ab, p.a_rs, p.M - m0, p.K, tid);
+    };
+    auto stage_a = [&](int tm, int buf) {
+        const int m0 = tm * kSkBM;
+        if (p.M - m0 < kSkBM || p.K < kSkK) mask_panel<kSkBM>(ra, p.M - m0, p.K, tid);
+        store_tile_lds<true, kSkBM, kSkK, kSkThreads>(lds_a[buf], ra, tid);
+    };
+
+    {
+        f32x4 rb[NCHB];
+        if (vec) load_panel<kSkBN, true>(rb, Bb, p.b_rs, p.N - n0, p.K, tid);
+        else load_panel<kSkBN, false>(rb, Bb, p.b_rs, p.N - n0, p.K, tid);
+        load_a(tm_first);
+        __builtin_amdgcn_sched_barrier(0);
+        if (p.N - n0 < kSkBN || p.K < kSkK) mask_panel<kSkBN>(rb, p.N - n0, p.K, tid);
+        // B goes in transposed: element (row n, k) to [k][n]
+#pragma unroll
+        for (int i = 0; i < NCHB; i++) {
+            const int c = tid + i * kSkThreads;
+            const int n = c >> 4;
+            const int k = (c & 15) * 4;
+#pragma unroll
+            for (int j = 0; j < 4; j++) lds_b[(k + j) * TileB::kStride + n] = rb[i][j];
+        }
+        stage_a(tm_first, 0);
+    }
+    alpha = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(alpha)));
+    leaky = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(leaky)));
+    __syncthreads();
+
+#pragma nounroll
+    for (int it = 0; it < ntile; it++) {
+        const int tm = tm_first + it;
+        const int m0 = tm * kSkBM;
+        const bool more = it + 1 < ntile;
+        if (more) load_a(tm + 1);   // in flight during the matrix work below
+        const float* la = lds_a[it & 1];
+
+        f32x16 acc[1][4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[0][j][r] = 0.f;
+        const bool rows_inside = m0 + wm0 < p.M;   // wave-uniform
+        if (rows_inside) {
+#pragma unroll
+            for (int kg = 0; kg < NG; kg++) {
+                Frag<true, 1> fa;
+                Frag<false, 4> fb;
+                read_frag<true, 1, kSkBM, kSkK>(fa, la, wm0, kg, l32, half);
+                read_frag<false, 4, kSkBN, kSkK>(fb, lds_b, 0, kg, l32, half);
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(0, t), fb.get(j, t), acc[0][j], 0, 0, 0);
+            }
+        }
+        // the next tile moves to LDS before this tile's stores are issued: the wait for its loads
+        // then never includes a store
+        if (more) stage_a(tm + 1, (it + 1) & 1);
+
+        if (rows_inside) {
+            if (FULL) {
+                gemm_epilogue<1, 4, true, false>(p, acc, m0, n0, c_off, wm0, 0, l32, half, alpha, leaky);
+            } else {
+                float* C = p.C + c_off;
+                const int col = n0 + 4 * l32;
+                static_for<0, 16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    const int row = m0 + wm0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    f32x4 o = {acc[0][0][r], acc[0][1][r], acc[0][2][r], acc[0][3][r]};
+                    o *= alpha;
+                    float* out = C + (int64_t)row * p.c_rs + col;
+                    if (row < p.M) {
+                        if (p.c_vec) {   // N % 4 == 0: the four columns are inside or outside together
+                            if (col < p.N) *reinterpret_cast<f32x4*>(out) = o;
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 4; j++)
+                                if (col + j < p.N) out[j] = o[j];
+                        }
+                    }
+                });
+            }
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace
+
+bool shortk_nt_applies(const GemmDesc& d) {
+    return d.a_ks == 1 && d.b_ks == 1 && d.c_cs == 1 && d.K >= 1 && d.K <= kSkK && d.rowsum == nullptr &&
+           d.k_part == 0 && d.M >= 64 && d.N >= 64;
+}
+
+int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream) {
+    p.tiles_m = (p.M + kSkBM - 1) / kSkBM;
+    p.tiles_n = (p.N + kSkBN - 1) / kSkBN;
+    if (p.tiles_m <= 0 || p.tiles_n <= 0 || nbatch <= 0) return KAI_OK;
+    // longest run of row tiles per workgroup that still leaves one workgroup per compute unit
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n * nbatch;
+    int64_t run = tiles / compute_units();
+    if (run > kSkMaxRun) run = kSkMaxRun;
+    if (run > p.tiles_m) run = p.tiles_m;
+    if (run < 1) run = 1;
+    p.group_m = (int)run;
+    const int64_t runs = (p.tiles_m + run - 1) / run;
+    const int64_t blocks = runs * p.tiles_n * nbatch;
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
+    const dim3 grid((unsigned)blocks, 1, 1);
+    const bool full = p.accflag || p.bias || p.C2 || p.act != kActNone;
+    if (p.K <= 32) {
+        if (full) shortk_nt_kernel<4, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+        else shortk_nt_kernel<4, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+    } else {
+        if (full) shortk_nt_kernel<8, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+        else shortk_nt_kernel<8, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+    }
+    return check_launch("shortk_nt_kernel");
+}
+
+}  // namespace kai

@@ -222,7 +222,9 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 9), (64, 64, 64), (65, 63, 66), (100, 3
           # 128-wide tiles: pipelined whole-tile kernel, then its edge variant
           (1024, 2048, 256), (1000, 2000, 130),
           # 256-wide tiles with edges in every dimension
-          (1500, 3000, 100)]
+          (1500, 3000, 100),
+          # short reductions (panel-resident kernel in the K-contiguous form): odd K, ragged rows and columns
+          (200, 130, 61), (513, 700, 64), (64, 1000, 8)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
