@@ -22,4 +22,8 @@ struct SkinnyParams {
 
 int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream);
 
+// skinny_stream.hip: aligned operands, K split over workgroups (uses the library's scratch memory)
+bool skinny_stream_applies(const SkinnyParams& p);
+int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream);
+
 }  // namespace kai

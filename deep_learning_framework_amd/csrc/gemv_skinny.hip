@@ -238,7 +238,7 @@ static int launch_slice(const SkinnyParams& p, hipStream_t stream) {
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int kMmWaves = 8;
-constexpr int kMmUnroll = 16;  // steps of 16 k (1 KiB of W and of X each) in flight per wave
+constexpr int kMmUnroll = 16;  // steps of 16 k (1 KiB of W and of X each) per chunk
 
 template <bool VEC>
 __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const SkinnyParams p) {
@@ -250,8 +250,8 @@ __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const Skinny
     const int64_t n0 = (int64_t)blockIdx.x * 16;
     const bool wvalid = n0 + r < p.N;
     const bool xvalid = r < p.M;
-    const float* __restrict__ wp = p.W + (wvalid ? (n0 + r) : 0) * p.ldw + 4 * g;
-    const float* __restrict__ xp = p.X + (int64_t)(xvalid ? r : 0) * p.ldx + 4 * g;
+    const float* __restrict__ wp = p.W + (wvalid ? (n0 + r) : 0) * p.ldw;
+    const float* __restrict__ xp = p.X + (int64_t)(xvalid ? r : 0) * p.ldx;
 
     // K split into 8 contiguous slices of whole 16-k steps
     const int steps = (p.K + 15) / 16;
@@ -260,40 +260,48 @@ __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const Skinny
     const int s_end = min(steps, s_begin + per);
 
     f32x4v acc = {0.f, 0.f, 0.f, 0.f};
-    auto load4 = [&](const float* base, int k, bool valid) -> f32x4v {
-        f32x4v v = {0.f, 0.f, 0.f, 0.f};
+    // Loads are raw: the address is clamped into the row, so that no branch sits between the loads
+    // of a chunk and all of them are in flight together.  What lies beyond the row, the slice or the
+    // matrix is zeroed when the value is consumed (bitwise, so that the load stays unconditional).
+    auto load4 = [&](const float* base, int k) -> f32x4v {
+        f32x4v v;
         if (VEC) {
             // K % 4 == 0: the float4 at k is entirely inside or outside
-            if (valid && k + 4 * g < p.K) v = *reinterpret_cast<const f32x4v*>(base + k);
+            v = *reinterpret_cast<const f32x4v*>(base + min(k, p.K - 4));
         } else {
-            if (valid) {
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (k + 4 * g + j < p.K) v[j] = base[k + j];
-            }
+            for (int j = 0; j < 4; j++) v[j] = base[min(k + j, p.K - 1)];
         }
         return v;
     };
-
-    // register ring of kMmUnroll steps: a slot is refilled with the step one ring-length ahead right
-    // after its MFMAs are issued, so kMmUnroll loads of W and of X stay in flight until the slice ends
-    f32x4v w[kMmUnroll], x[kMmUnroll];
+    auto masked = [&](f32x4v v, int k, bool valid) -> f32x4v {
+        f32x4v o;
 #pragma unroll
-    for (int u = 0; u < kMmUnroll; u++) {
-        const bool in = s_begin + u < s_end;
-        w[u] = load4(wp, (s_begin + u) * 16, wvalid && in);
-        x[u] = load4(xp, (s_begin + u) * 16, xvalid && in);
-    }
+        for (int j = 0; j < 4; j++) {
+            const int keep = (valid && k + j < p.K) ? -1 : 0;
+            const float e = v[j];
+            o[j] = __int_as_float(__float_as_int(e) & keep);
+        }
+        return o;
+    };
+
+    // chunks of kMmUnroll steps: all loads of W and of X of a chunk are issued back to back (32 KiB in
+    // flight per wave), then its MFMAs; the second wave of the SIMD computes meanwhile
     for (int base = s_begin; base < s_end; base += kMmUnroll) {
+        f32x4v w[kMmUnroll], x[kMmUnroll];
+#pragma unroll
+        for (int u = 0; u < kMmUnroll; u++) w[u] = load4(wp, (base + u) * 16 + 4 * g);
+#pragma unroll
+        for (int u = 0; u < kMmUnroll; u++) x[u] = load4(xp, (base + u) * 16 + 4 * g);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < kMmUnroll; u++) {
-            // steps past the end of the slice hold zeros and add nothing
+            const int k = (base + u) * 16 + 4 * g;
+            const bool in = base + u < s_end;   // steps past the end of the slice add nothing
+            const f32x4v wv = masked(w[u], k, wvalid && in);
+            const f32x4v xv = masked(x[u], k, xvalid && in);
 #pragma unroll
-            for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(x[u][t], w[u][t], acc, 0, 0, 0);
-            const int nxt = base + kMmUnroll + u;
-            const bool in = nxt < s_end;
-            w[u] = load4(wp, nxt * 16, wvalid && in);
-            x[u] = load4(xp, nxt * 16, xvalid && in);
+            for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[t], wv[t], acc, 0, 0, 0);
         }
     }
 
@@ -338,6 +346,7 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
         if (p.M == 2) return launch_slice<2>(p, stream);
         if (p.M <= 4) return launch_slice<4>(p, stream);
     }
+    if (skinny_stream_applies(p)) return launch_skinny_stream(p, stream);
     return launch_skinny_mfma(p, vec, stream);
 }
 
