@@ -157,27 +157,43 @@ __global__ void __launch_bounds__(64 * kSliceMaxWaves) skinny_slice_kernel(const
     for (int ks = wave * kSliceK; ks < p.K; ks += waves * kSliceK) {
         f32x4 w[RB][4];
         f32x4 x[MT][4];
+        // addresses are clamped into the row and the values masked afterwards (bitwise), so that no
+        // branch separates the loads
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int k = ks + 4 * lane + 256 * j;
-            const bool in = k < p.K;
+            const int k = min(ks + 4 * lane + 256 * j, p.K - 4);
 #pragma unroll
-            for (int r = 0; r < RB; r++) {
-                w[r][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-                if (in) w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + k));
-            }
+            for (int r = 0; r < RB; r++) w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + k));
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int k = ks + 4 * lane + 256 * j;
-            const bool in = k < p.K;
+            const int k = min(ks + 4 * lane + 256 * j, p.K - 4);
 #pragma unroll
-            for (int m = 0; m < MT; m++) {
-                x[m][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-                if (in && m < p.M) x[m][j] = *reinterpret_cast<const f32x4*>(p.X + (int64_t)m * p.ldx + k);
-            }
+            for (int m = 0; m < MT; m++)
+                x[m][j] = *reinterpret_cast<const f32x4*>(p.X + (int64_t)min(m, p.M - 1) * p.ldx + k);
         }
         __builtin_amdgcn_sched_barrier(0);   // all loads of the pass are in flight before the first multiply
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int keep_k = (ks + 4 * lane + 256 * j < p.K) ? -1 : 0;
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const int keep = (m < p.M) ? keep_k : 0;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float v = x[m][j][e];
+                    x[m][j][e] = __int_as_float(__float_as_int(v) & keep);
+                }
+            }
+            // W beyond K meets the zeros of X, but may hold anything: inf * 0 must not reach the sum
+#pragma unroll
+            for (int r = 0; r < RB; r++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float v = w[r][j][e];
+                    w[r][j][e] = __int_as_float(__float_as_int(v) & keep_k);
+                }
+        }
 #pragma unroll
         for (int m = 0; m < MT; m++)
 #pragma unroll
