@@ -123,14 +123,26 @@ __device__ __forceinline__ void load_tile_chunk(f32x4 (&reg)[ROWS * BK / 4 / NT]
     reg[i] = *reinterpret_cast<const f32x4*>(bi + toff);
 }
 
-// Predicated load: rows_left / k_left are the numbers of valid rows / k from the tile origin.
-// rs / ks are the element strides of the row index and the reduction index.
-template <bool KC, int ROWS, int BK, int NT>
+// General load of one operand tile: rows_left / k_left (both >= 1) are the numbers of valid rows / k
+// from the tile origin, rs / ks the element strides of the row index and the reduction index.
+// Every address is clamped into the matrix, so that no branch separates the loads of a tile (a load
+// under a condition makes the compiler wait for it before it issues the next one); what lies
+// outside the matrix is zeroed by mask_tile_edge() when the tile moves on to LDS, not here: a mask
+// right behind the load would bring the wait for it along.
+// true when 128-bit chunks may be used for every tile of a workgroup's operand: the operand allows
+// them at all and no chunk straddles the end of the index it runs along (k for KC, rows for MC)
+template <bool KC, int ROWS>
+__device__ __forceinline__ bool edge_operand_vec(int rows_left, int k_total, int vec_ok) {
+    return vec_ok && (KC ? (k_total & 3) == 0 : (rows_left >= ROWS || (rows_left & 3) == 0));
+}
+
+template <bool KC, int ROWS, int BK, int NT, bool VEC>
 __device__ __forceinline__ void load_tile_edge(f32x4 (&reg)[ROWS * BK / 4 / NT], const float* __restrict__ base,
-                                               int64_t rs, int64_t ks, int rows_left, int k_left, int vec_ok,
-                                               int tid) {
+                                               int64_t rs, int64_t ks, int rows_left, int k_left, int tid) {
     using TS = TileShape<KC, ROWS, BK>;
     constexpr int NCH = TS::kChunks / NT;
+    const int r_last = rows_left - 1, k_last = k_left - 1;
+    const int64_t klks = (int64_t)k_last * ks;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
         const int c = tid + i * NT;
@@ -138,31 +150,44 @@ __device__ __forceinline__ void load_tile_edge(f32x4 (&reg)[ROWS * BK / 4 / NT],
         const int off = (c % TS::kChunksPerLine) * 4;
         const int r = KC ? line : off;   // first row of the chunk
         const int k = KC ? off : line;   // first k of the chunk
-        f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        if (KC) {
-            if (r < rows_left) {
-                const float* p = base + (int64_t)r * rs + (int64_t)k * ks;
-                if (vec_ok && k + 3 < k_left) {
-                    v = *reinterpret_cast<const f32x4*>(p);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        if (k + j < k_left) v[j] = p[(int64_t)j * ks];
-                }
-            }
+        if (VEC) {
+            const int rc = KC ? min(r, r_last) : (r < rows_left ? r : 0);
+            const int kc = KC ? (k < k_left ? k : 0) : min(k, k_last);
+            reg[i] = *reinterpret_cast<const f32x4*>(base + (int64_t)rc * rs + (int64_t)kc * ks);
         } else {
-            if (k < k_left) {
-                const float* p = base + (int64_t)r * rs + (int64_t)k * ks;
-                if (vec_ok && r + 3 < rows_left) {
-                    v = *reinterpret_cast<const f32x4*>(p);
-                } else {
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        if (r + j < rows_left) v[j] = p[(int64_t)j * rs];
-                }
+            for (int j = 0; j < 4; j++) {
+                const int rj = KC ? r : r + j, kj = KC ? k + j : k;
+                // products of per-thread constants: they do not change from tile to tile, only the
+                // choice between them and the (uniform) offset of the last valid k does
+                const int64_t roff = (int64_t)min(rj, r_last) * rs;
+                const int64_t koff = kj <= k_last ? (int64_t)kj * ks : klks;
+                reg[i][j] = base[roff + koff];
             }
         }
-        reg[i] = v;
+    }
+}
+
+// Zeroes the elements of a tile loaded by load_tile_edge() that lie outside the matrix (bitwise, so
+// that the compiler cannot turn the mask back into a conditional load).
+template <bool KC, int ROWS, int BK, int NT>
+__device__ __forceinline__ void mask_tile_edge(f32x4 (&reg)[ROWS * BK / 4 / NT], int rows_left, int k_left, int tid) {
+    using TS = TileShape<KC, ROWS, BK>;
+    constexpr int NCH = TS::kChunks / NT;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * NT;
+        const int line = c / TS::kChunksPerLine;
+        const int off = (c % TS::kChunksPerLine) * 4;
+        const int r = KC ? line : off;
+        const int k = KC ? off : line;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int rj = KC ? r : r + j, kj = KC ? k + j : k;
+            const int keep = (rj < rows_left && kj < k_left) ? -1 : 0;
+            const float e = reg[i][j];
+            reg[i][j] = __int_as_float(__float_as_int(e) & keep);
+        }
     }
 }
 
@@ -413,9 +438,7 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     const int rows_b = p.N - n0;
     const int64_t a_ld = A_KC ? p.a_rs : p.a_ks;
     const int64_t b_ld = B_KC ? p.b_rs : p.b_ks;
-    // fast path: whole tile inside the matrix, aligned, and 32-bit thread offsets
-    const bool interior = !EDGE || ((rows_a >= BM) && (rows_b >= BN) && p.a_vec && p.b_vec &&
-                                    a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30));
+    // per-thread element offsets of the predicate-free loads (whole-tile kernels: they fit 32 bits)
     const uint32_t toff_a =
         (uint32_t)(tid / TA::kChunksPerLine) * (uint32_t)a_ld + (uint32_t)(tid % TA::kChunksPerLine) * 4u;
     const uint32_t toff_b =
@@ -440,33 +463,6 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     const int Kz = (EDGE && p.k_part > 0) ? min(p.k_part, p.K - z * p.k_part) : p.K;
     const int nkt = (Kz + BK - 1) / BK;
 
-    auto load_global_into = [&](int kt, f32x4(&da)[NCHA], f32x4(&db)[NCHB]) {
-        const int k0 = kt * BK;
-        const int k_left = Kz - k0;
-        const float* ap = Ab + (int64_t)k0 * p.a_ks;
-        const float* bp = Bb + (int64_t)k0 * p.b_ks;
-        if (!EDGE || (interior && k_left >= BK)) {
-            load_tile_fast<A_KC, BM, BK, NT>(da, ap, a_ld, toff_a);
-            load_tile_fast<B_KC, BN, BK, NT>(db, bp, b_ld, toff_b);
-        } else {
-            load_tile_edge<A_KC, BM, BK, NT>(da, ap, p.a_rs, p.a_ks, rows_a, k_left, p.a_vec, tid);
-            load_tile_edge<B_KC, BN, BK, NT>(db, bp, p.b_rs, p.b_ks, rows_b, k_left, p.b_vec, tid);
-        }
-    };
-    auto load_global = [&](int kt) { load_global_into(kt, ra, rb); };
-
-    // prologue: tiles 0 .. DEPTH-1 go to the staging slots, tile 0 on to LDS, and its slot is refilled
-    if (nkt > 0) {
-        static_for<0, DEPTH>([&](auto dc) {
-            constexpr int d = decltype(dc)::value;
-            if (d < nkt) load_global_into(d, rax[d], rbx[d]);
-        });
-        store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
-        store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
-        if (PIPE == 0 && DEPTH > 1 && DEPTH < nkt) load_global_into(DEPTH, ra, rb);
-    }
-    __syncthreads();
-
     constexpr int NKG = BK / 8;
     auto mfma_group = [&](const Frag<A_KC, NBM>& fa, const Frag<B_KC, NBN>& fb) {
 #pragma unroll
@@ -477,41 +473,103 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
                 for (int j = 0; j < NBN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(i, t), fb.get(j, t), acc[i][j], 0, 0, 0);
     };
+    // predicate-free load of tile kt (whole-tile kernels)
+    auto load_global = [&](int kt) {
+        load_tile_fast<A_KC, BM, BK, NT>(ra, Ab + (int64_t)kt * BK * p.a_ks, a_ld, toff_a);
+        load_tile_fast<B_KC, BN, BK, NT>(rb, Bb + (int64_t)kt * BK * p.b_ks, b_ld, toff_b);
+    };
 
     if (PIPE == 0) {
-        // At the top of tile kt: LDS[kt & 1] holds tile kt; slot (kt + j) % DEPTH holds tile kt + j for
-        // j = 1 .. DEPTH (slot kt % DEPTH was refilled with tile kt + DEPTH when tile kt left it).
-        // With DEPTH == 1 the single slot is refilled before the MFMAs of the tile instead.
-        for (int kt0 = 0; kt0 < nkt; kt0 += DEPTH) {
+        // The whole loop exists once per combination of 128-bit / element-wise loads of A and B.  The
+        // choice is made once per workgroup: a loop body that holds both kinds of load behind a branch
+        // makes the compiler wait for every load before the next tile's are issued, which turns the
+        // register staging into one memory round trip per tile.  For the same reason every load in the
+        // loop is unconditional: a tile index past the end is clamped (that tile is never stored).
+        auto pipe0 = [&](auto va_c, auto vb_c) {
+            constexpr bool VA = decltype(va_c)::value, VB = decltype(vb_c)::value;
+            auto load_into = [&](int kt, f32x4(&da)[NCHA], f32x4(&db)[NCHB]) {
+                const int ktc = min(kt, nkt - 1);
+                const int k0 = ktc * BK;
+                const float* ap = Ab + (int64_t)k0 * p.a_ks;
+                const float* bp = Bb + (int64_t)k0 * p.b_ks;
+                if (!EDGE) {
+                    load_tile_fast<A_KC, BM, BK, NT>(da, ap, a_ld, toff_a);
+                    load_tile_fast<B_KC, BN, BK, NT>(db, bp, b_ld, toff_b);
+                } else {
+                    load_tile_edge<A_KC, BM, BK, NT, VA>(da, ap, p.a_rs, p.a_ks, rows_a, Kz - k0, tid);
+                    load_tile_edge<B_KC, BN, BK, NT, VB>(db, bp, p.b_rs, p.b_ks, rows_b, Kz - k0, tid);
+                }
+            };
+            // a tile loaded by the general path still holds whatever the clamped addresses gave
+            auto mask_tile = [&](int kt, f32x4(&da)[NCHA], f32x4(&db)[NCHB]) {
+                const int k_left = Kz - kt * BK;
+                if (EDGE && (rows_a < BM || rows_b < BN || k_left < BK)) {
+                    mask_tile_edge<A_KC, BM, BK, NT>(da, rows_a, k_left, tid);
+                    mask_tile_edge<B_KC, BN, BK, NT>(db, rows_b, k_left, tid);
+                }
+            };
+
+            // prologue: tiles 0 .. DEPTH-1 go to the staging slots, tile 0 on to LDS, its slot is refilled
             static_for<0, DEPTH>([&](auto dc) {
                 constexpr int d = decltype(dc)::value;
-                constexpr int nslot = (d + 1) % DEPTH;
-                const int kt = kt0 + d;
-                if (kt < nkt) {
-                    const int cur = kt & 1;
-                    if (DEPTH == 1 && kt + 1 < nkt) load_global(kt + 1);
-                    const float* la = lds_a[cur];
-                    const float* lb = lds_b[cur];
-                    if (ROWSUM && do_rowsum) {   // rows and k beyond the matrix were stored as zeros
-#pragma unroll
-                        for (int kk = 0; kk < BK; kk++) rowsum += la[A_KC ? tid * TA::kStride + kk : kk * TA::kStride + tid];
-                    }
-#pragma unroll
-                    for (int kg = 0; kg < NKG; kg++) {
-                        Frag<A_KC, NBM> fa;
-                        Frag<B_KC, NBN> fb;
-                        read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
-                        read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
-                        mfma_group(fa, fb);
-                    }
-                    if (kt + 1 < nkt) {
-                        store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], rax[nslot], tid);
-                        store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rbx[nslot], tid);
-                        if (DEPTH > 1 && kt + 1 + DEPTH < nkt) load_global_into(kt + 1 + DEPTH, rax[nslot], rbx[nslot]);
-                    }
-                    __syncthreads();
-                }
+                load_into(d, rax[d], rbx[d]);
             });
+            mask_tile(0, ra, rb);
+            store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
+            store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
+            if (DEPTH > 1) load_into(DEPTH, ra, rb);
+            __syncthreads();
+
+            // At the top of tile kt: LDS[kt & 1] holds tile kt; slot (kt + j) % DEPTH holds tile kt + j for
+            // j = 1 .. DEPTH (slot kt % DEPTH was refilled with tile kt + DEPTH when tile kt left it).
+            // With DEPTH == 1 the single slot is refilled before the MFMAs of the tile instead.
+            for (int kt0 = 0; kt0 < nkt; kt0 += DEPTH) {
+                static_for<0, DEPTH>([&](auto dc) {
+                    constexpr int d = decltype(dc)::value;
+                    constexpr int nslot = (d + 1) % DEPTH;
+                    const int kt = kt0 + d;
+                    if (kt < nkt) {
+                        const int cur = kt & 1;
+                        if (DEPTH == 1) load_into(kt + 1, ra, rb);
+                        const float* la = lds_a[cur];
+                        const float* lb = lds_b[cur];
+                        if (ROWSUM && do_rowsum) {   // rows and k beyond the matrix were stored as zeros
+#pragma unroll
+                            for (int kk = 0; kk < BK; kk++)
+                                rowsum += la[A_KC ? tid * TA::kStride + kk : kk * TA::kStride + tid];
+                        }
+#pragma unroll
+                        for (int kg = 0; kg < NKG; kg++) {
+                            Frag<A_KC, NBM> fa;
+                            Frag<B_KC, NBN> fb;
+                            read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
+                            read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
+                            mfma_group(fa, fb);
+                        }
+                        if (kt + 1 < nkt) {
+                            mask_tile(kt + 1, rax[nslot], rbx[nslot]);
+                            store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], rax[nslot], tid);
+                            store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rbx[nslot], tid);
+                        }
+                        if (DEPTH > 1) load_into(kt + 1 + DEPTH, rax[nslot], rbx[nslot]);
+                        __syncthreads();
+                    }
+                });
+            }
+        };
+        using yes = std::integral_constant<bool, true>;
+        using no = std::integral_constant<bool, false>;
+        if (nkt > 0) {
+            if (!EDGE) {
+                pipe0(yes{}, yes{});
+            } else {
+                const bool va = edge_operand_vec<A_KC, BM>(rows_a, Kz, p.a_vec);
+                const bool vb = edge_operand_vec<B_KC, BN>(rows_b, Kz, p.b_vec);
+                if (va && vb) pipe0(yes{}, yes{});
+                else if (va) pipe0(yes{}, no{});
+                else if (vb) pipe0(no{}, yes{});
+                else pipe0(no{}, no{});
+            }
         }
     } else {
         static_assert(PIPE == 0 || NKG % 2 == 0, "the pipelined schedule needs an even number of groups per tile");
@@ -522,6 +580,12 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         constexpr int kMfma = 4 * NBM * NBN;                  // MFMAs per group
         Frag<A_KC, NBM> fa[2];
         Frag<B_KC, NBN> fb[2];
+        if (nkt > 0) {
+            load_global(0);
+            store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
+            store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
+        }
+        __syncthreads();
 
         // One group of the schedule: the MFMAs of the fragments in `use`, cut into slots; slot s is
         // preceded by the s-th LDS read of the fragments for the next group (into `fill`, from
