@@ -17,12 +17,18 @@
 //    so products always pair equal k, whatever the orientation mix.
 //  * v_mfma_f32_32x32x2_f32: every wave owns NBM x NBN blocks of 32x32 outputs held
 //    in accumulator registers (16 per lane per block).
-//  * Global -> register -> LDS staging, double buffered: the loads of tile t+1 are
-//    in flight while the MFMAs of tile t run; one barrier per K-tile.
-//  * Interior blocks with 16-byte aligned operands take a predicate-free 128-bit
-//    load path; edge blocks, ragged K and unaligned or strided operands take a
-//    predicated path (vector where a whole chunk is valid and aligned, scalar
-//    otherwise) that writes zeros into LDS outside the matrix.
+//  * Global -> register -> LDS staging, LDS double buffered, one barrier per K-tile.
+//    Two schedules (template parameter PIPE, described at the kernel): a simple one
+//    that keeps DEPTH tiles in flight in staging registers, for small tiles and
+//    general shapes, and a slot schedule that interleaves LDS reads, LDS stores and
+//    global loads with the MFMAs one by one, for large whole-tile products.
+//  * Shapes that are whole multiples of the tile with 16-byte aligned operands
+//    run a kernel variant with predicate-free 128-bit loads (EDGE = false).  The
+//    general variant loads through clamped addresses, 128-bit or element-wise as
+//    chosen once per workgroup, and zeroes what lies outside the matrix when the
+//    tile moves to LDS: no load in any loop sits behind a branch.
+//  * A single product can be cut along K over the batch dimension (k_part) and can
+//    sum the rows of A on the side (ROWSUM, the bias gradient of a dense layer).
 //  * Workgroup ids are remapped so that the workgroups that share one XCD (and its
 //    L2) cover a compact patch of C.
 //  * Epilogue in registers: alpha, C += (acc), bias add, optional store of the
