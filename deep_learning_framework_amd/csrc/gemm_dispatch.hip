@@ -121,6 +121,8 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
 
     const bool a_kc = plan.a_kc, b_kc = plan.b_kc;
     if (shortk_nt_applies(plan.dn)) return launch_gemm_shortk_nt(make_params(plan.dn, true, true), d.nbatch, stream);
+    if (shortk_heads_applies(plan.dn))
+        return launch_gemm_shortk_heads(make_params(plan.dn, true, true), d.nbatch, stream);
     if (plan.split >= 2) {
         const int64_t split = plan.split;
         float* part = nullptr;

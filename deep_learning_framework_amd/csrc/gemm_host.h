@@ -91,6 +91,9 @@ bool gemm_fuses_rowsum(const GemmDesc& d);
 // short reductions (K <= 64) with both operands K-contiguous and a contiguous output row: gemm_shortk.hip
 bool shortk_nt_applies(const GemmDesc& d);
 int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream);
+// the same with the inner batch index (heads) interleaved in C: element stride = number of heads
+bool shortk_heads_applies(const GemmDesc& d);
+int launch_gemm_shortk_heads(GemmParams p, int64_t nbatch, hipStream_t stream);
 
 // per-layout entry points (one translation unit each, to compile in parallel)
 enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2 };

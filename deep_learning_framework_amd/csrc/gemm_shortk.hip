@@ -209,6 +209,144 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
     }
 }
 
+
+// ---- the same product for several heads interleaved in C -------------------------------------------
+//
+// The engine keeps attention scores as P[batch, q, k, head] with the head index innermost
+// (vtensor.cpp:3005 of the reference), so the product of one head writes 4 bytes at a stride of
+// 4 * heads.  Here the four accumulators of a wave are four HEADS of the same 32 x 32 block of
+// (q, k): a lane then holds P[b, q, k, h .. h+3] and stores it as one 128-bit word.  A workgroup keeps
+// the rows of B (keys) of its 32-column panel for the four heads in LDS and streams the rows of A
+// (queries), one head slice of a 128-row tile at a time, through two LDS buffers; the stores of a
+// tile drain under the work on the next one.
+//
+// Batch index z = outer * bdiv + head (bdiv heads): A and B of head h start h * a_bs1 / h * b_bs1 past
+// the outer entry, C at + h (c_bs1 == 1) with element stride c_cs == bdiv.
+constexpr int kShHeads = 4;     // heads per workgroup
+constexpr int kShBN = 32;       // keys per workgroup
+
+using TileBh = TileShape<true, kShBN, kSkK>;   // [32][68]
+
+template <int NG>
+__global__ void __launch_bounds__(kSkThreads) shortk_heads_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) float lds_a[2][TileA::kFloats];
+    __shared__ __attribute__((aligned(16))) float lds_b[kShHeads][TileBh::kFloats];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    const int wm0 = wave * 32;
+
+    // grid: (outer batch, key panel, head group, run of query tiles), renumbered XCD-contiguous
+    const int run_len = p.group_m;
+    const int runs = (p.tiles_m + run_len - 1) / run_len;
+    const int hgroups = p.bdiv / kShHeads;
+    const int per_batch = runs * p.tiles_n * hgroups;
+    const int total = gridDim.x;
+    int id = blockIdx.x;
+    if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    const int zq = id / per_batch;
+    int rest = id - zq * per_batch;
+    const int tn = rest / (runs * hgroups);
+    rest -= tn * runs * hgroups;
+    const int hg = rest / runs;
+    const int tm_first = (rest - hg * runs) * run_len;
+    const int ntile = min(run_len, p.tiles_m - tm_first);
+    const int n0 = tn * kShBN;
+    const int h0 = hg * kShHeads;
+    const float* __restrict__ Az = p.A + zq * p.a_bs0 + h0 * p.a_bs1;
+    const float* __restrict__ Bz = p.B + zq * p.b_bs0 + h0 * p.b_bs1 + (int64_t)n0 * p.b_rs;
+    float* __restrict__ Cz = p.C + zq * p.c_bs0 + h0;
+
+    float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
+
+    constexpr int NCHA = kSkBM * kSkK / 4 / kSkThreads;   // 8
+    constexpr int NCHB = kShBN * kSkK / 4 / kSkThreads;   // 2
+    const bool vec = p.a_vec && p.b_vec && (p.K & 3) == 0;
+    f32x4 ra[NCHA];
+
+    // step s = tile * 4 + head: the A slice of head (s & 3) of query tile tm_first + (s >> 2)
+    auto load_a = [&](int s) {
+        const int m0 = (tm_first + (s >> 2)) * kSkBM;
+        const float* ab = Az + (s & 3) * p.a_bs1 + (int64_t)m0 * p.a_rs;
+        if (vec) load_panel<kSkBM, true>(ra, ab, p.a_rs, p.M - m0, p.K, tid);
+        else load_panel<kSkBM, false>(ra, ab, p.a_rs, p.M - m0, p.K, tid);
+    };
+    auto stage_a = [&](int s) {
+        const int m0 = (tm_first + (s >> 2)) * kSkBM;
+        if (p.M - m0 < kSkBM || p.K < kSkK) mask_panel<kSkBM>(ra, p.M - m0, p.K, tid);
+        store_tile_lds<true, kSkBM, kSkK, kSkThreads>(lds_a[s & 1], ra, tid);
+    };
+
+    {
+        f32x4 rb[kShHeads][NCHB];
+#pragma unroll
+        for (int j = 0; j < kShHeads; j++) {
+            if (vec) load_panel<kShBN, true>(rb[j], Bz + j * p.b_bs1, p.b_rs, p.N - n0, p.K, tid);
+            else load_panel<kShBN, false>(rb[j], Bz + j * p.b_bs1, p.b_rs, p.N - n0, p.K, tid);
+        }
+        load_a(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kShHeads; j++) {
+            if (p.N - n0 < kShBN || p.K < kSkK) mask_panel<kShBN>(rb[j], p.N - n0, p.K, tid);
+            store_tile_lds<true, kShBN, kSkK, kSkThreads>(lds_b[j], rb[j], tid);
+        }
+        stage_a(0);
+    }
+    alpha = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(alpha)));
+    __syncthreads();
+
+    const int nstep = ntile * kShHeads;
+#pragma nounroll
+    for (int it = 0; it < ntile; it++) {
+        const int m0 = (tm_first + it) * kSkBM;
+        const bool rows_inside = m0 + wm0 < p.M;   // wave-uniform
+        f32x16 acc[kShHeads];
+#pragma unroll
+        for (int j = 0; j < kShHeads; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+
+        static_for<0, kShHeads>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const int s = it * kShHeads + j;
+            const bool more = s + 1 < nstep;
+            if (more) load_a(s + 1);   // in flight during the matrix work below
+            const float* la = lds_a[s & 1];
+            if (rows_inside) {
+#pragma unroll
+                for (int kg = 0; kg < NG; kg++) {
+                    Frag<true, 1> fa, fb;
+                    read_frag<true, 1, kSkBM, kSkK>(fa, la, wm0, kg, l32, half);
+                    read_frag<true, 1, kShBN, kSkK>(fb, lds_b[j], 0, kg, l32, half);
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(0, t), fb.get(0, t), acc[j], 0, 0, 0);
+                }
+            }
+            // the next slice moves to LDS before this tile's stores are issued
+            if (more) stage_a(s + 1);
+            if (j + 1 < kShHeads) __syncthreads();
+        });
+
+        if (rows_inside) {
+            const int col = n0 + l32;
+            static_for<0, 16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                const int row = m0 + wm0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                f32x4 o = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
+                o *= alpha;
+                if (row < p.M && col < p.N)
+                    *reinterpret_cast<f32x4*>(Cz + (int64_t)row * p.c_rs + (int64_t)col * p.c_cs) = o;
+            });
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace
 
 bool shortk_nt_applies(const GemmDesc& d) {
@@ -240,6 +378,35 @@ int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream) {
         else shortk_nt_kernel<8, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     }
     return check_launch("shortk_nt_kernel");
+}
+
+bool shortk_heads_applies(const GemmDesc& d) {
+    return d.a_ks == 1 && d.b_ks == 1 && d.K >= 1 && d.K <= kSkK && d.bdiv >= kShHeads && d.bdiv % kShHeads == 0 &&
+           d.nbatch % d.bdiv == 0 && d.c_bs1 == 1 && d.c_cs == d.bdiv && d.c_rs % 4 == 0 && d.c_bs0 % 4 == 0 &&
+           aligned16(d.C) && !d.acc && !d.bias && !d.C2 && d.act == kActNone && d.rowsum == nullptr &&
+           d.k_part == 0 && d.M >= 64 && d.N >= kShBN;
+}
+
+int launch_gemm_shortk_heads(GemmParams p, int64_t nbatch, hipStream_t stream) {
+    p.tiles_m = (p.M + kSkBM - 1) / kSkBM;
+    p.tiles_n = (p.N + kShBN - 1) / kShBN;
+    const int64_t outer = nbatch / p.bdiv;
+    const int64_t hgroups = p.bdiv / kShHeads;
+    if (p.tiles_m <= 0 || p.tiles_n <= 0 || outer <= 0) return KAI_OK;
+    // longest run of query tiles per workgroup that still leaves one workgroup per compute unit
+    const int64_t units = (int64_t)p.tiles_m * p.tiles_n * hgroups * outer;
+    int64_t run = units / compute_units();
+    if (run > kSkMaxRun) run = kSkMaxRun;
+    if (run > p.tiles_m) run = p.tiles_m;
+    if (run < 1) run = 1;
+    p.group_m = (int)run;
+    const int64_t runs = (p.tiles_m + run - 1) / run;
+    const int64_t blocks = runs * p.tiles_n * hgroups * outer;
+    if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
+    const dim3 grid((unsigned)blocks, 1, 1);
+    if (p.K <= 32) shortk_heads_kernel<4><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+    else shortk_heads_kernel<8><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+    return check_launch("shortk_heads_kernel");
 }
 
 }  // namespace kai

@@ -407,8 +407,11 @@ def test_softmax_activation_rows():
 
 # ---- attention ops at small sizes, masks, backward --------------------------------------------------------------------
 
+# the last four run the kernel that writes four heads of a (q, k) pair as one word: ragged lengths, head sizes
+# that are not multiples of 8 or of 4, twelve heads
 @pytest.mark.parametrize("nbat,ntimes,nhead,npiece", [(2, 5, 1, 3), (3, 17, 4, 8), (1, 64, 2, 64), (2, 33, 3, 5),
-                                                      (1, 130, 1, 64), (1, 7, 200, 2)])
+                                                      (1, 130, 1, 64), (1, 7, 200, 2), (2, 100, 4, 16),
+                                                      (1, 130, 8, 64), (1, 70, 4, 6), (1, 96, 12, 24)])
 def test_attention_ops_small(nbat, ntimes, nhead, npiece):
     nvec = nhead * npiece
     rng = np.random.default_rng(nbat * 100 + ntimes * 10 + nhead)
