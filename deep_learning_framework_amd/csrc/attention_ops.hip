@@ -145,6 +145,21 @@ __global__ void __launch_bounds__(kTB) softmax_axis_block_kernel(float* __restri
 // (NV4 float4 per lane), so HBM sees exactly one 128-bit read and one 128-bit write per element.
 typedef float f32x4s __attribute__((ext_vector_type(4)));
 
+// v where keep, else `other` in every element.  Bitwise on purpose: with a select the compiler moves
+// the load that produced v under the condition, and a conditional load is waited for before the next
+// load is issued.
+__device__ __forceinline__ f32x4s keep_or(f32x4s v, bool keep, float other) {
+    const int m = keep ? -1 : 0;
+    const int o = __float_as_int(other) & ~m;
+    f32x4s r;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float e = v[j];
+        r[j] = __int_as_float((__float_as_int(e) & m) | o);
+    }
+    return r;
+}
+
 template <bool BACKWARD, int NV4>
 __global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __restrict__ io,
                                                                     const float* __restrict__ pp, int64_t nrow,
@@ -158,10 +173,20 @@ __global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __res
         f32x4s v[NV4];
 #pragma unroll
         for (int i = 0; i < NV4; i++) {
-            const int k = 4 * lane + 256 * i;
-            v[i] = f32x4s{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-            if (k < nvec) v[i] = *reinterpret_cast<const f32x4s*>(r + k);
+            const int k = 4 * lane + 256 * i;   // loads are unconditional (clamped), padding is masked below
+            v[i] = *reinterpret_cast<const f32x4s*>(r + min(k, nvec - 4));
         }
+        f32x4s q[NV4];   // backward only
+        if (BACKWARD) {
+            const float* __restrict__ pr = pp + row * nvec;
+#pragma unroll
+            for (int i = 0; i < NV4; i++) {
+                const int k = 4 * lane + 256 * i;
+                q[i] = *reinterpret_cast<const f32x4s*>(pr + min(k, nvec - 4));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NV4; i++) v[i] = keep_or(v[i], 4 * lane + 256 * i < nvec, BACKWARD ? 0.f : -INFINITY);
         if (!BACKWARD) {
             float mx = -FLT_MAX;
 #pragma unroll
@@ -182,17 +207,11 @@ __global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __res
                 if (k < nvec) *reinterpret_cast<f32x4s*>(r + k) = v[i] / sum;
             }
         } else {
-            const float* __restrict__ pr = pp + row * nvec;
-            f32x4s q[NV4];
             float dot = 0.f;
 #pragma unroll
             for (int i = 0; i < NV4; i++) {
-                const int k = 4 * lane + 256 * i;
-                q[i] = f32x4s{0.f, 0.f, 0.f, 0.f};
-                if (k < nvec) {
-                    q[i] = *reinterpret_cast<const f32x4s*>(pr + k);
-                    dot += q[i][0] * v[i][0] + q[i][1] * v[i][1] + q[i][2] * v[i][2] + q[i][3] * v[i][3];
-                }
+                q[i] = keep_or(q[i], 4 * lane + 256 * i < nvec, 0.f);
+                dot += q[i][0] * v[i][0] + q[i][1] * v[i][1] + q[i][2] * v[i][2] + q[i][3] * v[i][3];
             }
             dot = wsum(dot);
 #pragma unroll
@@ -268,6 +287,90 @@ __global__ void __launch_bounds__(kTB) softmax_axis_block_reg_kernel(float* __re
     }
 }
 
+// 4, 8, 16, ... 128 heads (a multiple of 4 whose quarter is a power of two), outer row (nvec*ncol
+// floats) at most 4*kTB*VN long: a thread keeps VN 128-bit chunks, each the same four heads of one
+// position, so that HBM sees one 128-bit read and one 128-bit write per four elements.  The four heads
+// are four independent reductions per thread; threads of one head group (t % G, G = ncol / 4) meet by
+// a butterfly over the lanes of a wave and one exchange through LDS.
+template <bool BACKWARD, int VN>
+__global__ void __launch_bounds__(kTB) softmax_axis_heads4_kernel(float* __restrict__ io,
+                                                                  const float* __restrict__ pp, int64_t nvec,
+                                                                  int ncol, const float* __restrict__ hcoef) {
+    __shared__ f32x4s red[2][kTB / 64][32];
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = t >> 6;
+    const int G = ncol >> 2;        // head groups: a power of two, at most 32
+    const int g = t & (G - 1);
+    const int len4 = (int)(nvec * ncol) >> 2;   // chunks in the row
+    float* __restrict__ r = io + (int64_t)blockIdx.x * (nvec * ncol);
+
+    // reduction over the threads of a head group, per component; `which` alternates the LDS buffer
+    auto fold = [&](f32x4s mine, bool is_max, int which) -> f32x4s {
+        for (int m = G; m < 64; m <<= 1) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float o = __shfl_xor(mine[j], m);
+                mine[j] = is_max ? fmaxf(mine[j], o) : mine[j] + o;
+            }
+        }
+        if (lane < G) red[which][wave][lane] = mine;
+        __syncthreads();
+        f32x4s a = red[which][0][g];
+#pragma unroll
+        for (int w = 1; w < kTB / 64; w++) {
+            const f32x4s b = red[which][w][g];
+#pragma unroll
+            for (int j = 0; j < 4; j++) a[j] = is_max ? fmaxf(a[j], b[j]) : a[j] + b[j];
+        }
+        return a;
+    };
+
+    f32x4s v[VN], q[VN];
+#pragma unroll
+    for (int i = 0; i < VN; i++) v[i] = *reinterpret_cast<const f32x4s*>(r + 4 * min(t + i * kTB, len4 - 1));
+    if (BACKWARD) {
+        const float* __restrict__ p = pp + (int64_t)blockIdx.x * (nvec * ncol);
+#pragma unroll
+        for (int i = 0; i < VN; i++) q[i] = *reinterpret_cast<const f32x4s*>(p + 4 * min(t + i * kTB, len4 - 1));
+    }
+#pragma unroll
+    for (int i = 0; i < VN; i++) v[i] = keep_or(v[i], t + i * kTB < len4, BACKWARD ? 0.f : -INFINITY);
+
+    if (!BACKWARD) {
+        f32x4s mx = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+#pragma unroll
+        for (int i = 0; i < VN; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) mx[j] = fmaxf(mx[j], v[i][j]);
+        mx = fold(mx, true, 0);
+        f32x4s sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < VN; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                v[i][j] = expf(v[i][j] - mx[j]);   // padding holds -inf: exp gives 0
+                sum[j] += v[i][j];
+            }
+        sum = fold(sum, false, 1);
+#pragma unroll
+        for (int i = 0; i < VN; i++)
+            if (t + i * kTB < len4) *reinterpret_cast<f32x4s*>(r + 4 * (t + i * kTB)) = v[i] / sum;
+    } else {
+        const float coef = hcoef ? *hcoef : 0.f;
+        f32x4s dot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < VN; i++) {
+            q[i] = keep_or(q[i], t + i * kTB < len4, 0.f);
+            dot += q[i] * v[i];
+        }
+        dot = fold(dot, false, 0);
+#pragma unroll
+        for (int i = 0; i < VN; i++)
+            if (t + i * kTB < len4) *reinterpret_cast<f32x4s*>(r + 4 * (t + i * kTB)) = coef * q[i] * (v[i] - dot);
+    }
+}
+
 template <bool BACKWARD>
 __global__ void __launch_bounds__(kTB) softmax_axis_thread_kernel(float* __restrict__ io,
                                                                   const float* __restrict__ pp, int64_t nrow,
@@ -314,7 +417,15 @@ static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, in
         if (nrow > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "softmax_direct_on_axis: too many rows");
         const int tb = (int)ncol * (kTB / (int)ncol);
         const int64_t len = nvec * ncol;
-        if (len <= (int64_t)tb * 16)
+        const int64_t quarter = ncol / 4;
+        const bool heads4 = ncol % 4 == 0 && (quarter & (quarter - 1)) == 0 && aligned16(io) &&
+                            (pp == nullptr || aligned16(pp)) && len <= 4 * kTB * 8;
+        if (heads4) {
+            const dim3 g((unsigned)nrow);
+            if (len <= 4 * kTB * 2) softmax_axis_heads4_kernel<BACKWARD, 2><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
+            else if (len <= 4 * kTB * 4) softmax_axis_heads4_kernel<BACKWARD, 4><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
+            else softmax_axis_heads4_kernel<BACKWARD, 8><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
+        } else if (len <= (int64_t)tb * 16)
             softmax_axis_block_reg_kernel<BACKWARD, 16><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol,
                                                                                                  tb, hcoef);
         else if (len <= (int64_t)tb * 32)
