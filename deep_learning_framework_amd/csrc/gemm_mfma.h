@@ -405,10 +405,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 // ROWSUM (PIPE 0 only): the workgroups of the first tile column also sum every row of their A tile
 // over K, one thread per row reading the tile from LDS, k ascending across tiles: a fixed order
 // that is the order of a sequential loop.
+//
+// WK (PIPE 0 only): waves along K.  With WK = 2 a second set of WM x WN waves shares the tiles in LDS
+// and takes every other group of 8 k, so that a SIMD holds two waves of the workgroup and one computes
+// while the other waits for LDS or the barrier; the two partial results meet in LDS at the end.  For
+// products whose grid gives a compute unit a single small workgroup.
 template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
-          int DEPTH = 1, bool ROWSUM = false>
-__global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const GemmParams p) {
-    constexpr int NT = 64 * WM * WN;
+          int DEPTH = 1, bool ROWSUM = false, int WK = 1>
+__global__ void __launch_bounds__(64 * WM * WN * WK, MINW) gemm_mfma_kernel(const GemmParams p) {
+    constexpr int NT = 64 * WM * WN * WK;
+    static_assert(WK == 1 || (WK == 2 && PIPE == 0 && (BK / 8) % 2 == 0), "two waves along K: PIPE 0, even group count");
     constexpr int BM = WM * NBM * 32;
     constexpr int BN = WN * NBN * 32;
     using TA = TileShape<A_KC, BM, BK>;
@@ -423,11 +429,13 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = WK == 1 ? (tid >> 6) : __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31;
     const int half = lane >> 5;
-    const int wm0 = (wave / WN) * (NBM * 32);
-    const int wn0 = (wave % WN) * (NBN * 32);
+    const int wk = wave / (WM * WN);           // which share of the k groups
+    const int wmn = wave % (WM * WN);
+    const int wm0 = (wmn / WN) * (NBM * 32);
+    const int wn0 = (wmn % WN) * (NBN * 32);
 
     int tm, tn;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
@@ -529,39 +537,52 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
             // At the top of tile kt: LDS[kt & 1] holds tile kt; slot (kt + j) % DEPTH holds tile kt + j for
             // j = 1 .. DEPTH (slot kt % DEPTH was refilled with tile kt + DEPTH when tile kt left it).
             // With DEPTH == 1 the single slot is refilled before the MFMAs of the tile instead.
-            for (int kt0 = 0; kt0 < nkt; kt0 += DEPTH) {
-                static_for<0, DEPTH>([&](auto dc) {
-                    constexpr int d = decltype(dc)::value;
-                    constexpr int nslot = (d + 1) % DEPTH;
-                    const int kt = kt0 + d;
-                    if (kt < nkt) {
-                        const int cur = kt & 1;
-                        if (DEPTH == 1) load_into(kt + 1, ra, rb);
-                        const float* la = lds_a[cur];
-                        const float* lb = lds_b[cur];
-                        if (ROWSUM && do_rowsum) {   // rows and k beyond the matrix were stored as zeros
-#pragma unroll
-                            for (int kk = 0; kk < BK; kk++)
-                                rowsum += la[A_KC ? tid * TA::kStride + kk : kk * TA::kStride + tid];
-                        }
-#pragma unroll
-                        for (int kg = 0; kg < NKG; kg++) {
-                            Frag<A_KC, NBM> fa;
-                            Frag<B_KC, NBN> fb;
-                            read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
-                            read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
-                            mfma_group(fa, fb);
-                        }
-                        if (kt + 1 < nkt) {
-                            mask_tile(kt + 1, rax[nslot], rbx[nslot]);
-                            store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], rax[nslot], tid);
-                            store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rbx[nslot], tid);
-                        }
-                        if (DEPTH > 1) load_into(kt + 1 + DEPTH, rax[nslot], rbx[nslot]);
-                        __syncthreads();
+            auto stage = [&](auto dc, int kt, bool last_tiles) {
+                constexpr int d = decltype(dc)::value;
+                constexpr int nslot = (d + 1) % DEPTH;
+                const int cur = kt & 1;
+                if (DEPTH == 1) load_into(kt + 1, ra, rb);
+                // With DEPTH > 1 the next tile has been in registers for a while: it goes to the free LDS
+                // buffer first, so that the store's latency runs under this tile's MFMAs instead of between
+                // them and the barrier.  (Every wave left that buffer before the last barrier.)  In the main
+                // loop the store is unconditional: past the last tile it moves a surplus copy of the last
+                // tile into the buffer nobody reads any more.
+                auto store_next = [&]() {
+                    if (!last_tiles || kt + 1 < nkt) {
+                        mask_tile(kt + 1, rax[nslot], rbx[nslot]);
+                        store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], rax[nslot], tid);
+                        store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rbx[nslot], tid);
                     }
-                });
-            }
+                    if (DEPTH > 1) load_into(kt + 1 + DEPTH, rax[nslot], rbx[nslot]);
+                };
+                if (DEPTH > 1) store_next();
+                const float* la = lds_a[cur];
+                const float* lb = lds_b[cur];
+                if (ROWSUM && do_rowsum) {   // rows and k beyond the matrix were stored as zeros
+#pragma unroll
+                    for (int kk = 0; kk < BK; kk++) rowsum += la[A_KC ? tid * TA::kStride + kk : kk * TA::kStride + tid];
+                }
+#pragma unroll
+                for (int kq = 0; kq < NKG / WK; kq++) {
+                    const int kg = WK * kq + wk;
+                    Frag<A_KC, NBM> fa;
+                    Frag<B_KC, NBN> fb;
+                    read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
+                    read_frag<B_KC, NBN, BN, BK>(fb, lb, wn0, kg, l32, half);
+                    mfma_group(fa, fb);
+                }
+                if (DEPTH == 1) store_next();
+                __syncthreads();
+            };
+            // Main loop: whole rounds of DEPTH tiles with no branch in the body, so that the compiler can
+            // count the loads in flight exactly across the back edge; with a conditional stage inside it
+            // waited for every load once per round.  The last, partial round follows.
+            int kt0 = 0;
+            for (; kt0 + DEPTH <= nkt; kt0 += DEPTH)
+                static_for<0, DEPTH>([&](auto dc) { stage(dc, kt0 + decltype(dc)::value, false); });
+            static_for<0, DEPTH>([&](auto dc) {
+                if (kt0 + decltype(dc)::value < nkt) stage(dc, kt0 + decltype(dc)::value, true);
+            });
         };
         using yes = std::integral_constant<bool, true>;
         using no = std::integral_constant<bool, false>;
@@ -681,6 +702,29 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     if (ROWSUM && do_rowsum && m0 + tid < p.M) {
         float* g = p.rowsum + m0 + tid;
         *g = p.rowsum_acc ? *g + rowsum : rowsum;
+    }
+    if (WK == 2) {
+        // the waves of the second share hand their accumulators over through the tile buffers (every
+        // wave is past its last fragment read: the loop ends with a barrier)
+        constexpr int kPerWave = NBM * NBN * 16 * 64;
+        static_assert(WK == 1 || WM * WN * kPerWave <= 2 * TA::kFloats, "partial results must fit the A tile buffers");
+        float* red = &lds_a[0][0] + wmn * kPerWave + lane;
+        if (wk == 1) {
+#pragma unroll
+            for (int i = 0; i < NBM; i++)
+#pragma unroll
+                for (int j = 0; j < NBN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) red[((i * NBN + j) * 16 + r) * 64] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (wk == 1) return;
+#pragma unroll
+        for (int i = 0; i < NBM; i++)
+#pragma unroll
+            for (int j = 0; j < NBN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += red[((i * NBN + j) * 16 + r) * 64];
     }
     const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
     const float leaky = p.leaky ? *p.leaky : 0.f;

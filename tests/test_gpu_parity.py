@@ -223,8 +223,9 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 9), (64, 64, 64), (65, 63, 66), (100, 3
           (1024, 2048, 256), (1000, 2000, 130),
           # 256-wide tiles with edges in every dimension
           (1500, 3000, 100),
-          # short reductions (panel-resident kernel in the K-contiguous form): odd K, ragged rows and columns
-          (200, 130, 61), (513, 700, 64), (64, 1000, 8)]
+          # short reductions: the tiled kernel below 4M outputs, the panel-resident kernel (K-contiguous form)
+          # above: odd K, ragged rows and columns
+          (200, 130, 61), (513, 700, 64), (64, 1000, 8), (2050, 2100, 61), (2048, 2048, 64), (4100, 1030, 24)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -407,11 +408,12 @@ def test_softmax_activation_rows():
 
 # ---- attention ops at small sizes, masks, backward --------------------------------------------------------------------
 
-# the last four run the kernel that writes four heads of a (q, k) pair as one word: ragged lengths, head sizes
-# that are not multiples of 8 or of 4, twelve heads
+# the last three are large enough (4M scores) for the panel-resident kernels: four heads of a (q, k) pair written
+# as one word, ragged lengths, head sizes that are not multiples of 8 or of 4; one head per batch entry
 @pytest.mark.parametrize("nbat,ntimes,nhead,npiece", [(2, 5, 1, 3), (3, 17, 4, 8), (1, 64, 2, 64), (2, 33, 3, 5),
                                                       (1, 130, 1, 64), (1, 7, 200, 2), (2, 100, 4, 16),
-                                                      (1, 130, 8, 64), (1, 70, 4, 6), (1, 96, 12, 24)])
+                                                      (1, 130, 8, 64), (1, 70, 4, 6), (1, 96, 12, 24),
+                                                      (2, 700, 8, 24), (1, 1100, 4, 6), (3, 1200, 1, 40)])
 def test_attention_ops_small(nbat, ntimes, nhead, npiece):
     nvec = nhead * npiece
     rng = np.random.default_rng(nbat * 100 + ntimes * 10 + nhead)
