@@ -68,7 +68,7 @@ inline bool fits_without_edges(const GemmParams& p, bool a_kc, bool b_kc, int BM
 }
 
 template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
-          int DEPTH = 1, bool ROWSUM = false, int WK = 1>
+          int DEPTH = 1, bool ROWSUM = false>
 int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t stream) {
     constexpr int BM = WM * NBM * 32, BN = WN * NBN * 32;
     p.tiles_m = (p.M + BM - 1) / BM;
@@ -78,8 +78,8 @@ int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t st
     if (tiles <= 0 || nbatch <= 0) return KAI_OK;
     if (tiles > kMaxDim || nbatch > 65535) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
     dim3 grid((unsigned)tiles, 1, (unsigned)nbatch);
-    gemm_mfma_kernel<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE, PIPE, MINW, DEPTH, ROWSUM, WK>
-        <<<grid, dim3(64 * WM * WN * WK), 0, stream>>>(p);
+    gemm_mfma_kernel<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE, PIPE, MINW, DEPTH, ROWSUM>
+        <<<grid, dim3(64 * WM * WN), 0, stream>>>(p);
     return check_launch("gemm_mfma_kernel");
 }
 

@@ -405,16 +405,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 // ROWSUM (PIPE 0 only): the workgroups of the first tile column also sum every row of their A tile
 // over K, one thread per row reading the tile from LDS, k ascending across tiles: a fixed order
 // that is the order of a sequential loop.
-//
-// WK (PIPE 0 only): waves along K.  With WK = 2 a second set of WM x WN waves shares the tiles in LDS
-// and takes every other group of 8 k, so that a SIMD holds two waves of the workgroup and one computes
-// while the other waits for LDS or the barrier; the two partial results meet in LDS at the end.  For
-// products whose grid gives a compute unit a single small workgroup.
 template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
-          int DEPTH = 1, bool ROWSUM = false, int WK = 1>
-__global__ void __launch_bounds__(64 * WM * WN * WK, MINW) gemm_mfma_kernel(const GemmParams p) {
-    constexpr int NT = 64 * WM * WN * WK;
-    static_assert(WK == 1 || (WK == 2 && PIPE == 0 && (BK / 8) % 2 == 0), "two waves along K: PIPE 0, even group count");
+          int DEPTH = 1, bool ROWSUM = false>
+__global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const GemmParams p) {
+    constexpr int NT = 64 * WM * WN;
     constexpr int BM = WM * NBM * 32;
     constexpr int BN = WN * NBN * 32;
     using TA = TileShape<A_KC, BM, BK>;
@@ -429,13 +423,11 @@ __global__ void __launch_bounds__(64 * WM * WN * WK, MINW) gemm_mfma_kernel(cons
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = WK == 1 ? (tid >> 6) : __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = tid >> 6;
     const int l32 = lane & 31;
     const int half = lane >> 5;
-    const int wk = wave / (WM * WN);           // which share of the k groups
-    const int wmn = wave % (WM * WN);
-    const int wm0 = (wmn / WN) * (NBM * 32);
-    const int wn0 = (wmn % WN) * (NBN * 32);
+    const int wm0 = (wave / WN) * (NBM * 32);
+    const int wn0 = (wave % WN) * (NBN * 32);
 
     int tm, tn;
     tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
@@ -563,8 +555,7 @@ __global__ void __launch_bounds__(64 * WM * WN * WK, MINW) gemm_mfma_kernel(cons
                     for (int kk = 0; kk < BK; kk++) rowsum += la[A_KC ? tid * TA::kStride + kk : kk * TA::kStride + tid];
                 }
 #pragma unroll
-                for (int kq = 0; kq < NKG / WK; kq++) {
-                    const int kg = WK * kq + wk;
+                for (int kg = 0; kg < NKG; kg++) {
                     Frag<A_KC, NBM> fa;
                     Frag<B_KC, NBN> fb;
                     read_frag<A_KC, NBM, BM, BK>(fa, la, wm0, kg, l32, half);
@@ -702,29 +693,6 @@ __global__ void __launch_bounds__(64 * WM * WN * WK, MINW) gemm_mfma_kernel(cons
     if (ROWSUM && do_rowsum && m0 + tid < p.M) {
         float* g = p.rowsum + m0 + tid;
         *g = p.rowsum_acc ? *g + rowsum : rowsum;
-    }
-    if (WK == 2) {
-        // the waves of the second share hand their accumulators over through the tile buffers (every
-        // wave is past its last fragment read: the loop ends with a barrier)
-        constexpr int kPerWave = NBM * NBN * 16 * 64;
-        static_assert(WK == 1 || WM * WN * kPerWave <= 2 * TA::kFloats, "partial results must fit the A tile buffers");
-        float* red = &lds_a[0][0] + wmn * kPerWave + lane;
-        if (wk == 1) {
-#pragma unroll
-            for (int i = 0; i < NBM; i++)
-#pragma unroll
-                for (int j = 0; j < NBN; j++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) red[((i * NBN + j) * 16 + r) * 64] = acc[i][j][r];
-        }
-        __syncthreads();
-        if (wk == 1) return;
-#pragma unroll
-        for (int i = 0; i < NBM; i++)
-#pragma unroll
-            for (int j = 0; j < NBN; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] += red[((i * NBN + j) * 16 + r) * 64];
     }
     const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
     const float leaky = p.leaky ? *p.leaky : 0.f;
