@@ -168,6 +168,10 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
         row(tag + "O = P.V (mix_values)",
             gpu_us(lambda: L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))),
             flops=fl, cpu=cpu_us(lambda: ko.mix_values(pbuf.cpu().numpy(), vc, nhead)))
+        row(tag + "all three fused, forward only (kai_attention_forward)",
+            gpu_us(lambda: L.kai_attention_forward(0, P(o), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
+                                                   P(coef), 0)),
+            flops=2 * fl)
     # cfg5: skinny (cold: six rotating weight buffers) and ragged
     K = N = 4096
     ws = [torch.rand((N, K), device=dev, generator=g) * 0.1 - 0.05 for _ in range(6)]

@@ -38,4 +38,12 @@ int launch_softmax_axis(float* pp, int64_t nrow, int64_t nvec, int64_t ncol, hip
 int launch_softmax_axis_backward(float* pgp, const float* pp, int64_t nrow, int64_t nvec, int64_t ncol,
                                  const float* hcoef, hipStream_t stream);
 
+
+// attention_fused.hip
+bool attention_fused_applies(const float* q, const float* k, const float* v, const float* o, int64_t ntimes,
+                             int64_t nvec, int64_t nhead, int64_t npiece);
+int launch_attention_fused(float* o, const float* q, const float* k, const float* v, int64_t nbat, int64_t ntimes,
+                           int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
+                           hipStream_t stream);
+
 }  // namespace kai

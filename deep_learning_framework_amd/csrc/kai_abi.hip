@@ -549,4 +549,23 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
     return KAI_OK;
 }
 
+int kai_attention_forward(int device, float* py, const float* pQ, const float* pK, const float* pV, int64_t nbat,
+                          int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
+                          int masked) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pQ); KAI_REQUIRE_PTR(pK); KAI_REQUIRE_PTR(pV);
+    if (attention_fused_applies(pQ, pK, pV, py, ntimes, nvec, nhead, npiece))
+        return launch_attention_fused(py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked != 0,
+                                      current_stream());
+    // any other shape: the separate kernels, probabilities in the library's scratch memory
+    float* pp = nullptr;
+    KAI_TRY(workspace(nbat * ntimes * ntimes * nhead * (int64_t)sizeof(float), &pp));
+    KAI_TRY(kai_mult_on_heads(device, pp, pK, pQ, nbat, ntimes, nvec, nhead, npiece, hCoef));
+    if (masked) KAI_TRY(kai_set_mh_attention_mask(device, pp, nbat, ntimes, nhead, 1));
+    KAI_TRY(kai_softmax_direct_on_axis(device, pp, nbat * ntimes, ntimes, nhead));
+    return kai_mix_values(device, py, pp, pV, nbat, ntimes, nvec, nhead, npiece);
+}
+
 }  // extern "C"

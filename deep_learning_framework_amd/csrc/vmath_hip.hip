@@ -82,6 +82,10 @@ void VMath::mix_values_backward_value(int device, float* pgV, float* pgy, float*
     raise_on(kai_mix_values_backward_value(device, pgV, pgy, pp, nbat, ntimes, nvec, nhead, npiece));
 }
 
+void VMath::attention_forward(int device, float* py, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked) {
+    raise_on(kai_attention_forward(device, py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked ? 1 : 0));
+}
+
 void VMath::dense_forward(int device, float* py, float* ppre, float* pw, float* pb, float* px, int64 yvec, int64 ndat, int64 xvec, int actFunc, HYPER h) {
     raise_on(kai_dense_forward(device, py, ppre, pw, pb, px, yvec, ndat, xvec, actFunc, h));
 }

@@ -61,6 +61,7 @@ SIGNATURES = {
     "kai_mix_values_backward_value": [_INT, _F, _F, _F, _I64, _I64, _I64, _I64, _I64],
     "kai_gemm_f32": [_INT, _INT, _INT, _I64, _I64, _I64, _F, _I64, _F, _I64, _F, _I64, _F, _INT, _F, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
+    "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
     "kai_dense_backward": [_INT, _F, _F, _F, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F, _INT],
 }
 
@@ -295,6 +296,11 @@ class VMath:
     def gemm_f32(device, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, bias, actFunc, hLeakyAlpha, acc):
         _ck(load().kai_gemm_f32(device, int(transA), int(transB), M, N, K, _addr(A), lda, _addr(B), ldb, _addr(C),
                                 ldc, _addr(bias), actFunc, _addr(hLeakyAlpha), int(acc)))
+
+    @staticmethod
+    def attention_forward(device, py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked):
+        _ck(load().kai_attention_forward(device, _addr(py), _addr(pQ), _addr(pK), _addr(pV), nbat, ntimes, nvec,
+                                         nhead, npiece, _addr(hCoef), int(bool(masked))))
 
     @staticmethod
     def dense_forward(device, py, ppre, pw, pb, px, yvec, ndat, xvec, actFunc, hLeakyAlpha):

@@ -194,6 +194,18 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
                        const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
                        int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc);
 
+/* Attention for forward-only use in one launch: py[nbat, ntimes, nhead*npiece] =
+ * mix_values(softmax_direct_on_axis(mask(mult_on_heads(K, Q, coef))), V), i.e. the middle of
+ * VTensor::mh_attention (vtensor.cpp:3036-3043), without materialising the
+ * [nbat, ntimes, ntimes, nhead] tensor (training needs that tensor and keeps the separate calls).
+ * masked != 0 applies the causal mask of set_mh_attention_mask.  Head sizes 16, 32 and 64 with
+ * 16-byte aligned operands run fused; any other shape runs the four separate kernels with the
+ * probabilities in the library's scratch memory.  The softmax is renormalised tile by tile, so the
+ * result equals the separate calls up to rounding. */
+int kai_attention_forward(int device, float* py, const float* pQ, const float* pK, const float* pV, int64_t nbat,
+                          int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
+                          int masked);
+
 #ifdef __cplusplus
 }
 #endif

@@ -78,6 +78,7 @@ public:
     static void mix_values_backward_value(int device, float* pV, float* pgy, float* pp, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece);
 
     /* additive: the `dense` layer formula activate(add(matmul(x,w),b)) (api/vconst.cpp:11) in one launch */
+    static void attention_forward(int device, float* py, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked);
     static void dense_forward(int device, float* py, float* ppre, float* pw, float* pb, float* px, int64 yvec, int64 ndat, int64 xvec, int actFunc, HYPER hLeakyAlpha);
     static void dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pga_work, float* pgy, float* pw, float* px, float* ppre, int64 yvec, int64 ndat, int64 xvec, int actFunc, HYPER hLeakyAlpha, bool acc);
 };

@@ -469,6 +469,30 @@ SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 51
                        (2, 1030, 2), (40, 64, 16)]
 
 
+# fused forward attention against the oracle's four separate steps: both cfg4 mappings, ragged lengths, the three
+# fused head sizes, the causal mask, and shapes that fall back to the separate kernels (head size 24, unaligned nvec)
+@pytest.mark.parametrize("nbat,ntimes,nhead,npiece,masked", [(32, 512, 1, 64, False), (4, 512, 8, 64, False),
+                                                             (2, 130, 4, 32, True), (3, 77, 2, 16, False),
+                                                             (1, 1000, 2, 64, True), (2, 64, 3, 64, True),
+                                                             (2, 100, 2, 24, True), (1, 50, 3, 7, False),
+                                                             (1, 1, 1, 16, True)])
+def test_attention_forward_fused(nbat, ntimes, nhead, npiece, masked):
+    nvec = nhead * npiece
+    rng = np.random.default_rng(nbat * 1000 + ntimes * 10 + nhead + npiece)
+    q = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    k = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    v = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    coef = 1.0 / np.sqrt(npiece)
+    s = ko.mult_on_heads(k, q, nhead, coef)
+    if masked:
+        s = ko.set_mh_attention_mask(s, True)
+    pr = ko.softmax_direct_on_axis(s, nbat * ntimes, ntimes, nhead).reshape(nbat, ntimes, ntimes, nhead)
+    ref = ko.mix_values(pr, v, nhead)
+    o = DB(nbat * ntimes * nvec * 4)
+    VMath.attention_forward(0, o, dev(q), dev(k), dev(v), nbat, ntimes, nvec, nhead, npiece, kai.hyper(coef), masked)
+    check(o.to_numpy((nbat, ntimes, nvec)), ref, what="fused attention")
+
+
 @pytest.mark.parametrize("nrow,nvec,ncol", SOFTMAX_AXIS_SHAPES)
 def test_softmax_axis_layouts(nrow, nvec, ncol):
     rng = np.random.default_rng(nrow + nvec + ncol)
