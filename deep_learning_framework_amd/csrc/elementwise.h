@@ -18,6 +18,15 @@ int launch_softmax_rows_backward(float* gx, const float* gy, const float* x, int
 int launch_fill_float(float* p, int64_t n, float value, hipStream_t stream);
 int launch_fill_int(int* p, int64_t n, int value, hipStream_t stream);
 
+// parameter update: VMath::accumulate_grad / subtract_param_grad / apply_decay / eval_adam_delta
+// (vmath.cu:364-490 of the reference); hyper-parameters are device scalars, null reads as 0
+int launch_accumulate_grad(float* y, const float* x, int64_t n, hipStream_t stream);
+int launch_subtract_param_grad(float* p, const float* g, int64_t n, const float* hlr, hipStream_t stream);
+int launch_apply_decay(float* d, const float* p, const float* g, int64_t n, const float* hl1, const float* hl2,
+                       hipStream_t stream);
+int launch_eval_adam_delta(float* a, const float* g, float* s, float* t, float* nstep, int64_t n, const float* hro1,
+                           const float* hro2, const float* heps, hipStream_t stream);
+
 // Final pass of a split-K product: C(m,n) (=|+=) act(alpha * sum_s part[s][m][n] + bias[n]), the
 // pre-activation value also to C2 when given.  `part` holds nsplit dense [M,N] matrices.
 struct SplitReduceParams {

@@ -244,6 +244,115 @@ int launch_fill_int(int* p, int64_t n, int value, hipStream_t stream) {
     return check_launch("fill_kernel");
 }
 
+// ---- parameter update ------------------------------------------------------------------------------
+//
+// Elementwise streams over the parameter, gradient and optimizer-state tensors.  The arithmetic keeps
+// the reference's rounding: its host build forbids contraction (-ffp-contract=off,
+// source/engine/CMakeLists.txt:196), so products and sums are rounded separately here too
+// (contraction is switched off below for the rest of this file; it must be this pragma around plain
+// operators: HIP's __fmul_rn / __fadd_rn are inline functions of a header outside its reach and get
+// fused after inlining) and the first three kernels are bit-identical to the host loops.
+// MODE selects the function; VEC = four elements per thread with 128-bit accesses.
+#pragma clang fp contract(off)
+
+enum UpdateMode { kUpdAccumulate = 0, kUpdSubtract = 1, kUpdDecay = 2 };
+
+struct UpdateParams {
+    float* out;         // accumulate: y (in place); subtract: p (in place); decay: d
+    const float* a;     // accumulate: x; subtract: g; decay: p
+    const float* b;     // decay: g
+    const float* h1;    // subtract: learning rate; decay: l1
+    const float* h2;    // decay: l2
+    int64_t n;
+};
+
+template <int MODE>
+__device__ __forceinline__ float update_one(float out, float a, float b, float h1, float h2) {
+    if (MODE == kUpdAccumulate) return out + a;
+    if (MODE == kUpdSubtract) return out - a * h1;
+    float delta = b;   // decay: a = p, b = g, h1 = l1, h2 = l2
+    if (h2 > 0) delta += h2 * a;
+    if (h1 > 0) delta += h1 * ((a > 0) ? 1.f : ((a < 0) ? -1.f : 0.f));
+    return delta;
+}
+
+template <int MODE, bool VEC>
+__global__ void __launch_bounds__(kEwThreads) update_kernel(UpdateParams p) {
+    const float h1 = p.h1 ? *p.h1 : 0.f;
+    const float h2 = p.h2 ? *p.h2 : 0.f;
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    const int64_t n = VEC ? p.n / 4 : p.n;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        if (VEC) {
+            f32x4 o = MODE == kUpdDecay ? f32x4{0.f, 0.f, 0.f, 0.f} : *reinterpret_cast<const f32x4*>(p.out + i * 4);
+            const f32x4 a = *reinterpret_cast<const f32x4*>(p.a + i * 4);
+            const f32x4 b = MODE == kUpdDecay ? *reinterpret_cast<const f32x4*>(p.b + i * 4) : a;
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[j] = update_one<MODE>(o[j], a[j], b[j], h1, h2);
+            *reinterpret_cast<f32x4*>(p.out + i * 4) = o;
+        } else {
+            const float o = MODE == kUpdDecay ? 0.f : p.out[i];
+            p.out[i] = update_one<MODE>(o, p.a[i], MODE == kUpdDecay ? p.b[i] : 0.f, h1, h2);
+        }
+    }
+}
+
+template <int MODE>
+static int launch_update(const UpdateParams& p, const char* name, hipStream_t stream) {
+    if (p.n <= 0) return KAI_OK;
+    const bool vec = p.n % 4 == 0 && aligned16(p.out) && aligned16(p.a) && (p.b == nullptr || aligned16(p.b));
+    if (vec) update_kernel<MODE, true><<<blocks_for(p.n / 4), kEwThreads, 0, stream>>>(p);
+    else update_kernel<MODE, false><<<blocks_for(p.n), kEwThreads, 0, stream>>>(p);
+    return check_launch(name);
+}
+
+int launch_accumulate_grad(float* y, const float* x, int64_t n, hipStream_t stream) {
+    UpdateParams p{y, x, nullptr, nullptr, nullptr, n};
+    return launch_update<kUpdAccumulate>(p, "accumulate_grad", stream);
+}
+
+int launch_subtract_param_grad(float* pp, const float* g, int64_t n, const float* hlr, hipStream_t stream) {
+    UpdateParams p{pp, g, nullptr, hlr, nullptr, n};
+    return launch_update<kUpdSubtract>(p, "subtract_param_grad", stream);
+}
+
+int launch_apply_decay(float* d, const float* pp, const float* g, int64_t n, const float* hl1, const float* hl2,
+                       hipStream_t stream) {
+    UpdateParams p{d, pp, g, hl1, hl2, n};
+    return launch_update<kUpdDecay>(p, "apply_decay", stream);
+}
+
+// One Adam step (vmath.cu:449-468): s and t are the moment tensors, nstep the per-element step count
+// (a float tensor in the engine), all updated in place; a receives the update direction.
+__global__ void __launch_bounds__(kEwThreads)
+    adam_delta_kernel(float* __restrict__ a, const float* __restrict__ g, float* __restrict__ s, float* __restrict__ t,
+                      float* __restrict__ nstep, int64_t n, const float* __restrict__ hro1,
+                      const float* __restrict__ hro2, const float* __restrict__ heps) {
+    const float ro1 = hro1 ? *hro1 : 0.f;
+    const float ro2 = hro2 ? *hro2 : 0.f;
+    const float eps = heps ? *heps : 0.f;
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        const float delta = g[i];
+        const float ns = nstep[i] + 1.f;
+        const float si = ro1 * s[i] + (1.f - ro1) * delta;
+        const float ti = ro2 * t[i] + (1.f - ro2) * delta * delta;
+        const float sterm = si / (1.f - powf(ro1, ns));
+        const float tterm = ti / (1.f - powf(ro2, ns));
+        s[i] = si;
+        t[i] = ti;
+        a[i] = sterm / (sqrtf(tterm) + eps);
+        nstep[i] = ns;
+    }
+}
+
+int launch_eval_adam_delta(float* a, const float* g, float* s, float* t, float* nstep, int64_t n, const float* hro1,
+                           const float* hro2, const float* heps, hipStream_t stream) {
+    if (n <= 0) return KAI_OK;
+    adam_delta_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(a, g, s, t, nstep, n, hro1, hro2, heps);
+    return check_launch("adam_delta_kernel");
+}
+
 // ---- split-K final pass ---------------------------------------------------------------------
 //
 // Sums the partial products in split order (fixed, so the result does not depend on scheduling)

@@ -549,6 +549,42 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
     return KAI_OK;
 }
 
+// ---- parameter update: what consumes dW and db ---------------------------------------------------
+
+int kai_accumulate_grad(int device, float* py, const float* px, int64_t nrow) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (nrow == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(px);
+    return launch_accumulate_grad(py, px, nrow, current_stream());
+}
+
+int kai_subtract_param_grad(int device, float* pp, const float* pg, int64_t nrow, const float* hLearningRate) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (nrow == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pp); KAI_REQUIRE_PTR(pg);
+    return launch_subtract_param_grad(pp, pg, nrow, hLearningRate, current_stream());
+}
+
+int kai_apply_decay(int device, float* pd, const float* pp, const float* pg, int64_t nrow, const float* hL1Decay,
+                    const float* hL2Decay) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (nrow == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pd); KAI_REQUIRE_PTR(pp); KAI_REQUIRE_PTR(pg);
+    return launch_apply_decay(pd, pp, pg, nrow, hL1Decay, hL2Decay, current_stream());
+}
+
+int kai_eval_adam_delta(int device, float* pa, const float* pg, float* ps, float* pt, float* pn, int64_t nrow,
+                        const float* hRo1, const float* hRo2, const float* hEpsilon) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (nrow == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pa); KAI_REQUIRE_PTR(pg); KAI_REQUIRE_PTR(ps); KAI_REQUIRE_PTR(pt); KAI_REQUIRE_PTR(pn);
+    return launch_eval_adam_delta(pa, pg, ps, pt, pn, nrow, hRo1, hRo2, hEpsilon, current_stream());
+}
+
 int kai_attention_forward(int device, float* py, const float* pQ, const float* pK, const float* pV, int64_t nbat,
                           int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
                           int masked) {

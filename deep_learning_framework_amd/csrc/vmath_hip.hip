@@ -82,6 +82,19 @@ void VMath::mix_values_backward_value(int device, float* pgV, float* pgy, float*
     raise_on(kai_mix_values_backward_value(device, pgV, pgy, pp, nbat, ntimes, nvec, nhead, npiece));
 }
 
+void VMath::accumulate_grad(int device, float* py, float* px, int64 nrow) {
+    raise_on(kai_accumulate_grad(device, py, px, nrow));
+}
+void VMath::subtract_param_grad(int device, float* pp, float* pg, int64 nrow, HYPER h) {
+    raise_on(kai_subtract_param_grad(device, pp, pg, nrow, h));
+}
+void VMath::apply_decay(int device, float* pd, float* pp, float* pg, int64 nrow, HYPER h1, HYPER h2) {
+    raise_on(kai_apply_decay(device, pd, pp, pg, nrow, h1, h2));
+}
+void VMath::eval_adam_delta(int device, float* pa, float* pg, float* ps, float* pt, float* pn, int64 nrow, HYPER hRo1, HYPER hRo2, HYPER hEpsilon) {
+    raise_on(kai_eval_adam_delta(device, pa, pg, ps, pt, pn, nrow, hRo1, hRo2, hEpsilon));
+}
+
 void VMath::attention_forward(int device, float* py, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked) {
     raise_on(kai_attention_forward(device, py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked ? 1 : 0));
 }

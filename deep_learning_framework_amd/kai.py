@@ -62,6 +62,10 @@ SIGNATURES = {
     "kai_gemm_f32": [_INT, _INT, _INT, _I64, _I64, _I64, _F, _I64, _F, _I64, _F, _I64, _F, _INT, _F, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
     "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
+    "kai_accumulate_grad": [_INT, _F, _F, _I64],
+    "kai_subtract_param_grad": [_INT, _F, _F, _I64, _F],
+    "kai_apply_decay": [_INT, _F, _F, _F, _I64, _F, _F],
+    "kai_eval_adam_delta": [_INT, _F, _F, _F, _F, _F, _I64, _F, _F, _F],
     "kai_dense_backward": [_INT, _F, _F, _F, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F, _INT],
 }
 
@@ -296,6 +300,23 @@ class VMath:
     def gemm_f32(device, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, bias, actFunc, hLeakyAlpha, acc):
         _ck(load().kai_gemm_f32(device, int(transA), int(transB), M, N, K, _addr(A), lda, _addr(B), ldb, _addr(C),
                                 ldc, _addr(bias), actFunc, _addr(hLeakyAlpha), int(acc)))
+
+    @staticmethod
+    def accumulate_grad(device, py, px, nrow):
+        _ck(load().kai_accumulate_grad(device, _addr(py), _addr(px), nrow))
+
+    @staticmethod
+    def subtract_param_grad(device, pp, pg, nrow, hLearningRate):
+        _ck(load().kai_subtract_param_grad(device, _addr(pp), _addr(pg), nrow, _addr(hLearningRate)))
+
+    @staticmethod
+    def apply_decay(device, pd, pp, pg, nrow, hL1Decay, hL2Decay):
+        _ck(load().kai_apply_decay(device, _addr(pd), _addr(pp), _addr(pg), nrow, _addr(hL1Decay), _addr(hL2Decay)))
+
+    @staticmethod
+    def eval_adam_delta(device, pa, pg, ps, pt, pn, nrow, hRo1, hRo2, hEpsilon):
+        _ck(load().kai_eval_adam_delta(device, _addr(pa), _addr(pg), _addr(ps), _addr(pt), _addr(pn), nrow,
+                                       _addr(hRo1), _addr(hRo2), _addr(hEpsilon)))
 
     @staticmethod
     def attention_forward(device, py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked):

@@ -194,6 +194,24 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
                        const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
                        int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc);
 
+/* ---- parameter update: the consumers of the weight and bias gradients (next to the path) ----------- */
+
+/* VMath::accumulate_grad, vmath.cu:364-382 (vmath.h:28).  py[n] += px[n]; sums the gradient shards of
+ * data-parallel replicas (vtensor.cpp:433-475). */
+int kai_accumulate_grad(int device, float* py, const float* px, int64_t nrow);
+/* VMath::subtract_param_grad, vmath.cu:385-404 (vmath.h:29).  pp[n] -= pg[n] * learningRate; the
+ * reference runs it on the host only (voptimizer.cpp:524,538), this entry point keeps the update on
+ * the device. */
+int kai_subtract_param_grad(int device, float* pp, const float* pg, int64_t nrow, const float* hLearningRate);
+/* VMath::apply_decay, vmath.cu:408-444 (vmath.h:30).  pd = pg + l2 * pp + l1 * sign(pp), each term only
+ * for a positive coefficient. */
+int kai_apply_decay(int device, float* pd, const float* pp, const float* pg, int64_t nrow, const float* hL1Decay,
+                    const float* hL2Decay);
+/* VMath::eval_adam_delta, vmath.cu:449-490 (vmath.h:31).  One Adam step: ps, pt (moments) and pn (step
+ * count, a float tensor) are updated in place, pa receives sterm / (sqrt(tterm) + epsilon). */
+int kai_eval_adam_delta(int device, float* pa, const float* pg, float* ps, float* pt, float* pn, int64_t nrow,
+                        const float* hRo1, const float* hRo2, const float* hEpsilon);
+
 /* Attention for forward-only use in one launch: py[nbat, ntimes, nhead*npiece] =
  * mix_values(softmax_direct_on_axis(mask(mult_on_heads(K, Q, coef))), V), i.e. the middle of
  * VTensor::mh_attention (vtensor.cpp:3036-3043), without materialising the

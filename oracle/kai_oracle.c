@@ -440,3 +440,57 @@ int ko_mix_values_backward_value(float* pgV, const float* pgy, const float* pp, 
     }
     return KO_OK;
 }
+
+/* ---- parameter update (next to the path: what consumes dW and db) ------------------------------ */
+
+#define KO_HYPER(h) ((h) ? *(h) : 0.0f)   /* HYPER_ACCESS, local_objects/vhypermanager.h:9 */
+
+int ko_accumulate_grad(float* py, const float* px, int64_t ndat) {
+    /* vmath.cu:364-368 */
+    for (int64_t nd = 0; nd < ndat; nd++) {
+        py[nd] += px[nd];
+    }
+    return KO_OK;
+}
+
+int ko_subtract_param_grad(float* pp, const float* pg, int64_t nrow, const float* hLearningRate) {
+    /* vmath.cu:385-390 */
+    float learningRate = KO_HYPER(hLearningRate);
+    for (int64_t n = 0; n < nrow; n++) {
+        pp[n] -= pg[n] * learningRate;
+    }
+    return KO_OK;
+}
+
+int ko_apply_decay(float* pd, const float* pp, const float* pg, int64_t nrow, const float* hL1Decay,
+                   const float* hL2Decay) {
+    /* vmath.cu:408-421 */
+    float l1Decay = KO_HYPER(hL1Decay);
+    float l2Decay = KO_HYPER(hL2Decay);
+    for (int64_t n = 0; n < nrow; n++) {
+        float delta = pg[n];
+        if (l2Decay > 0) delta += l2Decay * pp[n];
+        if (l1Decay > 0) delta += l1Decay * ((pp[n] > 0) ? 1 : ((pp[n] < 0) ? -1 : 0));
+        pd[n] = delta;
+    }
+    return KO_OK;
+}
+
+int ko_eval_adam_delta(float* pa, const float* pg, float* ps, float* pt, float* pn, int64_t nrow, const float* hRo1,
+                       const float* hRo2, const float* hEpsilon) {
+    /* vmath.cu:449-468 */
+    float ro1 = KO_HYPER(hRo1);
+    float ro2 = KO_HYPER(hRo2);
+    float epsilon = KO_HYPER(hEpsilon);
+    for (int64_t n = 0; n < nrow; n++) {
+        float delta = pg[n];
+        float nstep = pn[n] + 1;
+        ps[n] = ro1 * ps[n] + (1 - ro1) * delta;
+        pt[n] = ro2 * pt[n] + (1 - ro2) * delta * delta;
+        float sterm = ps[n] / (1 - powf(ro1, nstep));
+        float tterm = pt[n] / (1 - powf(ro2, nstep));
+        pa[n] = sterm / (sqrtf(tterm) + epsilon);
+        pn[n] = nstep;
+    }
+    return KO_OK;
+}

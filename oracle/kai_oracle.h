@@ -95,6 +95,14 @@ int ko_mix_values_backward_prop(float* pgp, const float* pgy, const float* pV, i
 int ko_mix_values_backward_value(float* pgV, const float* pgy, const float* pp, int64_t nbat, int64_t ntimes,
                                  int64_t nvec, int64_t nhead, int64_t npiece);
 
+/* vmath.cu:364-368, 385-390, 408-421, 449-468: what consumes the weight and bias gradients */
+int ko_accumulate_grad(float* py, const float* px, int64_t ndat);
+int ko_subtract_param_grad(float* pp, const float* pg, int64_t nrow, const float* hLearningRate);
+int ko_apply_decay(float* pd, const float* pp, const float* pg, int64_t nrow, const float* hL1Decay,
+                   const float* hL2Decay);
+int ko_eval_adam_delta(float* pa, const float* pg, float* ps, float* pt, float* pn, int64_t nrow, const float* hRo1,
+                       const float* hRo2, const float* hEpsilon);
+
 #ifdef __cplusplus
 }
 #endif

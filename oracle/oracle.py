@@ -56,6 +56,10 @@ def lib():
             "ko_mix_values": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
             "ko_mix_values_backward_prop": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
             "ko_mix_values_backward_value": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
+            "ko_accumulate_grad": [_F, _F, _I64],
+            "ko_subtract_param_grad": [_F, _F, _I64, _F],
+            "ko_apply_decay": [_F, _F, _F, _I64, _F, _F],
+            "ko_eval_adam_delta": [_F, _F, _F, _F, _F, _I64, _F, _F, _F],
         }
         for name, args in sig.items():
             fn = getattr(L, name)
@@ -256,3 +260,40 @@ def mix_values_backward_value(gy, p, nhead):
     gV = np.empty((nbat, ntimes, nvec), np.float32)
     _check(lib().ko_mix_values_backward_value(_p(gV), _p(gy), _p(p), nbat, ntimes, nvec, nhead, nvec // nhead))
     return gV
+
+
+def accumulate_grad(y, x):
+    """y + x elementwise (returns the new y)."""
+    y = _f32(y).copy()
+    x = _f32(x)
+    _check(lib().ko_accumulate_grad(_p(y), _p(x), y.size))
+    return y
+
+
+def subtract_param_grad(p, g, learning_rate):
+    p = _f32(p).copy()
+    g = _f32(g)
+    keep, h = _hyper(learning_rate)
+    _check(lib().ko_subtract_param_grad(_p(p), _p(g), p.size, h))
+    return p
+
+
+def apply_decay(p, g, l1_decay, l2_decay):
+    p, g = _f32(p), _f32(g)
+    d = np.zeros_like(g)
+    k1, h1 = _hyper(l1_decay)
+    k2, h2 = _hyper(l2_decay)
+    _check(lib().ko_apply_decay(_p(d), _p(p), _p(g), g.size, h1, h2))
+    return d
+
+
+def eval_adam_delta(g, s, t, n, ro1, ro2, epsilon):
+    """One Adam step: returns (delta, s', t', n'); s, t, n are the moment and step-count tensors."""
+    g = _f32(g)
+    s, t, n = _f32(s).copy(), _f32(t).copy(), _f32(n).copy()
+    a = np.zeros_like(g)
+    k1, h1 = _hyper(ro1)
+    k2, h2 = _hyper(ro2)
+    k3, h3 = _hyper(epsilon)
+    _check(lib().ko_eval_adam_delta(_p(a), _p(g), _p(s), _p(t), _p(n), g.size, h1, h2, h3))
+    return a, s, t, n

@@ -532,6 +532,41 @@ def test_split_k_scratch_survives_shutdown_and_growth():
         check(y.to_numpy((m, n))[rows], ko.matmul_rows(w, x, rows), what="split-K %dx%dx%d" % (m, n, k))
 
 
+# ---- parameter update: accumulate_grad, subtract_param_grad, apply_decay, eval_adam_delta ------------------------------
+
+@pytest.mark.parametrize("n", [1, 7, 1024, 4099, 1 << 20])
+def test_parameter_update_ops(n):
+    rng = np.random.default_rng(n)
+    p = rng.standard_normal(n).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    p[:: 5] = 0.0                                  # sign(0) = 0 in the L1 term
+    y = dev(p)
+    VMath.accumulate_grad(0, y, dev(g), n)
+    np.testing.assert_array_equal(y.to_numpy((n,)), ko.accumulate_grad(p, g))
+    y = dev(p)
+    VMath.subtract_param_grad(0, y, dev(g), n, kai.hyper(0.0123))
+    np.testing.assert_array_equal(y.to_numpy((n,)), ko.subtract_param_grad(p, g, 0.0123))   # product rounded first
+    y = dev(p)
+    VMath.subtract_param_grad(0, y, dev(g), n, None)                                        # null learning rate = 0
+    np.testing.assert_array_equal(y.to_numpy((n,)), p)
+    for l1, l2 in ((0.01, 0.02), (None, 0.5), (0.25, None), (None, None), (-1.0, -1.0)):
+        d = DB(n * 4)
+        VMath.apply_decay(0, d, dev(p), dev(g), n, kai.hyper(l1), kai.hyper(l2))
+        np.testing.assert_array_equal(d.to_numpy((n,)), ko.apply_decay(p, g, l1, l2))
+    # Adam: four steps, state carried on the device and in the oracle side by side
+    s, t, cnt = np.zeros(n, np.float32), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    ds, dt, dn, da = dev(s), dev(t), dev(cnt), DB(n * 4)
+    h1, h2, he = kai.hyper(0.9), kai.hyper(0.999), kai.hyper(1e-8)
+    for step in range(4):
+        gs = rng.standard_normal(n).astype(np.float32)
+        VMath.eval_adam_delta(0, da, dev(gs), ds, dt, dn, n, h1, h2, he)
+        a, s, t, cnt = ko.eval_adam_delta(gs, s, t, cnt, 0.9, 0.999, 1e-8)
+        np.testing.assert_array_equal(dn.to_numpy((n,)), cnt)
+        np.testing.assert_array_equal(ds.to_numpy((n,)), s)        # the moments use only +, * (rounded as in the oracle)
+        np.testing.assert_array_equal(dt.to_numpy((n,)), t)
+        np.testing.assert_allclose(da.to_numpy((n,)), a, rtol=2e-6, atol=1e-7)   # powf and sqrtf of two libraries
+
+
 # ---- memory helpers and errors ----------------------------------------------------------------------------------------
 
 def test_memory_helpers():

@@ -284,3 +284,52 @@ def test_attention_backward_closed_forms(nbat, ntimes, nhead, npiece):
     b = np.vdot(ko.mix_values_backward_prop(gy, v, nhead).astype(np.float64), p)
     c = np.vdot(ko.mix_values_backward_value(gy, p, nhead).astype(np.float64), v)
     assert abs(a - b) < 1e-4 * abs(a) + 1e-5 and abs(a - c) < 1e-4 * abs(a) + 1e-5
+
+
+# ---- parameter update (vmath.cu:364-490) --------------------------------------------------------------------------
+
+def test_accumulate_subtract_and_decay_exact_cases():
+    y = np.array([1, -2, 3.5, 0], np.float32)
+    x = np.array([4, 2, -0.5, -0.0], np.float32)
+    np.testing.assert_array_equal(ko.accumulate_grad(y, x), np.array([5, 0, 3, 0], np.float32))
+    # powers of two keep every product and difference exact
+    np.testing.assert_array_equal(ko.subtract_param_grad(y, x, 0.5), np.array([-1, -3, 3.75, 0], np.float32))
+    np.testing.assert_array_equal(ko.subtract_param_grad(y, x, None), y)          # null HYPER reads as 0
+    p = np.array([2, -4, 0, 1], np.float32)
+    g = np.array([1, 1, 1, -1], np.float32)
+    np.testing.assert_array_equal(ko.apply_decay(p, g, None, None), g)            # no decay: delta = g
+    np.testing.assert_array_equal(ko.apply_decay(p, g, 0.0, 0.25), g + 0.25 * p)  # L2 only
+    np.testing.assert_array_equal(ko.apply_decay(p, g, 0.5, 0.0), g + 0.5 * np.sign(p))   # L1 only: sign(0) = 0
+    np.testing.assert_array_equal(ko.apply_decay(p, g, 0.5, 0.25), g + 0.25 * p + 0.5 * np.sign(p))
+    np.testing.assert_array_equal(ko.apply_decay(p, g, -1.0, -1.0), g)            # non-positive coefficients are skipped
+
+
+def test_subtract_rounds_the_product_before_the_difference():
+    # p - g * lr with separately rounded product (no FMA): brute force in explicit fp32 steps
+    rng = np.random.default_rng(5)
+    p = rng.standard_normal(1000).astype(np.float32)
+    g = rng.standard_normal(1000).astype(np.float32)
+    lr = np.float32(0.0123)
+    want = (p - (g * lr).astype(np.float32)).astype(np.float32)
+    np.testing.assert_array_equal(ko.subtract_param_grad(p, g, float(lr)), want)
+
+
+def test_adam_first_step_closed_form_and_float64_recurrence():
+    rng = np.random.default_rng(6)
+    g = rng.standard_normal(500).astype(np.float32)
+    z = np.zeros(500, np.float32)
+    ro1, ro2, eps = 0.9, 0.999, 1e-8
+    a, s, t, n = ko.eval_adam_delta(g, z, z, z, ro1, ro2, eps)
+    # step 1: s / (1 - ro1) = g and t / (1 - ro2) = g^2, so the update direction is g / (|g| + eps)
+    np.testing.assert_allclose(a, g / (np.abs(g) + eps), rtol=2e-6)
+    np.testing.assert_array_equal(n, np.ones(500, np.float32))
+    # three more steps against a float64 recurrence
+    s64, t64 = s.astype(np.float64), t.astype(np.float64)
+    for step in range(2, 5):
+        g2 = rng.standard_normal(500).astype(np.float32)
+        a, s, t, n = ko.eval_adam_delta(g2, s, t, n, ro1, ro2, eps)
+        s64 = ro1 * s64 + (1 - ro1) * g2
+        t64 = ro2 * t64 + (1 - ro2) * g2.astype(np.float64) ** 2
+        want = (s64 / (1 - ro1 ** step)) / (np.sqrt(t64 / (1 - ro2 ** step)) + eps)
+        np.testing.assert_allclose(a, want, rtol=2e-5, atol=1e-6)
+        np.testing.assert_array_equal(n, np.full(500, step, np.float32))
