@@ -196,6 +196,22 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
     xc, wc = x.cpu().numpy(), w.cpu().numpy()
     row("cfg5 ragged 1000x777x333", gpu_us(lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0)),
         flops=2.0 * m * n * k, cpu=cpu_us(lambda: ko.matmul(wc, xc)))
+    # transposes next to the path: the head split [4,512,8,64] -> [4,8,512,64] of configuration 4 and a plain 4096^2
+    shape, axes = (4, 512, 8, 64), (0, 2, 1, 3)
+    x = torch.randn(shape, device=dev, generator=g)
+    y = torch.empty_like(x)
+    # the engine's table: per output axis (source axis, output elements per step), per source axis its source step
+    info = torch.tensor([[0, 512 * 8 * 64, 512 * 8 * 64], [2, 512 * 64, 8 * 64], [1, 64, 64], [3, 1, 1]],
+                        dtype=torch.int32, device=dev)
+    xc = x.cpu().numpy()
+    row("transpose [4,512,8,64] -> [4,8,512,64]",
+        gpu_us(lambda: L.kai_transpose(0, P(y), P(x), P(info), I(4), I(x.numel()))),
+        nbytes=8.0 * x.numel(), cpu=cpu_us(lambda: ko.transpose(xc, axes)))
+    x = torch.randn((4096, 4096), device=dev, generator=g)
+    y = torch.empty_like(x)
+    xc = x.cpu().numpy()
+    row("transpose_bin 4096 x 4096", gpu_us(lambda: L.kai_transpose_bin(0, P(y), P(x), I(4096), I(4096))),
+        nbytes=8.0 * x.numel(), cpu=cpu_us(lambda: ko.transpose_bin(xc, 4096, 4096)))
     return rows
 
 

@@ -27,6 +27,12 @@ int launch_apply_decay(float* d, const float* p, const float* g, int64_t n, cons
 int launch_eval_adam_delta(float* a, const float* g, float* s, float* t, float* nstep, int64_t n, const float* hro1,
                            const float* hro2, const float* heps, hipStream_t stream);
 
+// VMath::transpose / transpose_backward / transpose_bin (vmath.cu:9384-9510 of the reference); pn is the
+// engine's device table of axis_size x 3 ints
+int launch_transpose(float* y, const float* x, const int* pn, int64_t axis_size, int64_t n, bool backward,
+                     hipStream_t stream);
+int launch_transpose_bin(float* y, const float* x, int64_t nrow, int64_t ncol, hipStream_t stream);
+
 // Final pass of a split-K product: C(m,n) (=|+=) act(alpha * sum_s part[s][m][n] + bias[n]), the
 // pre-activation value also to C2 when given.  `part` holds nsplit dense [M,N] matrices.
 struct SplitReduceParams {

@@ -244,6 +244,78 @@ int launch_fill_int(int* p, int64_t n, int value, hipStream_t stream) {
     return check_launch("fill_kernel");
 }
 
+// ---- transposes -------------------------------------------------------------------------------------
+//
+// transpose_bin: y[nrow, ncol] = x[ncol, nrow]^T through a 32 x 33 LDS tile, so that both the reads and
+// the writes are 128-byte rows.  transpose / transpose_backward: the engine's general axis permutation,
+// driven by its device table (per output axis: source axis, output elements per step, and per SOURCE
+// axis: source elements per step); a thread owns one output element, writes (forward) or reads
+// (backward) are contiguous, the other side is a gather or scatter.
+
+constexpr int kTrTile = 32;
+constexpr int kTrMaxAxes = 8;
+
+__global__ void __launch_bounds__(kTrTile * 8) transpose_bin_kernel(float* __restrict__ y, const float* __restrict__ x,
+                                                                    int64_t nrow, int64_t ncol, int64_t tiles_c) {
+    __shared__ float tile[kTrTile][kTrTile + 1];
+    const int64_t tr = blockIdx.x / tiles_c, tc = blockIdx.x % tiles_c;   // tile of y: rows tr*32.., columns tc*32..
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;              // 32 x 8 threads
+    // x is [ncol, nrow]: read rows c of x (contiguous along r)
+#pragma unroll
+    for (int i = 0; i < kTrTile; i += 8) {
+        const int64_t c = tc * kTrTile + ty + i, r = tr * kTrTile + tx;
+        if (c < ncol && r < nrow) tile[ty + i][tx] = x[c * nrow + r];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kTrTile; i += 8) {
+        const int64_t r = tr * kTrTile + ty + i, c = tc * kTrTile + tx;
+        if (r < nrow && c < ncol) y[r * ncol + c] = tile[tx][ty + i];
+    }
+}
+
+int launch_transpose_bin(float* y, const float* x, int64_t nrow, int64_t ncol, hipStream_t stream) {
+    if (nrow <= 0 || ncol <= 0) return KAI_OK;
+    const int64_t tiles_r = (nrow + kTrTile - 1) / kTrTile, tiles_c = (ncol + kTrTile - 1) / kTrTile;
+    if (tiles_r * tiles_c > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "transpose_bin: matrix too large");
+    transpose_bin_kernel<<<dim3((unsigned)(tiles_r * tiles_c)), kTrTile * 8, 0, stream>>>(y, x, nrow, ncol, tiles_c);
+    return check_launch("transpose_bin_kernel");
+}
+
+template <bool BACKWARD>
+__global__ void __launch_bounds__(kEwThreads) transpose_axes_kernel(float* __restrict__ out,
+                                                                    const float* __restrict__ in,
+                                                                    const int* __restrict__ pn, int axis_size,
+                                                                    int64_t n) {
+    // the table is tiny and the same for every thread
+    __shared__ int64_t yblk[kTrMaxAxes], xblk[kTrMaxAxes];
+    if (threadIdx.x < axis_size) {
+        yblk[threadIdx.x] = pn[threadIdx.x * 3 + 1];
+        xblk[threadIdx.x] = pn[pn[threadIdx.x * 3] * 3 + 2];
+    }
+    __syncthreads();
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        int64_t xpos = 0, ypos = i;
+        for (int m = 0; m < axis_size; m++) {
+            const int64_t c = ypos / yblk[m];
+            ypos -= c * yblk[m];
+            xpos += c * xblk[m];
+        }
+        if (BACKWARD) out[xpos] = in[i];
+        else out[i] = in[xpos];
+    }
+}
+
+int launch_transpose(float* y, const float* x, const int* pn, int64_t axis_size, int64_t n, bool backward,
+                     hipStream_t stream) {
+    if (n <= 0) return KAI_OK;
+    if (axis_size < 1 || axis_size > kTrMaxAxes) return fail(KAI_ERR_INVALID_ARGUMENT, "transpose: 1 to 8 axes");
+    if (backward) transpose_axes_kernel<true><<<blocks_for(n), kEwThreads, 0, stream>>>(y, x, pn, (int)axis_size, n);
+    else transpose_axes_kernel<false><<<blocks_for(n), kEwThreads, 0, stream>>>(y, x, pn, (int)axis_size, n);
+    return check_launch("transpose_axes_kernel");
+}
+
 // ---- parameter update ------------------------------------------------------------------------------
 //
 // Elementwise streams over the parameter, gradient and optimizer-state tensors.  The arithmetic keeps

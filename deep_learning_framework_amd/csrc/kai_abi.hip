@@ -549,6 +549,34 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
     return KAI_OK;
 }
 
+// ---- transposes ----------------------------------------------------------------------------------
+
+int kai_transpose(int device, float* py, const float* px, const int* pn, int64_t axis_size, int64_t data_size) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(data_size >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (data_size == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(px); KAI_REQUIRE_PTR(pn);
+    return launch_transpose(py, px, pn, axis_size, data_size, false, current_stream());
+}
+
+int kai_transpose_backward(int device, float* pgx, const float* pgy, const int* pn, int64_t axis_size,
+                           int64_t data_size) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(data_size >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (data_size == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgx); KAI_REQUIRE_PTR(pgy); KAI_REQUIRE_PTR(pn);
+    return launch_transpose(pgx, pgy, pn, axis_size, data_size, true, current_stream());
+}
+
+int kai_transpose_bin(int device, float* py, const float* px, int64_t nrow, int64_t ncol) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (nrow == 0 || ncol == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(px);
+    KAI_REQUIRE(py != px, KAI_ERR_INVALID_ARGUMENT, "transpose_bin cannot run in place");
+    return launch_transpose_bin(py, px, nrow, ncol, current_stream());
+}
+
 // ---- parameter update: what consumes dW and db ---------------------------------------------------
 
 int kai_accumulate_grad(int device, float* py, const float* px, int64_t nrow) {

@@ -82,6 +82,15 @@ void VMath::mix_values_backward_value(int device, float* pgV, float* pgy, float*
     raise_on(kai_mix_values_backward_value(device, pgV, pgy, pp, nbat, ntimes, nvec, nhead, npiece));
 }
 
+void VMath::transpose(int device, float* py, float* px, int* pn, int64 axis_size, int64 data_size) {
+    raise_on(kai_transpose(device, py, px, pn, axis_size, data_size));
+}
+void VMath::transpose_backward(int device, float* pgx, float* pgy, int* pn, int64 axis_size, int64 data_size) {
+    raise_on(kai_transpose_backward(device, pgx, pgy, pn, axis_size, data_size));
+}
+void VMath::transpose_bin(int device, float* py, float* px, int64 nrow, int64 ncol) {
+    raise_on(kai_transpose_bin(device, py, px, nrow, ncol));
+}
 void VMath::accumulate_grad(int device, float* py, float* px, int64 nrow) {
     raise_on(kai_accumulate_grad(device, py, px, nrow));
 }

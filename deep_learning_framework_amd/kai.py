@@ -62,6 +62,9 @@ SIGNATURES = {
     "kai_gemm_f32": [_INT, _INT, _INT, _I64, _I64, _I64, _F, _I64, _F, _I64, _F, _I64, _F, _INT, _F, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
     "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
+    "kai_transpose": [_INT, _F, _F, _F, _I64, _I64],
+    "kai_transpose_backward": [_INT, _F, _F, _F, _I64, _I64],
+    "kai_transpose_bin": [_INT, _F, _F, _I64, _I64],
     "kai_accumulate_grad": [_INT, _F, _F, _I64],
     "kai_subtract_param_grad": [_INT, _F, _F, _I64, _F],
     "kai_apply_decay": [_INT, _F, _F, _F, _I64, _F, _F],
@@ -300,6 +303,18 @@ class VMath:
     def gemm_f32(device, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, bias, actFunc, hLeakyAlpha, acc):
         _ck(load().kai_gemm_f32(device, int(transA), int(transB), M, N, K, _addr(A), lda, _addr(B), ldb, _addr(C),
                                 ldc, _addr(bias), actFunc, _addr(hLeakyAlpha), int(acc)))
+
+    @staticmethod
+    def transpose(device, py, px, pn, axis_size, data_size):
+        _ck(load().kai_transpose(device, _addr(py), _addr(px), _addr(pn), axis_size, data_size))
+
+    @staticmethod
+    def transpose_backward(device, pgx, pgy, pn, axis_size, data_size):
+        _ck(load().kai_transpose_backward(device, _addr(pgx), _addr(pgy), _addr(pn), axis_size, data_size))
+
+    @staticmethod
+    def transpose_bin(device, py, px, nrow, ncol):
+        _ck(load().kai_transpose_bin(device, _addr(py), _addr(px), nrow, ncol))
 
     @staticmethod
     def accumulate_grad(device, py, px, nrow):

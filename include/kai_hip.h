@@ -194,6 +194,19 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
                        const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
                        int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc);
 
+/* ---- transposes (next to the path) ----------------------------------------------------------------- */
+
+/* VMath::transpose, vmath.cu:9384-9433 (vmath.h:309).  General axis permutation of a dense tensor of
+ * data_size elements.  pn is the DEVICE table of axis_size x 3 ints that VTensor::transpose builds
+ * (vtensor.cpp:5391-5417): pn[m*3] = source axis of output axis m, pn[m*3+1] = output elements per step
+ * of output axis m, pn[a*3+2] = source elements per step of source axis a.  1 <= axis_size <= 8. */
+int kai_transpose(int device, float* py, const float* px, const int* pn, int64_t axis_size, int64_t data_size);
+/* VMath::transpose_backward, vmath.cu:9436-9483: pgx[source position] = pgy[n] with the same table. */
+int kai_transpose_backward(int device, float* pgx, const float* pgy, const int* pn, int64_t axis_size,
+                           int64_t data_size);
+/* VMath::transpose_bin, vmath.cu:9487-9510: py[nrow, ncol] = px[ncol, nrow]^T (not in place). */
+int kai_transpose_bin(int device, float* py, const float* px, int64_t nrow, int64_t ncol);
+
 /* ---- parameter update: the consumers of the weight and bias gradients (next to the path) ----------- */
 
 /* VMath::accumulate_grad, vmath.cu:364-382 (vmath.h:28).  py[n] += px[n]; sums the gradient shards of

@@ -78,6 +78,9 @@ public:
     static void mix_values_backward_value(int device, float* pV, float* pgy, float* pp, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece);
 
     /* additive: the `dense` layer formula activate(add(matmul(x,w),b)) (api/vconst.cpp:11) in one launch */
+    static void transpose(int device, float* py, float* px, int* pn, int64 axis_size, int64 data_size);
+    static void transpose_backward(int device, float* pgx, float* pgy, int* pn, int64 axis_size, int64 data_size);
+    static void transpose_bin(int device, float* py, float* px, int64 nrow, int64 ncol);
     static void accumulate_grad(int device, float* py, float* px, int64 nrow);
     static void subtract_param_grad(int device, float* pp, float* pg, int64 nrow, HYPER hLearningRate);
     static void apply_decay(int device, float* pd, float* pp, float* pg, int64 nrow, HYPER hL1Decay, HYPER hL2Decay);

@@ -494,3 +494,53 @@ int ko_eval_adam_delta(float* pa, const float* pg, float* ps, float* pt, float* 
     }
     return KO_OK;
 }
+
+/* ---- transposes (next to the path) ------------------------------------------------------------------ */
+
+int ko_transpose(float* py, const float* px, const int* pn, int64_t axis_size, int64_t data_size) {
+    /* vmath.cu:9384-9403.  pn[m*3] = source axis of output axis m, pn[m*3+1] = elements per step of output
+       axis m, pn[a*3+2] = elements per step of SOURCE axis a (vtensor.cpp:5399-5417) */
+    for (int64_t n = 0; n < data_size; n++) {
+        int64_t xpos = 0;
+        int64_t ypos = n;
+        int64_t cood;
+        for (int64_t m = 0; m < axis_size; m++) {
+            int64_t y_block_size = pn[m * 3 + 1];
+            int64_t x_block_size = pn[pn[m * 3] * 3 + 2];
+            cood = ypos / y_block_size;
+            ypos = ypos % y_block_size;
+            xpos += cood * x_block_size;
+        }
+        py[n] = px[xpos];
+    }
+    return KO_OK;
+}
+
+int ko_transpose_backward(float* pgx, const float* pgy, const int* pn, int64_t axis_size, int64_t data_size) {
+    /* vmath.cu:9436-9455 */
+    for (int64_t n = 0; n < data_size; n++) {
+        int64_t xpos = 0;
+        int64_t ypos = n;
+        int64_t cood;
+        for (int64_t m = 0; m < axis_size; m++) {
+            int64_t y_block_size = pn[m * 3 + 1];
+            int64_t x_block_size = pn[pn[m * 3] * 3 + 2];
+            cood = ypos / y_block_size;
+            ypos = ypos % y_block_size;
+            xpos += cood * x_block_size;
+        }
+        pgx[xpos] = pgy[n];
+    }
+    return KO_OK;
+}
+
+int ko_transpose_bin(float* py, const float* px, int64_t nrow, int64_t ncol) {
+    /* vmath.cu:9487-9494 */
+    for (int64_t nr = 0, n = 0; nr < nrow; nr++) {
+        for (int64_t nc = 0; nc < ncol; nc++, n++) {
+            int64_t xpos = nc * nrow + nr;
+            py[n] = px[xpos];
+        }
+    }
+    return KO_OK;
+}

@@ -103,6 +103,11 @@ int ko_apply_decay(float* pd, const float* pp, const float* pg, int64_t nrow, co
 int ko_eval_adam_delta(float* pa, const float* pg, float* ps, float* pt, float* pn, int64_t nrow, const float* hRo1,
                        const float* hRo2, const float* hEpsilon);
 
+/* vmath.cu:9384-9403, 9436-9455, 9487-9494 */
+int ko_transpose(float* py, const float* px, const int* pn, int64_t axis_size, int64_t data_size);
+int ko_transpose_backward(float* pgx, const float* pgy, const int* pn, int64_t axis_size, int64_t data_size);
+int ko_transpose_bin(float* py, const float* px, int64_t nrow, int64_t ncol);
+
 #ifdef __cplusplus
 }
 #endif

@@ -56,6 +56,9 @@ def lib():
             "ko_mix_values": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
             "ko_mix_values_backward_prop": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
             "ko_mix_values_backward_value": [_F, _F, _F, _I64, _I64, _I64, _I64, _I64],
+            "ko_transpose": [_F, _F, ctypes.c_void_p, _I64, _I64],
+            "ko_transpose_backward": [_F, _F, ctypes.c_void_p, _I64, _I64],
+            "ko_transpose_bin": [_F, _F, _I64, _I64],
             "ko_accumulate_grad": [_F, _F, _I64],
             "ko_subtract_param_grad": [_F, _F, _I64, _F],
             "ko_apply_decay": [_F, _F, _F, _I64, _F, _F],
@@ -297,3 +300,41 @@ def eval_adam_delta(g, s, t, n, ro1, ro2, epsilon):
     k3, h3 = _hyper(epsilon)
     _check(lib().ko_eval_adam_delta(_p(a), _p(g), _p(s), _p(t), _p(n), g.size, h1, h2, h3))
     return a, s, t, n
+
+
+def transpose_axinfo(shape, axes):
+    """The [axis_size, 3] int32 table VTensor::transpose builds (vtensor.cpp:5391-5417): per output axis n the
+    source axis, the output elements per step of axis n, and the SOURCE elements per step of source axis n."""
+    shape = [int(v) for v in shape]
+    total = int(np.prod(shape))
+    rest, prod = total, total
+    info = np.zeros((len(shape), 3), np.int32)
+    for n, axis in enumerate(axes):
+        rest //= shape[axis]
+        prod //= shape[n]
+        info[n] = (axis, rest, prod)
+    return info
+
+
+def transpose(x, axes):
+    x = _f32(x)
+    info = transpose_axinfo(x.shape, axes)
+    y = np.zeros([x.shape[a] for a in axes], np.float32)
+    _check(lib().ko_transpose(_p(y), _p(x), info.ctypes.data, x.ndim, x.size))
+    return y
+
+
+def transpose_backward(gy, xshape, axes):
+    gy = _f32(gy)
+    info = transpose_axinfo(xshape, axes)
+    gx = np.zeros(xshape, np.float32)
+    _check(lib().ko_transpose_backward(_p(gx), _p(gy), info.ctypes.data, len(xshape), gy.size))
+    return gx
+
+
+def transpose_bin(x, nrow, ncol):
+    """x is [ncol, nrow]; returns [nrow, ncol]."""
+    x = _f32(x)
+    y = np.zeros((nrow, ncol), np.float32)
+    _check(lib().ko_transpose_bin(_p(y), _p(x), nrow, ncol))
+    return y

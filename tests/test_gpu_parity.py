@@ -532,6 +532,32 @@ def test_split_k_scratch_survives_shutdown_and_growth():
         check(y.to_numpy((m, n))[rows], ko.matmul_rows(w, x, rows), what="split-K %dx%dx%d" % (m, n, k))
 
 
+# ---- transposes ---------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape,axes", [((5,), (0,)), ((33, 70), (1, 0)), ((2, 3, 4), (2, 0, 1)), ((4, 512, 8, 64), (0, 2, 1, 3)),
+                                        ((3, 1, 5, 2), (3, 2, 1, 0)), ((2, 2, 2, 2, 3, 2, 2, 5), (7, 0, 6, 1, 5, 2, 4, 3))])
+def test_transpose_axes(shape, axes):
+    rng = np.random.default_rng(len(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    info = DB.from_numpy(ko.transpose_axinfo(shape, axes))            # raw int32 table, as the engine holds it
+    y = DB(x.size * 4)
+    VMath.transpose(0, y, dev(x), info, len(shape), x.size)
+    yshape = [shape[a] for a in axes]
+    np.testing.assert_array_equal(y.to_numpy(yshape), ko.transpose(x, axes))
+    gy = rng.standard_normal(yshape).astype(np.float32)
+    gx = DB(x.size * 4)
+    VMath.transpose_backward(0, gx, dev(gy), info, len(shape), x.size)
+    np.testing.assert_array_equal(gx.to_numpy(shape), ko.transpose_backward(gy, shape, axes))
+
+
+@pytest.mark.parametrize("nrow,ncol", [(1, 1), (32, 32), (33, 31), (5, 1000), (1000, 5), (1024, 4096)])
+def test_transpose_bin(nrow, ncol):
+    x = np.random.default_rng(nrow + ncol).standard_normal((ncol, nrow)).astype(np.float32)
+    y = DB(x.size * 4)
+    VMath.transpose_bin(0, y, dev(x), nrow, ncol)
+    np.testing.assert_array_equal(y.to_numpy((nrow, ncol)), ko.transpose_bin(x, nrow, ncol))
+
+
 # ---- parameter update: accumulate_grad, subtract_param_grad, apply_decay, eval_adam_delta ------------------------------
 
 @pytest.mark.parametrize("n", [1, 7, 1024, 4099, 1 << 20])

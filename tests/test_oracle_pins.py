@@ -333,3 +333,19 @@ def test_adam_first_step_closed_form_and_float64_recurrence():
         want = (s64 / (1 - ro1 ** step)) / (np.sqrt(t64 / (1 - ro2 ** step)) + eps)
         np.testing.assert_allclose(a, want, rtol=2e-5, atol=1e-6)
         np.testing.assert_array_equal(n, np.full(500, step, np.float32))
+
+
+# ---- transposes (vmath.cu:9384-9510) --------------------------------------------------------------------------------
+
+def test_transposes_equal_numpy():
+    rng = np.random.default_rng(8)
+    for shape, axes in [((5,), (0,)), ((3, 7), (1, 0)), ((2, 3, 4), (2, 0, 1)), ((2, 3, 4), (0, 2, 1)),
+                        ((3, 1, 5, 2), (3, 2, 1, 0)), ((4, 3, 2, 5), (0, 1, 2, 3))]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        y = ko.transpose(x, axes)
+        np.testing.assert_array_equal(y, np.transpose(x, axes))
+        # the backward pass scatters a gradient of y's shape back to x's positions: the inverse permutation
+        gy = rng.standard_normal(y.shape).astype(np.float32)
+        np.testing.assert_array_equal(ko.transpose_backward(gy, shape, axes), np.transpose(gy, np.argsort(axes)))
+    x = rng.standard_normal((37, 53)).astype(np.float32)            # [ncol, nrow]
+    np.testing.assert_array_equal(ko.transpose_bin(x, 53, 37), x.T)
