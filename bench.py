@@ -172,6 +172,27 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
             gpu_us(lambda: L.kai_attention_forward(0, P(o), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
                                                    P(coef), 0)),
             flops=2 * fl)
+        # the backward calls of the same block (vtensor.cpp:3142-3166 of the reference)
+        go = torch.randn((nbat, T, nvec), device=dev, generator=g)
+        gp = torch.empty_like(s0)
+        gv = torch.empty_like(v)
+        gq = torch.empty_like(q)
+        goc = go.cpu().numpy() if with_cpu else None
+        row(tag + "gP = gO.V^T (mix_values_backward_prop)",
+            gpu_us(lambda: L.kai_mix_values_backward_prop(0, P(gp), P(go), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))),
+            flops=fl, cpu=cpu_us(lambda: ko.mix_values_backward_prop(goc, vc, nhead)))
+        row(tag + "gV = P^T.gO (mix_values_backward_value)",
+            gpu_us(lambda: L.kai_mix_values_backward_value(0, P(gv), P(go), P(pbuf), I(nbat), I(T), I(nvec), I(nhead), I(D))),
+            flops=fl, cpu=cpu_us(lambda: ko.mix_values_backward_value(goc, pbuf.cpu().numpy(), nhead)))
+        gp0 = gp.clone()
+        row(tag + "softmax_direct_on_axis_backward (in place)",
+            gpu_us(lambda: L.kai_softmax_direct_on_axis_backward(0, P(gp), P(pbuf), I(nbat), I(T), I(nhead), P(coef)),
+                   iters=20, prep=lambda: gp.copy_(gp0)),
+            nbytes=12.0 * 32 * T * T,
+            cpu=cpu_us(lambda: ko.softmax_direct_on_axis_backward(gp0.cpu().numpy(), pbuf.cpu().numpy(), 0.125)))
+        row(tag + "gQ = gS.K (mult_on_heads_backward)",
+            gpu_us(lambda: L.kai_mult_on_heads_backward(0, P(gq), P(gp), P(k), I(nbat), I(T), I(nvec), I(nhead), I(D))),
+            flops=fl, cpu=cpu_us(lambda: ko.mult_on_heads_backward(gp.cpu().numpy(), kc, nhead)))
     # cfg5: skinny (cold: six rotating weight buffers) and ragged
     K = N = 4096
     ws = [torch.rand((N, K), device=dev, generator=g) * 0.1 - 0.05 for _ in range(6)]
