@@ -217,6 +217,33 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
     xc, wc = x.cpu().numpy(), w.cpu().numpy()
     row("cfg5 ragged 1000x777x333", gpu_us(lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0)),
         flops=2.0 * m * n * k, cpu=cpu_us(lambda: ko.matmul(wc, xc)))
+    # one LSTM layer forward as the engine's loop issues it (vtensor.cpp:2455-2492): 32 steps of 64 x 256 -> 4 x 256
+    nt_, nd_, ni_, nr_ = 32, 64, 256, 256
+    xs = torch.randn((nt_, nd_, ni_), device=dev, generator=g)
+    wi = torch.randn((4 * nr_, ni_), device=dev, generator=g) / 32
+    wr = torch.randn((4 * nr_, nr_), device=dev, generator=g) / 32
+    bi = torch.zeros(4 * nr_, device=dev)
+    aff = torch.zeros((nt_, nd_, 4 * nr_), device=dev)
+    rec = torch.zeros((nt_, nd_, nr_), device=dev)
+    sta = torch.zeros((nt_, nd_, nr_), device=dev)
+
+    def lstm_layer(batched):
+        L.kai_set_zero(0, P(aff), I(aff.numel() * 4))
+        if batched:
+            L.kai_matmul(0, P(aff), P(wi), P(xs), I(4 * nr_), I(nt_ * nd_), I(ni_), 0)
+        for t in range(nt_):
+            if t > 0:
+                L.kai_matmul(0, P(aff[t]), P(wr), P(rec[t - 1]), I(4 * nr_), I(nd_), I(nr_), int(batched))
+            if not batched:
+                L.kai_matmul(0, P(aff[t]), P(wi), P(xs[t]), I(4 * nr_), I(nd_), I(ni_), 1)
+            L.kai_add_bias(0, P(aff[t]), P(aff[t]), P(bi), I(nd_), I(4 * nr_))
+            L.kai_lstm_process(0, P(rec[t]), P(sta[t]), P(sta[t - 1]) if t > 0 else None, P(aff[t]), I(nd_), I(nr_), I(ni_))
+
+    lstm_flops = 2.0 * nt_ * nd_ * 4 * nr_ * (ni_ + nr_)
+    row("lstm layer forward, 32 steps x (64 x 256 -> 4 x 256), per-step calls", gpu_us(lambda: lstm_layer(False), iters=10),
+        flops=lstm_flops)
+    row("lstm layer forward, same, input products of all steps in one call", gpu_us(lambda: lstm_layer(True), iters=10),
+        flops=lstm_flops)
     # transposes next to the path: the head split [4,512,8,64] -> [4,8,512,64] of configuration 4 and a plain 4096^2
     shape, axes = (4, 512, 8, 64), (0, 2, 1, 3)
     x = torch.randn(shape, device=dev, generator=g)

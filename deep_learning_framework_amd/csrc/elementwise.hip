@@ -425,6 +425,117 @@ int launch_eval_adam_delta(float* a, const float* g, float* s, float* t, float* 
     return check_launch("adam_delta_kernel");
 }
 
+// ---- recurrent cells: what runs between the gate products of an RNN / LSTM / GRU step -------------------
+//
+// One thread per (row, unit); the gate pre-activations of a row lie nrec apart, so neighbouring threads
+// read neighbouring floats of every gate.
+
+__global__ void __launch_bounds__(kEwThreads) add_kernel(float* y, const float* a, const float* b, int64_t n) {
+    // y may alias a or b (the engine adds in place)
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) y[i] = a[i] + b[i];
+}
+
+int launch_add(float* y, const float* a, const float* b, int64_t n, hipStream_t stream) {
+    if (n <= 0) return KAI_OK;
+    add_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(y, a, b, n);
+    return check_launch("add_kernel");
+}
+
+__global__ void __launch_bounds__(kEwThreads)
+    lstm_process_kernel(float* __restrict__ r, float* s, const float* s1, const float* __restrict__ a, int64_t n,
+                        int64_t nrec) {
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        const int64_t nd = i / nrec, nr = i - nd * nrec;
+        const float* g = a + nd * 4 * nrec + nr;
+        const float state = s1 ? s1[i] : 0.f;
+        const float input_gate = act_sigmoid(g[0]);
+        const float forget_gate = act_sigmoid(g[nrec]);
+        const float input_block = act_tanh(g[2 * nrec]);
+        const float output_gate = act_sigmoid(g[3 * nrec]);
+        const float new_state = state * forget_gate + input_block * input_gate;
+        s[i] = new_state;
+        r[i] = act_tanh(new_state) * output_gate;
+    }
+}
+
+int launch_lstm_process(float* r, float* s, const float* s1, const float* a, int64_t ndat, int64_t nrec,
+                        hipStream_t stream) {
+    const int64_t n = ndat * nrec;
+    if (n <= 0) return KAI_OK;
+    lstm_process_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(r, s, s1, a, n, nrec);
+    return check_launch("lstm_process_kernel");
+}
+
+struct GruGates {
+    float Rt, Zt, Nt, Ht_1, par_n;
+};
+
+__device__ __forceinline__ GruGates gru_gates(const float* r, const float* ai, const float* ar, int64_t i, int64_t nt,
+                                              int64_t n, int64_t nrec, int64_t& gpos) {
+    const int64_t nd = i / nrec, ny = i - nd * nrec;
+    gpos = nd * 3 * nrec + ny;
+    GruGates g;
+    g.Rt = act_sigmoid(ai[gpos] + ar[gpos]);
+    g.Zt = act_sigmoid(ai[gpos + nrec] + ar[gpos + nrec]);
+    g.par_n = ar[gpos + 2 * nrec];
+    g.Nt = act_tanh(ai[gpos + 2 * nrec] + g.Rt * g.par_n);
+    g.Ht_1 = nt > 0 ? r[i - n] : 0.f;      // the previous time step lies one [ndat, nrec] block before r
+    return g;
+}
+
+__global__ void __launch_bounds__(kEwThreads)
+    gru_process_kernel(float* r, const float* __restrict__ ai, const float* __restrict__ ar, int64_t nt, int64_t n,
+                       int64_t nrec) {
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        int64_t gpos;
+        const GruGates g = gru_gates(r, ai, ar, i, nt, n, nrec, gpos);
+        r[i] = (1.0f - g.Zt) * g.Nt + g.Zt * g.Ht_1;
+    }
+}
+
+__global__ void __launch_bounds__(kEwThreads)
+    gru_process_backward_kernel(float* gr, float* __restrict__ gai, float* __restrict__ gar, const float* r,
+                                const float* __restrict__ ai, const float* __restrict__ ar, int64_t nt, int64_t n,
+                                int64_t nrec) {
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        int64_t gpos;
+        const GruGates g = gru_gates(r, ai, ar, i, nt, n, nrec, gpos);
+        const float gHt = gr[i];
+        const float gNt = (1 - g.Zt) * gHt;
+        const float gZt = (g.Ht_1 - g.Nt) * gHt;
+        const float gNt_seed = (1 + g.Nt) * (1 - g.Nt) * gNt;
+        const float gRt = g.par_n * gNt_seed;
+        const float dr = g.Rt * (1 - g.Rt) * gRt, dz = g.Zt * (1 - g.Zt) * gZt;
+        gai[gpos] = dr;
+        gar[gpos] = dr;
+        gai[gpos + nrec] = dz;
+        gar[gpos + nrec] = dz;
+        gai[gpos + 2 * nrec] = gNt_seed;
+        gar[gpos + 2 * nrec] = g.Rt * gNt_seed;
+        gr[i] = g.Zt * gHt;
+    }
+}
+
+int launch_gru_process(float* r, const float* ai, const float* ar, int64_t nt, int64_t ndat, int64_t nrec,
+                       hipStream_t stream) {
+    const int64_t n = ndat * nrec;
+    if (n <= 0) return KAI_OK;
+    gru_process_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(r, ai, ar, nt, n, nrec);
+    return check_launch("gru_process_kernel");
+}
+
+int launch_gru_process_backward(float* gr, float* gai, float* gar, const float* r, const float* ai, const float* ar,
+                                int64_t nt, int64_t ndat, int64_t nrec, hipStream_t stream) {
+    const int64_t n = ndat * nrec;
+    if (n <= 0) return KAI_OK;
+    gru_process_backward_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(gr, gai, gar, r, ai, ar, nt, n, nrec);
+    return check_launch("gru_process_backward_kernel");
+}
+
 // ---- split-K final pass ---------------------------------------------------------------------
 //
 // Sums the partial products in split order (fixed, so the result does not depend on scheduling)

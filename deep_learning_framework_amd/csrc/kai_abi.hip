@@ -549,6 +549,57 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
     return KAI_OK;
 }
 
+// ---- recurrent cells: the element-wise steps between the gate products -----------------------------
+
+int kai_copy(int device, float* py, const float* pa, int64_t ndat) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (ndat == 0 || py == pa) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pa);
+    // in stream order, like the reference's copy kernel
+    const hipError_t e = hipMemcpyAsync(py, pa, (size_t)ndat * sizeof(float), hipMemcpyDeviceToDevice, current_stream());
+    if (e != hipSuccess) return fail(KAI_ERR_GPU, std::string("copy: ") + hipGetErrorString(e));
+    return KAI_OK;
+}
+
+int kai_add(int device, float* py, const float* pa, const float* pb, int64_t ndat) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    if (ndat == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pa); KAI_REQUIRE_PTR(pb);
+    return launch_add(py, pa, pb, ndat, current_stream());
+}
+
+int kai_lstm_process(int device, float* pr, float* ps, const float* ps1, const float* pa, int64_t ndat, int64_t nrec,
+                     int64_t ninp) {
+    (void)ninp;   // carried by the reference's signature, not used by its loops either
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0 && nrec >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (ndat == 0 || nrec == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pr); KAI_REQUIRE_PTR(ps); KAI_REQUIRE_PTR(pa);
+    return launch_lstm_process(pr, ps, ps1, pa, ndat, nrec, current_stream());
+}
+
+int kai_gru_process(int device, float* pr, const float* pai, const float* par, int64_t nt, int64_t ntimes, int64_t ndat,
+                    int64_t nrec) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0 && nrec >= 0 && nt >= 0 && nt < ntimes, KAI_ERR_INVALID_ARGUMENT, "bad time step or dimension");
+    if (ndat == 0 || nrec == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pr); KAI_REQUIRE_PTR(pai); KAI_REQUIRE_PTR(par);
+    return launch_gru_process(pr, pai, par, nt, ndat, nrec, current_stream());
+}
+
+int kai_gru_process_backward(int device, float* pgr, float* pgai, float* pgar, const float* pr, const float* pai,
+                             const float* par, int64_t nt, int64_t ntimes, int64_t ndat, int64_t nrec) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0 && nrec >= 0 && nt >= 0 && nt < ntimes, KAI_ERR_INVALID_ARGUMENT, "bad time step or dimension");
+    if (ndat == 0 || nrec == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgr); KAI_REQUIRE_PTR(pgai); KAI_REQUIRE_PTR(pgar);
+    KAI_REQUIRE_PTR(pr); KAI_REQUIRE_PTR(pai); KAI_REQUIRE_PTR(par);
+    KAI_REQUIRE(pgai != pgar, KAI_ERR_INVALID_ARGUMENT, "gru_process_backward needs separate gate gradient buffers");
+    return launch_gru_process_backward(pgr, pgai, pgar, pr, pai, par, nt, ndat, nrec, current_stream());
+}
+
 // ---- transposes ----------------------------------------------------------------------------------
 
 int kai_transpose(int device, float* py, const float* px, const int* pn, int64_t axis_size, int64_t data_size) {

@@ -82,6 +82,18 @@ void VMath::mix_values_backward_value(int device, float* pgV, float* pgy, float*
     raise_on(kai_mix_values_backward_value(device, pgV, pgy, pp, nbat, ntimes, nvec, nhead, npiece));
 }
 
+void VMath::copy(int device, float* py, float* pa, int64 ndat) { raise_on(kai_copy(device, py, pa, ndat)); }
+void VMath::add(int device, float* py, float* pa, float* pb, int64 ndat) { raise_on(kai_add(device, py, pa, pb, ndat)); }
+void VMath::lstm_process(int device, float* pr, float* ps, float* ps1, float* pa, int64 ndat, int64 nrec, int64 ninp) {
+    raise_on(kai_lstm_process(device, pr, ps, ps1, pa, ndat, nrec, ninp));
+}
+void VMath::gru_process(int device, float* pr, float* pai, float* par, int64 nt, int64 ntimes, int64 ndat, int64 nrec) {
+    raise_on(kai_gru_process(device, pr, pai, par, nt, ntimes, ndat, nrec));
+}
+void VMath::gru_process_backward(int device, float* pgr, float* pgai, float* pgar, float* pr, float* pai, float* par,
+                                 int64 nt, int64 ntimes, int64 ndat, int64 nrec) {
+    raise_on(kai_gru_process_backward(device, pgr, pgai, pgar, pr, pai, par, nt, ntimes, ndat, nrec));
+}
 void VMath::transpose(int device, float* py, float* px, int* pn, int64 axis_size, int64 data_size) {
     raise_on(kai_transpose(device, py, px, pn, axis_size, data_size));
 }

@@ -62,6 +62,11 @@ SIGNATURES = {
     "kai_gemm_f32": [_INT, _INT, _INT, _I64, _I64, _I64, _F, _I64, _F, _I64, _F, _I64, _F, _INT, _F, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
     "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
+    "kai_copy": [_INT, _F, _F, _I64],
+    "kai_add": [_INT, _F, _F, _F, _I64],
+    "kai_lstm_process": [_INT, _F, _F, _F, _F, _I64, _I64, _I64],
+    "kai_gru_process": [_INT, _F, _F, _F, _I64, _I64, _I64, _I64],
+    "kai_gru_process_backward": [_INT, _F, _F, _F, _F, _F, _F, _I64, _I64, _I64, _I64],
     "kai_transpose": [_INT, _F, _F, _F, _I64, _I64],
     "kai_transpose_backward": [_INT, _F, _F, _F, _I64, _I64],
     "kai_transpose_bin": [_INT, _F, _F, _I64, _I64],
@@ -303,6 +308,27 @@ class VMath:
     def gemm_f32(device, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, bias, actFunc, hLeakyAlpha, acc):
         _ck(load().kai_gemm_f32(device, int(transA), int(transB), M, N, K, _addr(A), lda, _addr(B), ldb, _addr(C),
                                 ldc, _addr(bias), actFunc, _addr(hLeakyAlpha), int(acc)))
+
+    @staticmethod
+    def copy(device, py, pa, ndat):
+        _ck(load().kai_copy(device, _addr(py), _addr(pa), ndat))
+
+    @staticmethod
+    def add(device, py, pa, pb, ndat):
+        _ck(load().kai_add(device, _addr(py), _addr(pa), _addr(pb), ndat))
+
+    @staticmethod
+    def lstm_process(device, pr, ps, ps1, pa, ndat, nrec, ninp):
+        _ck(load().kai_lstm_process(device, _addr(pr), _addr(ps), _addr(ps1), _addr(pa), ndat, nrec, ninp))
+
+    @staticmethod
+    def gru_process(device, pr, pai, par, nt, ntimes, ndat, nrec):
+        _ck(load().kai_gru_process(device, _addr(pr), _addr(pai), _addr(par), nt, ntimes, ndat, nrec))
+
+    @staticmethod
+    def gru_process_backward(device, pgr, pgai, pgar, pr, pai, par, nt, ntimes, ndat, nrec):
+        _ck(load().kai_gru_process_backward(device, _addr(pgr), _addr(pgai), _addr(pgar), _addr(pr), _addr(pai),
+                                            _addr(par), nt, ntimes, ndat, nrec))
 
     @staticmethod
     def transpose(device, py, px, pn, axis_size, data_size):

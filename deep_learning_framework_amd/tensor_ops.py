@@ -8,6 +8,7 @@ lists exactly as the reference's ``VTensor`` methods do and issue the same seque
 * ``add`` / ``add_backprop``         -- api_objects/vtensor.cpp:3395-3485
 * ``activate`` / ``activate_backprop`` -- api_objects/vtensor.cpp:5674-5718
 * ``mh_attention`` / ``mh_attention_backprop`` -- api_objects/vtensor.cpp:2978-3227
+* ``rnn`` / ``rnn_backprop`` (module level)  -- api_objects/vtensor.cpp:2350-2522, 2524-2717
 
 Shape errors raise ``KaiError`` with the reference's codes (VERR_BAD_SHAPE_TENSOR = 10003).
 The graph, autograd queue and tracer of the engine are not rebuilt: backprop methods
@@ -234,3 +235,147 @@ def dense(x, w, b, actfunc="relu", leaky_alpha=None, fused=True, keep_pre=False)
     VMath.dense_forward(x.device, y.ptr, pre.ptr if pre else None, w.ptr, b.ptr if b is not None else None, x.ptr,
                         yvec, ndat, xvec, code, h)
     return y, pre
+
+
+# ---- recurrent layers: vtensor.cpp:2350-2522 (m_rnn) and 2524-2717 (m_rnn_backprop) ----------------------
+
+VERR_SHAPE_RNN = 1307
+_NGATES = {"rnn": 1, "lstm": 4, "gru": 3}
+
+
+def rnn(x, wi, wr, bi, br, cell_type, rec_size, actfunc="tanh", leaky_alpha=None, forward=True, timesteps=None,
+        use_state=False, batch_input_projection=False):
+    """One direction of a recurrent layer, as the engine's per-time-step loop issues it.
+
+    ``x`` is ``[ntimes, ndat, ninp]`` (a sequence) or ``[ndat, ninp]`` (the same input at each of ``timesteps``
+    steps); ``wi [ngates*nrec, ninp]``, ``wr [ngates*nrec, nrec]``, ``bi``/``br`` ``[ngates*nrec]`` or None.
+    Per step: the recurrent gate product with acc = 0, the input gate product with acc = 1 (rnn and lstm keep
+    both in one buffer), the bias adds, then the cell.  ``batch_input_projection=True`` is the additive fusion:
+    the input products of all steps are issued as ONE call over ``ntimes*ndat`` rows before the loop and the
+    recurrent product accumulates onto it, which gives the same sums (a + b == b + a).
+    Returns the ``[ndat, nrec]`` output and the tensors the backward pass needs."""
+    if cell_type not in _NGATES:
+        raise KaiError(8, "rnn cell type")
+    ngates = _NGATES[cell_type]
+    nrec = int(rec_size)
+    in_seq = len(x.shape) == 3
+    if len(wi.shape) != 2 or len(wr.shape) != 2:
+        raise KaiError(VERR_SHAPE_RNN, "rnn")
+    ntimes = x.shape[0] if in_seq else int(timesteps)
+    ndat = x.shape[1] if in_seq else x.shape[0]
+    ninp = x.shape[-1]
+    if wi.shape != (ngates * nrec, ninp) or wr.shape != (ngates * nrec, nrec):
+        raise KaiError(VERR_SHAPE_RNN, "rnn")
+    use_bias = bi is not None
+    if use_bias and (bi.shape != (ngates * nrec,) or br.shape != (ngates * nrec,)):
+        raise KaiError(VERR_SHAPE_RNN, "rnn")
+    dev = x.device
+    code = ACT[actfunc] if isinstance(actfunc, str) else int(actfunc)
+    halpha = kai.hyper(leaky_alpha, dev)
+    recurs = Tensor((ntimes, ndat, nrec), dev)
+    iaffines = Tensor((ntimes, ndat, ngates * nrec), dev)
+    raffines = iaffines
+    VMath.set_zero(dev, recurs.ptr, recurs.total_size() * 4)
+    VMath.set_zero(dev, iaffines.ptr, iaffines.total_size() * 4)
+    if cell_type == "gru":
+        raffines = Tensor((ntimes, ndat, ngates * nrec), dev)
+        VMath.set_zero(dev, raffines.ptr, raffines.total_size() * 4)
+    states = None
+    if cell_type == "lstm":
+        states = Tensor((ntimes, ndat, nrec), dev)
+        VMath.set_zero(dev, states.ptr, states.total_size() * 4)
+    xsize, ysize = ndat * ninp, ndat * nrec
+    asize = ngates * ysize
+    f4 = 4
+    batched = batch_input_projection and in_seq
+    if batched:
+        VMath.matmul(dev, iaffines.ptr, wi.ptr, x.ptr, ngates * nrec, ntimes * ndat, ninp, False)
+    for n in range(ntimes):
+        nt = n if forward else ntimes - n - 1
+        pr = recurs.buf.offset(nt * ysize * f4)
+        pai = iaffines.buf.offset(nt * asize * f4)
+        par = raffines.buf.offset(nt * asize * f4)
+        px = x.buf.offset(nt * xsize * f4) if in_seq else x.ptr
+        if n > 0:
+            pr_prev = recurs.buf.offset((nt - 1 if forward else nt + 1) * ysize * f4)
+            # with the input products already in place the recurrent one accumulates (rnn, lstm: same buffer)
+            VMath.matmul(dev, par, wr.ptr, pr_prev, ngates * nrec, ndat, nrec, batched and raffines is iaffines)
+        if not batched:
+            VMath.matmul(dev, pai, wi.ptr, px, ngates * nrec, ndat, ninp, True)
+        if use_bias:
+            VMath.add_bias(dev, par, par, br.ptr, ndat, ngates * nrec)
+            VMath.add_bias(dev, pai, pai, bi.ptr, ndat, ngates * nrec)
+        if cell_type == "rnn":
+            VMath.copy(dev, pr, pai, ysize)
+            VMath.add(dev, pr, pr, pai, ysize)
+            VMath.activate(dev, pr, pr, ndat, nrec, code, halpha)
+        elif cell_type == "lstm":
+            ps = states.buf.offset(nt * ysize * f4)
+            ps_prev = states.buf.offset((nt - 1 if forward else nt + 1) * ysize * f4) if n > 0 else None
+            VMath.lstm_process(dev, pr, ps, ps_prev, pai, ndat, nrec, ninp)
+        else:
+            VMath.gru_process(dev, pr, pai, par, nt, ntimes, ndat, nrec)
+    y = Tensor((ndat, nrec), dev)
+    src = states if (use_state and states is not None) else recurs
+    VMath.copy(dev, y.ptr, src.buf.offset(((ntimes - 1) if forward else 0) * ysize * f4), ysize)
+    saved = {"cell_type": cell_type, "forward": forward, "x": x, "wi": wi, "wr": wr, "use_bias": use_bias,
+             "recurs": recurs, "iaffines": iaffines, "raffines": raffines, "states": states, "actfunc": code,
+             "leaky_alpha": halpha, "ngates": ngates}
+    return y, saved
+
+
+def rnn_backprop(saved, ygrad, ytgrad):
+    """vtensor.cpp:2524-2717 for the rnn and gru cells.  ``ygrad [ndat, nrec]`` is used in place as the running
+    gradient of the recurrent output, as there; ``ytgrad [ntimes, ndat, nrec]`` is the per-step gradient.
+    Returns {x, wi, wr[, bi, br]} gradients.  The lstm cell has no backward here: the reference's
+    lstm_process_backward indexes outside its gate-gradient buffer (vmath.cu:4890-4893)."""
+    cell_type = saved["cell_type"]
+    if cell_type == "lstm":
+        raise KaiError(VERR_UNDEFINED, "lstm backward is not built")
+    forward, ngates = saved["forward"], saved["ngates"]
+    x, wi, wr = saved["x"], saved["wi"], saved["wr"]
+    recurs, iaffines, raffines = saved["recurs"], saved["iaffines"], saved["raffines"]
+    ntimes, ndat, nrec = ytgrad.shape
+    ninp = x.shape[-1]
+    in_seq = len(x.shape) == 3
+    dev = x.device
+    is_gru = cell_type == "gru"
+    xgrad, wigrad, wrgrad = Tensor(x.shape, dev), Tensor(wi.shape, dev), Tensor(wr.shape, dev)
+    aigrad = Tensor((ndat, ngates * nrec), dev)
+    for t in (xgrad, wigrad, wrgrad):
+        VMath.set_zero(dev, t.ptr, t.total_size() * 4)
+    argrad = aigrad
+    if is_gru:
+        argrad = Tensor((ndat, ngates * nrec), dev)
+        VMath.set_zero(dev, argrad.ptr, argrad.total_size() * 4)
+    out = {"x": xgrad, "wi": wigrad, "wr": wrgrad}
+    if saved["use_bias"]:
+        out["bi"], out["br"] = Tensor((ngates * nrec,), dev), Tensor((ngates * nrec,), dev)
+        VMath.set_zero(dev, out["bi"].ptr, ngates * nrec * 4)
+        VMath.set_zero(dev, out["br"].ptr, ngates * nrec * 4)
+    pgr = ygrad.ptr
+    xsize, ysize = ndat * ninp, ndat * nrec
+    asize = ngates * ysize
+    f4 = 4
+    for n in range(ntimes):
+        nt = ntimes - n - 1 if forward else n
+        pr = recurs.buf.offset(nt * ysize * f4)
+        pai = iaffines.buf.offset(nt * asize * f4)
+        par = raffines.buf.offset(nt * asize * f4)
+        px = x.buf.offset(nt * xsize * f4) if in_seq else x.ptr
+        pgx = xgrad.buf.offset(nt * xsize * f4) if in_seq else xgrad.ptr
+        VMath.add(dev, pgr, pgr, ytgrad.buf.offset(nt * ysize * f4), ysize)
+        if cell_type == "rnn":
+            VMath.activate_backward_with_y(dev, aigrad.ptr, pgr, pr, ndat, nrec, saved["actfunc"], saved["leaky_alpha"])
+        else:
+            VMath.gru_process_backward(dev, pgr, aigrad.ptr, argrad.ptr, pr, pai, par, nt, ntimes, ndat, nrec)
+        if saved["use_bias"]:
+            VMath.add_bias_backward_b(dev, out["bi"].ptr, aigrad.ptr, ndat, ngates * nrec, True)
+            VMath.add_bias_backward_b(dev, out["br"].ptr, argrad.ptr, ndat, ngates * nrec, True)
+        VMath.matmul_backward_w(dev, wigrad.ptr, aigrad.ptr, px, ngates * nrec, ndat, ninp, True)
+        if n < ntimes - 1:
+            pr_prev = recurs.buf.offset((nt - 1 if forward else nt + 1) * ysize * f4)
+            VMath.matmul_backward_w(dev, wrgrad.ptr, argrad.ptr, pr_prev, ngates * nrec, ndat, nrec, True)
+        VMath.matmul_backward_x(dev, pgx, aigrad.ptr, wi.ptr, ngates * nrec, ndat, ninp, False)
+        VMath.matmul_backward_x(dev, pgr, argrad.ptr, wr.ptr, ngates * nrec, ndat, nrec, is_gru)
+    return out

@@ -194,6 +194,28 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
                        const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
                        int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc);
 
+/* ---- recurrent layers (next to the path): the steps between the gate products ---------------------- */
+/* VTensor's rnn/lstm/gru loop (vtensor.cpp:2455-2492, 2657-2701) issues, per time step, kai_matmul with
+ * acc = 0 and 1 on sub-buffers at t * size offsets, kai_add_bias in place, and the calls below. */
+
+/* VMath::copy, vmath.cu:732-752.  py[n] = pa[n], in stream order. */
+int kai_copy(int device, float* py, const float* pa, int64_t ndat);
+/* VMath::add, vmath.cu:774-794.  py[n] = pa[n] + pb[n]; py may be pa or pb. */
+int kai_add(int device, float* py, const float* pa, const float* pb, int64_t ndat);
+/* VMath::lstm_process, vmath.cu:4807-4857.  pa[ndat, 4*nrec] holds the pre-activations of the input, forget,
+ * block and output gates; ps = ps1 * f + g * i (ps1 null: 0), pr = tanh(ps) * o.  ninp is unused, as there. */
+int kai_lstm_process(int device, float* pr, float* ps, const float* ps1, const float* pa, int64_t ndat, int64_t nrec,
+                     int64_t ninp);
+/* VMath::gru_process, vmath.cu:4946-4996.  pr points at step nt of [ntimes, ndat, nrec] and the previous step is
+ * read ndat*nrec floats before it when nt > 0; pai/par[ndat, 3*nrec]: reset, update, candidate. */
+int kai_gru_process(int device, float* pr, const float* pai, const float* par, int64_t nt, int64_t ntimes, int64_t ndat,
+                    int64_t nrec);
+/* VMath::gru_process_backward, vmath.cu:4999-5080.  pgr is replaced by the gradient of the previous step's output.
+ * VMath::lstm_process_backward (vmath.cu:4860-4943) has no counterpart: its gate-gradient index expression
+ * (apos * g + n * nrec) leaves the [ndat, 4*nrec] buffer for nrec > 4. */
+int kai_gru_process_backward(int device, float* pgr, float* pgai, float* pgar, const float* pr, const float* pai,
+                             const float* par, int64_t nt, int64_t ntimes, int64_t ndat, int64_t nrec);
+
 /* ---- transposes (next to the path) ----------------------------------------------------------------- */
 
 /* VMath::transpose, vmath.cu:9384-9433 (vmath.h:309).  General axis permutation of a dense tensor of

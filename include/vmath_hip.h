@@ -78,6 +78,12 @@ public:
     static void mix_values_backward_value(int device, float* pV, float* pgy, float* pp, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece);
 
     /* additive: the `dense` layer formula activate(add(matmul(x,w),b)) (api/vconst.cpp:11) in one launch */
+    static void copy(int device, float* py, float* pa, int64 ndat);
+    static void add(int device, float* py, float* pa, float* pb, int64 ndat);
+    static void lstm_process(int device, float* pr, float* ps, float* ps1, float* pa, int64 ndat, int64 nrec, int64 ninp);
+    static void gru_process(int device, float* pr, float* pai, float* par, int64 nt, int64 ntimes, int64 ndat, int64 nrec);
+    static void gru_process_backward(int device, float* pgr, float* pgai, float* pgar, float* pr, float* pai, float* par,
+                                     int64 nt, int64 ntimes, int64 ndat, int64 nrec);
     static void transpose(int device, float* py, float* px, int* pn, int64 axis_size, int64 data_size);
     static void transpose_backward(int device, float* pgx, float* pgy, int* pn, int64 axis_size, int64 data_size);
     static void transpose_bin(int device, float* py, float* px, int64 nrow, int64 ncol);

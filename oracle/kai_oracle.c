@@ -544,3 +544,84 @@ int ko_transpose_bin(float* py, const float* px, int64_t nrow, int64_t ncol) {
     }
     return KO_OK;
 }
+
+/* ---- recurrent cells: what runs between the gate products of an RNN/LSTM/GRU step ----------- */
+
+int ko_copy(float* py, const float* pa, int64_t ndat) {
+    /* vmath.cu:732-736 */
+    for (int64_t n = 0; n < ndat; n++) py[n] = pa[n];
+    return KO_OK;
+}
+
+int ko_add(float* py, const float* pa, const float* pb, int64_t ndat) {
+    /* vmath.cu:774-778 */
+    for (int64_t nd = 0; nd < ndat; nd++) py[nd] = pa[nd] + pb[nd];
+    return KO_OK;
+}
+
+int ko_lstm_process(float* pr, float* ps, const float* ps1, const float* pa, int64_t ndat, int64_t nrec) {
+    /* vmath.cu:4807-4826; gate order in pa[ndat, 4*nrec]: input, forget, block, output */
+    for (int64_t nd = 0, n = 0; nd < ndat; nd++) {
+        for (int64_t nr = 0; nr < nrec; nr++, n++) {
+            int64_t apos = nd * 4 * nrec + nr;
+            float state = ps1 ? ps1[n] : 0;
+            float input_gate = ko_sigmoid(pa[apos + 0 * nrec]);
+            float forget_gate = ko_sigmoid(pa[apos + 1 * nrec]);
+            float input_block = ko_tanh(pa[apos + 2 * nrec]);
+            float output_gate = ko_sigmoid(pa[apos + 3 * nrec]);
+            float new_state = state * forget_gate + input_block * input_gate;
+            float new_recur = ko_tanh(new_state) * output_gate;
+            ps[n] = new_state;
+            pr[n] = new_recur;
+        }
+    }
+    return KO_OK;
+}
+
+int ko_gru_process(float* pr, const float* pai, const float* par, int64_t nt, int64_t ndat, int64_t nrec) {
+    /* vmath.cu:4946-4965; pr points at time step nt of [ntimes, ndat, nrec], the previous step lies ndat*nrec
+     * floats before it; gate order in pai/par[ndat, 3*nrec]: reset, update, candidate */
+    for (int64_t nd = 0; nd < ndat; nd++) {
+        for (int64_t ny = 0; ny < nrec; ny++) {
+            int64_t rpos = nd * nrec + ny;
+            int64_t rgpos = nd * 3 * nrec + ny;
+            int64_t zgpos = nd * 3 * nrec + nrec + ny;
+            int64_t ngpos = nd * 3 * nrec + 2 * nrec + ny;
+            float Rt = ko_sigmoid(pai[rgpos] + par[rgpos]);
+            float Zt = ko_sigmoid(pai[zgpos] + par[zgpos]);
+            float Nt = ko_tanh(pai[ngpos] + Rt * par[ngpos]);
+            float Ht = (nt > 0) ? pr[rpos - ndat * nrec] : 0;
+            pr[rpos] = (1.0f - Zt) * Nt + Zt * Ht;
+        }
+    }
+    return KO_OK;
+}
+
+int ko_gru_process_backward(float* pgr, float* pgai, float* pgar, const float* pr, const float* pai,
+                            const float* par, int64_t nt, int64_t ndat, int64_t nrec) {
+    /* vmath.cu:4999-5033 */
+    for (int64_t nd = 0; nd < ndat; nd++) {
+        for (int64_t ny = 0; ny < nrec; ny++) {
+            int64_t rpos = nd * nrec + ny;
+            int64_t rgpos = nd * 3 * nrec + ny;
+            int64_t zgpos = nd * 3 * nrec + nrec + ny;
+            int64_t ngpos = nd * 3 * nrec + 2 * nrec + ny;
+            float Rt = ko_sigmoid(pai[rgpos] + par[rgpos]);
+            float Zt = ko_sigmoid(pai[zgpos] + par[zgpos]);
+            float Nt = ko_tanh(pai[ngpos] + Rt * par[ngpos]);
+            float Ht_1 = (nt > 0) ? pr[rpos - ndat * nrec] : 0;
+            float gHt = pgr[rpos];
+            float gNt = (1 - Zt) * gHt;
+            float gZt = (Ht_1 - Nt) * gHt;
+            float gHt_1 = Zt * gHt;
+            float gNt_seed = (1 + Nt) * (1 - Nt) * gNt;
+            float gRt = par[ngpos] * gNt_seed;
+            pgai[rgpos] = pgar[rgpos] = Rt * (1 - Rt) * gRt;
+            pgai[zgpos] = pgar[zgpos] = Zt * (1 - Zt) * gZt;
+            pgai[ngpos] = gNt_seed;
+            pgar[ngpos] = Rt * gNt_seed;
+            pgr[rpos] = gHt_1;
+        }
+    }
+    return KO_OK;
+}

@@ -108,6 +108,16 @@ int ko_transpose(float* py, const float* px, const int* pn, int64_t axis_size, i
 int ko_transpose_backward(float* pgx, const float* pgy, const int* pn, int64_t axis_size, int64_t data_size);
 int ko_transpose_bin(float* py, const float* px, int64_t nrow, int64_t ncol);
 
+/* recurrent cells (vmath.cu:732-736, 774-778, 4807-4826, 4946-4965, 4999-5033).  lstm_process_backward
+ * (vmath.cu:4860-4897) is not restated: its gate-gradient index expression (apos * g + n * nrec) leaves
+ * the [ndat, 4*nrec] buffer for nrec > 4. */
+int ko_copy(float* py, const float* pa, int64_t ndat);
+int ko_add(float* py, const float* pa, const float* pb, int64_t ndat);
+int ko_lstm_process(float* pr, float* ps, const float* ps1, const float* pa, int64_t ndat, int64_t nrec);
+int ko_gru_process(float* pr, const float* pai, const float* par, int64_t nt, int64_t ndat, int64_t nrec);
+int ko_gru_process_backward(float* pgr, float* pgai, float* pgar, const float* pr, const float* pai,
+                            const float* par, int64_t nt, int64_t ndat, int64_t nrec);
+
 #ifdef __cplusplus
 }
 #endif

@@ -59,6 +59,11 @@ def lib():
             "ko_transpose": [_F, _F, ctypes.c_void_p, _I64, _I64],
             "ko_transpose_backward": [_F, _F, ctypes.c_void_p, _I64, _I64],
             "ko_transpose_bin": [_F, _F, _I64, _I64],
+            "ko_copy": [_F, _F, _I64],
+            "ko_add": [_F, _F, _F, _I64],
+            "ko_lstm_process": [_F, _F, _F, _F, _I64, _I64],
+            "ko_gru_process": [_F, _F, _F, _I64, _I64, _I64],
+            "ko_gru_process_backward": [_F, _F, _F, _F, _F, _F, _I64, _I64, _I64],
             "ko_accumulate_grad": [_F, _F, _I64],
             "ko_subtract_param_grad": [_F, _F, _I64, _F],
             "ko_apply_decay": [_F, _F, _F, _I64, _F, _F],
@@ -338,3 +343,49 @@ def transpose_bin(x, nrow, ncol):
     y = np.zeros((nrow, ncol), np.float32)
     _check(lib().ko_transpose_bin(_p(y), _p(x), nrow, ncol))
     return y
+
+
+# ---- recurrent cells -------------------------------------------------------------------------------
+
+def copy(a):
+    a = _f32(a)
+    y = np.zeros_like(a)
+    _check(lib().ko_copy(_p(y), _p(a), a.size))
+    return y
+
+
+def add(a, b):
+    a, b = _f32(a), _f32(b)
+    y = np.zeros_like(a)
+    _check(lib().ko_add(_p(y), _p(a), _p(b), a.size))
+    return y
+
+
+def lstm_process(affine, prev_state=None):
+    """affine [ndat, 4*nrec] (input, forget, block, output); returns (recurrent, state), each [ndat, nrec]."""
+    affine = _f32(affine)
+    ndat, nrec = affine.shape[0], affine.shape[1] // 4
+    r = np.zeros((ndat, nrec), np.float32)
+    st = np.zeros((ndat, nrec), np.float32)
+    ps1 = None if prev_state is None else _p(_f32(prev_state))
+    _check(lib().ko_lstm_process(_p(r), _p(st), ps1, _p(affine), ndat, nrec))
+    return r, st
+
+
+def gru_process(recurs, pai, par, nt):
+    """recurs [ntimes, ndat, nrec] is updated in place at step nt (reads step nt-1 when nt > 0)."""
+    assert recurs.dtype == np.float32 and recurs.flags["C_CONTIGUOUS"]
+    pai, par = _f32(pai), _f32(par)
+    _, ndat, nrec = recurs.shape
+    _check(lib().ko_gru_process(_p(recurs[nt]), _p(pai), _p(par), nt, ndat, nrec))
+    return recurs
+
+
+def gru_process_backward(gr, recurs, pai, par, nt):
+    """gr [ndat, nrec] is replaced by the gradient of the previous step's output; returns (gr, gai, gar)."""
+    gr = _f32(gr).copy()
+    pai, par = _f32(pai), _f32(par)
+    _, ndat, nrec = recurs.shape
+    gai, gar = np.zeros_like(pai), np.zeros_like(par)
+    _check(lib().ko_gru_process_backward(_p(gr), _p(gai), _p(gar), _p(recurs[nt]), _p(pai), _p(par), nt, ndat, nrec))
+    return gr, gai, gar

@@ -532,6 +532,130 @@ def test_split_k_scratch_survives_shutdown_and_growth():
         check(y.to_numpy((m, n))[rows], ko.matmul_rows(w, x, rows), what="split-K %dx%dx%d" % (m, n, k))
 
 
+# ---- recurrent layers: cells and the per-time-step loop ---------------------------------------------------------
+
+def test_recurrent_cells():
+    rng = np.random.default_rng(21)
+    for ndat, nrec in ((3, 5), (64, 256), (1, 1)):
+        n = ndat * nrec
+        a, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+        y = dev(a)
+        VMath.add(0, y, y, dev(b), n)                       # in place, as the engine's gradient sum does
+        np.testing.assert_array_equal(y.to_numpy(n), ko.add(a, b))
+        c = DB(n * 4)
+        VMath.copy(0, c, y, n)
+        np.testing.assert_array_equal(c.to_numpy(n), a + b)
+        aff = (rng.standard_normal((ndat, 4 * nrec)) * 2).astype(np.float32)
+        s0 = rng.standard_normal((ndat, nrec)).astype(np.float32)
+        for prev in (s0, None):
+            r, st = DB(n * 4), DB(n * 4)
+            VMath.lstm_process(0, r, st, None if prev is None else dev(prev), dev(aff), ndat, nrec, 7)
+            want_r, want_s = ko.lstm_process(aff, prev)
+            check(st.to_numpy((ndat, nrec)), want_s, what="lstm state")
+            check(r.to_numpy((ndat, nrec)), want_r, what="lstm recurrent")
+        ai = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
+        ar = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
+        recurs = np.zeros((3, ndat, nrec), np.float32)
+        recurs[0] = rng.standard_normal((ndat, nrec)).astype(np.float32)
+        for nt in (0, 1):
+            rbuf = dev(recurs)
+            VMath.gru_process(0, rbuf.offset(nt * n * 4), dev(ai), dev(ar), nt, 3, ndat, nrec)
+            check(rbuf.to_numpy(recurs.shape), ko.gru_process(recurs.copy(), ai, ar, nt), what="gru step %d" % nt)
+            gh = rng.standard_normal((ndat, nrec)).astype(np.float32)
+            want = ko.gru_process_backward(gh, recurs, ai, ar, nt)
+            g, gai, gar, rsrc = dev(gh), DB(ai.nbytes), DB(ar.nbytes), dev(recurs)
+            VMath.gru_process_backward(0, g, gai, gar, rsrc.offset(nt * n * 4), dev(ai), dev(ar), nt, 3, ndat, nrec)
+            for got, ref, name in ((g.to_numpy(gh.shape), want[0], "gH"), (gai.to_numpy(ai.shape), want[1], "gai"),
+                                   (gar.to_numpy(ar.shape), want[2], "gar")):
+                check(got, ref, what="gru backward %s step %d" % (name, nt))
+
+
+def _oracle_rnn(x, wi, wr, bi, br, cell, nrec, forward, act="tanh"):
+    """The reference's per-step loop (vtensor.cpp:2455-2492) issued against the oracle."""
+    ntimes, ndat, _ = x.shape
+    ngates = {"rnn": 1, "lstm": 4, "gru": 3}[cell]
+    recurs = np.zeros((ntimes, ndat, nrec), np.float32)
+    states = np.zeros((ntimes, ndat, nrec), np.float32)
+    ia = np.zeros((ntimes, ndat, ngates * nrec), np.float32)
+    ra = np.zeros_like(ia) if cell == "gru" else ia
+    for n in range(ntimes):
+        nt = n if forward else ntimes - n - 1
+        prev = nt - 1 if forward else nt + 1
+        if n > 0:
+            ra[nt] = ko.matmul(wr, recurs[prev])
+        ia[nt] = ko.matmul(wi, x[nt], acc_into=ia[nt].copy())
+        if bi is not None:
+            ra[nt] = ko.add_bias(ra[nt], br)
+            ia[nt] = ko.add_bias(ia[nt], bi)
+        if cell == "rnn":
+            recurs[nt] = ko.activate(ko.add(ko.copy(ia[nt]), ia[nt]), act)
+        elif cell == "lstm":
+            recurs[nt], states[nt] = ko.lstm_process(ia[nt], states[prev] if n > 0 else None)
+        else:
+            ko.gru_process(recurs, ia[nt], ra[nt], nt)
+    return recurs, ia, ra
+
+
+def _oracle_rnn_backprop(x, wi, wr, use_bias, cell, recurs, ia, ra, gy, gyt, forward, act="tanh"):
+    """vtensor.cpp:2657-2701 issued against the oracle."""
+    ntimes, ndat, nrec = gyt.shape
+    gx, gwi, gwr = np.zeros_like(x), np.zeros_like(wi), np.zeros_like(wr)
+    gbi = np.zeros(wi.shape[0], np.float32)
+    gbr = np.zeros(wi.shape[0], np.float32)
+    gr = gy.copy()
+    for n in range(ntimes):
+        nt = ntimes - n - 1 if forward else n
+        prev = nt - 1 if forward else nt + 1
+        gr = ko.add(gr, gyt[nt])
+        if cell == "rnn":
+            gai = ko.activate_backward_with_y(gr, recurs[nt], act)
+            gar = gai
+        else:
+            gr, gai, gar = ko.gru_process_backward(gr, recurs, ia[nt], ra[nt], nt)
+        if use_bias:
+            gbi = ko.add_bias_backward_b(gai, gai.shape[1], acc_into=gbi)
+            gbr = ko.add_bias_backward_b(gar, gar.shape[1], acc_into=gbr)
+        gwi = ko.matmul_backward_w(gai, x[nt], wi.shape[0], wi.shape[1], acc_into=gwi)
+        if n < ntimes - 1:
+            gwr = ko.matmul_backward_w(gar, recurs[prev], wr.shape[0], wr.shape[1], acc_into=gwr)
+        gx[nt] = ko.matmul_backward_x(gai, wi)
+        gr = ko.matmul_backward_x(gar, wr, acc_into=gr if cell == "gru" else None)
+    return {"x": gx, "wi": gwi, "wr": gwr, "bi": gbi, "br": gbr}
+
+
+@pytest.mark.parametrize("cell", ["rnn", "lstm", "gru"])
+@pytest.mark.parametrize("ntimes,ndat,ninp,nrec,forward,bias", [(4, 3, 7, 5, True, True),       # sub-buffers at odd offsets
+                                                                (6, 16, 64, 32, False, False),
+                                                                (5, 64, 96, 128, True, True)])
+def test_rnn_layer_loop(cell, ntimes, ndat, ninp, nrec, forward, bias):
+    from deep_learning_framework_amd import tensor_ops as T
+    rng = np.random.default_rng(ntimes * 100 + ndat)
+    ngates = {"rnn": 1, "lstm": 4, "gru": 3}[cell]
+    x = rng.standard_normal((ntimes, ndat, ninp)).astype(np.float32)
+    wi = (rng.standard_normal((ngates * nrec, ninp)) / np.sqrt(ninp) * 0.5).astype(np.float32)
+    wr = (rng.standard_normal((ngates * nrec, nrec)) / np.sqrt(nrec) * 0.5).astype(np.float32)
+    bi = (rng.standard_normal(ngates * nrec) * 0.1).astype(np.float32) if bias else None
+    br = (rng.standard_normal(ngates * nrec) * 0.1).astype(np.float32) if bias else None
+    recurs, ia, ra = _oracle_rnn(x, wi, wr, bi, br, cell, nrec, forward)
+    tn = lambda a: None if a is None else T.Tensor.from_numpy(a)
+    for batched in (False, True):
+        y, saved = T.rnn(tn(x), tn(wi), tn(wr), tn(bi), tn(br), cell, nrec, forward=forward,
+                         batch_input_projection=batched)
+        check(saved["recurs"].numpy(), recurs, what="%s recurrent outputs (batched=%s)" % (cell, batched))
+        check(saved["iaffines"].numpy(), ia, what="%s gate pre-activations" % cell)
+        check(y.numpy(), recurs[-1 if forward else 0], what="%s output" % cell)
+    if cell == "lstm":
+        with pytest.raises(T.KaiError):
+            T.rnn_backprop(saved, tn(recurs[0]), tn(recurs))
+        return
+    gy = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    gyt = (rng.standard_normal((ntimes, ndat, nrec)) * 0.5).astype(np.float32)
+    want = _oracle_rnn_backprop(x, wi, wr, bias, cell, recurs, ia, ra, gy, gyt, forward)
+    got = T.rnn_backprop(saved, tn(gy), tn(gyt))
+    for name in got:
+        check(got[name].numpy(), want[name], tol=2e-5, what="%s backprop %s" % (cell, name))
+
+
 # ---- transposes ---------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("shape,axes", [((5,), (0,)), ((33, 70), (1, 0)), ((2, 3, 4), (2, 0, 1)), ((4, 512, 8, 64), (0, 2, 1, 3)),

@@ -349,3 +349,71 @@ def test_transposes_equal_numpy():
         np.testing.assert_array_equal(ko.transpose_backward(gy, shape, axes), np.transpose(gy, np.argsort(axes)))
     x = rng.standard_normal((37, 53)).astype(np.float32)            # [ncol, nrow]
     np.testing.assert_array_equal(ko.transpose_bin(x, 53, 37), x.T)
+
+
+# ---- recurrent cells (vmath.cu:732-778, 4807-4826, 4946-5033) --------------------------------------------------------
+
+def _sig64(v):
+    return 1.0 / (1.0 + np.exp(-np.asarray(v, np.float64)))
+
+
+def _gru64(ai, ar, hprev):
+    nrec = hprev.shape[1]
+    r = _sig64(ai[:, :nrec] + ar[:, :nrec])
+    z = _sig64(ai[:, nrec:2 * nrec] + ar[:, nrec:2 * nrec])
+    cand = np.tanh(ai[:, 2 * nrec:] + r * ar[:, 2 * nrec:])
+    return (1 - z) * cand + z * hprev
+
+
+def test_copy_and_add_exact():
+    a = np.arange(-5, 6, dtype=np.float32)
+    b = np.arange(11, dtype=np.float32) * 3
+    np.testing.assert_array_equal(ko.copy(a), a)
+    np.testing.assert_array_equal(ko.add(a, b), a + b)
+
+
+def test_lstm_cell_equals_textbook_float64():
+    rng = np.random.default_rng(9)
+    ndat, nrec = 5, 7
+    a = (rng.standard_normal((ndat, 4 * nrec)) * 2).astype(np.float32)
+    s0 = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    i, f, g, o = (a[:, k * nrec:(k + 1) * nrec].astype(np.float64) for k in range(4))
+    for prev in (s0, None):
+        r, s = ko.lstm_process(a, prev)
+        want_s = (0 if prev is None else prev) * _sig64(f) + np.tanh(g) * _sig64(i)
+        np.testing.assert_allclose(s, want_s, rtol=0, atol=5e-7)
+        np.testing.assert_allclose(r, np.tanh(want_s) * _sig64(o), rtol=0, atol=5e-7)
+    # a gate order mistake would show here: only the forget gate open keeps the state, output gate shut gives 0
+    a2 = np.full((1, 4), -40.0, np.float32)
+    a2[0, 1] = 40.0
+    r, s = ko.lstm_process(a2, np.array([[0.75]], np.float32))
+    assert s[0, 0] == 0.75 and abs(r[0, 0]) < 1e-12
+
+
+def test_gru_cell_and_its_backward():
+    rng = np.random.default_rng(10)
+    ntimes, ndat, nrec = 3, 4, 6
+    ai = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
+    ar = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
+    recurs = np.zeros((ntimes, ndat, nrec), np.float32)
+    recurs[0] = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    # step 0 sees no previous output, step 1 reads step 0
+    first = ko.gru_process(np.zeros_like(recurs), ai, ar, 0)[0]
+    np.testing.assert_allclose(first, _gru64(ai, ar, np.zeros((ndat, nrec))), rtol=0, atol=5e-7)
+    ko.gru_process(recurs, ai, ar, 1)
+    np.testing.assert_allclose(recurs[1], _gru64(ai, ar, recurs[0]), rtol=0, atol=5e-7)
+    # backward against central differences of the float64 closed form
+    gh = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    gprev, gai, gar = ko.gru_process_backward(gh, recurs, ai, ar, 1)
+    loss = lambda ai_, ar_, hp_: float((_gru64(ai_, ar_, hp_) * gh).sum())
+    eps = 1e-6
+    base = (ai.astype(np.float64), ar.astype(np.float64), recurs[0].astype(np.float64))
+    for which, got in ((0, gai), (1, gar), (2, gprev)):
+        num = np.zeros_like(base[which])
+        for idx in np.ndindex(num.shape):
+            hi = [b.copy() for b in base]
+            lo = [b.copy() for b in base]
+            hi[which][idx] += eps
+            lo[which][idx] -= eps
+            num[idx] = (loss(*hi) - loss(*lo)) / (2 * eps)
+        np.testing.assert_allclose(got, num, rtol=0, atol=2e-6)
