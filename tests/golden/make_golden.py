@@ -1,6 +1,7 @@
 #!/usr/bin/env python3
 """Writes tests/golden/matmul_path_small.npz: inputs and expected outputs of every operator of
-the matmul path at small shapes.
+the matmul path at small shapes, and tests/golden/next_to_path_small.npz: the same for the operators
+either side of it (parameter update, transposes, recurrent cells).
 
 The reference ships no golden vectors, known-answer tests or fixtures for this path and cannot be
 built or run here, so the expected outputs are produced by the CPU oracle (oracle/kai_oracle.c),
@@ -66,6 +67,53 @@ def main():
     f["att_gk"] = ko.mult_on_heads_backward(f["att_gscores"], q, nhead)
     f["att_gq"] = ko.mult_on_heads_backward(f["att_gscores"], k, nhead)
     out = os.path.join(HERE, "matmul_path_small.npz")
+    np.savez_compressed(out, **f)
+    print("wrote", out, os.path.getsize(out), "bytes,", len(f), "arrays")
+    next_to_path()
+
+
+def next_to_path():
+    rng = np.random.default_rng(20240608)
+    f = {}
+    # parameter update on 37 elements
+    n = 37
+    p = rng.standard_normal(n).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    s = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    t = (rng.random(n) * 0.01).astype(np.float32)
+    steps = np.full(n, 3, np.float32)
+    f.update(upd_p=p, upd_g=g, upd_s=s, upd_t=t, upd_steps=steps,
+             upd_hyper=np.array([0.01, 0.001, 0.0005, 0.9, 0.999, 1e-8], np.float32))   # lr, l1, l2, ro1, ro2, eps
+    f["upd_accumulate"] = ko.accumulate_grad(p, g)
+    f["upd_subtract"] = ko.subtract_param_grad(p, g, 0.01)
+    f["upd_decay"] = ko.apply_decay(p, g, 0.001, 0.0005)
+    f["adam_delta"], f["adam_s"], f["adam_t"], f["adam_steps"] = ko.eval_adam_delta(g, s, t, steps, 0.9, 0.999, 1e-8)
+    # transposes
+    x = rng.standard_normal((2, 3, 4, 5)).astype(np.float32)
+    axes = (2, 0, 3, 1)
+    f.update(tr_x=x, tr_axes=np.array(axes, np.int64), tr_table=ko.transpose_axinfo(x.shape, axes))
+    f["tr_y"] = ko.transpose(x, axes)
+    gy = rng.standard_normal(f["tr_y"].shape).astype(np.float32)
+    f.update(tr_gy=gy, tr_gx=ko.transpose_backward(gy, x.shape, axes))
+    xb = rng.standard_normal((7, 13)).astype(np.float32)          # [ncol, nrow]
+    f.update(trbin_x=xb, trbin_y=ko.transpose_bin(xb, 13, 7))
+    # recurrent cells: ndat 3, nrec 5
+    ndat, nrec = 3, 5
+    a4 = (rng.standard_normal((ndat, 4 * nrec)) * 2).astype(np.float32)
+    st = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    f.update(lstm_affine=a4, lstm_prev_state=st)
+    f["lstm_recur"], f["lstm_state"] = ko.lstm_process(a4, st)
+    f["lstm_recur_first"], f["lstm_state_first"] = ko.lstm_process(a4, None)
+    ai = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
+    ar = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
+    recurs = np.zeros((2, ndat, nrec), np.float32)
+    recurs[0] = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    gh = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    f.update(gru_ai=ai, gru_ar=ar, gru_recurs_in=recurs.copy(), gru_gh=gh)
+    f["gru_recurs_out"] = ko.gru_process(recurs, ai, ar, 1).copy()
+    f["gru_gprev"], f["gru_gai"], f["gru_gar"] = ko.gru_process_backward(gh, f["gru_recurs_out"], ai, ar, 1)
+    f["add"] = ko.add(p, g)
+    out = os.path.join(HERE, "next_to_path_small.npz")
     np.savez_compressed(out, **f)
     print("wrote", out, os.path.getsize(out), "bytes,", len(f), "arrays")
 

@@ -9,6 +9,7 @@ import pytest
 from util import REL_FRO_TOL, ROOT, ko, rel_fro
 
 G = np.load(os.path.join(ROOT, "tests", "golden", "matmul_path_small.npz"), allow_pickle=False)
+G2 = np.load(os.path.join(ROOT, "tests", "golden", "next_to_path_small.npz"), allow_pickle=False)
 ACTS = ["none", "relu", "leaky", "sigmoid", "tanh", "gelu", "selu", "mish", "swish"]
 
 
@@ -112,3 +113,93 @@ def test_hip_path_matches_the_fixture():
     VMath.mult_on_heads_backward(0, gq, dgs, dk, nbat, ntimes, nvec, nhead, npiece)
     assert rel_fro(gk.to_numpy(G["att_gk"].shape), G["att_gk"]) <= REL_FRO_TOL
     assert rel_fro(gq.to_numpy(G["att_gq"].shape), G["att_gq"]) <= REL_FRO_TOL
+
+
+# ---- the operators either side of the path: tests/golden/next_to_path_small.npz ----------------------------------
+
+def test_oracle_reproduces_the_second_fixture_bit_for_bit():
+    p, g, s, t, steps = (G2[k] for k in ("upd_p", "upd_g", "upd_s", "upd_t", "upd_steps"))
+    lr, l1, l2, ro1, ro2, eps = (float(v) for v in G2["upd_hyper"])
+    assert np.array_equal(ko.accumulate_grad(p, g), G2["upd_accumulate"])
+    assert np.array_equal(ko.subtract_param_grad(p, g, lr), G2["upd_subtract"])
+    assert np.array_equal(ko.apply_decay(p, g, l1, l2), G2["upd_decay"])
+    for got, name in zip(ko.eval_adam_delta(g, s, t, steps, ro1, ro2, eps), ("adam_delta", "adam_s", "adam_t", "adam_steps")):
+        assert np.array_equal(got, G2[name]), name
+    axes = tuple(int(a) for a in G2["tr_axes"])
+    assert np.array_equal(ko.transpose_axinfo(G2["tr_x"].shape, axes), G2["tr_table"])
+    assert np.array_equal(ko.transpose(G2["tr_x"], axes), G2["tr_y"])
+    assert np.array_equal(ko.transpose_backward(G2["tr_gy"], G2["tr_x"].shape, axes), G2["tr_gx"])
+    assert np.array_equal(ko.transpose_bin(G2["trbin_x"], 13, 7), G2["trbin_y"])
+    r, st = ko.lstm_process(G2["lstm_affine"], G2["lstm_prev_state"])
+    assert np.array_equal(r, G2["lstm_recur"]) and np.array_equal(st, G2["lstm_state"])
+    assert np.array_equal(ko.gru_process(G2["gru_recurs_in"].copy(), G2["gru_ai"], G2["gru_ar"], 1), G2["gru_recurs_out"])
+    for got, name in zip(ko.gru_process_backward(G2["gru_gh"], G2["gru_recurs_out"], G2["gru_ai"], G2["gru_ar"], 1),
+                         ("gru_gprev", "gru_gai", "gru_gar")):
+        assert np.array_equal(got, G2[name]), name
+
+
+def test_second_fixture_satisfies_closed_forms():
+    axes = tuple(int(a) for a in G2["tr_axes"])
+    assert np.array_equal(G2["tr_y"], np.transpose(G2["tr_x"], axes))
+    assert np.array_equal(G2["trbin_y"], G2["trbin_x"].T)
+    lr = np.float32(G2["upd_hyper"][0])
+    assert np.array_equal(G2["upd_subtract"], G2["upd_p"] - G2["upd_g"] * lr)
+    assert np.array_equal(G2["adam_steps"], G2["upd_steps"] + 1)
+    sig = lambda v: 1 / (1 + np.exp(-v.astype(np.float64)))
+    i, f, g, o = (G2["lstm_affine"][:, k * 5:(k + 1) * 5] for k in range(4))
+    assert np.allclose(G2["lstm_state"], G2["lstm_prev_state"] * sig(f) + np.tanh(g.astype(np.float64)) * sig(i), atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_hip_path_matches_the_second_fixture():
+    from deep_learning_framework_amd import kai
+    from deep_learning_framework_amd.kai import DeviceBuffer as DB, VMath
+    kai.load()
+    kai.set_device(0)
+    dev = lambda a: DB.from_numpy(np.ascontiguousarray(a))
+    p, g, s, t, steps = (G2[k] for k in ("upd_p", "upd_g", "upd_s", "upd_t", "upd_steps"))
+    n = p.size
+    lr, l1, l2, ro1, ro2, eps = (kai.hyper(float(v)) for v in G2["upd_hyper"])
+    y = dev(p)
+    VMath.accumulate_grad(0, y, dev(g), n)
+    assert np.array_equal(y.to_numpy(n), G2["upd_accumulate"])
+    y = dev(p)
+    VMath.subtract_param_grad(0, y, dev(g), n, lr)
+    assert np.array_equal(y.to_numpy(n), G2["upd_subtract"])
+    d = DB(n * 4)
+    VMath.apply_decay(0, d, dev(p), dev(g), n, l1, l2)
+    assert np.array_equal(d.to_numpy(n), G2["upd_decay"])
+    a, ds, dt, dn = DB(n * 4), dev(s), dev(t), dev(steps)
+    VMath.eval_adam_delta(0, a, dev(g), ds, dt, dn, n, ro1, ro2, eps)
+    assert np.array_equal(ds.to_numpy(n), G2["adam_s"]) and np.array_equal(dt.to_numpy(n), G2["adam_t"])
+    assert np.array_equal(dn.to_numpy(n), G2["adam_steps"])
+    assert rel_fro(a.to_numpy(n), G2["adam_delta"]) <= REL_FRO_TOL
+    x = G2["tr_x"]
+    table = dev(G2["tr_table"])
+    out = DB(x.nbytes)
+    VMath.transpose(0, out, dev(x), table, x.ndim, x.size)
+    assert np.array_equal(out.to_numpy(G2["tr_y"].shape), G2["tr_y"])
+    VMath.transpose_backward(0, out, dev(G2["tr_gy"]), table, x.ndim, x.size)
+    assert np.array_equal(out.to_numpy(x.shape), G2["tr_gx"])
+    ob = DB(G2["trbin_x"].nbytes)
+    VMath.transpose_bin(0, ob, dev(G2["trbin_x"]), 13, 7)
+    assert np.array_equal(ob.to_numpy((13, 7)), G2["trbin_y"])
+    ndat, nrec = G2["lstm_prev_state"].shape
+    r, st = DB(ndat * nrec * 4), DB(ndat * nrec * 4)
+    VMath.lstm_process(0, r, st, dev(G2["lstm_prev_state"]), dev(G2["lstm_affine"]), ndat, nrec, 0)
+    assert rel_fro(r.to_numpy((ndat, nrec)), G2["lstm_recur"]) <= REL_FRO_TOL
+    assert rel_fro(st.to_numpy((ndat, nrec)), G2["lstm_state"]) <= REL_FRO_TOL
+    VMath.lstm_process(0, r, st, None, dev(G2["lstm_affine"]), ndat, nrec, 0)
+    assert rel_fro(r.to_numpy((ndat, nrec)), G2["lstm_recur_first"]) <= REL_FRO_TOL
+    rec = dev(G2["gru_recurs_in"])
+    ai, ar = dev(G2["gru_ai"]), dev(G2["gru_ar"])
+    VMath.gru_process(0, rec.offset(ndat * nrec * 4), ai, ar, 1, 2, ndat, nrec)
+    assert rel_fro(rec.to_numpy(G2["gru_recurs_out"].shape), G2["gru_recurs_out"]) <= REL_FRO_TOL
+    gh, gai, gar, rec2 = dev(G2["gru_gh"]), DB(G2["gru_ai"].nbytes), DB(G2["gru_ar"].nbytes), dev(G2["gru_recurs_out"])
+    VMath.gru_process_backward(0, gh, gai, gar, rec2.offset(ndat * nrec * 4), ai, ar, 1, 2, ndat, nrec)
+    assert rel_fro(gh.to_numpy((ndat, nrec)), G2["gru_gprev"]) <= REL_FRO_TOL
+    assert rel_fro(gai.to_numpy(G2["gru_ai"].shape), G2["gru_gai"]) <= REL_FRO_TOL
+    assert rel_fro(gar.to_numpy(G2["gru_ar"].shape), G2["gru_gar"]) <= REL_FRO_TOL
+    s2 = DB(n * 4)
+    VMath.add(0, s2, dev(p), dev(g), n)
+    assert np.array_equal(s2.to_numpy(n), G2["add"])
