@@ -43,6 +43,11 @@ int launch_gru_process(float* r, const float* ai, const float* ar, int64_t nt, i
 int launch_gru_process_backward(float* gr, float* gai, float* gar, const float* r, const float* ai, const float* ar,
                                 int64_t nt, int64_t ndat, int64_t nrec, hipStream_t stream);
 
+// VMath::cosinesim (vmath.cu:6459-6513 of the reference) after the row-pair products are in y: the norms of
+// the nrow1 + nrow2 rows go to norms, then y[i,j] /= norms[i] * norms[nrow1 + j] + 1e-20
+int launch_cosine_norms_and_scale(float* y, float* norms, const float* x1, const float* x2, int64_t nrow1,
+                                  int64_t nrow2, int64_t ncol, hipStream_t stream);
+
 // Final pass of a split-K product: C(m,n) (=|+=) act(alpha * sum_s part[s][m][n] + bias[n]), the
 // pre-activation value also to C2 when given.  `part` holds nsplit dense [M,N] matrices.
 struct SplitReduceParams {

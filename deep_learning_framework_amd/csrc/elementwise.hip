@@ -536,6 +536,46 @@ int launch_gru_process_backward(float* gr, float* gai, float* gar, const float* 
     return check_launch("gru_process_backward_kernel");
 }
 
+// ---- cosine similarity: the two passes around the row-pair product ---------------------------------------
+//
+// y[i,j] = <a_i, b_j> / (|a_i| |b_j| + 1e-20).  The products come from the GEMM; row_norm_kernel writes
+// |row| for the rows of both operands (a wave per row), cosine_scale_kernel divides.
+
+__global__ void __launch_bounds__(256) row_norm_kernel(float* __restrict__ out, const float* __restrict__ x1,
+                                                       int64_t nrow1, const float* __restrict__ x2, int64_t nrow2,
+                                                       int64_t ncol) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= nrow1 + nrow2) return;
+    const float* xr = row < nrow1 ? x1 + row * ncol : x2 + (row - nrow1) * ncol;
+    float s = 0.f;
+    for (int64_t c = lane; c < ncol; c += 64) s += xr[c] * xr[c];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    if (lane == 0) out[row] = sqrtf(s);
+}
+
+__global__ void __launch_bounds__(kEwThreads) cosine_scale_kernel(float* __restrict__ y, const float* __restrict__ norms,
+                                                                  int64_t nrow1, int64_t nrow2) {
+    const int64_t n = nrow1 * nrow2;
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        const int64_t r1 = i / nrow2, r2 = i - r1 * nrow2;
+        y[i] = y[i] / (norms[r1] * norms[nrow1 + r2] + 1e-20f);
+    }
+}
+
+int launch_cosine_norms_and_scale(float* y, float* norms, const float* x1, const float* x2, int64_t nrow1,
+                                  int64_t nrow2, int64_t ncol, hipStream_t stream) {
+    const int64_t rows = nrow1 + nrow2;
+    if (rows <= 0 || nrow1 * nrow2 <= 0) return KAI_OK;
+    if ((rows + 3) / 4 > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "cosinesim: too many rows");
+    row_norm_kernel<<<dim3((unsigned)((rows + 3) / 4)), 256, 0, stream>>>(norms, x1, nrow1, x2, nrow2, ncol);
+    KAI_TRY(check_launch("row_norm_kernel"));
+    cosine_scale_kernel<<<blocks_for(nrow1 * nrow2), kEwThreads, 0, stream>>>(y, norms, nrow1, nrow2);
+    return check_launch("cosine_scale_kernel");
+}
+
 // ---- split-K final pass ---------------------------------------------------------------------
 //
 // Sums the partial products in split order (fixed, so the result does not depend on scheduling)

@@ -549,6 +549,24 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
     return KAI_OK;
 }
 
+// ---- cosine similarity ------------------------------------------------------------------------------
+
+int kai_cosinesim(int device, float* py, const float* px1, const float* px2, int64_t nrow1, int64_t nrow2,
+                  int64_t ncol) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(nrow1 >= 0 && nrow2 >= 0 && ncol >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (nrow1 == 0 || nrow2 == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py);
+    if (ncol == 0) return launch_fill_float(py, nrow1 * nrow2, 0.0f, current_stream());   // 0 / 1e-20
+    KAI_REQUIRE_PTR(px1); KAI_REQUIRE_PTR(px2);
+    // the products are y = x1 . x2^T, the same NT product as matmul with x2 in the weight's place
+    KAI_TRY(kai_matmul(device, py, px2, px1, nrow2, nrow1, ncol, 0));
+    // the product may have used the scratch for its own partial sums; in stream order it is free again here
+    float* norms = nullptr;
+    KAI_TRY(workspace((nrow1 + nrow2) * (int64_t)sizeof(float), &norms));
+    return launch_cosine_norms_and_scale(py, norms, px1, px2, nrow1, nrow2, ncol, current_stream());
+}
+
 // ---- recurrent cells: the element-wise steps between the gate products -----------------------------
 
 int kai_copy(int device, float* py, const float* pa, int64_t ndat) {

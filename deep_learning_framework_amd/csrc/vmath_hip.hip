@@ -82,6 +82,9 @@ void VMath::mix_values_backward_value(int device, float* pgV, float* pgy, float*
     raise_on(kai_mix_values_backward_value(device, pgV, pgy, pp, nbat, ntimes, nvec, nhead, npiece));
 }
 
+void VMath::cosinesim(int device, float* py, float* px1, float* px2, int64 nrow1, int64 nrow2, int64 ncol) {
+    raise_on(kai_cosinesim(device, py, px1, px2, nrow1, nrow2, ncol));
+}
 void VMath::copy(int device, float* py, float* pa, int64 ndat) { raise_on(kai_copy(device, py, pa, ndat)); }
 void VMath::add(int device, float* py, float* pa, float* pb, int64 ndat) { raise_on(kai_add(device, py, pa, pb, ndat)); }
 void VMath::lstm_process(int device, float* pr, float* ps, float* ps1, float* pa, int64 ndat, int64 nrec, int64 ninp) {

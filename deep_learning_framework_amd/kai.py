@@ -62,6 +62,7 @@ SIGNATURES = {
     "kai_gemm_f32": [_INT, _INT, _INT, _I64, _I64, _I64, _F, _I64, _F, _I64, _F, _I64, _F, _INT, _F, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
     "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
+    "kai_cosinesim": [_INT, _F, _F, _F, _I64, _I64, _I64],
     "kai_copy": [_INT, _F, _F, _I64],
     "kai_add": [_INT, _F, _F, _F, _I64],
     "kai_lstm_process": [_INT, _F, _F, _F, _F, _I64, _I64, _I64],
@@ -308,6 +309,10 @@ class VMath:
     def gemm_f32(device, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, bias, actFunc, hLeakyAlpha, acc):
         _ck(load().kai_gemm_f32(device, int(transA), int(transB), M, N, K, _addr(A), lda, _addr(B), ldb, _addr(C),
                                 ldc, _addr(bias), actFunc, _addr(hLeakyAlpha), int(acc)))
+
+    @staticmethod
+    def cosinesim(device, py, px1, px2, nrow1, nrow2, ncol):
+        _ck(load().kai_cosinesim(device, _addr(py), _addr(px1), _addr(px2), nrow1, nrow2, ncol))
 
     @staticmethod
     def copy(device, py, pa, ndat):

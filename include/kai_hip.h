@@ -194,6 +194,14 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
                        const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
                        int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc);
 
+/* ---- cosine similarity (next to the path) ------------------------------------------------------------ */
+
+/* VMath::cosinesim, vmath.cu:6459-6513 (vmath.h:226; driver VTensor::cosinesim, vtensor.cpp:5864-5890).
+ * py[nrow1, nrow2] = <x1_i, x2_j> / (|x1_i| |x2_j| + 1e-20): the NT product of the path, the row norms and a
+ * scaling pass.  Forward only, as in the reference (its backprop throws VERR_NOT_IMPLEMENTED_YET). */
+int kai_cosinesim(int device, float* py, const float* px1, const float* px2, int64_t nrow1, int64_t nrow2,
+                  int64_t ncol);
+
 /* ---- recurrent layers (next to the path): the steps between the gate products ---------------------- */
 /* VTensor's rnn/lstm/gru loop (vtensor.cpp:2455-2492, 2657-2701) issues, per time step, kai_matmul with
  * acc = 0 and 1 on sub-buffers at t * size offsets, kai_add_bias in place, and the calls below. */

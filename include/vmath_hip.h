@@ -78,6 +78,7 @@ public:
     static void mix_values_backward_value(int device, float* pV, float* pgy, float* pp, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece);
 
     /* additive: the `dense` layer formula activate(add(matmul(x,w),b)) (api/vconst.cpp:11) in one launch */
+    static void cosinesim(int device, float* py, float* px1, float* px2, int64 nrow1, int64 nrow2, int64 ncol);
     static void copy(int device, float* py, float* pa, int64 ndat);
     static void add(int device, float* py, float* pa, float* pb, int64 ndat);
     static void lstm_process(int device, float* pr, float* ps, float* ps1, float* pa, int64 ndat, int64 nrec, int64 ninp);

@@ -625,3 +625,25 @@ int ko_gru_process_backward(float* pgr, float* pgai, float* pgar, const float* p
     }
     return KO_OK;
 }
+
+/* ---- cosine similarity of every row pair ------------------------------------------------------ */
+
+int ko_cosinesim(float* py, const float* px1, const float* px2, int64_t nrow1, int64_t nrow2, int64_t ncol) {
+    /* vmath.cu:6459-6480 */
+    for (int64_t nr1 = 0, n = 0; nr1 < nrow1; nr1++) {
+        for (int64_t nr2 = 0; nr2 < nrow2; nr2++, n++) {
+            float aa_sum = 0;
+            float bb_sum = 0;
+            float ab_sum = 0;
+            for (int64_t nc = 0; nc < ncol; nc++) {
+                float a = px1[nr1 * ncol + nc];
+                float b = px2[nr2 * ncol + nc];
+                aa_sum += a * a;
+                bb_sum += b * b;
+                ab_sum += a * b;
+            }
+            py[n] = ab_sum / (sqrtf(aa_sum) * sqrtf(bb_sum) + 1e-20f);
+        }
+    }
+    return KO_OK;
+}

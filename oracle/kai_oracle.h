@@ -108,6 +108,9 @@ int ko_transpose(float* py, const float* px, const int* pn, int64_t axis_size, i
 int ko_transpose_backward(float* pgx, const float* pgy, const int* pn, int64_t axis_size, int64_t data_size);
 int ko_transpose_bin(float* py, const float* px, int64_t nrow, int64_t ncol);
 
+/* cosine similarity of every row of x1[nrow1, ncol] with every row of x2[nrow2, ncol] (vmath.cu:6459-6480) */
+int ko_cosinesim(float* py, const float* px1, const float* px2, int64_t nrow1, int64_t nrow2, int64_t ncol);
+
 /* recurrent cells (vmath.cu:732-736, 774-778, 4807-4826, 4946-4965, 4999-5033).  lstm_process_backward
  * (vmath.cu:4860-4897) is not restated: its gate-gradient index expression (apos * g + n * nrec) leaves
  * the [ndat, 4*nrec] buffer for nrec > 4. */

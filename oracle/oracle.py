@@ -59,6 +59,7 @@ def lib():
             "ko_transpose": [_F, _F, ctypes.c_void_p, _I64, _I64],
             "ko_transpose_backward": [_F, _F, ctypes.c_void_p, _I64, _I64],
             "ko_transpose_bin": [_F, _F, _I64, _I64],
+            "ko_cosinesim": [_F, _F, _F, _I64, _I64, _I64],
             "ko_copy": [_F, _F, _I64],
             "ko_add": [_F, _F, _F, _I64],
             "ko_lstm_process": [_F, _F, _F, _F, _I64, _I64],
@@ -342,6 +343,16 @@ def transpose_bin(x, nrow, ncol):
     x = _f32(x)
     y = np.zeros((nrow, ncol), np.float32)
     _check(lib().ko_transpose_bin(_p(y), _p(x), nrow, ncol))
+    return y
+
+
+def cosinesim(x1, x2):
+    """y[nrow1, nrow2]: cosine of every row of x1 with every row of x2 (last axis = the vector)."""
+    x1, x2 = _f32(x1), _f32(x2)
+    ncol = x1.shape[-1]
+    nrow1, nrow2 = x1.size // ncol, x2.size // ncol
+    y = np.zeros((nrow1, nrow2), np.float32)
+    _check(lib().ko_cosinesim(_p(y), _p(x1), _p(x2), nrow1, nrow2, ncol))
     return y
 
 

@@ -532,6 +532,23 @@ def test_split_k_scratch_survives_shutdown_and_growth():
         check(y.to_numpy((m, n))[rows], ko.matmul_rows(w, x, rows), what="split-K %dx%dx%d" % (m, n, k))
 
 
+# ---- cosinesim ----------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("nrow1,nrow2,ncol", [(1, 1, 1), (6, 4, 33), (64, 512, 784), (300, 70, 1000), (2048, 2048, 64), (5, 4100, 128)])
+def test_cosinesim(nrow1, nrow2, ncol):
+    rng = np.random.default_rng(nrow1 + ncol)
+    a = rng.standard_normal((nrow1, ncol)).astype(np.float32)
+    b = rng.standard_normal((nrow2, ncol)).astype(np.float32)
+    if nrow2 > 2:
+        b[1] = 0                                           # a zero row: 0 through the 1e-20 guard
+    y = DB(nrow1 * nrow2 * 4)
+    VMath.cosinesim(0, y, dev(a), dev(b), nrow1, nrow2, ncol)
+    got = y.to_numpy((nrow1, nrow2))
+    check(got, ko.cosinesim(a, b), what="cosinesim")
+    if nrow2 > 2:
+        assert (got[:, 1] == 0).all()
+
+
 # ---- recurrent layers: cells and the per-time-step loop ---------------------------------------------------------
 
 def test_recurrent_cells():

@@ -417,3 +417,20 @@ def test_gru_cell_and_its_backward():
             lo[which][idx] -= eps
             num[idx] = (loss(*hi) - loss(*lo)) / (2 * eps)
         np.testing.assert_allclose(got, num, rtol=0, atol=2e-6)
+
+
+# ---- cosinesim (vmath.cu:6459-6480) ----------------------------------------------------------------------------------
+
+def test_cosinesim_against_float64_and_special_rows():
+    rng = np.random.default_rng(12)
+    a = rng.standard_normal((6, 33)).astype(np.float32)
+    b = rng.standard_normal((4, 33)).astype(np.float32)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    want = (a64 @ b64.T) / (np.linalg.norm(a64, axis=1)[:, None] * np.linalg.norm(b64, axis=1)[None, :])
+    np.testing.assert_allclose(ko.cosinesim(a, b), want, rtol=0, atol=1e-6)
+    # a row with itself is 1, with its negative -1, with an orthogonal one 0; a zero row gives 0 (the 1e-20 guard)
+    e = np.array([[3, 4, 0], [-3, -4, 0], [0, 0, 2], [0, 0, 0]], np.float32)
+    got = ko.cosinesim(e[:1], e)
+    np.testing.assert_array_equal(got, np.array([[1, -1, 0, 0]], np.float32))
+    # leading axes fold into rows (vtensor.cpp:5878-5880)
+    assert ko.cosinesim(a.reshape(2, 3, 33), b).shape == (6, 4)
