@@ -227,11 +227,14 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
     rec = torch.zeros((nt_, nd_, nr_), device=dev)
     sta = torch.zeros((nt_, nd_, nr_), device=dev)
 
-    def lstm_layer(batched):
+    def lstm_layer(batched, fused=False):
         L.kai_set_zero(0, P(aff), I(aff.numel() * 4))
         if batched:
             L.kai_matmul(0, P(aff), P(wi), P(xs), I(4 * nr_), I(nt_ * nd_), I(ni_), 0)
-        for t in range(nt_):
+        for t in range(nt_ if fused else 0):
+            L.kai_lstm_step(0, P(rec[t]), P(sta[t]), P(sta[t - 1]) if t > 0 else None, P(aff[t]), P(wr),
+                            P(rec[t - 1]) if t > 0 else None, P(bi), None, I(nd_), I(nr_))
+        for t in range(0 if fused else nt_):
             if t > 0:
                 L.kai_matmul(0, P(aff[t]), P(wr), P(rec[t - 1]), I(4 * nr_), I(nd_), I(nr_), int(batched))
             if not batched:
@@ -244,6 +247,18 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
         flops=lstm_flops)
     row("lstm layer forward, same, input products of all steps in one call", gpu_us(lambda: lstm_layer(True), iters=10),
         flops=lstm_flops)
+    row("lstm layer forward, same, one kai_lstm_step per step", gpu_us(lambda: lstm_layer(True, True), iters=10),
+        flops=lstm_flops)
+    # the same calls recorded once into a HIP graph and replayed (the counterpart of the engine's call replay)
+    side = torch.cuda.Stream()
+    for fused, name in ((False, "three calls per step"), (True, "one kai_lstm_step per step")):
+        kai.set_stream(side.cuda_stream)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            lstm_layer(True, fused)
+        kai.set_stream(stream.cuda_stream)
+        row("lstm layer forward, %s, replayed from a HIP graph" % name, gpu_us(graph.replay, iters=10), flops=lstm_flops)
+        del graph
     # transposes next to the path: the head split [4,512,8,64] -> [4,8,512,64] of configuration 4 and a plain 4096^2
     shape, axes = (4, 512, 8, 64), (0, 2, 1, 3)
     x = torch.randn(shape, device=dev, generator=g)

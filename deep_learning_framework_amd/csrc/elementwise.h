@@ -43,6 +43,19 @@ int launch_gru_process(float* r, const float* ai, const float* ar, int64_t nt, i
 int launch_gru_process_backward(float* gr, float* gai, float* gar, const float* r, const float* ai, const float* ar,
                                 int64_t nt, int64_t ndat, int64_t nrec, hipStream_t stream);
 
+// One LSTM / GRU time step in one launch (recurrent_step.hip): recurrent gate product + biases + cell.
+// r_prev null: no recurrent product (first step).  recurrent_step_applies: operand alignment and the sizes up
+// to which the single launch beats the separate calls.
+constexpr int64_t kRecStepMaxRows = 256, kRecStepMaxUnits = 1024;
+bool recurrent_step_applies(const float* wr, const float* r_prev, int64_t ndat, int64_t nrec);
+int launch_lstm_step(float* r, float* s, const float* s1, float* a, const float* wr, const float* r_prev,
+                     const float* bi, const float* br, int64_t ndat, int64_t nrec, hipStream_t stream);
+int launch_gru_step(float* r, float* ai, float* ar, const float* wr, const float* r_prev, const float* h_prev,
+                    const float* bi, const float* br, int64_t ndat, int64_t nrec, hipStream_t stream);
+// gru_process with the previous output given by pointer (null: 0) instead of by position
+int launch_gru_process_from(float* r, const float* h_prev, const float* ai, const float* ar, int64_t ndat, int64_t nrec,
+                            hipStream_t stream);
+
 // VMath::cosinesim (vmath.cu:6459-6513 of the reference) after the row-pair products are in y: the norms of
 // the nrow1 + nrow2 rows go to norms, then y[i,j] /= norms[i] * norms[nrow1 + j] + 1e-20
 int launch_cosine_norms_and_scale(float* y, float* norms, const float* x1, const float* x2, int64_t nrow1,

@@ -472,8 +472,8 @@ struct GruGates {
     float Rt, Zt, Nt, Ht_1, par_n;
 };
 
-__device__ __forceinline__ GruGates gru_gates(const float* r, const float* ai, const float* ar, int64_t i, int64_t nt,
-                                              int64_t n, int64_t nrec, int64_t& gpos) {
+__device__ __forceinline__ GruGates gru_gates(const float* h_prev, const float* ai, const float* ar, int64_t i,
+                                              int64_t nrec, int64_t& gpos) {
     const int64_t nd = i / nrec, ny = i - nd * nrec;
     gpos = nd * 3 * nrec + ny;
     GruGates g;
@@ -481,29 +481,28 @@ __device__ __forceinline__ GruGates gru_gates(const float* r, const float* ai, c
     g.Zt = act_sigmoid(ai[gpos + nrec] + ar[gpos + nrec]);
     g.par_n = ar[gpos + 2 * nrec];
     g.Nt = act_tanh(ai[gpos + 2 * nrec] + g.Rt * g.par_n);
-    g.Ht_1 = nt > 0 ? r[i - n] : 0.f;      // the previous time step lies one [ndat, nrec] block before r
+    g.Ht_1 = h_prev ? h_prev[i] : 0.f;
     return g;
 }
 
 __global__ void __launch_bounds__(kEwThreads)
-    gru_process_kernel(float* r, const float* __restrict__ ai, const float* __restrict__ ar, int64_t nt, int64_t n,
-                       int64_t nrec) {
+    gru_process_kernel(float* r, const float* h_prev, const float* __restrict__ ai, const float* __restrict__ ar,
+                       int64_t n, int64_t nrec) {
     const int64_t stride = (int64_t)gridDim.x * kEwThreads;
     for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
         int64_t gpos;
-        const GruGates g = gru_gates(r, ai, ar, i, nt, n, nrec, gpos);
+        const GruGates g = gru_gates(h_prev, ai, ar, i, nrec, gpos);
         r[i] = (1.0f - g.Zt) * g.Nt + g.Zt * g.Ht_1;
     }
 }
 
 __global__ void __launch_bounds__(kEwThreads)
-    gru_process_backward_kernel(float* gr, float* __restrict__ gai, float* __restrict__ gar, const float* r,
-                                const float* __restrict__ ai, const float* __restrict__ ar, int64_t nt, int64_t n,
-                                int64_t nrec) {
+    gru_process_backward_kernel(float* gr, float* __restrict__ gai, float* __restrict__ gar, const float* h_prev,
+                                const float* __restrict__ ai, const float* __restrict__ ar, int64_t n, int64_t nrec) {
     const int64_t stride = (int64_t)gridDim.x * kEwThreads;
     for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
         int64_t gpos;
-        const GruGates g = gru_gates(r, ai, ar, i, nt, n, nrec, gpos);
+        const GruGates g = gru_gates(h_prev, ai, ar, i, nrec, gpos);
         const float gHt = gr[i];
         const float gNt = (1 - g.Zt) * gHt;
         const float gZt = (g.Ht_1 - g.Nt) * gHt;
@@ -524,7 +523,16 @@ int launch_gru_process(float* r, const float* ai, const float* ar, int64_t nt, i
                        hipStream_t stream) {
     const int64_t n = ndat * nrec;
     if (n <= 0) return KAI_OK;
-    gru_process_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(r, ai, ar, nt, n, nrec);
+    // the previous time step lies one [ndat, nrec] block before r (vmath.cu:4961)
+    gru_process_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(r, nt > 0 ? r - n : nullptr, ai, ar, n, nrec);
+    return check_launch("gru_process_kernel");
+}
+
+int launch_gru_process_from(float* r, const float* h_prev, const float* ai, const float* ar, int64_t ndat, int64_t nrec,
+                            hipStream_t stream) {
+    const int64_t n = ndat * nrec;
+    if (n <= 0) return KAI_OK;
+    gru_process_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(r, h_prev, ai, ar, n, nrec);
     return check_launch("gru_process_kernel");
 }
 
@@ -532,7 +540,8 @@ int launch_gru_process_backward(float* gr, float* gai, float* gar, const float* 
                                 int64_t nt, int64_t ndat, int64_t nrec, hipStream_t stream) {
     const int64_t n = ndat * nrec;
     if (n <= 0) return KAI_OK;
-    gru_process_backward_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(gr, gai, gar, r, ai, ar, nt, n, nrec);
+    gru_process_backward_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(gr, gai, gar, nt > 0 ? r - n : nullptr, ai, ar, n,
+                                                                          nrec);
     return check_launch("gru_process_backward_kernel");
 }
 

@@ -618,6 +618,41 @@ int kai_gru_process_backward(int device, float* pgr, float* pgai, float* pgar, c
     return launch_gru_process_backward(pgr, pgai, pgar, pr, pai, par, nt, ndat, nrec, current_stream());
 }
 
+// ---- one recurrent time step per launch (additive) ----------------------------------------------------
+
+int kai_lstm_step(int device, float* pr, float* ps, const float* ps_prev, float* pa, const float* pwr,
+                  const float* pr_prev, const float* pbi, const float* pbr, int64_t ndat, int64_t nrec) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0 && nrec >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (ndat == 0 || nrec == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pr); KAI_REQUIRE_PTR(ps); KAI_REQUIRE_PTR(pa);
+    if (pr_prev) KAI_REQUIRE_PTR(pwr);
+    if (recurrent_step_applies(pwr, pr_prev, ndat, nrec))
+        return launch_lstm_step(pr, ps, ps_prev, pa, pwr, pr_prev, pbi, pbr, ndat, nrec, current_stream());
+    // the separate calls, in the engine's order (vtensor.cpp:2468-2483)
+    if (pr_prev) KAI_TRY(kai_matmul(device, pa, pwr, pr_prev, 4 * nrec, ndat, nrec, 1));
+    if (pbr) KAI_TRY(kai_add_bias(device, pa, pa, pbr, ndat, 4 * nrec));
+    if (pbi) KAI_TRY(kai_add_bias(device, pa, pa, pbi, ndat, 4 * nrec));
+    return kai_lstm_process(device, pr, ps, ps_prev, pa, ndat, nrec, 0);
+}
+
+int kai_gru_step(int device, float* pr, float* pai, float* par, const float* pwr, const float* pr_prev,
+                 const float* ph_prev, const float* pbi, const float* pbr, int64_t ndat, int64_t nrec) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0 && nrec >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (ndat == 0 || nrec == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pr); KAI_REQUIRE_PTR(pai); KAI_REQUIRE_PTR(par);
+    KAI_REQUIRE(pai != par, KAI_ERR_INVALID_ARGUMENT, "the gru keeps input and recurrent sums in separate buffers");
+    if (pr_prev) KAI_REQUIRE_PTR(pwr);
+    if (recurrent_step_applies(pwr, pr_prev, ndat, nrec))
+        return launch_gru_step(pr, pai, par, pwr, pr_prev, ph_prev, pbi, pbr, ndat, nrec, current_stream());
+    if (pr_prev) KAI_TRY(kai_matmul(device, par, pwr, pr_prev, 3 * nrec, ndat, nrec, 0));
+    else KAI_TRY(kai_set_zero(device, par, ndat * 3 * nrec * (int64_t)sizeof(float)));
+    if (pbr) KAI_TRY(kai_add_bias(device, par, par, pbr, ndat, 3 * nrec));
+    if (pbi) KAI_TRY(kai_add_bias(device, pai, pai, pbi, ndat, 3 * nrec));
+    return launch_gru_process_from(pr, ph_prev, pai, par, ndat, nrec, current_stream());
+}
+
 // ---- transposes ----------------------------------------------------------------------------------
 
 int kai_transpose(int device, float* py, const float* px, const int* pn, int64_t axis_size, int64_t data_size) {

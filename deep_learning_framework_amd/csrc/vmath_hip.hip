@@ -97,6 +97,14 @@ void VMath::gru_process_backward(int device, float* pgr, float* pgai, float* pga
                                  int64 nt, int64 ntimes, int64 ndat, int64 nrec) {
     raise_on(kai_gru_process_backward(device, pgr, pgai, pgar, pr, pai, par, nt, ntimes, ndat, nrec));
 }
+void VMath::lstm_step(int device, float* pr, float* ps, float* ps_prev, float* pa, float* pwr, float* pr_prev, float* pbi,
+                      float* pbr, int64 ndat, int64 nrec) {
+    raise_on(kai_lstm_step(device, pr, ps, ps_prev, pa, pwr, pr_prev, pbi, pbr, ndat, nrec));
+}
+void VMath::gru_step(int device, float* pr, float* pai, float* par, float* pwr, float* pr_prev, float* ph_prev, float* pbi,
+                     float* pbr, int64 ndat, int64 nrec) {
+    raise_on(kai_gru_step(device, pr, pai, par, pwr, pr_prev, ph_prev, pbi, pbr, ndat, nrec));
+}
 void VMath::transpose(int device, float* py, float* px, int* pn, int64 axis_size, int64 data_size) {
     raise_on(kai_transpose(device, py, px, pn, axis_size, data_size));
 }

@@ -68,6 +68,8 @@ SIGNATURES = {
     "kai_lstm_process": [_INT, _F, _F, _F, _F, _I64, _I64, _I64],
     "kai_gru_process": [_INT, _F, _F, _F, _I64, _I64, _I64, _I64],
     "kai_gru_process_backward": [_INT, _F, _F, _F, _F, _F, _F, _I64, _I64, _I64, _I64],
+    "kai_lstm_step": [_INT, _F, _F, _F, _F, _F, _F, _F, _F, _I64, _I64],
+    "kai_gru_step": [_INT, _F, _F, _F, _F, _F, _F, _F, _F, _I64, _I64],
     "kai_transpose": [_INT, _F, _F, _F, _I64, _I64],
     "kai_transpose_backward": [_INT, _F, _F, _F, _I64, _I64],
     "kai_transpose_bin": [_INT, _F, _F, _I64, _I64],
@@ -334,6 +336,16 @@ class VMath:
     def gru_process_backward(device, pgr, pgai, pgar, pr, pai, par, nt, ntimes, ndat, nrec):
         _ck(load().kai_gru_process_backward(device, _addr(pgr), _addr(pgai), _addr(pgar), _addr(pr), _addr(pai),
                                             _addr(par), nt, ntimes, ndat, nrec))
+
+    @staticmethod
+    def lstm_step(device, pr, ps, ps_prev, pa, pwr, pr_prev, pbi, pbr, ndat, nrec):
+        _ck(load().kai_lstm_step(device, _addr(pr), _addr(ps), _addr(ps_prev), _addr(pa), _addr(pwr), _addr(pr_prev),
+                                 _addr(pbi), _addr(pbr), ndat, nrec))
+
+    @staticmethod
+    def gru_step(device, pr, pai, par, pwr, pr_prev, ph_prev, pbi, pbr, ndat, nrec):
+        _ck(load().kai_gru_step(device, _addr(pr), _addr(pai), _addr(par), _addr(pwr), _addr(pr_prev), _addr(ph_prev),
+                                _addr(pbi), _addr(pbr), ndat, nrec))
 
     @staticmethod
     def transpose(device, py, px, pn, axis_size, data_size):

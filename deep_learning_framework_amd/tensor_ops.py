@@ -244,7 +244,7 @@ _NGATES = {"rnn": 1, "lstm": 4, "gru": 3}
 
 
 def rnn(x, wi, wr, bi, br, cell_type, rec_size, actfunc="tanh", leaky_alpha=None, forward=True, timesteps=None,
-        use_state=False, batch_input_projection=False):
+        use_state=False, batch_input_projection=False, fused_step=False):
     """One direction of a recurrent layer, as the engine's per-time-step loop issues it.
 
     ``x`` is ``[ntimes, ndat, ninp]`` (a sequence) or ``[ndat, ninp]`` (the same input at each of ``timesteps``
@@ -253,6 +253,8 @@ def rnn(x, wi, wr, bi, br, cell_type, rec_size, actfunc="tanh", leaky_alpha=None
     both in one buffer), the bias adds, then the cell.  ``batch_input_projection=True`` is the additive fusion:
     the input products of all steps are issued as ONE call over ``ntimes*ndat`` rows before the loop and the
     recurrent product accumulates onto it, which gives the same sums (a + b == b + a).
+    ``fused_step=True`` (lstm, gru; implies the batched input products for a sequence input) replaces the
+    remaining calls of a step by ONE kai_lstm_step / kai_gru_step.
     Returns the ``[ndat, nrec]`` output and the tensors the backward pass needs."""
     if cell_type not in _NGATES:
         raise KaiError(8, "rnn cell type")
@@ -287,7 +289,8 @@ def rnn(x, wi, wr, bi, br, cell_type, rec_size, actfunc="tanh", leaky_alpha=None
     xsize, ysize = ndat * ninp, ndat * nrec
     asize = ngates * ysize
     f4 = 4
-    batched = batch_input_projection and in_seq
+    fused_step = fused_step and cell_type in ("lstm", "gru")
+    batched = (batch_input_projection or fused_step) and in_seq
     if batched:
         VMath.matmul(dev, iaffines.ptr, wi.ptr, x.ptr, ngates * nrec, ntimes * ndat, ninp, False)
     for n in range(ntimes):
@@ -296,6 +299,19 @@ def rnn(x, wi, wr, bi, br, cell_type, rec_size, actfunc="tanh", leaky_alpha=None
         pai = iaffines.buf.offset(nt * asize * f4)
         par = raffines.buf.offset(nt * asize * f4)
         px = x.buf.offset(nt * xsize * f4) if in_seq else x.ptr
+        if fused_step:
+            pr_prev = recurs.buf.offset((nt - 1 if forward else nt + 1) * ysize * f4) if n > 0 else None
+            if not batched:
+                VMath.matmul(dev, pai, wi.ptr, px, ngates * nrec, ndat, ninp, True)
+            pbi, pbr = (bi.ptr, br.ptr) if use_bias else (None, None)
+            if cell_type == "lstm":
+                ps = states.buf.offset(nt * ysize * f4)
+                ps_prev = states.buf.offset((nt - 1 if forward else nt + 1) * ysize * f4) if n > 0 else None
+                VMath.lstm_step(dev, pr, ps, ps_prev, pai, wr.ptr, pr_prev, pbi, pbr, ndat, nrec)
+            else:
+                ph_prev = recurs.buf.offset((nt - 1) * ysize * f4) if nt > 0 else None   # vmath.cu:4961
+                VMath.gru_step(dev, pr, pai, par, wr.ptr, pr_prev, ph_prev, pbi, pbr, ndat, nrec)
+            continue
         if n > 0:
             pr_prev = recurs.buf.offset((nt - 1 if forward else nt + 1) * ysize * f4)
             # with the input products already in place the recurrent one accumulates (rnn, lstm: same buffer)

@@ -224,6 +224,21 @@ int kai_gru_process(int device, float* pr, const float* pai, const float* par, i
 int kai_gru_process_backward(int device, float* pgr, float* pgai, float* pgar, const float* pr, const float* pai,
                              const float* par, int64_t nt, int64_t ntimes, int64_t ndat, int64_t nrec);
 
+/* One time step of the loop above in one launch (additive, no counterpart call in the reference):
+ *   kai_lstm_step == [pr_prev: kai_matmul(pa, pwr, pr_prev, 4*nrec, ndat, nrec, acc = 1)], [kai_add_bias(pa, pbr)],
+ *                    [kai_add_bias(pa, pbi)], kai_lstm_process(pr, ps, ps_prev, pa)
+ * with pa[ndat, 4*nrec] holding the input products of this step on entry (kai_matmul over all time steps at
+ * once, or per step) and the gate sums the cell saw on return, as the backward pass needs them.  pr_prev null:
+ * first step, no recurrent product.  pbi, pbr, ps_prev may be null. */
+int kai_lstm_step(int device, float* pr, float* ps, const float* ps_prev, float* pa, const float* pwr,
+                  const float* pr_prev, const float* pbi, const float* pbr, int64_t ndat, int64_t nrec);
+/*   kai_gru_step == par = pr_prev . pwr^T (zero when pr_prev is null), [kai_add_bias(par, pbr)],
+ *                   [kai_add_bias(pai, pbi)], kai_gru_process with ph_prev as the previous output (null: 0).
+ * pr_prev and ph_prev are separate because the engine's loop reads the output of step nt - 1 in both
+ * directions (vmath.cu:4961) while the product takes the step processed before (vtensor.cpp:2464). */
+int kai_gru_step(int device, float* pr, float* pai, float* par, const float* pwr, const float* pr_prev,
+                 const float* ph_prev, const float* pbi, const float* pbr, int64_t ndat, int64_t nrec);
+
 /* ---- transposes (next to the path) ----------------------------------------------------------------- */
 
 /* VMath::transpose, vmath.cu:9384-9433 (vmath.h:309).  General axis permutation of a dense tensor of

@@ -85,6 +85,11 @@ public:
     static void gru_process(int device, float* pr, float* pai, float* par, int64 nt, int64 ntimes, int64 ndat, int64 nrec);
     static void gru_process_backward(int device, float* pgr, float* pgai, float* pgar, float* pr, float* pai, float* par,
                                      int64 nt, int64 ntimes, int64 ndat, int64 nrec);
+    // additive: one recurrent time step per launch (see kai_lstm_step / kai_gru_step)
+    static void lstm_step(int device, float* pr, float* ps, float* ps_prev, float* pa, float* pwr, float* pr_prev,
+                          float* pbi, float* pbr, int64 ndat, int64 nrec);
+    static void gru_step(int device, float* pr, float* pai, float* par, float* pwr, float* pr_prev, float* ph_prev,
+                         float* pbi, float* pbr, int64 ndat, int64 nrec);
     static void transpose(int device, float* py, float* px, int* pn, int64 axis_size, int64 data_size);
     static void transpose_backward(int device, float* pgx, float* pgy, int* pn, int64 axis_size, int64 data_size);
     static void transpose_bin(int device, float* py, float* px, int64 nrow, int64 ncol);

@@ -643,7 +643,8 @@ def _oracle_rnn_backprop(x, wi, wr, use_bias, cell, recurs, ia, ra, gy, gyt, for
 @pytest.mark.parametrize("cell", ["rnn", "lstm", "gru"])
 @pytest.mark.parametrize("ntimes,ndat,ninp,nrec,forward,bias", [(4, 3, 7, 5, True, True),       # sub-buffers at odd offsets
                                                                 (6, 16, 64, 32, False, False),
-                                                                (5, 64, 96, 128, True, True)])
+                                                                (5, 64, 96, 128, True, True),
+                                                                (3, 40, 32, 100, True, True)])       # ragged tiles
 def test_rnn_layer_loop(cell, ntimes, ndat, ninp, nrec, forward, bias):
     from deep_learning_framework_amd import tensor_ops as T
     rng = np.random.default_rng(ntimes * 100 + ndat)
@@ -655,12 +656,15 @@ def test_rnn_layer_loop(cell, ntimes, ndat, ninp, nrec, forward, bias):
     br = (rng.standard_normal(ngates * nrec) * 0.1).astype(np.float32) if bias else None
     recurs, ia, ra = _oracle_rnn(x, wi, wr, bi, br, cell, nrec, forward)
     tn = lambda a: None if a is None else T.Tensor.from_numpy(a)
-    for batched in (False, True):
+    for batched, fused in ((True, True), (False, False), (True, False)):
         y, saved = T.rnn(tn(x), tn(wi), tn(wr), tn(bi), tn(br), cell, nrec, forward=forward,
-                         batch_input_projection=batched)
-        check(saved["recurs"].numpy(), recurs, what="%s recurrent outputs (batched=%s)" % (cell, batched))
-        check(saved["iaffines"].numpy(), ia, what="%s gate pre-activations" % cell)
-        check(y.numpy(), recurs[-1 if forward else 0], what="%s output" % cell)
+                         batch_input_projection=batched, fused_step=fused)
+        mode = "batched=%s fused=%s" % (batched, fused)
+        check(saved["recurs"].numpy(), recurs, what="%s recurrent outputs (%s)" % (cell, mode))
+        check(saved["iaffines"].numpy(), ia, what="%s gate pre-activations (%s)" % (cell, mode))
+        if cell == "gru":
+            check(saved["raffines"].numpy(), ra, what="gru recurrent gate sums (%s)" % mode)
+        check(y.numpy(), recurs[-1 if forward else 0], what="%s output (%s)" % (cell, mode))
     if cell == "lstm":
         with pytest.raises(T.KaiError):
             T.rnn_backprop(saved, tn(recurs[0]), tn(recurs))
