@@ -123,6 +123,7 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
     if (shortk_nt_applies(plan.dn)) return launch_gemm_shortk_nt(make_params(plan.dn, true, true), d.nbatch, stream);
     if (shortk_heads_applies(plan.dn))
         return launch_gemm_shortk_heads(make_params(plan.dn, true, true), d.nbatch, stream);
+    if (heads_pv_applies(d)) return launch_heads_pv(d, stream);
     if (plan.split >= 2) {
         const int64_t split = plan.split;
         float* part = nullptr;

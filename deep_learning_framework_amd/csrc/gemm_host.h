@@ -96,6 +96,10 @@ int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream);
 bool shortk_heads_applies(const GemmDesc& d);
 int launch_gemm_shortk_heads(GemmParams p, int64_t nbatch, hipStream_t stream);
 
+// products of the head-interleaved attention tensor with several heads per batch entry: heads_pv.hip
+bool heads_pv_applies(const GemmDesc& d);
+int launch_heads_pv(const GemmDesc& d, hipStream_t stream);
+
 // per-layout entry points (one translation unit each, to compile in parallel)
 enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2 };
 int launch_gemm_kc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
