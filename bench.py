@@ -168,6 +168,12 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
         row(tag + "O = P.V (mix_values)",
             gpu_us(lambda: L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))),
             flops=fl, cpu=cpu_us(lambda: ko.mix_values(pbuf.cpu().numpy(), vc, nhead)))
+        def three_calls():
+            L.kai_mult_on_heads(0, P(pbuf), P(k), P(q), I(nbat), I(T), I(nvec), I(nhead), I(D), P(coef))
+            L.kai_softmax_direct_on_axis(0, P(pbuf), I(nbat * T), I(T), I(nhead))
+            L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))
+
+        row(tag + "the three calls back to back", gpu_us(three_calls), flops=2 * fl)
         row(tag + "all three fused, forward only (kai_attention_forward)",
             gpu_us(lambda: L.kai_attention_forward(0, P(o), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
                                                    P(coef), 0)),

@@ -270,7 +270,7 @@ __global__ void __launch_bounds__(kTrTile * 8) transpose_bin_kernel(float* __res
 #pragma unroll
     for (int i = 0; i < kTrTile; i += 8) {
         const int64_t r = tr * kTrTile + ty + i, c = tc * kTrTile + tx;
-        if (r < nrow && c < ncol) y[r * ncol + c] = tile[tx][ty + i];
+        if (r < nrow && c < ncol) __builtin_nontemporal_store(tile[tx][ty + i], y + r * ncol + c);
     }
 }
 

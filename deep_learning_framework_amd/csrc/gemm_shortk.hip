@@ -195,7 +195,9 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
                     float* out = C + (int64_t)row * p.c_rs + col;
                     if (row < p.M) {
                         if (p.c_vec) {   // N % 4 == 0: the four columns are inside or outside together
-                            if (col < p.N) *reinterpret_cast<f32x4*>(out) = o;
+                            // streaming: whole 512-byte rows that this kernel never reads again; otherwise the
+                            // dirty lines pile up in L2 and are written back after the last wave has ended
+                            if (col < p.N) __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(out));
                         } else {
 #pragma unroll
                             for (int j = 0; j < 4; j++)
