@@ -413,7 +413,7 @@ def test_softmax_activation_rows():
 @pytest.mark.parametrize("nbat,ntimes,nhead,npiece", [(2, 5, 1, 3), (3, 17, 4, 8), (1, 64, 2, 64), (2, 33, 3, 5),
                                                       (1, 130, 1, 64), (1, 7, 200, 2), (2, 100, 4, 16),
                                                       (1, 130, 8, 64), (1, 70, 4, 6), (1, 96, 12, 24),
-                                                      (2, 700, 8, 24), (1, 1100, 4, 6), (3, 1200, 1, 40),
+                                                      (2, 700, 8, 24), (1, 1100, 4, 6), (3, 1200, 1, 40), (1, 608, 12, 8),
                                                       # several heads per batch entry, lengths and head sizes in whole
                                                       # 32s: the kernels that take four heads per workgroup
                                                       (2, 64, 4, 32), (1, 96, 8, 64), (3, 32, 12, 32), (4, 128, 4, 96)])
