@@ -318,48 +318,132 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         return v;
     };
     const bool vec_store = !B_KC && NBN == 4 && p.c_vec;
+    // Per 32-row block: everything that has to be loaded (the old C for acc, the bias) is loaded first, at
+    // clamped addresses and under workgroup-uniform conditions only, then all stores follow back to back.
+    // Written element by element (load, wait, store, next load ...) every store waited for the one before it:
+    // the 16 stores of a 64x64 tile took 2.7 us.
+    const bool has_alpha = p.has_alpha != 0, accf = p.accflag != 0, has_bias = p.bias != nullptr;
+    auto activate_cheap = [&](float& v) {   // act is uniform: the branch is taken once per call site by all lanes
+        v = cheap_act(v);
+    };
 
     static_for<0, NBM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        static_for<0, 16>([&](auto rc) {
-            constexpr int r = decltype(rc)::value;
-            const int row = row_of(i, r);
-            const bool row_ok = row < p.M;
-            if (vec_store) {
-                const int col = col_of(0);
-                if (row_ok && col < p.N) {   // N % 4 == 0 under c_vec, so the whole chunk is inside
-                    const int64_t idx = (int64_t)row * p.c_rs + col;
-                    f32x4 o;
-                    static_for<0, 4>([&](auto jc) {
-                        constexpr int j = decltype(jc)::value;
-                        o[j] = acc[i][j % NBN][r];
-                    });
-                    if (p.has_alpha) o *= alpha;
-                    if (p.accflag) o += *reinterpret_cast<const f32x4*>(C + idx);
-                    if (p.bias) o += *reinterpret_cast<const f32x4*>(p.bias + col);
-                    if (C2) *reinterpret_cast<f32x4*>(C2 + idx) = o;
-                    static_for<0, 4>([&](auto jc) {
-                        constexpr int j = decltype(jc)::value;
-                        o[j] = cheap_act(o[j]);
-                    });
-                    *reinterpret_cast<f32x4*>(C + idx) = o;
-                }
-            } else {
-                static_for<0, NBN>([&](auto jc) {
+        int rows[16];
+        int64_t rowbase[16], rowbase_c[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            rows[r] = row_of(i, r);
+            rowbase[r] = (int64_t)rows[r] * p.c_rs;
+            rowbase_c[r] = (int64_t)(rows[r] < p.M ? rows[r] : p.M - 1) * p.c_rs;
+        }
+        if (vec_store) {
+            const int col = col_of(0);
+            const bool col_ok = col < p.N;       // N % 4 == 0 under c_vec: a chunk is inside or outside as a whole
+            const int colc = col_ok ? col : 0;
+            f32x4 o[16];
+            static_for<0, 16>([&](auto rc) {
+                constexpr int r = decltype(rc)::value;
+                static_for<0, 4>([&](auto jc) {
                     constexpr int j = decltype(jc)::value;
-                    const int col = col_of(j);
-                    if (row_ok && col < p.N) {
-                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
-                        float v = acc[i][j][r];
-                        if (p.has_alpha) v *= alpha;
-                        if (p.accflag) v += C[idx];
-                        if (p.bias) v += p.bias[col];
-                        if (C2) C2[idx] = v;
-                        C[idx] = cheap_act(v);
-                    }
+                    o[r][j] = acc[i][j % NBN][r];
                 });
+            });
+            if (has_alpha) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[r] *= alpha;
             }
-        });
+            if (accf) {
+                f32x4 cin[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) cin[r] = *reinterpret_cast<const f32x4*>(C + rowbase_c[r] + colc);
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[r] += cin[r];
+            }
+            if (has_bias) {
+                const f32x4 bv = *reinterpret_cast<const f32x4*>(p.bias + colc);
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[r] += bv;
+            }
+            if (C2) {
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (rows[r] < p.M && col_ok) *reinterpret_cast<f32x4*>(C2 + rowbase[r] + col) = o[r];
+            }
+            if (act != kActNone) {
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float v = o[r][j];
+                        activate_cheap(v);
+                        o[r][j] = v;
+                    }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                if (rows[r] < p.M && col_ok) *reinterpret_cast<f32x4*>(C + rowbase[r] + col) = o[r];
+        } else {
+            float v[NBN][16];
+            int cols[NBN];
+            int64_t coloff[NBN], coloff_c[NBN];
+#pragma unroll
+            for (int j = 0; j < NBN; j++) {
+                cols[j] = col_of(j);
+                coloff[j] = (int64_t)cols[j] * p.c_cs;
+                coloff_c[j] = (int64_t)(cols[j] < p.N ? cols[j] : 0) * p.c_cs;
+            }
+            static_for<0, NBN>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                static_for<0, 16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    v[j][r] = acc[i][j][r];
+                });
+            });
+            if (has_alpha) {
+#pragma unroll
+                for (int j = 0; j < NBN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) v[j][r] *= alpha;
+            }
+            if (accf) {
+                float cin[NBN][16];
+#pragma unroll
+                for (int j = 0; j < NBN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) cin[j][r] = C[rowbase_c[r] + coloff_c[j]];
+#pragma unroll
+                for (int j = 0; j < NBN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) v[j][r] += cin[j][r];
+            }
+            if (has_bias) {
+#pragma unroll
+                for (int j = 0; j < NBN; j++) {
+                    const float bv = p.bias[cols[j] < p.N ? cols[j] : 0];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) v[j][r] += bv;
+                }
+            }
+            if (C2) {
+#pragma unroll
+                for (int j = 0; j < NBN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        if (rows[r] < p.M && cols[j] < p.N) C2[rowbase[r] + coloff[j]] = v[j][r];
+            }
+            if (act != kActNone) {
+#pragma unroll
+                for (int j = 0; j < NBN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) activate_cheap(v[j][r]);
+            }
+#pragma unroll
+            for (int j = 0; j < NBN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (rows[r] < p.M && cols[j] < p.N) C[rowbase[r] + coloff[j]] = v[j][r];
+        }
     });
 
     if (slow_act) {
