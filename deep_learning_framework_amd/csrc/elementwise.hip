@@ -590,7 +590,7 @@ int launch_cosine_norms_and_scale(float* y, float* norms, const float* x1, const
 // Sums the partial products in split order (fixed, so the result does not depend on scheduling)
 // and applies the GEMM epilogue.  VEC: four consecutive columns per thread with 128-bit accesses.
 
-template <bool VEC>
+template <bool VEC, int NMAX>
 __global__ void __launch_bounds__(kEwThreads) splitk_reduce_kernel(SplitReduceParams p) {
     constexpr int W = VEC ? 4 : 1;
     const int64_t total = p.M * p.N;
@@ -599,17 +599,35 @@ __global__ void __launch_bounds__(kEwThreads) splitk_reduce_kernel(SplitReducePa
     const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.0f) : 1.0f;
     const float leaky = p.leaky ? *p.leaky : 0.0f;
     const int64_t m = e / p.N, n = e - m * p.N;
+    const int64_t idx = m * p.c_rs + n * p.c_cs;
+    // all NMAX >= nsplit partial sums are requested before the first one is used (parts beyond nsplit repeat
+    // the last one and are masked out of the sum), so the loads overlap instead of queueing behind the adds
     float v[W];
     if (VEC) {
-        f32x4 s = *reinterpret_cast<const f32x4*>(p.part + e);
-        for (int k = 1; k < p.nsplit; k++) s += *reinterpret_cast<const f32x4*>(p.part + k * total + e);
+        f32x4 part[NMAX];
+#pragma unroll
+        for (int k = 0; k < NMAX; k++)
+            part[k] = *reinterpret_cast<const f32x4*>(p.part + (k < p.nsplit ? k : p.nsplit - 1) * total + e);
+        f32x4 s = part[0];
+#pragma unroll
+        for (int k = 1; k < NMAX; k++) {
+            const int keep = k < p.nsplit ? -1 : 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float x = part[k][j];
+                s[j] += __int_as_float(__float_as_int(x) & keep);
+            }
+        }
         for (int j = 0; j < W; j++) v[j] = s[j];
     } else {
-        float s = p.part[e];
-        for (int k = 1; k < p.nsplit; k++) s += p.part[k * total + e];
+        float part[NMAX];
+#pragma unroll
+        for (int k = 0; k < NMAX; k++) part[k] = p.part[(k < p.nsplit ? k : p.nsplit - 1) * total + e];
+        float s = part[0];
+#pragma unroll
+        for (int k = 1; k < NMAX; k++) s += __int_as_float(__float_as_int(part[k]) & (k < p.nsplit ? -1 : 0));
         v[0] = s;
     }
-    const int64_t idx = m * p.c_rs + n * p.c_cs;
     for (int j = 0; j < W; j++) {
         float o = p.has_alpha ? v[j] * alpha : v[j];
         if (p.accflag) o += p.C[idx + j * p.c_cs];
@@ -627,16 +645,22 @@ __global__ void __launch_bounds__(kEwThreads) splitk_reduce_kernel(SplitReducePa
     }
 }
 
+template <int NMAX>
+static int launch_splitk_reduce_n(const SplitReduceParams& p, bool vec, int64_t total, hipStream_t stream) {
+    if (vec) splitk_reduce_kernel<true, NMAX><<<blocks_for(total / 4), kEwThreads, 0, stream>>>(p);
+    else splitk_reduce_kernel<false, NMAX><<<blocks_for(total), kEwThreads, 0, stream>>>(p);
+    return check_launch("splitk_reduce_kernel");
+}
+
 int launch_splitk_reduce(const SplitReduceParams& p, hipStream_t stream) {
     const int64_t total = p.M * p.N;
     if (total <= 0) return KAI_OK;
+    if (p.nsplit < 1 || p.nsplit > 16) return fail(KAI_ERR_INVALID_ARGUMENT, "split-K: 1 to 16 parts");
     const bool vec = p.c_cs == 1 && p.N % 4 == 0 && p.c_rs % 4 == 0 && aligned16(p.part) && aligned16(p.C) &&
                      (!p.C2 || aligned16(p.C2)) && (!p.bias || aligned16(p.bias));
-    if (vec)
-        splitk_reduce_kernel<true><<<blocks_for(total / 4), kEwThreads, 0, stream>>>(p);
-    else
-        splitk_reduce_kernel<false><<<blocks_for(total), kEwThreads, 0, stream>>>(p);
-    return check_launch("splitk_reduce_kernel");
+    if (p.nsplit <= 4) return launch_splitk_reduce_n<4>(p, vec, total, stream);
+    if (p.nsplit <= 8) return launch_splitk_reduce_n<8>(p, vec, total, stream);
+    return launch_splitk_reduce_n<16>(p, vec, total, stream);
 }
 
 }  // namespace kai
