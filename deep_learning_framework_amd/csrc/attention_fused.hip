@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
     const int qc = min(q, T - 1);
     f32x4 qf[DB];
 #pragma unroll
-    for (int s = 0; s < DB; s++) qf[s] = *reinterpret_cast<const f32x4*>(Qb + (int64_t)qc * p.nvec + 16 * s + 4 * g);
+    for (int s = 0; s < DB; s++) qf[s] = c2 * *reinterpret_cast<const f32x4*>(Qb + (int64_t)qc * p.nvec + 16 * s + 4 * g);
 
     // key tiles that hold an unmasked key for some query of this workgroup
     const int q_last = min(q0 + kFaQ, T) - 1;
@@ -119,9 +119,14 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
             const int kl = c / kChunksPerKey;
             const int d = (c % kChunksPerKey) * 4;
             if (!kPartial || c < kTileChunks) {
-                const bool inside = kt * kFaKeys + kl < T;   // keys past the end: zeros (their scores are masked)
-                *reinterpret_cast<f32x4*>(&lds_k[buf][kl * kKStride + d]) = keep4(rk[i], inside);
-                *reinterpret_cast<f32x4*>(&lds_v[buf][kl * kVStride + d]) = keep4(rv[i], inside);
+                if (kt * kFaKeys + kFaKeys <= T) {   // uniform: only the last tile can reach past the end
+                    *reinterpret_cast<f32x4*>(&lds_k[buf][kl * kKStride + d]) = rk[i];
+                    *reinterpret_cast<f32x4*>(&lds_v[buf][kl * kVStride + d]) = rv[i];
+                } else {
+                    const bool inside = kt * kFaKeys + kl < T;   // keys past the end: zeros (their scores are masked)
+                    *reinterpret_cast<f32x4*>(&lds_k[buf][kl * kKStride + d]) = keep4(rk[i], inside);
+                    *reinterpret_cast<f32x4*>(&lds_v[buf][kl * kVStride + d]) = keep4(rv[i], inside);
+                }
             }
         }
     };
@@ -159,21 +164,23 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
                     for (int kb = 0; kb < 2; kb++)
                         sc[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[kb][e], qf[s][e], sc[kb], 0, 0, 0);
             }
-            // sc[kb][v] = score of (query q, key key0 + 16*kb + 4*g + v), kept in the base-2 domain:
-            // exp(coef * s - m) = 2^(c2 * s - m2) with c2 = coef * log2(e), one v_exp_f32 per element
+            // sc[kb][v] = score of (query q, key key0 + 16*kb + 4*g + v) in the base-2 domain (Q was scaled by
+            // c2 = coef * log2(e) when it was loaded): exp(coef * s - m) = 2^(c2 * s - m2), one v_exp_f32 per element
             const bool edge_tile = key0 + 32 > T || (p.masked && key0 + 31 > q0 + 16 * qg);   // wave-uniform
-            float m_tile = -INFINITY;
+            // fp32 MFMAs and vector ALU instructions take turns on a SIMD (measured: their times add up), so the
+            // 16 compares and selects of the mask are kept off the tiles that do not need them by a real branch
+            if (edge_tile) {   // keys past the end or above the diagonal of some query of this wave
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    sc[kb][v] *= c2;
-                    if (edge_tile) {   // keys past the end or above the diagonal of some query of this wave
+                    for (int v = 0; v < 4; v++) {
                         const int key = key0 + 16 * kb + 4 * g + v;
                         if (key >= T || (p.masked && key > q)) sc[kb][v] = -INFINITY;
                     }
-                    m_tile = fmaxf(m_tile, sc[kb][v]);
-                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            float m_tile = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
+                                 fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16));
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32));
             const float m_new = fmaxf(m_run, m_tile);
@@ -190,8 +197,11 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
             l_run = l_run * rescale + l_tile;
             m_run = m_new;
             // O^T[d, q] = O^T * rescale + sum_key V[key, d] * P[q, key]
+            // the running maximum rarely moves after the first tiles: skip the 4*DB multiplies when no lane needs them
+            if (__builtin_amdgcn_ballot_w64(rescale != 1.0f) != 0) {
 #pragma unroll
-            for (int db = 0; db < DB; db++) acc_o[db] *= rescale;
+                for (int db = 0; db < DB; db++) acc_o[db] *= rescale;
+            }
             // V^T[d = 16*db + r16][key = 16*kb + 4*g + e]: 32-bit reads down a column of the tile (consecutive
             // lanes, consecutive d: no bank conflict); a transposed tile would allow 128-bit reads but costs
             // element-wise LDS stores with 8-way conflicts on the way in.  The DB output blocks alternate.
