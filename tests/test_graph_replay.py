@@ -17,7 +17,7 @@ import pytest
 
 @pytest.mark.gpu
 def test_training_step_graph_replays_equal_eager():
-    out = subprocess.run([sys.executable, "-u", os.path.abspath(__file__)], capture_output=True, text=True, timeout=170)
+    out = subprocess.run([sys.executable, "-u", os.path.abspath(__file__)], capture_output=True, text=True, timeout=280)
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-3000:]
     assert "graph replays equal eager" in out.stdout
 
