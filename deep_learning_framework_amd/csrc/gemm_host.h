@@ -67,6 +67,14 @@ inline bool fits_without_edges(const GemmParams& p, bool a_kc, bool b_kc, int BM
            a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30);
 }
 
+// The pipelined kernels address their operands as a 32-bit byte offset from the first row of the workgroup's
+// tile (buffer loads): the whole extent of a tile row block must stay below 2 GiB.
+inline bool fits_buffer_offsets(const GemmParams& p, bool a_kc, bool b_kc, int BM, int BN) {
+    const int64_t a_span = a_kc ? (BM - 1) * p.a_rs + p.K : (p.K - 1) * p.a_ks + BM;
+    const int64_t b_span = b_kc ? (BN - 1) * p.b_rs + p.K : (p.K - 1) * p.b_ks + BN;
+    return a_span * 4 < (1ll << 31) && b_span * 4 < (1ll << 31);
+}
+
 template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
           int DEPTH = 1, bool ROWSUM = false>
 int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t stream) {

@@ -29,11 +29,11 @@ template <bool A_KC, bool B_KC>
 int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream) {
     switch (tile) {
     case kTileLarge:
-        if (fits_without_edges(p, A_KC, B_KC, 256, 256, 16))
+        if (fits_without_edges(p, A_KC, B_KC, 256, 256, 16) && fits_buffer_offsets(p, A_KC, B_KC, 256, 256))
             return launch_gemm_config<2, 4, 4, 2, 16, A_KC, B_KC, false, 1>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<2, 4, 4, 2, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);
     case kTileMedium:
-        if (fits_without_edges(p, A_KC, B_KC, 128, 128, 32))
+        if (fits_without_edges(p, A_KC, B_KC, 128, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 128, 128))
             return launch_gemm_config<2, 2, 2, 2, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<2, 2, 2, 2, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);
     default:

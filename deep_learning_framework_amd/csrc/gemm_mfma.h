@@ -119,6 +119,20 @@ __device__ __forceinline__ void load_tile_fast(f32x4 (&reg)[ROWS * BK / 4 / NT],
     }
 }
 
+// The same chunk through a buffer load: address = resource base + a uniform byte offset (scalar registers) +
+// the thread's constant byte offset.  In the pipelined loop this leaves NO vector instruction per load; with
+// flat addresses the compiler keeps a 64-bit pointer per load in vector registers and advances each of them
+// every tile, and vector instructions take their time from the fp32 MFMAs.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+template <bool KC, int ROWS, int BK, int NT>
+__device__ __forceinline__ void load_tile_chunk_buf(f32x4 (&reg)[ROWS * BK / 4 / NT], __amdgpu_buffer_rsrc_t rsrc,
+                                                    int tile_off, int ld_bytes, int toff_bytes, int i) {
+    using TS = TileShape<KC, ROWS, BK>;
+    constexpr int kLinesPerPass = NT / TS::kChunksPerLine;
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, toff_bytes, tile_off + i * kLinesPerPass * ld_bytes, 0);
+    reg[i] = __builtin_bit_cast(f32x4, v);
+}
+
 // One chunk of the predicate-free load (chunk i of the calling thread).
 template <bool KC, int ROWS, int BK, int NT>
 __device__ __forceinline__ void load_tile_chunk(f32x4 (&reg)[ROWS * BK / 4 / NT], const float* __restrict__ base,
@@ -682,6 +696,19 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         constexpr int kMfma = 4 * NBM * NBN;                  // MFMAs per group
         Frag<A_KC, NBM> fa[2];
         Frag<B_KC, NBN> fb[2];
+        // buffer resources over the two operands from this workgroup's tile rows on (the host has checked that
+        // every offset of the tile row fits 31 bits); stride 0, no bounds beyond 4 GiB, raw 32-bit data format
+        // (the bases are the same in every lane; saying so keeps the compiler from looping over "distinct" resources)
+        auto uniform_ptr = [](const float* q) -> float* {
+            const uint64_t a = reinterpret_cast<uint64_t>(q);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+            const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+            return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
+        };
+        const __amdgpu_buffer_rsrc_t rsrc_a =
+            __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Ab), 0, (int)0xFFFFFFFFu, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rsrc_b =
+            __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Bb), 0, (int)0xFFFFFFFFu, 0x00020000);
         if (nkt > 0) {
             load_global(0);
             store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
@@ -697,8 +724,7 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         auto group = [&](int use, int fill, bool read, int rbuf, int rkg, bool store, int wbuf, bool gload, int gkt) {
             const int memops = (store || gload) ? kWrites : 0;
             const int slots = (read ? kReads : 0) > memops ? (read ? kReads : 0) : memops;
-            const float* gap = Ab + (int64_t)gkt * BK * p.a_ks;
-            const float* gbp = Bb + (int64_t)gkt * BK * p.b_ks;
+            const int ga_off = gkt * BK * (int)p.a_ks * 4, gb_off = gkt * BK * (int)p.b_ks * 4;   // bytes, uniform
             const int per = slots > 0 ? kMfma / slots : kMfma;
             int q = 0;
 #pragma unroll
@@ -715,8 +741,8 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
                         else store_tile_chunk<B_KC, BN, BK, NT>(lds_b[wbuf], rb, tid, sl - NCHA);
                     }
                     if (gload && sl < kWrites) {
-                        if (sl < NCHA) load_tile_chunk<A_KC, BM, BK, NT>(ra, gap, a_ld, toff_a, sl);
-                        else load_tile_chunk<B_KC, BN, BK, NT>(rb, gbp, b_ld, toff_b, sl - NCHA);
+                        if (sl < NCHA) load_tile_chunk_buf<A_KC, BM, BK, NT>(ra, rsrc_a, ga_off, (int)a_ld * 4, (int)toff_a * 4, sl);
+                        else load_tile_chunk_buf<B_KC, BN, BK, NT>(rb, rsrc_b, gb_off, (int)b_ld * 4, (int)toff_b * 4, sl - NCHA);
                     }
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
