@@ -331,7 +331,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         if (act == kActLeaky) return (v > 0) ? v : v * leaky;
         return v;
     };
-    const bool vec_store = !B_KC && NBN == 4 && p.c_vec;
+    const bool vec_store = !B_KC && (NBN == 4 || NBN == 2) && p.c_vec;
     // Per 32-row block: everything that has to be loaded (the old C for acc, the bias) is loaded first, at
     // clamped addresses and under workgroup-uniform conditions only, then all stores follow back to back.
     // Written element by element (load, wait, store, next load ...) every store waited for the one before it:
@@ -352,13 +352,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             rowbase_c[r] = (int64_t)(rows[r] < p.M ? rows[r] : p.M - 1) * p.c_rs;
         }
         if (vec_store) {
+            // the NBN columns of a lane are adjacent in memory: one store of NBN floats per row
+            constexpr int VW = (NBN == 2 || NBN == 4) ? NBN : 4;
+            typedef float vecw __attribute__((ext_vector_type(VW)));
             const int col = col_of(0);
             const bool col_ok = col < p.N;       // N % 4 == 0 under c_vec: a chunk is inside or outside as a whole
             const int colc = col_ok ? col : 0;
-            f32x4 o[16];
+            vecw o[16];
             static_for<0, 16>([&](auto rc) {
                 constexpr int r = decltype(rc)::value;
-                static_for<0, 4>([&](auto jc) {
+                static_for<0, VW>([&](auto jc) {
                     constexpr int j = decltype(jc)::value;
                     o[r][j] = acc[i][j % NBN][r];
                 });
@@ -368,27 +371,27 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                 for (int r = 0; r < 16; r++) o[r] *= alpha;
             }
             if (accf) {
-                f32x4 cin[16];
+                vecw cin[16];
 #pragma unroll
-                for (int r = 0; r < 16; r++) cin[r] = *reinterpret_cast<const f32x4*>(C + rowbase_c[r] + colc);
+                for (int r = 0; r < 16; r++) cin[r] = *reinterpret_cast<const vecw*>(C + rowbase_c[r] + colc);
 #pragma unroll
                 for (int r = 0; r < 16; r++) o[r] += cin[r];
             }
             if (has_bias) {
-                const f32x4 bv = *reinterpret_cast<const f32x4*>(p.bias + colc);
+                const vecw bv = *reinterpret_cast<const vecw*>(p.bias + colc);
 #pragma unroll
                 for (int r = 0; r < 16; r++) o[r] += bv;
             }
             if (C2) {
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    if (rows[r] < p.M && col_ok) *reinterpret_cast<f32x4*>(C2 + rowbase[r] + col) = o[r];
+                    if (rows[r] < p.M && col_ok) *reinterpret_cast<vecw*>(C2 + rowbase[r] + col) = o[r];
             }
             if (act != kActNone) {
 #pragma unroll
                 for (int r = 0; r < 16; r++)
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
+                    for (int j = 0; j < VW; j++) {
                         float v = o[r][j];
                         activate_cheap(v);
                         o[r][j] = v;
@@ -396,7 +399,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             }
 #pragma unroll
             for (int r = 0; r < 16; r++)
-                if (rows[r] < p.M && col_ok) *reinterpret_cast<f32x4*>(C + rowbase[r] + col) = o[r];
+                if (rows[r] < p.M && col_ok) *reinterpret_cast<vecw*>(C + rowbase[r] + col) = o[r];
         } else {
             float v[NBN][16];
             int cols[NBN];
