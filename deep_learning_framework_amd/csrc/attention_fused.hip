@@ -42,18 +42,6 @@ struct FusedParams {
     int masked;
 };
 
-// v where keep, else zeros: bitwise, so that the load that produced v stays unconditional
-__device__ __forceinline__ f32x4 keep4(f32x4 v, bool keep) {
-    const int m = keep ? -1 : 0;
-    f32x4 r;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const float e = v[j];
-        r[j] = __int_as_float(__float_as_int(e) & m);
-    }
-    return r;
-}
-
 // DB = npiece / 16.  Two sets of four waves share a tile of 64 keys, 32 keys each, and keep separate
 // running maxima, sums and outputs that are merged once at the end: a SIMD then holds two waves of
 // the workgroup, and the softmax arithmetic and LDS waits of one run under the MFMAs of the other.
@@ -98,17 +86,34 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
     const int q_last = min(q0 + kFaQ, T) - 1;
     const int nkt = p.masked ? q_last / kFaKeys + 1 : (T + kFaKeys - 1) / kFaKeys;
 
-    // tile loads: chunk c of a thread = (key c / (D/4), d 4 * (c % (D/4))), the same for K and V
+    // tile loads: chunk c of a thread = (key c / (D/4), d 4 * (c % (D/4))), the same for K and V.  Buffer loads:
+    // resource = this (batch entry, head)'s rows of K / V up to the last key, lane offset constant, tile offset
+    // scalar, so a tile costs no vector instruction for addresses, and keys past the end read as zeros (their
+    // scores are masked) without a clamp or a mask.  Vector instructions take their time from the fp32 MFMAs.
+    auto uniform_ptr = [](const float* q) -> float* {
+        const uint64_t a = reinterpret_cast<uint64_t>(q);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
+    };
+    const int extent = (int)(((int64_t)(T - 1) * p.nvec + D) * 4);   // bytes; the host keeps it below 2 GiB
+    const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Kb), 0, extent, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Vb), 0, extent, 0x00020000);
+    const int tile_bytes = kFaKeys * (int)p.nvec * 4;
+    int choff[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * kFaThreads;
+        choff[i] = ((c / kChunksPerKey) * (int)p.nvec + (c % kChunksPerKey) * 4) * 4;
+    }
     f32x4 rk[NCH], rv[NCH];
     auto load_tile = [&](int kt) {
 #pragma unroll
         for (int i = 0; i < NCH; i++) {
             const int c = tid + i * kFaThreads;
-            const int key = min(kt * kFaKeys + c / kChunksPerKey, T - 1);
-            const int d = (c % kChunksPerKey) * 4;
             if (!kPartial || c < kTileChunks) {
-                rk[i] = *reinterpret_cast<const f32x4*>(Kb + (int64_t)key * p.nvec + d);
-                rv[i] = *reinterpret_cast<const f32x4*>(Vb + (int64_t)key * p.nvec + d);
+                rk[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, choff[i], kt * tile_bytes, 0));
+                rv[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_v, choff[i], kt * tile_bytes, 0));
             }
         }
     };
@@ -119,14 +124,8 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
             const int kl = c / kChunksPerKey;
             const int d = (c % kChunksPerKey) * 4;
             if (!kPartial || c < kTileChunks) {
-                if (kt * kFaKeys + kFaKeys <= T) {   // uniform: only the last tile can reach past the end
-                    *reinterpret_cast<f32x4*>(&lds_k[buf][kl * kKStride + d]) = rk[i];
-                    *reinterpret_cast<f32x4*>(&lds_v[buf][kl * kVStride + d]) = rv[i];
-                } else {
-                    const bool inside = kt * kFaKeys + kl < T;   // keys past the end: zeros (their scores are masked)
-                    *reinterpret_cast<f32x4*>(&lds_k[buf][kl * kKStride + d]) = keep4(rk[i], inside);
-                    *reinterpret_cast<f32x4*>(&lds_v[buf][kl * kVStride + d]) = keep4(rv[i], inside);
-                }
+                *reinterpret_cast<f32x4*>(&lds_k[buf][kl * kKStride + d]) = rk[i];
+                *reinterpret_cast<f32x4*>(&lds_v[buf][kl * kVStride + d]) = rv[i];
             }
         }
     };
@@ -258,6 +257,7 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
 bool attention_fused_applies(const float* q, const float* k, const float* v, const float* o, int64_t ntimes,
                              int64_t nvec, int64_t nhead, int64_t npiece) {
     return (npiece == 16 || npiece == 32 || npiece == 64) && nvec % 4 == 0 && ntimes >= 1 && ntimes <= kMaxDim &&
+           ntimes * nvec * 4 < (1ll << 31) &&
            nhead >= 1 && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o);
 }
 
