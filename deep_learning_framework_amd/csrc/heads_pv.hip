@@ -64,22 +64,35 @@ __global__ void __launch_bounds__(kHpThreads) heads_pv_kernel(HeadsPvParams p) {
     const int nkt = p.T / kHpTile;
 
     // per-thread coordinates of the 128-bit pieces: P piece c = position (second axis pq, third axis pk),
-    // X piece c = (reduction row xr, head xh, four columns from 4 * xd)
-    int64_t poff[kHpChunks], xoff[kHpChunks];
+    // X piece c = (reduction row xr, head xh, four columns from 4 * xd).  Buffer loads: resource = this batch
+    // entry's part of P / X from the workgroup's heads on, lane offsets constant, tile offset scalar, so that a
+    // tile costs no vector instruction for addresses (they would take their time from the fp32 MFMAs).
+    int poff[kHpChunks], xoff[kHpChunks];   // bytes
     int plds[kHpChunks], xlds[kHpChunks];
 #pragma unroll
     for (int c = 0; c < kHpChunks; c++) {
         const int idx = tid + kHpThreads * c;
         const int pk = idx & 31, pq = idx >> 5;
         // plain: rows pq are the workgroup's output rows, pk walks the reduction; transposed: the other way round
-        poff[c] = TRANS ? ((int64_t)pq * T + (o0 + pk)) * H : ((int64_t)(o0 + pq) * T + pk) * H;
+        poff[c] = (int)((TRANS ? ((int64_t)pq * T + (o0 + pk)) * H : ((int64_t)(o0 + pq) * T + pk) * H) * 4);
         plds[c] = pq * kHpPStride + pk;
         const int xd = idx & 7, xh = (idx >> 3) & 3, xr = idx >> 5;
-        xoff[c] = (int64_t)xr * HD + (int64_t)xh * p.D + 4 * xd;
+        xoff[c] = (int)(((int64_t)xr * HD + (int64_t)xh * p.D + 4 * xd) * 4);
         xlds[c] = xh * (kHpTile * kHpXStride) + xr * kHpXStride + 4 * xd;
     }
-    const int64_t pstep = TRANS ? (int64_t)kHpTile * T * H : (int64_t)kHpTile * H;   // one tile along the reduction
-    const int64_t xstep = (int64_t)kHpTile * HD;
+    const int pstep = (int)((TRANS ? (int64_t)kHpTile * T * H : (int64_t)kHpTile * H) * 4);   // one tile along the reduction
+    const int xstep = (int)((int64_t)kHpTile * HD * 4);
+    auto uniform_ptr = [](const float* q) -> float* {
+        const uint64_t a = reinterpret_cast<uint64_t>(q);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
+    };
+    // (the host keeps a batch entry of P and of X below 2 GiB)
+    const __amdgpu_buffer_rsrc_t rsrc_p =
+        __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Pb), 0, (int)(T * T * H * 4 - kHpHeads * g * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+        uniform_ptr(Xb), 0, (int)(T * HD * 4 - ((int64_t)(kHpHeads * g) * p.D + kHpTile * db) * 4), 0x00020000);
 
     f32x4 rp[kHpDepth][kHpChunks], rx[kHpDepth][kHpChunks];
     f32x16 acc;
@@ -89,12 +102,12 @@ __global__ void __launch_bounds__(kHpThreads) heads_pv_kernel(HeadsPvParams p) {
     // every load is unconditional: a tile index past the end repeats the last tile, which is never stored
     auto load_into = [&](int kt, f32x4(&dp)[kHpChunks], f32x4(&dx)[kHpChunks]) {
         const int ktc = kt < nkt ? kt : nkt - 1;
-        const float* pp = Pb + ktc * pstep;
-        const float* xp = Xb + ktc * xstep;
 #pragma unroll
-        for (int c = 0; c < kHpChunks; c++) dp[c] = *reinterpret_cast<const f32x4*>(pp + poff[c]);
+        for (int c = 0; c < kHpChunks; c++)
+            dp[c] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, poff[c], ktc * pstep, 0));
 #pragma unroll
-        for (int c = 0; c < kHpChunks; c++) dx[c] = *reinterpret_cast<const f32x4*>(xp + xoff[c]);
+        for (int c = 0; c < kHpChunks; c++)
+            dx[c] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, xoff[c], ktc * xstep, 0));
     };
     auto store_lds = [&](int buf, const f32x4(&sp)[kHpChunks], const f32x4(&sx)[kHpChunks]) {
 #pragma unroll
@@ -175,7 +188,7 @@ bool heads_pv_applies(const GemmDesc& d) {
     if (d.c_cs != 1 || d.c_rs != H * D || d.c_bs1 != D || d.c_bs0 != T * H * D) return false;
     if (d.acc || d.bias || d.C2 || d.act != kActNone || d.has_alpha || d.rowsum || d.k_part != 0) return false;
     if (!aligned16(d.A) || !aligned16(d.B)) return false;
-    return T <= (1 << 20) && D <= (1 << 20);
+    return T * T * H * 4 < (1ll << 31) && T * H * D * 4 < (1ll << 31);
 }
 
 int launch_heads_pv(const GemmDesc& d, hipStream_t stream) {
