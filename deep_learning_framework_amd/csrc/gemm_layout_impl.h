@@ -20,7 +20,7 @@ template <bool A_KC, bool B_KC>
 int launch_gemm_layout_rowsum(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream) {
     if (tile == kTileMedium)
         return launch_gemm_config<2, 2, 2, 2, 16, A_KC, B_KC, true, 0, 1, 1, true>(p, nbatch, kGroupM, stream);
-    if (fits_without_edges(p, A_KC, B_KC, 64, 64, 16))
+    if (fits_without_edges(p, A_KC, B_KC, 64, 64, 16) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
         return launch_gemm_config<2, 2, 1, 1, 16, A_KC, B_KC, false, 0, 2, 8, true>(p, nbatch, kGroupM, stream);
     return launch_gemm_config<2, 2, 1, 1, 16, A_KC, B_KC, true, 0, 1, 1, true>(p, nbatch, kGroupM, stream);
 }
@@ -39,9 +39,9 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
     default:
         // a 64x64x16 tile computes for ~0.25 us, a global load takes ~1-2 us: 128 reduction steps in flight
         // (measured with whole tiles of 32 steps against 16 and 64: 15.5 / 16.9 / 16.0 us for 256x1024x1024)
-        if (fits_without_edges(p, A_KC, B_KC, 64, 64, 32))
+        if (fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
             return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, false, 0, 2, 4>(p, nbatch, kGroupM, stream);
-        if (fits_without_edges(p, A_KC, B_KC, 64, 64, 16))
+        if (fits_without_edges(p, A_KC, B_KC, 64, 64, 16) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
             return launch_gemm_config<2, 2, 1, 1, 16, A_KC, B_KC, false, 0, 2, 8>(p, nbatch, kGroupM, stream);
         // 32-step tiles halve the number of rounds; with an operand that is strided in both directions (one
         // head of an interleaved tensor) the element-wise loads of a tile cost more than the round saves

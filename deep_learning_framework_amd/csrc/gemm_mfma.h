@@ -586,6 +586,21 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         load_tile_fast<B_KC, BN, BK, NT>(rb, Bb + (int64_t)kt * BK * p.b_ks, b_ld, toff_b);
     };
 
+    // Whole-tile kernels read their operand tiles with buffer loads: resources over the two operands from this
+    // workgroup's tile rows on (the host has checked that every offset of the tile row block fits 31 bits); stride 0,
+    // no bounds below 4 GiB, raw 32-bit data format.  The bases are the same in every lane; saying so keeps the
+    // compiler from looping over "distinct" resources.
+    auto uniform_ptr = [](const float* q) -> float* {
+        const uint64_t a = reinterpret_cast<uint64_t>(q);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
+    };
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Ab), 0, (int)0xFFFFFFFFu, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Bb), 0, (int)0xFFFFFFFFu, 0x00020000);
+
     if (PIPE == 0) {
         // The whole loop exists once per combination of 128-bit / element-wise loads of A and B.  The
         // choice is made once per workgroup: a loop body that holds both kinds of load behind a branch
@@ -600,8 +615,12 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
                 const float* ap = Ab + (int64_t)k0 * p.a_ks;
                 const float* bp = Bb + (int64_t)k0 * p.b_ks;
                 if (!EDGE) {
-                    load_tile_fast<A_KC, BM, BK, NT>(da, ap, a_ld, toff_a);
-                    load_tile_fast<B_KC, BN, BK, NT>(db, bp, b_ld, toff_b);
+#pragma unroll
+                    for (int i = 0; i < NCHA; i++)
+                        load_tile_chunk_buf<A_KC, BM, BK, NT>(da, rsrc_a, k0 * (int)p.a_ks * 4, (int)a_ld * 4, (int)toff_a * 4, i);
+#pragma unroll
+                    for (int i = 0; i < NCHB; i++)
+                        load_tile_chunk_buf<B_KC, BN, BK, NT>(db, rsrc_b, k0 * (int)p.b_ks * 4, (int)b_ld * 4, (int)toff_b * 4, i);
                 } else {
                     load_tile_edge<A_KC, BM, BK, NT, VA>(da, ap, p.a_rs, p.a_ks, rows_a, Kz - k0, tid);
                     load_tile_edge<B_KC, BN, BK, NT, VB>(db, bp, p.b_rs, p.b_ks, rows_b, Kz - k0, tid);
@@ -699,19 +718,6 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         constexpr int kMfma = 4 * NBM * NBN;                  // MFMAs per group
         Frag<A_KC, NBM> fa[2];
         Frag<B_KC, NBN> fb[2];
-        // buffer resources over the two operands from this workgroup's tile rows on (the host has checked that
-        // every offset of the tile row fits 31 bits); stride 0, no bounds beyond 4 GiB, raw 32-bit data format
-        // (the bases are the same in every lane; saying so keeps the compiler from looping over "distinct" resources)
-        auto uniform_ptr = [](const float* q) -> float* {
-            const uint64_t a = reinterpret_cast<uint64_t>(q);
-            const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
-            const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
-            return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
-        };
-        const __amdgpu_buffer_rsrc_t rsrc_a =
-            __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Ab), 0, (int)0xFFFFFFFFu, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rsrc_b =
-            __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Bb), 0, (int)0xFFFFFFFFu, 0x00020000);
         if (nkt > 0) {
             load_global(0);
             store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
