@@ -141,7 +141,9 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
             const int n = c >> 4;
             const int k = (c & 15) * 4;
 #pragma unroll
-            for (int j = 0; j < 4; j++) lds_b[(k + j) * TileB::kStride + n] = rb[i][j];
+            // plain epilogue: the scale goes into the panel once per workgroup instead of into every output (64
+            // multiplies per lane and tile, which would take their time from the MFMAs)
+            for (int j = 0; j < 4; j++) lds_b[(k + j) * TileB::kStride + n] = FULL ? rb[i][j] : rb[i][j] * alpha;
         }
         stage_a(tm_first, 0);
     }
@@ -158,24 +160,25 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
         const float* la = lds_a[it & 1];
 
         f32x16 acc[1][4];
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[0][j][r] = 0.f;
         const bool rows_inside = m0 + wm0 < p.M;   // wave-uniform
         if (rows_inside) {
-#pragma unroll
-            for (int kg = 0; kg < NG; kg++) {
+            static_for<0, NG>([&](auto kgc) {
+                constexpr int kg = decltype(kgc)::value;
                 Frag<true, 1> fa;
                 Frag<false, 4> fb;
                 read_frag<true, 1, kSkBM, kSkK>(fa, la, wm0, kg, l32, half);
                 read_frag<false, 4, kSkBN, kSkK>(fb, lds_b, 0, kg, l32, half);
+                static_for<0, 4>([&](auto tc) {
+                    constexpr int t = decltype(tc)::value;
 #pragma unroll
-                for (int t = 0; t < 4; t++)
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(0, t), fb.get(j, t), acc[0][j], 0, 0, 0);
-            }
+                    for (int j = 0; j < 4; j++) {
+                        // the first product of an accumulator starts from a zero constant: no 64 moves to clear them
+                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(0, t), fb.get(j, t),
+                                                                        (kg == 0 && t == 0) ? zero : acc[0][j], 0, 0, 0);
+                    }
+                });
+            });
         }
         // the next tile moves to LDS before this tile's stores are issued: the wait for its loads
         // then never includes a store
@@ -190,8 +193,7 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
                 static_for<0, 16>([&](auto rc) {
                     constexpr int r = decltype(rc)::value;
                     const int row = m0 + wm0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    f32x4 o = {acc[0][0][r], acc[0][1][r], acc[0][2][r], acc[0][3][r]};
-                    o *= alpha;
+                    const f32x4 o = {acc[0][0][r], acc[0][1][r], acc[0][2][r], acc[0][3][r]};   // scaled through B
                     float* out = C + (int64_t)row * p.c_rs + col;
                     if (row < p.M) {
                         if (p.c_vec) {   // N % 4 == 0: the four columns are inside or outside together
