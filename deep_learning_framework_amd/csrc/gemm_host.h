@@ -79,6 +79,12 @@ template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool E
           int DEPTH = 1, bool ROWSUM = false>
 int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t stream) {
     constexpr int BM = WM * NBM * 32, BN = WN * NBN * 32;
+    {
+        // byte span of one tile of each operand (its lane offsets are 32-bit in the buffer-load variants)
+        const int64_t a_span = ((BM - 1) * p.a_rs + (BK - 1) * p.a_ks + 1) * 4;
+        const int64_t b_span = ((BN - 1) * p.b_rs + (BK - 1) * p.b_ks + 1) * 4;
+        p.edge_buf = a_span < (1ll << 31) && b_span < (1ll << 31);
+    }
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     p.group_m = group_m < 1 ? 1 : group_m;

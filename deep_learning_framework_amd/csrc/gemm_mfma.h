@@ -74,6 +74,7 @@ struct GemmParams {
     int64_t a_bs0, a_bs1, b_bs0, b_bs1, c_bs0, c_bs1;
     int bdiv;
     int a_vec, b_vec, c_vec;  // 128-bit access along the contiguous index is legal
+    int edge_buf;             // general kernels: a tile of either operand spans less than 2 GiB (buffer loads)
     int act;
     int accflag;
     int has_alpha;        // 1: multiply by (*alpha, or 0 if alpha is null)
@@ -207,6 +208,56 @@ __device__ __forceinline__ void mask_tile_edge(f32x4 (&reg)[ROWS * BK / 4 / NT],
             const int keep = (rj < rows_left && kj < k_left) ? -1 : 0;
             const float e = reg[i][j];
             reg[i][j] = __int_as_float(__float_as_int(e) & keep);
+        }
+    }
+}
+
+// The general tile through buffer loads.  A thread's byte offsets inside a tile do not change from tile to tile
+// (edge_offsets, computed once); the tile itself is addressed by a resource that starts at the tile and ends with
+// the operand (edge_resource, scalar arithmetic), so nothing is clamped: an address past the end of the operand
+// returns zero instead of faulting, an address that wraps into a neighbouring row returns data that mask_tile_edge
+// removes.  No vector instruction per load is left in the loop, where they would take their time from the MFMAs;
+// the flat version above spends about six per element on clamps and 64-bit sums.
+template <bool KC, int ROWS, int BK, int NT, bool VEC>
+__device__ __forceinline__ void edge_offsets(int (&voff)[ROWS * BK / 4 / NT][VEC ? 1 : 4], int64_t rs, int64_t ks, int tid) {
+    using TS = TileShape<KC, ROWS, BK>;
+    constexpr int NCH = TS::kChunks / NT;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * NT;
+        const int line = c / TS::kChunksPerLine;
+        const int off = (c % TS::kChunksPerLine) * 4;
+        const int r = KC ? line : off;
+        const int k = KC ? off : line;
+#pragma unroll
+        for (int j = 0; j < (VEC ? 1 : 4); j++) {
+            const int rj = KC ? r : r + j, kj = KC ? k + j : k;
+            voff[i][j] = (int)(((int64_t)rj * rs + (int64_t)kj * ks) * 4);   // the host has checked the tile's span
+        }
+    }
+}
+
+// base: address of element (row 0 of the workgroup's rows, k = 0) as an integer known to be uniform;
+// rows_total: rows from there to the end of the operand; k_total: reduction length from k = 0
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t edge_resource(uint64_t base, int64_t rs, int64_t ks, int rows_total,
+                                                                int k_total, int k0) {
+    const uint64_t addr = base + (uint64_t)((int64_t)k0 * ks * 4);
+    int64_t ext = ((int64_t)(rows_total - 1) * rs + (int64_t)(k_total - k0 - 1) * ks + 1) * 4;
+    if (ext > 0xFFFFFFFFll) ext = 0xFFFFFFFFll;   // a tile's own span is below 2 GiB: then all of it is inside
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(addr), 0, (int)(uint32_t)ext, 0x00020000);
+}
+
+template <int NCH, bool VEC>
+__device__ __forceinline__ void load_tile_edge_buf(f32x4 (&reg)[NCH], __amdgpu_buffer_rsrc_t rsrc,
+                                                   const int (&voff)[NCH][VEC ? 1 : 4]) {
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        if (VEC) {
+            reg[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff[i][0], 0, 0));
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                reg[i][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voff[i][j], 0, 0));
         }
     }
 }
@@ -607,14 +658,26 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         // makes the compiler wait for every load before the next tile's are issued, which turns the
         // register staging into one memory round trip per tile.  For the same reason every load in the
         // loop is unconditional: a tile index past the end is clamped (that tile is never stored).
-        auto pipe0 = [&](auto va_c, auto vb_c) {
+        auto pipe0 = [&](auto va_c, auto vb_c, auto buf_c) {
             constexpr bool VA = decltype(va_c)::value, VB = decltype(vb_c)::value;
+            constexpr bool BUF = EDGE && decltype(buf_c)::value;   // general tiles through buffer loads
+            int voa[NCHA][VA ? 1 : 4], vob[NCHB][VB ? 1 : 4];
+            uint64_t a_base = 0, b_base = 0;
+            if (BUF) {
+                edge_offsets<A_KC, BM, BK, NT, VA>(voa, p.a_rs, p.a_ks, tid);
+                edge_offsets<B_KC, BN, BK, NT, VB>(vob, p.b_rs, p.b_ks, tid);
+                a_base = reinterpret_cast<uint64_t>(uniform_ptr(Ab));
+                b_base = reinterpret_cast<uint64_t>(uniform_ptr(Bb));
+            }
             auto load_into = [&](int kt, f32x4(&da)[NCHA], f32x4(&db)[NCHB]) {
                 const int ktc = min(kt, nkt - 1);
                 const int k0 = ktc * BK;
                 const float* ap = Ab + (int64_t)k0 * p.a_ks;
                 const float* bp = Bb + (int64_t)k0 * p.b_ks;
-                if (!EDGE) {
+                if (BUF) {
+                    load_tile_edge_buf<NCHA, VA>(da, edge_resource(a_base, p.a_rs, p.a_ks, p.M - m0, Kz, k0), voa);
+                    load_tile_edge_buf<NCHB, VB>(db, edge_resource(b_base, p.b_rs, p.b_ks, p.N - n0, Kz, k0), vob);
+                } else if (!EDGE) {
 #pragma unroll
                     for (int i = 0; i < NCHA; i++)
                         load_tile_chunk_buf<A_KC, BM, BK, NT>(da, rsrc_a, k0 * (int)p.a_ks * 4, (int)a_ld * 4, (int)toff_a * 4, i);
@@ -699,14 +762,16 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         using no = std::integral_constant<bool, false>;
         if (nkt > 0) {
             if (!EDGE) {
-                pipe0(yes{}, yes{});
+                pipe0(yes{}, yes{}, no{});
+            } else if (!p.edge_buf) {
+                pipe0(no{}, no{}, no{});   // a tile spans 2 GiB or more: flat element-wise loads
             } else {
                 const bool va = edge_operand_vec<A_KC, BM>(rows_a, Kz, p.a_vec);
                 const bool vb = edge_operand_vec<B_KC, BN>(rows_b, Kz, p.b_vec);
-                if (va && vb) pipe0(yes{}, yes{});
-                else if (va) pipe0(yes{}, no{});
-                else if (vb) pipe0(no{}, yes{});
-                else pipe0(no{}, no{});
+                if (va && vb) pipe0(yes{}, yes{}, yes{});
+                else if (va) pipe0(yes{}, no{}, yes{});
+                else if (vb) pipe0(no{}, yes{}, yes{});
+                else pipe0(no{}, no{}, yes{});
             }
         }
     } else {
