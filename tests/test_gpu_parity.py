@@ -537,6 +537,29 @@ def test_split_k_scratch_survives_shutdown_and_growth():
         check(y.to_numpy((m, n))[rows], ko.matmul_rows(w, x, rows), what="split-K %dx%dx%d" % (m, n, k))
 
 
+# ---- operands whose tiles span 2 GiB: the flat-load fallback of the buffer-load kernels ---------------------------
+
+def test_matmul_with_a_two_gib_tile_span():
+    """64 x 64 outputs over K = 8.6M: 64 rows of either operand span 2.2 GB, more than the 31-bit lane offsets of
+    the buffer-load variants, so dispatch must take the general kernel with flat loads (cut along K as usual).
+    Inputs are -1 / 0 / 1: every partial sum is an integer below 2^24, so any summation order is exact and the
+    comparison with float64 is bit for bit."""
+    m = n = 64
+    k = 8_600_064
+    rng = np.random.default_rng(77)
+    x = rng.integers(-1, 2, (m, k), dtype=np.int8).astype(np.float32)
+    w = rng.integers(-1, 2, (n, k), dtype=np.int8).astype(np.float32)
+    y = DB(m * n * 4)
+    dx, dw = dev(x), dev(w)
+    VMath.matmul(0, y, dw, dx, n, m, k, False)
+    got = y.to_numpy((m, n))
+    rows = [0, 17, 63]
+    want = np.stack([w.astype(np.float64) @ x[r].astype(np.float64) for r in rows])
+    np.testing.assert_array_equal(got[rows], want.astype(np.float32))
+    # and the whole matrix against the oracle's own (sequential, equally exact) sums on one more row
+    np.testing.assert_array_equal(got[40], ko.matmul_rows(w, x, [40])[0])
+
+
 # ---- cosinesim ----------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("nrow1,nrow2,ncol", [(1, 1, 1), (6, 4, 33), (64, 512, 784), (300, 70, 1000), (2048, 2048, 64), (5, 4100, 128)])
