@@ -1,0 +1,115 @@
+"""Seeded sweeps over shapes, operand forms, leading dimensions and epilogue flags: kai_gemm_f32 against the
+oracle's loops (and float64 for the one form the engine never issues), and the attention entry points against
+the oracle at random geometries.  The fixed cases of test_gpu_parity.py aim at kernel variants one by one; this
+walks the dispatch at large."""
+import numpy as np
+import pytest
+
+from util import REL_FRO_TOL, ko, rel_fro
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 96, 100, 127, 128, 129, 200, 255, 256, 257,
+         300, 384, 500, 512, 513, 640, 777, 1000, 1024, 1030, 2048]
+
+
+def _kai():
+    from deep_learning_framework_amd import kai
+    from deep_learning_framework_amd.kai import DeviceBuffer, VMath
+    kai.load()
+    kai.set_device(0)
+    return kai, DeviceBuffer, VMath
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_gemm_f32_random_shapes(seed):
+    kai, DB, VMath = _kai()
+    rng = np.random.default_rng(seed)
+    leaky = kai.hyper(0.1)
+    for _ in range(60):
+        M, N = int(rng.choice(SIZES)), int(rng.choice(SIZES))
+        K = int(rng.choice(SIZES + [3000, 4096]))
+        if M * N * K > 4e7:                                   # keeps the oracle's scalar loops to seconds
+            K = max(1, int(4e7 // (M * N)))
+        tA, tB = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        pads = [int(rng.choice([0, 0, 1, 3, 4, 8])) for _ in range(3)]
+        acc, use_bias, act = int(rng.integers(0, 2)), int(rng.integers(0, 2)), int(rng.choice([0, 0, 1, 2]))
+        A = rng.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+        B = rng.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+        lda, ldb, ldc = A.shape[1] + pads[0], B.shape[1] + pads[1], N + pads[2]
+        Ap = np.full((A.shape[0], lda), np.nan, np.float32)      # what lies between the rows must never be read as data
+        Ap[:, :A.shape[1]] = A
+        Bp = np.full((B.shape[0], ldb), np.nan, np.float32)
+        Bp[:, :B.shape[1]] = B
+        C0 = rng.standard_normal((M, ldc)).astype(np.float32)
+        bias = rng.standard_normal(N).astype(np.float32)
+        dC = DB.from_numpy(C0)
+        VMath.gemm_f32(0, tA, tB, M, N, K, DB.from_numpy(Ap), lda, DB.from_numpy(Bp), ldb, dC, ldc,
+                       DB.from_numpy(bias) if use_bias else None, act, leaky, acc)
+        got = dC.to_numpy((M, ldc))
+        start = np.ascontiguousarray(C0[:, :N]) if acc else None
+        if (tA, tB) == (0, 1):
+            ref = ko.matmul(B, A, acc_into=start)
+        elif (tA, tB) == (0, 0):
+            ref = ko.matmul_backward_x(A, B, acc_into=start)
+        elif (tA, tB) == (1, 0):
+            ref = ko.matmul_backward_w(A, B, M, N, acc_into=start)
+        else:
+            ref = (A.T.astype(np.float64) @ B.T.astype(np.float64) + (start if acc else 0)).astype(np.float32)
+        if use_bias:
+            ref = ko.add_bias(ref, bias)
+        ref = ko.activate(ref, ["none", "relu", "leaky"][act], 0.1)
+        what = "M=%d N=%d K=%d tA=%d tB=%d ld=%d/%d/%d acc=%d bias=%d act=%d" % (M, N, K, tA, tB, lda, ldb, ldc, acc,
+                                                                                use_bias, act)
+        assert np.isfinite(got[:, :N]).all(), what
+        assert rel_fro(got[:, :N], ref) <= 2 * REL_FRO_TOL, what      # K up to 4096 with unit-variance inputs
+        assert np.array_equal(got[:, N:], C0[:, N:]), what + ": wrote between the rows of C"
+
+
+def test_attention_random_geometries():
+    kai, DB, VMath = _kai()
+    rng = np.random.default_rng(21)
+    dev = lambda a: DB.from_numpy(np.ascontiguousarray(a, np.float32))
+    done = 0
+    while done < 24:
+        nhead = int(rng.choice([1, 2, 3, 4, 8, 12]))
+        npiece = int(rng.choice([4, 6, 16, 24, 32, 64, 96]))
+        T = int(rng.choice([5, 32, 33, 64, 96, 100, 128, 160, 256, 300, 512]))
+        nbat = int(rng.choice([1, 2, 3, 5]))
+        if nbat * T * T * nhead > 4e6:
+            nbat = 1
+        if nbat * T * T * nhead * npiece > 2e8:
+            continue
+        done += 1
+        nvec = nhead * npiece
+        q, k, v, gy = (rng.standard_normal((nbat, T, nvec)).astype(np.float32) for _ in range(4))
+        coef = 1.0 / np.sqrt(npiece)
+        hc = kai.hyper(coef)
+        masked = bool(rng.integers(0, 2))
+        ps = (nbat, T, T, nhead)
+        what = "nbat=%d T=%d nhead=%d npiece=%d masked=%s: " % (nbat, T, nhead, npiece, masked)
+        p = DB(int(np.prod(ps)) * 4)
+        VMath.mult_on_heads(0, p, dev(k), dev(q), nbat, T, nvec, nhead, npiece, hc)
+        ref_s = ko.mult_on_heads(k, q, nhead, coef)
+        assert rel_fro(p.to_numpy(ps), ref_s) <= REL_FRO_TOL, what + "scores"
+        if masked:
+            VMath.set_mh_attention_mask(0, p, nbat, T, nhead, True)
+            ref_s = ko.set_mh_attention_mask(ref_s, True)
+        VMath.softmax_direct_on_axis(0, p, nbat * T, T, nhead)
+        ref_p = ko.softmax_direct_on_axis(ref_s, nbat * T, T, nhead)
+        assert rel_fro(p.to_numpy(ps), ref_p) <= REL_FRO_TOL, what + "softmax"
+        dp, o = dev(ref_p), DB(nbat * T * nvec * 4)
+        VMath.mix_values(0, o, dp, dev(v), nbat, T, nvec, nhead, npiece)
+        ref_o = ko.mix_values(ref_p, v, nhead)
+        assert rel_fro(o.to_numpy((nbat, T, nvec)), ref_o) <= REL_FRO_TOL, what + "mix_values"
+        VMath.attention_forward(0, o, dev(q), dev(k), dev(v), nbat, T, nvec, nhead, npiece, hc, masked)
+        assert rel_fro(o.to_numpy((nbat, T, nvec)), ref_o) <= REL_FRO_TOL, what + "attention_forward"
+        g = DB(nbat * T * nvec * 4)
+        VMath.mix_values_backward_value(0, g, dev(gy), dp, nbat, T, nvec, nhead, npiece)
+        assert rel_fro(g.to_numpy((nbat, T, nvec)), ko.mix_values_backward_value(gy, ref_p, nhead)) <= REL_FRO_TOL, what + "gV"
+        gp = DB(int(np.prod(ps)) * 4)
+        VMath.mix_values_backward_prop(0, gp, dev(gy), dev(v), nbat, T, nvec, nhead, npiece)
+        ref_gp = ko.mix_values_backward_prop(gy, v, nhead)
+        assert rel_fro(gp.to_numpy(ps), ref_gp) <= REL_FRO_TOL, what + "gP"
+        VMath.mult_on_heads_backward(0, g, dev(ref_gp), dev(k), nbat, T, nvec, nhead, npiece)
+        assert rel_fro(g.to_numpy((nbat, T, nvec)), ko.mult_on_heads_backward(ref_gp, k, nhead)) <= REL_FRO_TOL, what + "gQ"
