@@ -50,10 +50,18 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     plan.a_kc = operand_is_kc(dn.a_rs, dn.a_ks);
     plan.b_kc = operand_is_kc(dn.b_rs, dn.b_ks);
 
-    // largest tile that still yields about one workgroup per compute unit and is not mostly padding
+    // Largest tile that still yields about one workgroup per compute unit and is not mostly padding.  Between
+    // the two big tiles the number of rounds decides: both run at the same rate per compute unit (measured:
+    // 149 TFLOP/s either way at 8192^3), a compute unit works through its 256x256 tiles one at a time and
+    // through 128x128 tiles at a quarter of that each (two resident ones share its rate), so the last, partly
+    // filled round costs four times less with the medium tile (4100^3: 1.85 ms against 1.19 ms).  On a tie the
+    // large tile wins: it moves half as much through LDS per flop (8000^3: 7.1 against 7.5 ms).
     const int64_t short_side = d.M < d.N ? d.M : d.N;
-    if (short_side > 128 && tiles_of(d.M, d.N, d.nbatch, 256) >= 192) plan.tile = kTileLarge;
-    else if (short_side > 64 && tiles_of(d.M, d.N, d.nbatch, 128) >= 128) plan.tile = kTileMedium;
+    const int64_t cus = compute_units();
+    const int64_t t256 = tiles_of(d.M, d.N, d.nbatch, 256), t128 = tiles_of(d.M, d.N, d.nbatch, 128);
+    if (short_side > 128 && t256 >= (3 * cus) / 4 && 4 * ((t256 + cus - 1) / cus) <= (t128 + cus - 1) / cus)
+        plan.tile = kTileLarge;
+    else if (short_side > 64 && t128 >= cus / 2) plan.tile = kTileMedium;
 
     // Split-K: a single product whose output tiles leave most compute units idle is cut along K
     // into `split` equal parts that run as the batch dimension of the same kernel and write raw

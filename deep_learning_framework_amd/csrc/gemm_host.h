@@ -75,6 +75,15 @@ inline bool fits_buffer_offsets(const GemmParams& p, bool a_kc, bool b_kc, int B
     return a_span * 4 < (1ll << 31) && b_span * 4 < (1ll << 31);
 }
 
+// true when the pipelined kernel's general variant may run the problem: 128-bit loads are legal for both
+// operands (M, N and K themselves are arbitrary: rows past the end are never stored, the last partial K-tile
+// is masked) and the reduction is not cut over the batch index
+inline bool fits_ragged_pipe(const GemmParams& p, bool a_kc, bool b_kc, int BM, int BN) {
+    const int64_t a_ld = a_kc ? p.a_rs : p.a_ks, b_ld = b_kc ? p.b_rs : p.b_ks;
+    return p.k_part == 0 && p.a_vec && p.b_vec && p.K > 0 && a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30) &&
+           fits_buffer_offsets(p, a_kc, b_kc, BM, BN);
+}
+
 template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
           int DEPTH = 1, bool ROWSUM = false>
 int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t stream) {

@@ -31,10 +31,14 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
     case kTileLarge:
         if (fits_without_edges(p, A_KC, B_KC, 256, 256, 16) && fits_buffer_offsets(p, A_KC, B_KC, 256, 256))
             return launch_gemm_config<2, 4, 4, 2, 16, A_KC, B_KC, false, 1>(p, nbatch, kGroupM, stream);
+        if (fits_ragged_pipe(p, A_KC, B_KC, 256, 256))
+            return launch_gemm_config<2, 4, 4, 2, 16, A_KC, B_KC, true, 1>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<2, 4, 4, 2, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);
     case kTileMedium:
         if (fits_without_edges(p, A_KC, B_KC, 128, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 128, 128))
             return launch_gemm_config<2, 2, 2, 2, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
+        if (fits_ragged_pipe(p, A_KC, B_KC, 128, 128))
+            return launch_gemm_config<2, 2, 2, 2, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<2, 2, 2, 2, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);
     default:
         // a 64x64x16 tile computes for ~0.25 us, a global load takes ~1-2 us: 128 reduction steps in flight

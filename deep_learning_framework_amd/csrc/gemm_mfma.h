@@ -647,10 +647,17 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
         return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
     };
+    // The pipelined schedule on general shapes (PIPE 1 with EDGE): the resources end with the operand, so a
+    // row past the last one reads as zero or as other rows' data of the same operand; either only ever reaches
+    // output rows and columns that are not stored.  The loop then runs over the whole K-tiles without any
+    // predicate, and the rest of K follows as one masked tile.
+    constexpr bool RAGGED_PIPE = EDGE && PIPE == 1;
     const __amdgpu_buffer_rsrc_t rsrc_a =
-        __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Ab), 0, (int)0xFFFFFFFFu, 0x00020000);
+        RAGGED_PIPE ? edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Ab)), p.a_rs, p.a_ks, p.M - m0, p.K, 0)
+                    : __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Ab), 0, (int)0xFFFFFFFFu, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b =
-        __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Bb), 0, (int)0xFFFFFFFFu, 0x00020000);
+        RAGGED_PIPE ? edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Bb)), p.b_rs, p.b_ks, p.N - n0, p.K, 0)
+                    : __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Bb), 0, (int)0xFFFFFFFFu, 0x00020000);
 
     if (PIPE == 0) {
         // The whole loop exists once per combination of 128-bit / element-wise loads of A and B.  The
@@ -776,15 +783,29 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         }
     } else {
         static_assert(PIPE == 0 || NKG % 2 == 0, "the pipelined schedule needs an even number of groups per tile");
-        static_assert(PIPE == 0 || !EDGE, "the pipelined schedule uses the predicate-free loads only");
+        // whole K-tiles of the pipelined loop; a general shape's last, partial tile follows it
+        const int nkt_all = nkt;
+        const int nkt = RAGGED_PIPE ? p.K / BK : nkt_all;
         constexpr int kReadsA = A_KC ? NBM : 4;
         constexpr int kReads = kReadsA + (B_KC ? NBN : 4);   // LDS reads per group
         constexpr int kWrites = NCHA + NCHB;                  // LDS stores per tile and thread
         constexpr int kMfma = 4 * NBM * NBN;                  // MFMAs per group
         Frag<A_KC, NBM> fa[2];
         Frag<B_KC, NBN> fb[2];
+        auto load_whole = [&](int kt) {
+            if (RAGGED_PIPE) {   // flat loads could fault on the rows past the operand
+#pragma unroll
+                for (int i = 0; i < NCHA; i++)
+                    load_tile_chunk_buf<A_KC, BM, BK, NT>(ra, rsrc_a, kt * BK * (int)p.a_ks * 4, (int)a_ld * 4, (int)toff_a * 4, i);
+#pragma unroll
+                for (int i = 0; i < NCHB; i++)
+                    load_tile_chunk_buf<B_KC, BN, BK, NT>(rb, rsrc_b, kt * BK * (int)p.b_ks * 4, (int)b_ld * 4, (int)toff_b * 4, i);
+            } else {
+                load_global(kt);
+            }
+        };
         if (nkt > 0) {
-            load_global(0);
+            load_whole(0);
             store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
             store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
         }
@@ -847,7 +868,7 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
         // them into the free LDS buffer, one store per slot; the last group refills them with tile
         // kt+2, one global load per slot, so that the waves of a workgroup never queue all their
         // loads on the address unit at once and every load has most of a tile to land.
-        if (nkt > 1) load_global(1);
+        if (nkt > 1) load_whole(1);
         if (nkt > 0) {
             read_frag<A_KC, NBM, BM, BK>(fa[0], lds_a[0], wm0, 0, l32, half);
             read_frag<B_KC, NBN, BN, BK>(fb[0], lds_b[0], wn0, 0, l32, half);
@@ -871,6 +892,32 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
             const int cur = (nkt - 1) & 1;
 #pragma unroll
             for (int kg = 0; kg < NKG; kg++) group(kg & 1, (kg + 1) & 1, kg + 1 < NKG, cur, kg + 1, false, 0, false, 0);
+        }
+        if constexpr (RAGGED_PIPE) {
+            const int k0 = nkt * BK, k_left = p.K - k0;
+            if (k_left > 0) {   // uniform
+                int voa[NCHA][4], vob[NCHB][4];
+                edge_offsets<A_KC, BM, BK, NT, false>(voa, p.a_rs, p.a_ks, tid);
+                edge_offsets<B_KC, BN, BK, NT, false>(vob, p.b_rs, p.b_ks, tid);
+                load_tile_edge_buf<NCHA, false>(
+                    ra, edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Ab)), p.a_rs, p.a_ks, p.M - m0, p.K, k0), voa);
+                load_tile_edge_buf<NCHB, false>(
+                    rb, edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Bb)), p.b_rs, p.b_ks, p.N - n0, p.K, k0), vob);
+                mask_tile_edge<A_KC, BM, BK, NT>(ra, rows_a, k_left, tid);
+                mask_tile_edge<B_KC, BN, BK, NT>(rb, rows_b, k_left, tid);
+                __syncthreads();   // every wave has read its last fragments of the whole tiles
+                store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
+                store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
+                __syncthreads();
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    Frag<A_KC, NBM> ta;
+                    Frag<B_KC, NBN> tb;
+                    read_frag<A_KC, NBM, BM, BK>(ta, lds_a[0], wm0, kg, l32, half);
+                    read_frag<B_KC, NBN, BN, BK>(tb, lds_b[0], wn0, kg, l32, half);
+                    mfma_group(ta, tb);
+                }
+            }
         }
     }
 

@@ -66,6 +66,59 @@ def test_gemm_f32_random_shapes(seed):
         assert np.array_equal(got[:, N:], C0[:, N:]), what + ": wrote between the rows of C"
 
 
+# Products big enough for the 256x256 and 128x128 tiles whose sides are no multiples of the tile: the pipelined
+# kernels then read past the last row (never stored) and finish K with one masked tile.  Leading dimensions that
+# are multiples of 4 keep the 128-bit loads; the cases with other ones take the element-wise variant of the same tile.
+BIG_RAGGED = [
+    # M, N, K, tA, tB, pads (A, B, C), acc, bias, act
+    (3000, 4200, 36, 0, 1, (0, 0, 0), 0, 1, 1),     # large tile, two whole K-tiles and a rest of 4
+    (3100, 4100, 8, 0, 0, (0, 0, 0), 1, 0, 0),      # large tile, K shorter than one K-tile
+    (3001, 4204, 32, 1, 0, (3, 0, 0), 0, 0, 2),     # large tile, whole K-tiles, 128-bit chunks that straddle the last row
+    (2900, 4400, 20, 1, 1, (0, 0, 1), 0, 1, 0),     # large tile, the form the engine never issues
+    (3000, 4200, 18, 0, 1, (1, 0, 0), 0, 0, 0),     # large tile, unaligned rows of A: element-wise loads
+    (1000, 3000, 200, 0, 1, (0, 0, 0), 0, 1, 1),    # medium tile, six whole K-tiles and a rest of 8
+    (1001, 2999, 77, 0, 0, (3, 1, 0), 1, 1, 0),     # medium tile, K no multiple of 4 behind aligned rows
+    (1500, 1300, 44, 1, 0, (0, 0, 3), 0, 0, 1),     # medium tile
+    (1100, 1900, 20, 1, 1, (0, 0, 0), 0, 0, 0),     # medium tile, only the masked K-tile
+]
+
+
+@pytest.mark.parametrize("case", BIG_RAGGED, ids=lambda c: "%dx%dx%d-%d%d" % c[:5])
+def test_gemm_f32_big_ragged_tiles(case):
+    kai, DB, VMath = _kai()
+    M, N, K, tA, tB, pads, acc, use_bias, act = case
+    rng = np.random.default_rng(M + N + K)
+    leaky = kai.hyper(0.1)
+    A = rng.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+    B = rng.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    lda, ldb, ldc = A.shape[1] + pads[0], B.shape[1] + pads[1], N + pads[2]
+    Ap = np.full((A.shape[0], lda), np.nan, np.float32)
+    Ap[:, :A.shape[1]] = A
+    Bp = np.full((B.shape[0], ldb), np.nan, np.float32)
+    Bp[:, :B.shape[1]] = B
+    C0 = rng.standard_normal((M, ldc)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    dC = DB.from_numpy(C0)
+    VMath.gemm_f32(0, tA, tB, M, N, K, DB.from_numpy(Ap), lda, DB.from_numpy(Bp), ldb, dC, ldc,
+                   DB.from_numpy(bias) if use_bias else None, act, leaky, acc)
+    got = dC.to_numpy((M, ldc))
+    start = np.ascontiguousarray(C0[:, :N]) if acc else None
+    if (tA, tB) == (0, 1):
+        ref = ko.matmul(B, A, acc_into=start)
+    elif (tA, tB) == (0, 0):
+        ref = ko.matmul_backward_x(A, B, acc_into=start)
+    elif (tA, tB) == (1, 0):
+        ref = ko.matmul_backward_w(A, B, M, N, acc_into=start)
+    else:
+        ref = (A.T.astype(np.float64) @ B.T.astype(np.float64) + (start if acc else 0)).astype(np.float32)
+    if use_bias:
+        ref = ko.add_bias(ref, bias)
+    ref = ko.activate(ref, ["none", "relu", "leaky"][act], 0.1)
+    assert np.isfinite(got[:, :N]).all()
+    assert rel_fro(got[:, :N], ref) <= REL_FRO_TOL
+    assert np.array_equal(got[:, N:], C0[:, N:]), "wrote between the rows of C"
+
+
 def test_attention_random_geometries():
     kai, DB, VMath = _kai()
     rng = np.random.default_rng(21)
