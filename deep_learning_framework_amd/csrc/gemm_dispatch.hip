@@ -61,7 +61,14 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     const int64_t t256 = tiles_of(d.M, d.N, d.nbatch, 256), t128 = tiles_of(d.M, d.N, d.nbatch, 128);
     if (short_side > 128 && t256 >= (3 * cus) / 4 && 4 * ((t256 + cus - 1) / cus) <= (t128 + cus - 1) / cus)
         plan.tile = kTileLarge;
-    else if (short_side > 64 && t128 >= cus / 2) plan.tile = kTileMedium;
+    else if (short_side > 64 && t128 >= cus / 2) {
+        // The same count between the 128- and the 64-wide tile, which runs at about 0.88 of the medium tile's
+        // rate per compute unit (2048^3: 134 against 123 us): the small tile wins where its finer grain saves
+        // a round (1024x2048x512, 128 medium tiles on 256 units: 36 -> 24 us; 1536^3 91 -> 77; 3000^3 540 -> 485).
+        const int64_t t64 = tiles_of(d.M, d.N, d.nbatch, 64);
+        const int64_t rounds_m = (t128 + cus - 1) / cus, rounds_s = (t64 + cus - 1) / cus;
+        if (100 * rounds_s >= 340 * rounds_m) plan.tile = kTileMedium;
+    }
 
     // Split-K: a single product whose output tiles leave most compute units idle is cut along K
     // into `split` equal parts that run as the batch dimension of the same kernel and write raw

@@ -5,8 +5,9 @@
 //   large  256x256 tile, 8 waves of 128x64 (2 waves per SIMD)  -- big, compute-bound products
 //   medium 128x128 tile, 4 waves of 64x64, 2 workgroups per CU -- fills the chip at mid sizes
 //   small   64x64  tile, 4 waves of 32x32                      -- small or very ragged products
-// Shapes that are whole multiples of the tile with aligned operands run the pipelined,
-// predicate-free kernel; everything else the general one.
+// On the two bigger tiles, operands that allow 128-bit loads run the pipelined kernel: predicate-free
+// when the shape is a whole multiple of the tile, else with range-checked buffer resources and one
+// masked K-tile at the end.  Everything else runs the general kernel with the simple schedule.
 #pragma once
 
 #include "gemm_host.h"

@@ -24,9 +24,12 @@
 //    global loads with the MFMAs one by one, for large whole-tile products.
 //  * Shapes that are whole multiples of the tile with 16-byte aligned operands
 //    run a kernel variant with predicate-free 128-bit loads (EDGE = false).  The
-//    general variant loads through clamped addresses, 128-bit or element-wise as
-//    chosen once per workgroup, and zeroes what lies outside the matrix when the
-//    tile moves to LDS: no load in any loop sits behind a branch.
+//    general variant loads through buffer resources that end with the operand (or
+//    through clamped addresses), 128-bit or element-wise as chosen once per
+//    workgroup, and zeroes what lies outside the matrix when the tile moves to
+//    LDS: no load in any loop sits behind a branch.  With the slot schedule it
+//    masks only the last, partial K-tile: rows past the operand never reach a
+//    stored output.
 //  * A single product can be cut along K over the batch dimension (k_part) and can
 //    sum the rows of A on the side (ROWSUM, the bias gradient of a dense layer).
 //  * Workgroup ids are remapped so that the workgroups that share one XCD (and its
@@ -536,7 +539,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 
 // EDGE = false: the host has checked that M, N, K are multiples of the tile, that both operands
 // allow aligned 128-bit loads and that a tile's offsets fit 32 bits; the kernel then holds no
-// predicated load code at all (fewer registers).  EDGE = true: general shapes.
+// predicated load code at all (fewer registers).  EDGE = true: general shapes (with PIPE 1: any
+// M, N, K, but operands that allow aligned 128-bit loads and 32-bit offsets, checked by the host).
 //
 // PIPE selects the schedule of the main loop:
 //   0  per K-tile: all fragment reads of a group, then its MFMAs; LDS stores and the barrier at the
