@@ -2,6 +2,8 @@
 // most 16 rows against a K-contiguous weight matrix, otherwise the MFMA kernel in the LDS
 // orientation pair that matches how the operands lie in memory, with the largest tile that still
 // fills the 256 compute units.
+#include <algorithm>
+
 #include "elementwise.h"
 #include "gemm_host.h"
 #include "gemv_skinny.h"
@@ -35,7 +37,24 @@ struct GemmPlan {
     int64_t k_part = 0;
     bool ragged_parts = false;   // the last part is shorter than k_part
     GemmDesc dn;   // the product with batch strides normalised
+    int wavesplit_edge = 0;   // 16 or 32: the product runs on the kernel that cuts K over the waves of a workgroup
 };
+
+// Expected duration in microseconds of the wave-split kernel with T x T blocks, from measurements over 60 shapes
+// (a fixed cost, then the larger of the stream of operand bytes through the compute units' address units and
+// one wave's chain of rounds along K; an operand that is not K-contiguous adds about an eighth), or a negative
+// value outside the measured range.
+double wavesplit_estimate(const GemmDesc& d, int T) {
+    const int64_t wgs = ((d.M + T - 1) / T) * ((d.N + T - 1) / T);
+    const double K = (double)d.K;
+    const double forms = 1.0 + 0.12 * ((d.a_ks != 1) + (d.b_ks != 1));
+    if (T == 16) {
+        if (d.K > 2048 || wgs > 1024) return -1.0;
+        return (3.8 + std::max(1.3e-5 * (double)wgs * K, 3.3e-3 * K)) * forms;
+    }
+    if (d.K > 1024 || wgs > 512 || (d.K < 256 && wgs > 256)) return -1.0;
+    return (4.0 + std::max(2.7e-5 * (double)wgs * K, 6.45e-3 * K)) * forms;
+}
 
 GemmPlan plan_gemm(const GemmDesc& d) {
     GemmPlan plan;
@@ -68,6 +87,18 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         const int64_t t64 = tiles_of(d.M, d.N, d.nbatch, 64);
         const int64_t rounds_m = (t128 + cus - 1) / cus, rounds_s = (t64 + cus - 1) / cus;
         if (100 * rounds_s >= 340 * rounds_m) plan.tile = kTileMedium;
+    }
+
+    // Small products: one launch of the wave-split kernel where it is expected to finish before the tiled
+    // kernel (plus, for long K, its second launch) could: measured, it wins wherever its estimate stays below
+    // ~12.5 us (64x512x784 9.8 -> 4.9 us, 256x1024x1024 14.3 -> 11.0, its backward_x form 14.3 -> 12.4,
+    // 300^3 11.1 -> 4.9), and against the skinny kernels for 5..16 rows below ~7 us (16x1024x1024 7.8 -> 5.9).
+    if (wavesplit_applies(dn)) {
+        const double e16 = wavesplit_estimate(dn, 16), e32 = wavesplit_estimate(dn, 32);
+        const bool take16 = e16 > 0 && (e32 < 0 || e16 <= e32);
+        const double best = take16 ? e16 : e32;
+        const double limit = plan.skinny ? (d.M <= 4 ? 0.0 : 7.0) : 12.5;
+        if (best > 0 && best <= limit) plan.wavesplit_edge = take16 ? 16 : 32;
     }
 
     // Split-K: a single product whose output tiles leave most compute units idle is cut along K
@@ -110,7 +141,7 @@ bool valid_dims(const GemmDesc& d) {
 bool gemm_fuses_rowsum(const GemmDesc& d) {
     if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
     const GemmPlan plan = plan_gemm(d);
-    return !plan.skinny && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge && plan.split == 1;
+    return !plan.skinny && !plan.wavesplit_edge && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge && plan.split == 1;
 }
 
 int launch_gemm(const GemmDesc& d, hipStream_t stream) {
@@ -125,6 +156,7 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
     if (d.rowsum && !gemm_fuses_rowsum(d))
         return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: this product cannot carry the fused row sum");
 
+    if (plan.wavesplit_edge) return launch_gemm_wavesplit(plan.dn, plan.wavesplit_edge, stream);
     if (plan.skinny) {
         SkinnyParams s{};
         s.W = d.B; s.X = d.A; s.Y = d.C; s.Y2 = d.C2; s.bias = d.bias; s.leaky = d.leaky;

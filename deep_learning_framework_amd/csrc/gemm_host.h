@@ -119,6 +119,11 @@ int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream);
 bool shortk_heads_applies(const GemmDesc& d);
 int launch_gemm_shortk_heads(GemmParams p, int64_t nbatch, hipStream_t stream);
 
+// small products with a long reduction, both operands K-contiguous: the reduction is cut over the waves of a
+// workgroup (gemm_wavesplit.hip); block_edge is 32 or 16
+bool wavesplit_applies(const GemmDesc& d);
+int launch_gemm_wavesplit(const GemmDesc& d, int block_edge, hipStream_t stream);
+
 // products of the head-interleaved attention tensor with several heads per batch entry: heads_pv.hip
 bool heads_pv_applies(const GemmDesc& d);
 int launch_heads_pv(const GemmDesc& d, hipStream_t stream);

@@ -522,19 +522,90 @@ def test_softmax_axis_backward_layouts(nbat, ntimes, nhead):
 
 
 def test_split_k_scratch_survives_shutdown_and_growth():
-    # a product cut along K uses scratch memory of the library: small first, then a larger one (the buffer
-    # grows), then released and created again
+    # a product cut along K over workgroups (reductions too long for the single-launch small-product kernel) uses
+    # scratch memory of the library; an attention forward with a head size outside the fused kernel's keeps its
+    # probabilities there and needs more of it (the buffer grows); then it is released and created again
     rng = np.random.default_rng(99)
-    for (m, n, k), release in [((64, 64, 2048), False), ((1024, 2048, 1024), False), ((64, 128, 2048), True),
-                               ((64, 128, 2048), False)]:
+
+    def split_k(m, n, k):
         x = rng.standard_normal((m, k)).astype(np.float32)
         w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
         y = DB(m * n * 4)
-        if release:
-            kai.shutdown()
         VMath.matmul(0, y, dev(w), dev(x), n, m, k, False)
         rows = list(range(0, m, max(1, m // 64)))
         check(y.to_numpy((m, n))[rows], ko.matmul_rows(w, x, rows), what="split-K %dx%dx%d" % (m, n, k))
+
+    def attention_with_scratch():
+        nbat, T, nhead, npiece = 2, 384, 4, 24            # 2 * 384 * 384 * 4 floats = 4.5 MiB of probabilities
+        q, k, v = (rng.standard_normal((nbat, T, nhead * npiece)).astype(np.float32) for _ in range(3))
+        coef = 1.0 / np.sqrt(npiece)
+        o = DB(nbat * T * nhead * npiece * 4)
+        VMath.attention_forward(0, o, dev(q), dev(k), dev(v), nbat, T, nhead * npiece, nhead, npiece, kai.hyper(coef), False)
+        probs = ko.softmax_direct_on_axis(ko.mult_on_heads(k, q, nhead, coef), nbat * T, T, nhead)
+        check(o.to_numpy((nbat, T, nhead * npiece)), ko.mix_values(probs, v, nhead), what="attention through the scratch")
+
+    split_k(64, 64, 4096)
+    split_k(256, 512, 4096)
+    attention_with_scratch()
+    split_k(64, 128, 8192)
+    kai.shutdown()
+    split_k(64, 128, 8192)
+    attention_with_scratch()
+
+
+# ---- small products: the reduction cut over the waves of one workgroup ---------------------------------------
+
+WAVE_SPLIT = [
+    # M, N, K: 16 x 16 blocks (few workgroups) and 32 x 32 blocks (more of them), whole and ragged blocks, K with and
+    # without a rest after the last round, K shorter than one round, K no multiple of 4 (forms without a K-contiguous
+    # operand only; the others run the tiled kernel there)
+    (64, 512, 784), (256, 1024, 1024), (100, 300, 1000), (17, 33, 44), (31, 77, 1001), (300, 300, 300),
+    (16, 16, 2048), (50, 70, 4), (33, 17, 1), (512, 1024, 512), (192, 1000, 1000), (9, 200, 1030), (128, 512, 260),
+]
+
+
+@pytest.mark.parametrize("m,n,k", WAVE_SPLIT)
+def test_small_products_every_form_and_epilogue(m, n, k):
+    rng = np.random.default_rng(m * 7919 + n * 31 + k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    bt, at = np.ascontiguousarray(b.T), np.ascontiguousarray(a.T)
+    ref = ko.matmul(bt, a)
+    ref_pre = ko.add_bias(ko.matmul(bt, a, acc_into=c0), bias)
+    da, dat, dbm, dbt, dbias = dev(a), dev(at), dev(b), dev(bt), dev(bias)
+    alpha = kai.hyper(0.1)
+    for ta, tb, A, lda, B, ldb in [(0, 1, da, k, dbt, k), (0, 0, da, k, dbm, n), (1, 0, dat, m, dbm, n),
+                                   (1, 1, dat, m, dbt, k)]:
+        what = "form (%d,%d) %dx%dx%d" % (ta, tb, m, n, k)
+        c = DB.from_numpy(np.full((m, n), np.nan, np.float32))
+        VMath.gemm_f32(0, ta, tb, m, n, k, A, lda, B, ldb, c, n, None, 0, None, False)
+        check(c.to_numpy((m, n)), ref, what=what)
+        for act in ("leaky", "sigmoid", "gelu"):
+            c = dev(c0)
+            VMath.gemm_f32(0, ta, tb, m, n, k, A, lda, B, ldb, c, n, dbias, kai.ACT[act], alpha, True)
+            check(c.to_numpy((m, n)), ko.activate(ref_pre, act, 0.1), what=what + " acc+bias+" + act)
+    # the engine's calls, the fused forward with its pre-activation output, a padded output row
+    w, x = bt, a
+    y, pre = DB(m * n * 4), DB(m * n * 4)
+    VMath.dense_forward(0, y, pre, dev(w), dbias, dev(x), n, m, k, kai.ACT["relu"], None)
+    ref_pre2 = ko.add_bias(ko.matmul(w, x), bias)
+    check(pre.to_numpy((m, n)), ref_pre2, what="pre-activation")
+    check(y.to_numpy((m, n)), ko.activate(ref_pre2, "relu"), what="relu")
+    gy = rng.standard_normal((m, n)).astype(np.float32)
+    gx, gw = DB(m * k * 4), DB(n * k * 4)
+    VMath.matmul_backward_x(0, gx, dev(gy), dev(w), n, m, k, False)
+    VMath.matmul_backward_w(0, gw, dev(gy), dev(x), n, m, k, False)
+    check(gx.to_numpy((m, k)), ko.matmul_backward_x(gy, w), what="backward_x")
+    check(gw.to_numpy((n, k)), ko.matmul_backward_w(gy, x, n, k), what="backward_w")
+    ldc = n + 5
+    cp0 = rng.standard_normal((m, ldc)).astype(np.float32)
+    cp = DB.from_numpy(cp0)
+    VMath.gemm_f32(0, 0, 1, m, n, k, da, k, dbt, k, cp, ldc, None, 0, None, False)
+    got = cp.to_numpy((m, ldc))
+    check(got[:, :n], ref, what="padded output rows")
+    assert np.array_equal(got[:, n:], cp0[:, n:]), "wrote between the rows of C"
 
 
 # ---- operands whose tiles span 2 GiB: the flat-load fallback of the buffer-load kernels ---------------------------
