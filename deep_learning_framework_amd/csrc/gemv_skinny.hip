@@ -471,6 +471,11 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
     const bool vec = p.K % 4 == 0 && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X);
     if (vec && p.K >= 256) {
         if (p.M == 1) return launch_gemv_rows(p, stream);
+        // 3 and 4 rows: the streaming kernel once its workgroups (16 rows of W each) cover the chip (measured at
+        // 4096 x 4096: 12.6 against 16.0 us, 11008 x 4096: 30 against 40; at 2048 x 8192, 128 workgroups:
+        // 19.8 against 15.3); 2 rows run as fast either way
+        if (p.M >= 3 && p.N >= 16 * (int64_t)compute_units() && skinny_stream_applies(p))
+            return launch_skinny_stream(p, stream);
         if (p.M == 2) return launch_slice<2>(p, stream);
         if (p.M <= 4) return launch_slice<4>(p, stream);
     }

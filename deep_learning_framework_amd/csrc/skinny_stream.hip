@@ -4,14 +4,16 @@
 //
 // A workgroup of eight waves owns 16 rows of W and all of K; wave w owns the slices of 512 reduction
 // steps number w, w+8, ...  Everything up to the final sum is private to a wave, so there is no
-// barrier in the stream: a wave loads its slice tile by tile (16 x 128 of W and of X, 512 contiguous
-// bytes per row and load; rows of X beyond M are not loaded), W three tiles and X two tiles ahead of
-// the tile it is working on, and passes both through its own LDS tiles into the operand layout of
+// barrier in the stream: a wave loads its slice tile by tile (16 x 64 of W and of X, 256 contiguous
+// bytes per row and load; rows of X beyond M are not loaded), two tiles ahead of the tile it is
+// working on, and passes both through its own LDS tiles into the operand layout of
 // v_mfma_f32_16x16x4_f32 (row = lane % 16, k group = lane / 16).  Loading in operand layout directly
 // would touch 64 bytes per row and load, which costs a third of the bandwidth.  The matrix core only
 // removes the per-row wave reductions and the X broadcasts a vector-ALU version would need; the
 // kernel is bound by HBM.  The eight partial 16 x 16 results meet in LDS once, in wave order.
 #include "gemv_skinny.h"
+
+#include <type_traits>
 
 #include "act_funcs.h"
 
@@ -24,9 +26,21 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kSsWaves = 8;
 constexpr int kSsThreads = 64 * kSsWaves;
 constexpr int kSsSlice = 512;                 // reduction steps per wave and pass of the pipeline: four tiles
-constexpr int kSsTileK = 128;                 // k per staged tile: 512 contiguous bytes per row
+constexpr int kSsTileK = 32;                  // k per staged tile: 256 contiguous bytes per row
+constexpr int kSsTiles = kSsSlice / kSsTileK; // tiles per slice
+constexpr int kSsRing = 3;                    // tiles of a wave in registers: one at work, the others on their way
+constexpr int kSsLanesPerRow = kSsTileK / 4;
+constexpr int kSsRowsPerLoad = 64 / kSsLanesPerRow;
 constexpr int kSsTileStride = kSsTileK + 4;
 constexpr int kSsLoadsPerTile = 16 * kSsTileK / 4 / 64;   // 128-bit loads per lane and tile: 8
+
+template <int B, int E, typename F>
+__device__ __forceinline__ void ss_static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        ss_static_for<B + 1, E>(f);
+    }
+}
 
 __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
     const int m = keep ? -1 : 0;
@@ -49,15 +63,15 @@ __global__ void __launch_bounds__(kSsThreads) skinny_stream_kernel(const SkinnyP
     const int r = lane & 15;    // row of W inside the block's 16 / row of X
     const int g = lane >> 4;    // k group of the MFMA operand
     const int64_t n0 = (int64_t)blockIdx.x * 16;
-    const int lrow = lane >> 5;          // a load covers 2 rows x 128 k
-    const int lk = (lane & 31) * 4;
+    const int lrow = lane / kSsLanesPerRow;          // a load covers kSsRowsPerLoad rows x kSsTileK k
+    const int lk = (lane % kSsLanesPerRow) * 4;
     float* tw = lds_w[wave];
     float* tx = lds_x[wave];
 
     // rows of X that are never loaded stay zero in the tile
 #pragma unroll
     for (int j = 0; j < kSsLoadsPerTile; j++)
-        *reinterpret_cast<f32x4*>(tx + (2 * j + lrow) * kSsTileStride + lk) = f32x4{0.f, 0.f, 0.f, 0.f};
+        *reinterpret_cast<f32x4*>(tx + (kSsRowsPerLoad * j + lrow) * kSsTileStride + lk) = f32x4{0.f, 0.f, 0.f, 0.f};
 
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     // One tile = 16 rows x 128 k of W and of X, eight 128-bit loads per lane each.  Addresses past K are
@@ -65,7 +79,7 @@ __global__ void __launch_bounds__(kSsThreads) skinny_stream_kernel(const SkinnyP
     auto load_w = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
 #pragma unroll
         for (int j = 0; j < kSsLoadsPerTile; j++) {
-            const int64_t n = n0 + 2 * j + lrow;
+            const int64_t n = n0 + kSsRowsPerLoad * j + lrow;
             const float* src = p.W + (n < p.N ? n : p.N - 1) * p.ldw + min(kt + lk, p.K - 4);
             dst[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src));
         }
@@ -73,8 +87,8 @@ __global__ void __launch_bounds__(kSsThreads) skinny_stream_kernel(const SkinnyP
     auto load_x = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
 #pragma unroll
         for (int j = 0; j < kSsLoadsPerTile; j++) {
-            if (2 * j < p.M) {   // uniform: this pair of rows holds a row of X
-                const int m = 2 * j + lrow;
+            if (kSsRowsPerLoad * j < p.M) {   // uniform: these rows hold a row of X
+                const int m = kSsRowsPerLoad * j + lrow;
                 dst[j] = *reinterpret_cast<const f32x4*>(p.X + (int64_t)min(m, p.M - 1) * p.ldx + min(kt + lk, p.K - 4));
             }
         }
@@ -83,11 +97,10 @@ __global__ void __launch_bounds__(kSsThreads) skinny_stream_kernel(const SkinnyP
         if (kt < p.K) {   // uniform
 #pragma unroll
             for (int j = 0; j < kSsLoadsPerTile; j++) {
-                const int64_t n = n0 + 2 * j + lrow;
-                *reinterpret_cast<f32x4*>(tw + (2 * j + lrow) * kSsTileStride + lk) = keep_if(w[j], n < p.N && kt + lk < p.K);
-                if (2 * j < p.M)
-                    *reinterpret_cast<f32x4*>(tx + (2 * j + lrow) * kSsTileStride + lk) =
-                        keep_if(x[j], 2 * j + lrow < p.M && kt + lk < p.K);
+                const int row = kSsRowsPerLoad * j + lrow;
+                *reinterpret_cast<f32x4*>(tw + row * kSsTileStride + lk) = keep_if(w[j], n0 + row < p.N && kt + lk < p.K);
+                if (kSsRowsPerLoad * j < p.M)
+                    *reinterpret_cast<f32x4*>(tx + row * kSsTileStride + lk) = keep_if(x[j], row < p.M && kt + lk < p.K);
             }
             __builtin_amdgcn_wave_barrier();   // LDS serves a wave's accesses in order; the compiler must too
 #pragma unroll
@@ -100,30 +113,29 @@ __global__ void __launch_bounds__(kSsThreads) skinny_stream_kernel(const SkinnyP
             __builtin_amdgcn_wave_barrier();
         }
     };
-    // Software pipeline over the four tiles of a slice: W runs three tiles ahead (it comes from HBM), X two
-    // (it comes from L2), so the stream of a wave goes on while the wave passes a tile through LDS and the
-    // matrix core.  Loads return in order, which is why the X tile is issued before the W tile that follows it.
+    // Software pipeline over the tiles of a slice: a ring of kSsRing tiles per wave, the loads of tile t + kSsRing
+    // issued as soon as tile t has left its registers, so the stream of a wave goes on while the wave passes a
+    // tile through LDS and the matrix core.  A deeper ring does not help: a wave that asks for more than the
+    // compute unit's memory pipeline takes at once stalls at the issue of its loads, in front of the tile that
+    // has long arrived.
     for (int k0 = wave * kSsSlice; k0 < p.K; k0 += kSsWaves * kSsSlice) {
-        f32x4 w0[kSsLoadsPerTile], w1[kSsLoadsPerTile], w2[kSsLoadsPerTile];
-        f32x4 x0[kSsLoadsPerTile], x1[kSsLoadsPerTile];
-        load_w(w0, k0);
-        load_x(x0, k0);
-        load_w(w1, k0 + kSsTileK);
-        load_x(x1, k0 + kSsTileK);
-        load_w(w2, k0 + 2 * kSsTileK);
-        __builtin_amdgcn_sched_barrier(0);
-        consume(w0, x0, k0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_x(x0, k0 + 2 * kSsTileK);
-        load_w(w0, k0 + 3 * kSsTileK);
-        __builtin_amdgcn_sched_barrier(0);
-        consume(w1, x1, k0 + kSsTileK);
-        __builtin_amdgcn_sched_barrier(0);
-        load_x(x1, k0 + 3 * kSsTileK);
-        __builtin_amdgcn_sched_barrier(0);
-        consume(w2, x0, k0 + 2 * kSsTileK);
-        __builtin_amdgcn_sched_barrier(0);
-        consume(w0, x1, k0 + 3 * kSsTileK);
+        f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kSsLoadsPerTile];
+        ss_static_for<0, kSsRing>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            load_w(w[t], k0 + t * kSsTileK);
+            load_x(x[t], k0 + t * kSsTileK);
+        });
+        ss_static_for<0, kSsTiles>([&](auto tc) {
+            constexpr int t = decltype(tc)::value;
+            constexpr int slot = t % kSsRing;
+            __builtin_amdgcn_sched_barrier(0);
+            consume(w[slot], x[slot], k0 + t * kSsTileK);
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (t + kSsRing < kSsTiles) {
+                load_w(w[slot], k0 + (t + kSsRing) * kSsTileK);
+                load_x(x[slot], k0 + (t + kSsRing) * kSsTileK);
+            }
+        });
     }
 
     // acc[v] = D[m = 4 * g + v][n = n0 + r]; the tiles are free now: wave w parks its result in its W tile
