@@ -109,33 +109,39 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
             load_operand(b[u], brow, p.b_ks, k, std::integral_constant<bool, B_KC>{});
         }
     };
-    // rounds of U groups per wave; the next round's loads are issued before this round's MFMAs
-    // Every load is unconditional (a round past the end reads k = 0 again): a load under a condition is waited
-    // for at the join before anything else issues.
-    int g0 = wave * (T == 32 ? 1 : U);
-    load(g0);
-    while (g0 < ngroups) {
-        f32x4 a_now[U], b_now[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            a_now[u] = a[u];
-            b_now[u] = b[u];
-        }
-        load(g0 + U * kWsWaves);
+    // Rounds of U groups per wave; the next round's loads are issued before this round's MFMAs.  No load sits
+    // under a condition inside the loop (it would be waited for at the join before anything else issues); the
+    // last round runs after the loop, without a prefetch.
+    auto multiply = [&](const f32x4(&av)[U], const f32x4(&bv)[U], int g0) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int k = (g0 + u * GS) * KG + 4 * kq;
-            const f32x4 av = mask_operand(a_now[u], k, std::integral_constant<bool, A_KC>{});
-            const f32x4 bv = mask_operand(b_now[u], k, std::integral_constant<bool, B_KC>{});
+            const f32x4 am = mask_operand(av[u], k, std::integral_constant<bool, A_KC>{});
+            const f32x4 bm = mask_operand(bv[u], k, std::integral_constant<bool, B_KC>{});
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 if constexpr (T == 32)
-                    acc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[j], bv[j], acc[u & 1], 0, 0, 0);
+                    acc[u & 1] = __builtin_amdgcn_mfma_f32_32x32x2f32(am[j], bm[j], acc[u & 1], 0, 0, 0);
                 else
-                    acc[u & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[j], bv[j], acc[u & 1], 0, 0, 0);
+                    acc[u & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(am[j], bm[j], acc[u & 1], 0, 0, 0);
             }
         }
-        g0 += U * kWsWaves;
+    };
+    int g0 = wave * (T == 32 ? 1 : U);
+    if (g0 < ngroups) {   // uniform per wave
+        load(g0);
+        for (int next = g0 + U * kWsWaves; next < ngroups; next += U * kWsWaves) {
+            f32x4 a_now[U], b_now[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                a_now[u] = a[u];
+                b_now[u] = b[u];
+            }
+            load(next);
+            multiply(a_now, b_now, g0);
+            g0 = next;
+        }
+        multiply(a, b, g0);
     }
 
 #pragma unroll
