@@ -4,8 +4,8 @@
 //
 // A workgroup of eight waves owns 16 rows of W and all of K; wave w owns the slices of 512 reduction
 // steps number w, w+8, ...  Everything up to the final sum is private to a wave, so there is no
-// barrier in the stream: a wave loads its slice tile by tile (16 x 64 of W and of X, 256 contiguous
-// bytes per row and load; rows of X beyond M are not loaded), two tiles ahead of the tile it is
+// barrier in the stream: a wave loads its slice tile by tile (16 x 32 of W and of X, one 128-byte
+// line per row and load; rows of X beyond M are not loaded), two tiles ahead of the tile it is
 // working on, and passes both through its own LDS tiles into the operand layout of
 // v_mfma_f32_16x16x4_f32 (row = lane % 16, k group = lane / 16).  Loading in operand layout directly
 // would touch 64 bytes per row and load, which costs a third of the bandwidth.  The matrix core only
@@ -25,14 +25,14 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kSsWaves = 8;
 constexpr int kSsThreads = 64 * kSsWaves;
-constexpr int kSsSlice = 512;                 // reduction steps per wave and pass of the pipeline: four tiles
-constexpr int kSsTileK = 32;                  // k per staged tile: 256 contiguous bytes per row
+constexpr int kSsSlice = 512;                 // reduction steps per wave and pass of the pipeline
+constexpr int kSsTileK = 32;                  // k per staged tile: one 128-byte line per row
 constexpr int kSsTiles = kSsSlice / kSsTileK; // tiles per slice
 constexpr int kSsRing = 3;                    // tiles of a wave in registers: one at work, the others on their way
 constexpr int kSsLanesPerRow = kSsTileK / 4;
 constexpr int kSsRowsPerLoad = 64 / kSsLanesPerRow;
 constexpr int kSsTileStride = kSsTileK + 4;
-constexpr int kSsLoadsPerTile = 16 * kSsTileK / 4 / 64;   // 128-bit loads per lane and tile: 8
+constexpr int kSsLoadsPerTile = 16 * kSsTileK / 4 / 64;   // 128-bit loads per lane and tile
 
 template <int B, int E, typename F>
 __device__ __forceinline__ void ss_static_for(F&& f) {
@@ -74,8 +74,8 @@ __global__ void __launch_bounds__(kSsThreads) skinny_stream_kernel(const SkinnyP
         *reinterpret_cast<f32x4*>(tx + (kSsRowsPerLoad * j + lrow) * kSsTileStride + lk) = f32x4{0.f, 0.f, 0.f, 0.f};
 
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    // One tile = 16 rows x 128 k of W and of X, eight 128-bit loads per lane each.  Addresses past K are
-    // clamped into the row (every load is unconditional); what they return is zeroed on the way to LDS.
+    // One tile = 16 rows x kSsTileK k of W and of X, kSsLoadsPerTile 128-bit loads per lane each.  Addresses past
+    // K are clamped into the row (every load is unconditional); what they return is zeroed on the way to LDS.
     auto load_w = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
 #pragma unroll
         for (int j = 0; j < kSsLoadsPerTile; j++) {
