@@ -1,7 +1,8 @@
 // Chooses the kernel for one (batched) product: the bandwidth-bound skinny kernel for at
-// most 16 rows against a K-contiguous weight matrix, otherwise the MFMA kernel in the LDS
-// orientation pair that matches how the operands lie in memory, with the largest tile that still
-// fills the 256 compute units.
+// most 16 rows against a K-contiguous weight matrix, the wave-split kernel for small products that
+// one launch can finish in a few microseconds, otherwise the MFMA kernel in the LDS orientation
+// pair that matches how the operands lie in memory, with the tile that needs the fewest rounds
+// over the compute units.
 #include <algorithm>
 
 #include "elementwise.h"
@@ -111,8 +112,6 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         int64_t split = compute_units() / tiles;
         if (split > d.K / kSplitMinK) split = d.K / kSplitMinK;
         if (split > kSplitMax) split = kSplitMax;
-        // equal parts of whole 16-step tiles if some part count allows it, else parts that at least keep
-        // the operands' 16-byte alignment
         // equal parts of whole 16-step tiles if some part count allows it; else parts of whole tiles with a
         // shorter last one, which the general kernel variant handles
         int64_t whole = split;
