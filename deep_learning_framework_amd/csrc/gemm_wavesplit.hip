@@ -1,8 +1,9 @@
 // Small products with a long reduction: C[M,N] (=|+=) act(alpha * sum_k A(m,k) B(n,k) + bias) for the engine's
 // dense layer (VMath::matmul / matmul_backward_x / matmul_backward_w, vmath.cu:2961-3093 of the reference), when
 // the output has too few tiles to fill the chip and the tiled kernel would cut K over workgroups and sum the
-// parts in a second launch.  Each operand is either K-contiguous ("KC": one 128-bit load gives a lane its four k)
-// or contiguous along its output index ("MC": four 32-bit loads, the lanes of a row group side by side).
+// parts in a second launch.  Each operand is either K-contiguous ("KC": one 128-bit load gives a lane its four k;
+// rows may start at any float address) or contiguous along its output index ("MC": four 32-bit loads, the lanes
+// of a row group side by side).
 //
 // Here the reduction is cut over the WAVES of one workgroup instead.  A workgroup owns one T x T block of C
 // (T = 32 on v_mfma_f32_32x32x2_f32, T = 16 on v_mfma_f32_16x16x4_f32).  K is dealt out in rounds of
@@ -21,6 +22,8 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+// four consecutive floats at any float address: global memory takes 128-bit loads at 4-byte alignment
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
 
 constexpr int kWsWaves = 16;
 constexpr int kWsFlight = 4;   // k-groups per wave in flight
@@ -68,7 +71,6 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
     // rows past the end are read from the last row and never stored
     const float* __restrict__ arow = p.A + (int64_t)min(m0 + r, p.M - 1) * p.a_rs;
     const float* __restrict__ brow = p.B + (int64_t)min(n0 + r, p.N - 1) * p.b_rs;
-    const int ngroups = (p.K + KG - 1) / KG;
 
     typedef typename std::conditional<T == 32, f32x16, f32x4>::type acc_t;
     acc_t acc[2];
@@ -77,26 +79,29 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
 #pragma unroll
         for (int i = 0; i < NR; i++) acc[h][i] = 0.f;
 
-    // A KC operand needs K to be a multiple of 4 (host check): a lane's chunk is inside the row as a whole or not
-    // at all.  What lies past the end of K is loaded from k = 0 (every load is unconditional) and zeroed.
+    // The rounds cover K4 = K rounded down to a multiple of 4, so that a KC operand's chunk is inside the row as a
+    // whole or not at all; wave 0 adds the last one to three k afterwards.  What lies past the end is loaded
+    // from k = 0 (every load is unconditional) and zeroed.
+    const int K4 = (A_KC || B_KC) ? (p.K & ~3) : p.K;
+    const int ngroups = (K4 + KG - 1) / KG;
     f32x4 a[U], b[U];
     auto load_operand = [&](f32x4& dst, const float* __restrict__ row, int64_t ks, int k, auto kc_tag) {
         if constexpr (decltype(kc_tag)::value) {
-            dst = *reinterpret_cast<const f32x4*>(row + (k < p.K ? k : 0));
+            dst = *reinterpret_cast<const f32x4u*>(row + (k < K4 ? k : 0));
         } else {
 #pragma unroll
-            for (int j = 0; j < 4; j++) dst[j] = row[(int64_t)(k + j < p.K ? k + j : 0) * ks];
+            for (int j = 0; j < 4; j++) dst[j] = row[(int64_t)(k + j < K4 ? k + j : 0) * ks];
         }
     };
     auto mask_operand = [&](f32x4 v, int k, auto kc_tag) -> f32x4 {
         if constexpr (decltype(kc_tag)::value) {
-            return keep_if(v, k < p.K);
+            return keep_if(v, k < K4);
         } else {
             f32x4 o;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const float e = v[j];
-                o[j] = __int_as_float(__float_as_int(e) & (k + j < p.K ? -1 : 0));
+                o[j] = __int_as_float(__float_as_int(e) & (k + j < K4 ? -1 : 0));
             }
             return o;
         }
@@ -143,6 +148,23 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
         }
         multiply(a, b, g0);
     }
+    if ((A_KC || B_KC) && wave == 0 && K4 < p.K) {   // uniform: the one to three k past K4, in the lanes of k group 0
+        f32x4 at = {0.f, 0.f, 0.f, 0.f}, bt = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            if (kq == 0 && K4 + j < p.K) {
+                at[j] = arow[(int64_t)(K4 + j) * p.a_ks];
+                bt[j] = brow[(int64_t)(K4 + j) * p.b_ks];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            if constexpr (T == 32)
+                acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(at[j], bt[j], acc[0], 0, 0, 0);
+            else
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(at[j], bt[j], acc[0], 0, 0, 0);
+        }
+    }
 
 #pragma unroll
     for (int i = 0; i < NR; i++) red[(wave * NR + i) * 64 + lane] = acc[0][i] + acc[1][i];
@@ -172,14 +194,11 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
 
 }  // namespace
 
-// Each operand K-contiguous with 128-bit loads legal, or contiguous along its output index; a contiguous output
-// row, one product.  Whether the product is small enough for this kernel to win is the dispatcher's decision.
+// Each operand K-contiguous or contiguous along its output index; a contiguous output row, one product.  Whether the product is small enough for this kernel to win is the dispatcher's decision.
 bool wavesplit_applies(const GemmDesc& d) {
-    const bool a_kc = d.a_ks == 1 && d.a_rs % 4 == 0 && aligned16(d.A) && d.K % 4 == 0;
-    const bool b_kc = d.b_ks == 1 && d.b_rs % 4 == 0 && aligned16(d.B) && d.K % 4 == 0;
-    const bool a_mc = d.a_rs == 1 && d.a_ks != 1, b_mc = d.b_rs == 1 && d.b_ks != 1;
-    return d.nbatch == 1 && (a_kc || a_mc) && (b_kc || b_mc) && d.c_cs == 1 && d.rowsum == nullptr && d.k_part == 0 &&
-           d.K >= 1 && d.K <= (1 << 24) && d.act >= kActNone && d.act <= kActSwish;
+    const bool a_ok = d.a_ks == 1 || d.a_rs == 1, b_ok = d.b_ks == 1 || d.b_rs == 1;
+    return d.nbatch == 1 && a_ok && b_ok && d.c_cs == 1 && d.rowsum == nullptr && d.k_part == 0 && d.K >= 1 &&
+           d.K <= (1 << 24) && d.act >= kActNone && d.act <= kActSwish;
 }
 
 template <int T>

@@ -557,10 +557,11 @@ def test_split_k_scratch_survives_shutdown_and_growth():
 
 WAVE_SPLIT = [
     # M, N, K: 16 x 16 blocks (few workgroups) and 32 x 32 blocks (more of them), whole and ragged blocks, K with and
-    # without a rest after the last round, K shorter than one round, K no multiple of 4 (forms without a K-contiguous
-    # operand only; the others run the tiled kernel there)
+    # without a rest after the last round, K shorter than one round
     (64, 512, 784), (256, 1024, 1024), (100, 300, 1000), (17, 33, 44), (31, 77, 1001), (300, 300, 300),
     (16, 16, 2048), (50, 70, 4), (33, 17, 1), (512, 1024, 512), (192, 1000, 1000), (9, 200, 1030), (128, 512, 260),
+    # rows that start at odd float addresses (128-bit loads at 4-byte alignment) and one to three k after the rounds
+    (64, 512, 783), (256, 1024, 1023), (1000, 333, 777), (130, 70, 2),
 ]
 
 
