@@ -49,6 +49,8 @@ inline GemmParams make_params(const GemmDesc& d, bool a_kc, bool b_kc) {
     const int64_t b_cont = b_kc ? d.b_ks : d.b_rs, b_ld = b_kc ? d.b_rs : d.b_ks;
     p.a_vec = a_cont == 1 && a_ld % 4 == 0 && d.a_bs0 % 4 == 0 && d.a_bs1 % 4 == 0 && aligned16(d.A);
     p.b_vec = b_cont == 1 && b_ld % 4 == 0 && d.b_bs0 % 4 == 0 && d.b_bs1 % 4 == 0 && aligned16(d.B);
+    p.a_cont = a_cont == 1;
+    p.b_cont = b_cont == 1;
     p.c_vec = d.c_cs == 1 && d.c_rs % 4 == 0 && d.N % 4 == 0 && d.c_bs0 % 4 == 0 && d.c_bs1 % 4 == 0 &&
               aligned16(d.C) && (d.C2 == nullptr || aligned16(d.C2)) && (d.bias == nullptr || aligned16(d.bias));
     p.act = d.act;
@@ -75,12 +77,13 @@ inline bool fits_buffer_offsets(const GemmParams& p, bool a_kc, bool b_kc, int B
     return a_span * 4 < (1ll << 31) && b_span * 4 < (1ll << 31);
 }
 
-// true when the pipelined kernel's general variant may run the problem: 128-bit loads are legal for both
-// operands (M, N and K themselves are arbitrary: rows past the end are never stored, the last partial K-tile
-// is masked) and the reduction is not cut over the batch index
+// true when the pipelined kernel's general variant may run the problem: both operands have a unit stride (its
+// buffer loads fetch 128 bits at any 4-byte aligned address; M, N, K and the leading dimensions are arbitrary:
+// rows past the end are never stored, the last partial K-tile is masked) and the reduction is not cut over
+// the batch index
 inline bool fits_ragged_pipe(const GemmParams& p, bool a_kc, bool b_kc, int BM, int BN) {
     const int64_t a_ld = a_kc ? p.a_rs : p.a_ks, b_ld = b_kc ? p.b_rs : p.b_ks;
-    return p.k_part == 0 && p.a_vec && p.b_vec && p.K > 0 && a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30) &&
+    return p.k_part == 0 && p.a_cont && p.b_cont && p.K > 0 && a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30) &&
            fits_buffer_offsets(p, a_kc, b_kc, BM, BN);
 }
 

@@ -24,12 +24,14 @@
 //    global loads with the MFMAs one by one, for large whole-tile products.
 //  * Shapes that are whole multiples of the tile with 16-byte aligned operands
 //    run a kernel variant with predicate-free 128-bit loads (EDGE = false).  The
-//    general variant loads through buffer resources that end with the operand (or
-//    through clamped addresses), 128-bit or element-wise as chosen once per
-//    workgroup, and zeroes what lies outside the matrix when the tile moves to
-//    LDS: no load in any loop sits behind a branch.  With the slot schedule it
-//    masks only the last, partial K-tile: rows past the operand never reach a
-//    stored output.
+//    general variant loads through buffer resources that end with the operand:
+//    128 bits at a time for an operand with a unit stride (any 4-byte aligned
+//    address will do, and the range is checked dword by dword), element-wise for
+//    one that is strided both ways, as chosen once per workgroup; it zeroes what
+//    lies outside the matrix when the tile moves to LDS: no load in any loop sits
+//    behind a branch.  With the slot schedule it masks only the last, partial
+//    K-tile: rows past the operand never reach a stored output.  (A tile that
+//    spans 2 GiB or more falls back to flat, clamped, element-wise loads.)
 //  * A single product can be cut along K over the batch dimension (k_part) and can
 //    sum the rows of A on the side (ROWSUM, the bias gradient of a dense layer).
 //  * Workgroup ids are remapped so that the workgroups that share one XCD (and its
@@ -76,7 +78,8 @@ struct GemmParams {
     // batch z = blockIdx.z is split as (z / bdiv, z % bdiv); offset = q*bs0 + r*bs1
     int64_t a_bs0, a_bs1, b_bs0, b_bs1, c_bs0, c_bs1;
     int bdiv;
-    int a_vec, b_vec, c_vec;  // 128-bit access along the contiguous index is legal
+    int a_vec, b_vec, c_vec;  // 16-byte aligned 128-bit access along the contiguous index is legal
+    int a_cont, b_cont;       // the operand has a unit stride (then buffer loads may fetch 128 bits at 4-byte alignment)
     int edge_buf;             // general kernels: a tile of either operand spans less than 2 GiB (buffer loads)
     int act;
     int accflag;
@@ -153,13 +156,6 @@ __device__ __forceinline__ void load_tile_chunk(f32x4 (&reg)[ROWS * BK / 4 / NT]
 // under a condition makes the compiler wait for it before it issues the next one); what lies
 // outside the matrix is zeroed by mask_tile_edge() when the tile moves on to LDS, not here: a mask
 // right behind the load would bring the wait for it along.
-// true when 128-bit chunks may be used for every tile of a workgroup's operand: the operand allows
-// them at all and no chunk straddles the end of the index it runs along (k for KC, rows for MC)
-template <bool KC, int ROWS>
-__device__ __forceinline__ bool edge_operand_vec(int rows_left, int k_total, int vec_ok) {
-    return vec_ok && (KC ? (k_total & 3) == 0 : (rows_left >= ROWS || (rows_left & 3) == 0));
-}
-
 template <bool KC, int ROWS, int BK, int NT, bool VEC>
 __device__ __forceinline__ void load_tile_edge(f32x4 (&reg)[ROWS * BK / 4 / NT], const float* __restrict__ base,
                                                int64_t rs, int64_t ks, int rows_left, int k_left, int tid) {
@@ -777,8 +773,9 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
             } else if (!p.edge_buf) {
                 pipe0(no{}, no{}, no{});   // a tile spans 2 GiB or more: flat element-wise loads
             } else {
-                const bool va = edge_operand_vec<A_KC, BM>(rows_a, Kz, p.a_vec);
-                const bool vb = edge_operand_vec<B_KC, BN>(rows_b, Kz, p.b_vec);
+                // Buffer loads fetch 128 bits at any 4-byte aligned address, a chunk that runs past the end of
+                // its row or of the operand brings data that the mask removes or zeros: a unit stride is enough.
+                const bool va = p.a_cont != 0, vb = p.b_cont != 0;
                 if (va && vb) pipe0(yes{}, yes{}, yes{});
                 else if (va) pipe0(yes{}, no{}, yes{});
                 else if (vb) pipe0(no{}, yes{}, yes{});
