@@ -57,6 +57,28 @@ double wavesplit_estimate(const GemmDesc& d, int T) {
     return (4.0 + std::max(2.7e-5 * (double)wgs * K, 6.45e-3 * K)) * forms;
 }
 
+// Number of parts for a long reduction on the 64x64 tile.  A compute unit that holds one workgroup spends
+// 0.53 us per 32 reduction steps (store to LDS, barrier, read, 16 dependent MFMAs: a chain), one that holds two
+// or more 0.43 us per 32 steps of any of them (the MFMA rate); the parts cost a second launch and their
+// traffic (5 us + 0.5 us per part, measured).  So cutting K pays twice where it turns a partly filled round over
+// the compute units into full ones or brings a second workgroup onto each (768^2 x 4096: 76 -> 59 us with 4
+// parts, 1536^2 x 4096: 190 -> 158, 1024^2 x 8192: 154 -> 134), and not where the tiles already do both.
+int64_t small_tile_split(int64_t tiles, int64_t K, int64_t cus) {
+    int64_t best = 1;
+    double best_cost = 0.0;
+    for (int64_t s = 1; s <= kSplitMax; s *= 2) {
+        if (s > 1 && K / s < 256) break;
+        const int64_t per_cu = (tiles * s + cus - 1) / cus;
+        const double cost = (double)per_cu * ((double)K / (double)s / 32.0) * (per_cu >= 2 ? 0.43 : 0.53) +
+                            (s > 1 ? 5.0 + 0.5 * (double)s : 0.0);
+        if (s == 1 || cost < 0.97 * best_cost) {
+            best = s;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
 GemmPlan plan_gemm(const GemmDesc& d) {
     GemmPlan plan;
     // skinny: y = x . w^T with both operands K-contiguous, a contiguous output row, no scaling
@@ -110,6 +132,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         const int64_t edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
         const int64_t tiles = tiles_of(d.M, d.N, 1, edge);
         int64_t split = compute_units() / tiles;
+        if (plan.tile == kTileSmall && d.K >= 1024) split = small_tile_split(tiles, d.K, cus);
         if (split > d.K / kSplitMinK) split = d.K / kSplitMinK;
         if (split > kSplitMax) split = kSplitMax;
         // equal parts of whole 16-step tiles if some part count allows it; else parts of whole tiles with a
