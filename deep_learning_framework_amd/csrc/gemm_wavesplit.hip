@@ -8,11 +8,12 @@
 // Here the reduction is cut over the WAVES of one workgroup instead.  A workgroup owns one T x T block of C
 // (T = 32 on v_mfma_f32_32x32x2_f32, T = 16 on v_mfma_f32_16x16x4_f32).  K is dealt out in rounds of
 // WAVES x kWsFlight k-groups (a group = one 128-bit load per lane and operand, 8 or 16 consecutive k); in every
-// round a wave takes kWsFlight of them, consecutive ones (T = 16) or every WAVES-th (T = 32; measured, see the
-// dispatcher), straight from global memory into the MFMA operands: a lane's four consecutive k feed four successive MFMAs, and both operands use the same
-// lane -> k mapping, so products pair equal k.  No LDS staging, no barrier in the loop.  The partial blocks meet
-// in LDS, one thread per output element adds them in wave order (a fixed order: results do not depend on timing)
-// and runs the epilogue.  One launch, and its critical path is one wave's share of K.
+// round a wave takes kWsFlight of them -- consecutive ones for T = 16, every WAVES-th for T = 32, each the faster
+// choice where the dispatcher uses that block size -- straight from global memory into the MFMA operands: a
+// lane's four consecutive k feed four successive MFMAs, and both operands use the same lane -> k mapping, so
+// products pair equal k.  No LDS staging, no barrier in the loop.  The partial blocks meet in LDS, one thread
+// per output element adds them in wave order (a fixed order: results do not depend on timing) and runs the
+// epilogue.  One launch, and its critical path is one wave's share of K.
 #include "act_funcs.h"
 #include "gemm_host.h"
 
