@@ -20,6 +20,7 @@ static int64_t tiles_of(int64_t M, int64_t N, int64_t nbatch, int64_t t) {
 constexpr int64_t kSplitFromK = 512;
 constexpr int64_t kSplitMinK = 64;
 constexpr int64_t kSplitMax = 16;
+constexpr int64_t kSplitScratchMax = 64ll << 20;   // bytes of partial sums a product may ask of the library scratch
 
 static int launch_layout(const GemmParams& p, bool a_kc, bool b_kc, int64_t nbatch, int tile, hipStream_t stream) {
     if (a_kc && b_kc) return launch_gemm_kc_kc(p, nbatch, tile, stream);
@@ -133,6 +134,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         const int64_t tiles = tiles_of(d.M, d.N, 1, edge);
         int64_t split = compute_units() / tiles;
         if (plan.tile == kTileSmall && d.K >= 1024) split = small_tile_split(tiles, d.K, cus);
+        while (split > 1 && split * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) split /= 2;
         if (split > d.K / kSplitMinK) split = d.K / kSplitMinK;
         if (split > kSplitMax) split = kSplitMax;
         // equal parts of whole 16-step tiles if some part count allows it; else parts of whole tiles with a
