@@ -4,6 +4,7 @@
 // pair that matches how the operands lie in memory, with the tile that needs the fewest rounds
 // over the compute units.
 #include <algorithm>
+#include <string>
 
 #include "elementwise.h"
 #include "gemm_host.h"
@@ -52,7 +53,7 @@ double wavesplit_estimate(const GemmDesc& d, int T) {
     const double forms = 1.0 + 0.12 * ((d.a_ks != 1) + (d.b_ks != 1));
     if (T == 16) {
         if (d.K > 2048 || wgs > 1024) return -1.0;
-        return (3.8 + std::max(1.3e-5 * (double)wgs * K, 3.3e-3 * K)) * forms;
+        return (3.8 + std::max(1.3e-5 * (double)wgs * K, 3.1e-3 * std::max(0.0, K - 256.0))) * forms;
     }
     if (d.K > 1024 || wgs > 512 || (d.K < 256 && wgs > 256)) return -1.0;
     return (4.0 + std::max(2.7e-5 * (double)wgs * K, 6.45e-3 * K)) * forms;
@@ -166,6 +167,43 @@ bool gemm_fuses_rowsum(const GemmDesc& d) {
     if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
     const GemmPlan plan = plan_gemm(d);
     return !plan.skinny && !plan.wavesplit_edge && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge && plan.split == 1;
+}
+
+// What launch_gemm would do with this product, as text: the kernel family and, for the tiled kernel, tile,
+// variant and the number of parts K is cut into.  Host arithmetic only, nothing is launched or allocated.
+std::string describe_gemm(const GemmDesc& d) {
+    if (!valid_dims(d)) return "invalid";
+    if (d.M == 0 || d.N == 0 || d.nbatch == 0) return "nothing";
+    const GemmPlan plan = plan_gemm(d);
+    if (plan.wavesplit_edge) return "wavesplit " + std::to_string(plan.wavesplit_edge);
+    if (plan.skinny) return "skinny";
+    if (shortk_nt_applies(plan.dn)) return "shortk_nt";
+    if (shortk_heads_applies(plan.dn)) return "shortk_heads";
+    if (heads_pv_applies(d)) return "heads_pv";
+    const bool a_kc = plan.a_kc, b_kc = plan.b_kc;
+    GemmDesc dt = plan.dn;
+    if (plan.split >= 2) {
+        if (plan.ragged_parts) dt.k_part = plan.k_part;
+        else dt.K = plan.k_part;
+        dt.nbatch = plan.split; dt.bdiv = 1;
+        dt.a_bs0 = plan.k_part * d.a_ks; dt.b_bs0 = plan.k_part * d.b_ks; dt.c_bs0 = d.M * d.N;
+        dt.a_bs1 = dt.b_bs1 = dt.c_bs1 = 0;
+        dt.c_rs = d.N; dt.c_cs = 1;
+    }
+    const GemmParams p = make_params(dt, a_kc, b_kc);
+    const int edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
+    const char* tile = plan.tile == kTileLarge ? "large" : plan.tile == kTileMedium ? "medium" : "small";
+    const char* variant = "general";
+    if (plan.tile != kTileSmall) {
+        const int bk = plan.tile == kTileLarge ? 16 : 32;
+        if (fits_without_edges(p, a_kc, b_kc, edge, edge, bk) && fits_buffer_offsets(p, a_kc, b_kc, edge, edge))
+            variant = "whole pipelined";
+        else if (fits_ragged_pipe(p, a_kc, b_kc, edge, edge)) variant = "ragged pipelined";
+    } else if ((fits_without_edges(p, a_kc, b_kc, 64, 64, 32) || fits_without_edges(p, a_kc, b_kc, 64, 64, 16)) &&
+               fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
+        variant = "whole";
+    }
+    return std::string("mfma ") + tile + " " + variant + " split " + std::to_string(plan.split);
 }
 
 int launch_gemm(const GemmDesc& d, hipStream_t stream) {

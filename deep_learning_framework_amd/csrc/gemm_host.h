@@ -2,6 +2,8 @@
 // configuration.  Used by gemm_dispatch.hip, which picks the configuration.
 #pragma once
 
+#include <string>
+
 #include "gemm_mfma.h"
 #include "kai_common.h"
 
@@ -111,6 +113,8 @@ int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t st
 
 // picks kernel family, tile and variant; defined in gemm_dispatch.hip
 int launch_gemm(const GemmDesc& d, hipStream_t stream);
+// the decision of launch_gemm as text (host arithmetic only)
+std::string describe_gemm(const GemmDesc& d);
 // true when launch_gemm would compute GemmDesc::rowsum inside the product's own launch (d.rowsum is
 // not looked at); otherwise the caller runs a separate column-sum kernel and leaves rowsum null
 bool gemm_fuses_rowsum(const GemmDesc& d);

@@ -285,6 +285,29 @@ int kai_gemm_f32(int device, int transA, int transB, int64_t M, int64_t N, int64
     return launch_gemm(d, current_stream());
 }
 
+int kai_gemm_plan(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                  int has_bias, int actFunc, int acc, char* out, int buflen) {
+    KAI_REQUIRE_PTR(out);
+    KAI_REQUIRE(buflen > 0, KAI_ERR_INVALID_ARGUMENT, "buflen <= 0");
+    KAI_REQUIRE_DIM(M); KAI_REQUIRE_DIM(N); KAI_REQUIRE_DIM(K);
+    KAI_REQUIRE(act_is_elementwise(actFunc), KAI_ERR_CONDITIONAL_STATEMENT, "activation code must be 0..8");
+    KAI_REQUIRE(lda >= (transA ? M : K) && ldb >= (transB ? K : N) && ldc >= N, KAI_ERR_INVALID_ARGUMENT,
+                "leading dimension smaller than the row length");
+    // stand-ins for 16-byte aligned operands; nothing dereferences them
+    static float dummy[16] __attribute__((aligned(64)));
+    GemmDesc d;
+    d.A = dummy; d.B = dummy; d.C = dummy; d.bias = has_bias ? dummy : nullptr;
+    d.M = M; d.N = N; d.K = K;
+    if (transA) { d.a_rs = 1; d.a_ks = lda; } else { d.a_rs = lda; d.a_ks = 1; }
+    if (transB) { d.b_rs = ldb; d.b_ks = 1; } else { d.b_rs = 1; d.b_ks = ldb; }
+    d.c_rs = ldc; d.c_cs = 1;
+    d.act = actFunc; d.acc = acc != 0;
+    const std::string text = describe_gemm(d);
+    std::strncpy(out, text.c_str(), (size_t)buflen - 1);
+    out[buflen - 1] = 0;
+    return KAI_OK;
+}
+
 int kai_matmul(int device, float* py, const float* pw, const float* px, int64_t yvec, int64_t ndat, int64_t xvec,
                int acc) {
     // y[ndat,yvec] = x[ndat,xvec] . w[yvec,xvec]^T : A = x (K-contiguous), B = w stored [N,K]

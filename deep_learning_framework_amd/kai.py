@@ -60,6 +60,7 @@ SIGNATURES = {
     "kai_mix_values_backward_prop": [_INT, _F, _F, _F, _I64, _I64, _I64, _I64, _I64],
     "kai_mix_values_backward_value": [_INT, _F, _F, _F, _I64, _I64, _I64, _I64, _I64],
     "kai_gemm_f32": [_INT, _INT, _INT, _I64, _I64, _I64, _F, _I64, _F, _I64, _F, _I64, _F, _INT, _F, _INT],
+    "kai_gemm_plan": [_INT, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _INT, _INT, _INT, ctypes.c_char_p, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
     "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
     "kai_cosinesim": [_INT, _F, _F, _F, _I64, _I64, _I64],
@@ -311,6 +312,17 @@ class VMath:
     def gemm_f32(device, transA, transB, M, N, K, A, lda, B, ldb, C, ldc, bias, actFunc, hLeakyAlpha, acc):
         _ck(load().kai_gemm_f32(device, int(transA), int(transB), M, N, K, _addr(A), lda, _addr(B), ldb, _addr(C),
                                 ldc, _addr(bias), actFunc, _addr(hLeakyAlpha), int(acc)))
+
+    @staticmethod
+    def gemm_plan(transA, transB, M, N, K, lda=None, ldb=None, ldc=None, has_bias=False, actFunc=0, acc=False):
+        """Text naming the kernel kai_gemm_f32 would launch for aligned operands of this shape (no GPU needed)."""
+        lda = (M if transA else K) if lda is None else lda
+        ldb = (K if transB else N) if ldb is None else ldb
+        ldc = N if ldc is None else ldc
+        buf = ctypes.create_string_buffer(128)
+        _ck(load().kai_gemm_plan(int(transA), int(transB), M, N, K, lda, ldb, ldc, int(has_bias), actFunc, int(acc),
+                                 buf, 128))
+        return buf.value.decode()
 
     @staticmethod
     def cosinesim(device, py, px1, px2, nrow1, nrow2, ncol):

@@ -180,6 +180,14 @@ int kai_gemm_f32(int device, int transA, int transB, int64_t M, int64_t N, int64
                  const float* B, int64_t ldb, float* C, int64_t ldc, const float* bias, int actFunc,
                  const float* hLeakyAlpha, int acc);
 
+/* No counterpart in the reference (its kernels are one per method).  Writes into `out` which kernel
+ * kai_gemm_f32 would launch for 16-byte aligned operands of this shape, as text: "wavesplit 16",
+ * "skinny", "shortk_nt", "mfma large whole pipelined split 1", "mfma small general split 4" ...  Host
+ * arithmetic only: nothing is launched or allocated and no GPU is needed (without one the choice is made
+ * for 256 compute units).  For maintainers and tests of the dispatch rules. */
+int kai_gemm_plan(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                  int has_bias, int actFunc, int acc, char* out, int buflen);
+
 /* The engine's `dense` layer formula activate(add(matmul(x,w),b)) (api/vconst.cpp:11) in one launch:
  * py = act(x . w^T + b).  ppre, if not null, receives the pre-activation x . w^T + b that
  * VTensor::activate_backprop needs (vtensor.cpp:5697-5718).  pb may be null (no bias). */

@@ -129,3 +129,56 @@ def test_tensor_operator_argument_derivation(monkeypatch):
     xg, wg = y.matmul_backprop(T.Tensor((6, 5, 3), buf=FakeBuf()))
     assert calls[-2][0] == "matmul_backward_x" and calls[-2][5:9] == (3, 30, 8, False)
     assert calls[-1][0] == "matmul_backward_w" and wg.shape == (3, 8) and xg.shape == (6, 5, 8)
+
+
+# ---- which kernel a product gets: the dispatcher's rules, from its host-only description ------------------
+
+GEMM_PLANS = [
+    # transA, transB, M, N, K -> kernel (for 256 compute units, aligned operands, tight leading dimensions)
+    ((0, 1, 64, 512, 784), "wavesplit 16"),                          # configuration 1: one launch, 16 x 16 blocks
+    ((0, 1, 256, 1024, 1024), "wavesplit 32"),                       # configuration 2 forward
+    ((0, 0, 256, 1024, 1024), "wavesplit 32"),                       # configuration 2 dX: one operand not K-contiguous
+    ((1, 0, 1024, 1024, 256), "mfma small whole split 1"),           # configuration 2 dW: 256 tiles of 64 x 64
+    ((0, 0, 8192, 8192, 8192), "mfma large whole pipelined split 1"),  # the headline product
+    ((0, 1, 8192, 8192, 8192), "mfma large whole pipelined split 1"),
+    ((0, 0, 8191, 8191, 8191), "mfma large ragged pipelined split 1"),  # odd sizes keep the pipelined loop
+    ((0, 1, 4100, 4100, 4100), "mfma medium ragged pipelined split 1"),  # 289 large tiles would need two rounds
+    ((0, 1, 4096, 4096, 4096), "mfma large whole pipelined split 1"),   # exactly one round of large tiles
+    ((0, 1, 3072, 4096, 4096), "mfma medium whole pipelined split 1"),  # 192 large tiles leave a quarter of the chip idle
+    ((0, 1, 2048, 2048, 2048), "mfma medium whole pipelined split 1"),
+    ((0, 1, 1024, 2048, 512), "mfma small whole split 1"),           # 128 medium tiles on 256 units: the finer tile
+    ((0, 1, 1, 4096, 4096), "skinny"),                               # configuration 5
+    ((0, 1, 4, 4096, 4096), "skinny"),
+    ((0, 1, 16, 4096, 4096), "skinny"),
+    ((0, 1, 16, 1024, 1024), "wavesplit 16"),                        # 5..16 rows against a small weight matrix
+    ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
+    ((0, 1, 1000, 333, 777), "wavesplit 32"),                        # configuration 5, ragged: unaligned rows are fine
+    ((0, 1, 64, 64, 8192), "mfma small whole split 16"),             # one tile, a long reduction
+    ((0, 1, 768, 768, 4096), "mfma small whole split 8"),            # K cut to fill the rounds
+    ((0, 1, 1024, 1024, 8192), "mfma small whole split 2"),          # K cut to bring a second workgroup onto each unit
+    ((0, 1, 1024, 1024, 1024), "mfma small whole split 1"),
+    ((0, 1, 128, 128, 4096), "mfma small whole split 8"),            # too long for the one-launch kernel
+    ((0, 1, 0, 5, 5), "nothing"),
+]
+
+
+@pytest.mark.parametrize("args,expected", GEMM_PLANS, ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else None)
+def test_gemm_dispatch_rules(args, expected):
+    assert kai.VMath.gemm_plan(*args) == expected
+
+
+def test_gemm_dispatch_never_cuts_k_beyond_the_scratch_limit():
+    # partial sums of one product stay within 64 MiB of library scratch
+    for m, n, k in [(1536, 1536, 8192), (2000, 2000, 16384), (4000, 1000, 16384), (700, 6000, 32768)]:
+        plan = kai.VMath.gemm_plan(0, 1, m, n, k)
+        split = int(plan.rsplit(" ", 1)[1])
+        assert split == 1 or split * m * n * 4 <= 64 << 20, plan
+
+
+def test_gemm_plan_checks_its_arguments():
+    L = kai.load()
+    buf = ctypes.create_string_buffer(64)
+    assert L.kai_gemm_plan(0, 1, 4, 4, 4, 3, 4, 4, 0, 0, 0, buf, 64) == 510      # lda < K
+    assert L.kai_gemm_plan(0, 1, 4, 4, 4, 4, 4, 4, 0, 9, 0, buf, 64) != 0        # softmax is no element-wise code
+    assert L.kai_gemm_plan(0, 1, 4, 4, 4, 4, 4, 4, 0, 0, 0, None, 64) != 0       # null output
+    assert L.kai_gemm_plan(0, 1, 4, 4, 4, 4, 4, 4, 0, 0, 0, buf, 4) == 0 and len(buf.value) == 3   # truncated, terminated
