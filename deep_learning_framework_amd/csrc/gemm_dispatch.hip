@@ -113,6 +113,9 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         const int64_t rounds_m = (t128 + cus - 1) / cus, rounds_s = (t64 + cus - 1) / cus;
         if (100 * rounds_s >= 340 * rounds_m) plan.tile = kTileMedium;
     }
+    // 17..32 rows against at least 256 columns: a 64-row tile would spend half of its MFMAs on padding, and these
+    // products are bound by the stream of the other operand (32 x 4096 x 4096: 30.6 us with 64 x 64 tiles)
+    if (plan.tile == kTileSmall && d.M <= 32 && d.N >= 256) plan.tile = kTileFlat;
 
     // Small products: one launch of the wave-split kernel where it is expected to finish before the tiled
     // kernel (plus, for long K, its second launch) could: measured, it wins wherever its estimate stays below
@@ -132,9 +135,9 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // applies the epilogue.
     if (!plan.skinny && d.nbatch == 1 && d.K >= kSplitFromK) {
         const int64_t edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
-        const int64_t tiles = tiles_of(d.M, d.N, 1, edge);
+        const int64_t tiles = plan.tile == kTileFlat ? ((d.M + 31) / 32) * ((d.N + 127) / 128) : tiles_of(d.M, d.N, 1, edge);
         int64_t split = compute_units() / tiles;
-        if (plan.tile == kTileSmall && d.K >= 1024) split = small_tile_split(tiles, d.K, cus);
+        if ((plan.tile == kTileSmall || plan.tile == kTileFlat) && d.K >= 1024) split = small_tile_split(tiles, d.K, cus);
         while (split > 1 && split * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) split /= 2;
         if (split > d.K / kSplitMinK) split = d.K / kSplitMinK;
         if (split > kSplitMax) split = kSplitMax;
@@ -166,7 +169,8 @@ bool valid_dims(const GemmDesc& d) {
 bool gemm_fuses_rowsum(const GemmDesc& d) {
     if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
     const GemmPlan plan = plan_gemm(d);
-    return !plan.skinny && !plan.wavesplit_edge && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge && plan.split == 1;
+    return !plan.skinny && !plan.wavesplit_edge && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge &&
+           plan.tile != kTileFlat && plan.split == 1;
 }
 
 // What launch_gemm would do with this product, as text: the kernel family and, for the tiled kernel, tile,
@@ -192,9 +196,12 @@ std::string describe_gemm(const GemmDesc& d) {
     }
     const GemmParams p = make_params(dt, a_kc, b_kc);
     const int edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
-    const char* tile = plan.tile == kTileLarge ? "large" : plan.tile == kTileMedium ? "medium" : "small";
+    const char* tile = plan.tile == kTileLarge ? "large" : plan.tile == kTileMedium ? "medium" :
+                       plan.tile == kTileFlat ? "flat" : "small";
     const char* variant = "general";
-    if (plan.tile != kTileSmall) {
+    if (plan.tile == kTileFlat) {
+        if (fits_without_edges(p, a_kc, b_kc, 32, 128, 32) && fits_buffer_offsets(p, a_kc, b_kc, 32, 128)) variant = "whole";
+    } else if (plan.tile != kTileSmall) {
         const int bk = plan.tile == kTileLarge ? 16 : 32;
         if (fits_without_edges(p, a_kc, b_kc, edge, edge, bk) && fits_buffer_offsets(p, a_kc, b_kc, edge, edge))
             variant = "whole pipelined";

@@ -136,7 +136,7 @@ bool heads_pv_applies(const GemmDesc& d);
 int launch_heads_pv(const GemmDesc& d, hipStream_t stream);
 
 // per-layout entry points (one translation unit each, to compile in parallel)
-enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2 };
+enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2, kTileFlat = 3 };   // flat: 32 rows x 128 columns
 int launch_gemm_kc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
 int launch_gemm_kc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
 int launch_gemm_mc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);

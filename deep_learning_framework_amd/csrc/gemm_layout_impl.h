@@ -5,6 +5,7 @@
 //   large  256x256 tile, 8 waves of 128x64 (2 waves per SIMD)  -- big, compute-bound products
 //   medium 128x128 tile, 4 waves of 64x64, 2 workgroups per CU -- fills the chip at mid sizes
 //   small   64x64  tile, 4 waves of 32x32                      -- small or very ragged products
+//   flat    32x128 tile, 4 waves of 32x32 side by side         -- at most 32 rows against many columns
 // On the two bigger tiles, operands that allow 128-bit loads run the pipelined kernel: predicate-free
 // when the shape is a whole multiple of the tile, else with range-checked buffer resources and one
 // masked K-tile at the end.  Everything else runs the general kernel with the simple schedule.
@@ -41,6 +42,12 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
         if (fits_ragged_pipe(p, A_KC, B_KC, 128, 128))
             return launch_gemm_config<2, 2, 2, 2, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<2, 2, 2, 2, 16, A_KC, B_KC, true>(p, nbatch, kGroupM, stream);
+    case kTileFlat:
+        // at most 32 rows against many columns (a batch of 17..32 rows against a weight matrix): four waves side
+        // by side, so that the matrix cores do not spend half their time on rows that do not exist
+        if (fits_without_edges(p, A_KC, B_KC, 32, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 32, 128))
+            return launch_gemm_config<1, 4, 1, 1, 32, A_KC, B_KC, false, 0, 2, 4>(p, nbatch, kGroupM, stream);
+        return launch_gemm_config<1, 4, 1, 1, 32, A_KC, B_KC, true, 0, 1, 4>(p, nbatch, kGroupM, stream);
     default:
         // a 64x64x16 tile computes for ~0.25 us, a global load takes ~1-2 us: 128 reduction steps in flight
         // (measured with whole tiles of 32 steps against 16 and 64: 15.5 / 16.9 / 16.0 us for 256x1024x1024)

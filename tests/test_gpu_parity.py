@@ -223,6 +223,8 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 9), (64, 64, 64), (65, 63, 66), (100, 3
           (1024, 2048, 256), (1000, 2000, 130),
           # 256-wide tiles with edges in every dimension
           (1500, 3000, 100),
+          # at most 32 rows against many columns, too long for the one-launch kernel: the 32 x 128 tile, whole and ragged
+          (32, 2048, 2304), (20, 1030, 2100),
           # short reductions: the tiled kernel below 4M outputs, the panel-resident kernel (K-contiguous form)
           # above: odd K, ragged rows and columns
           (200, 130, 61), (513, 700, 64), (64, 1000, 8), (2050, 2100, 61), (2048, 2048, 64), (4100, 1030, 24)]
