@@ -156,6 +156,7 @@ GEMM_PLANS = [
     ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
     ((0, 1, 17, 11008, 4096), "mfma flat general split 8"),
     ((0, 1, 48, 4096, 4096), "mfma small general split 8"),
+    ((0, 1, 96, 4096, 4096), "mfma flat whole split 8"),             # 65..96 rows: three row tiles of 32, not two of 64
     ((0, 1, 64, 64, 8192), "mfma small whole split 16"),             # one tile, a long reduction
     ((0, 1, 768, 768, 4096), "mfma small whole split 8"),            # K cut to fill the rounds
     ((0, 1, 1024, 1024, 8192), "mfma small whole split 2"),          # K cut to bring a second workgroup onto each unit
