@@ -170,7 +170,7 @@ bool valid_dims(const GemmDesc& d) {
 bool gemm_fuses_rowsum(const GemmDesc& d) {
     if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
     const GemmPlan plan = plan_gemm(d);
-    return !plan.skinny && !plan.wavesplit_edge && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge &&
+    return !plan.skinny && !plan.wavesplit_edge && !skinny_rows_applies(plan.dn) && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge &&
            plan.tile != kTileFlat && plan.split == 1;
 }
 
@@ -181,6 +181,7 @@ std::string describe_gemm(const GemmDesc& d) {
     if (d.M == 0 || d.N == 0 || d.nbatch == 0) return "nothing";
     const GemmPlan plan = plan_gemm(d);
     if (plan.wavesplit_edge) return "wavesplit " + std::to_string(plan.wavesplit_edge);
+    if (skinny_rows_applies(plan.dn)) return "skinny rows";
     if (plan.skinny) return "skinny";
     if (shortk_nt_applies(plan.dn)) return "shortk_nt";
     if (shortk_heads_applies(plan.dn)) return "shortk_heads";
@@ -227,6 +228,7 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
         return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: this product cannot carry the fused row sum");
 
     if (plan.wavesplit_edge) return launch_gemm_wavesplit(plan.dn, plan.wavesplit_edge, stream);
+    if (skinny_rows_applies(plan.dn)) return launch_skinny_rows(plan.dn, stream);
     if (plan.skinny) {
         SkinnyParams s{};
         s.W = d.B; s.X = d.A; s.Y = d.C; s.Y2 = d.C2; s.bias = d.bias; s.leaky = d.leaky;

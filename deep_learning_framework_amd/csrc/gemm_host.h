@@ -131,6 +131,10 @@ int launch_gemm_shortk_heads(GemmParams p, int64_t nbatch, hipStream_t stream);
 bool wavesplit_applies(const GemmDesc& d);
 int launch_gemm_wavesplit(const GemmDesc& d, int block_edge, hipStream_t stream);
 
+// at most 16 rows against a matrix stored [K, N] (skinny_rows.hip; uses the library's scratch memory)
+bool skinny_rows_applies(const GemmDesc& d);
+int launch_skinny_rows(const GemmDesc& d, hipStream_t stream);
+
 // products of the head-interleaved attention tensor with several heads per batch entry: heads_pv.hip
 bool heads_pv_applies(const GemmDesc& d);
 int launch_heads_pv(const GemmDesc& d, hipStream_t stream);

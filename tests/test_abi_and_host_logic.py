@@ -150,6 +150,9 @@ GEMM_PLANS = [
     ((0, 1, 1, 4096, 4096), "skinny"),                               # configuration 5
     ((0, 1, 4, 4096, 4096), "skinny"),
     ((0, 1, 16, 4096, 4096), "skinny"),
+    ((0, 0, 4, 4096, 4096), "skinny rows"),                          # backward_x at a small batch: b stored [K, N]
+    ((0, 0, 16, 11008, 4096), "skinny rows"),
+    ((0, 0, 17, 4096, 4096), "mfma flat general split 8"),
     ((0, 1, 16, 1024, 1024), "wavesplit 16"),                        # 5..16 rows against a small weight matrix
     ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
     ((0, 1, 1000, 333, 777), "wavesplit 32"),                        # configuration 5, ragged: unaligned rows are fine

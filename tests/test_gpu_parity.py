@@ -304,6 +304,29 @@ def test_skinny_shapes_bias_act_acc(m, k, n):
     check(ya.to_numpy((m, n)), ko.matmul(w, x, acc_into=y0), what="skinny acc")
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 4096), (4, 2500, 4100), (5, 2100, 1500), (9, 9000, 1024), (16, 3000, 1028),
+                                   (13, 4096, 2048), (2, 8200, 1100)])
+def test_skinny_products_against_a_row_major_k_by_n_matrix(m, k, n):
+    # at most 16 rows against b[K, N]: matmul_backward_x at small batches (reduction over yvec = k here) and the
+    # forward product in the transposed weight layout; K beyond one LDS chunk per part, ragged column slices
+    rng = np.random.default_rng(m * 31 + k + n)
+    gy = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.uniform(-0.05, 0.05, (k, n)).astype(np.float32)        # the engine's w[yvec, xvec]
+    gx0 = rng.standard_normal((m, n)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    dgy, dw = dev(gy), dev(w)
+    gx = DB(m * n * 4)
+    VMath.matmul_backward_x(0, gx, dgy, dw, k, m, n, False)
+    check(gx.to_numpy((m, n)), ko.matmul_backward_x(gy, w), what="backward_x")
+    gxa = dev(gx0)
+    VMath.matmul_backward_x(0, gxa, dgy, dw, k, m, n, True)
+    check(gxa.to_numpy((m, n)), ko.matmul_backward_x(gy, w, acc_into=gx0), what="backward_x acc")
+    y = dev(gx0)
+    VMath.gemm_f32(0, 0, 0, m, n, k, dgy, k, dw, n, y, n, dev(b), kai.ACT["leaky"], kai.hyper(0.1), True)
+    ref = ko.activate(ko.add_bias(ko.matmul_backward_x(gy, w, acc_into=gx0), b), "leaky", 0.1)
+    check(y.to_numpy((m, n)), ref, what="[K,N] layout, acc + bias + leaky")
+
+
 def test_empty_and_degenerate_sizes():
     d = dev(np.ones(16, np.float32))
     out = dev(np.full(16, 7.0, np.float32))
