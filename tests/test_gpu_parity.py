@@ -325,6 +325,18 @@ def test_skinny_products_against_a_row_major_k_by_n_matrix(m, k, n):
     VMath.gemm_f32(0, 0, 0, m, n, k, dgy, k, dw, n, y, n, dev(b), kai.ACT["leaky"], kai.hyper(0.1), True)
     ref = ko.activate(ko.add_bias(ko.matmul_backward_x(gy, w, acc_into=gx0), b), "leaky", 0.1)
     check(y.to_numpy((m, n)), ref, what="[K,N] layout, acc + bias + leaky")
+    # leading dimensions beyond the row lengths and operands that start 4 bytes past a 16-byte boundary
+    lda, ldb, ldc = k + 3, n + 5, n + 2
+    ap = np.full((m, lda), np.nan, np.float32); ap[:, :k] = gy
+    bp = np.full((k, ldb), np.nan, np.float32); bp[:, :n] = w
+    cp0 = rng.standard_normal((m, ldc)).astype(np.float32)
+    ba = dev(np.concatenate([np.zeros(1, np.float32), ap.ravel()]))
+    bb = dev(np.concatenate([np.zeros(1, np.float32), bp.ravel()]))
+    bc = dev(np.concatenate([np.zeros(1, np.float32), cp0.ravel()]))
+    VMath.gemm_f32(0, 0, 0, m, n, k, ba.offset(4), lda, bb.offset(4), ldb, bc.offset(4), ldc, None, 0, None, False)
+    got = bc.to_numpy((1 + m * ldc,))[1:].reshape(m, ldc)
+    check(got[:, :n], ko.matmul_backward_x(gy, w), what="[K,N] layout, padded rows, unaligned operands")
+    assert np.array_equal(got[:, n:], cp0[:, n:]), "wrote between the rows of C"
 
 
 def test_empty_and_degenerate_sizes():
