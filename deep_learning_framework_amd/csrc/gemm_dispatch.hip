@@ -138,7 +138,13 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         const int64_t edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
         const int64_t tiles = plan.tile == kTileFlat ? ((d.M + 31) / 32) * ((d.N + 127) / 128) : tiles_of(d.M, d.N, 1, edge);
         int64_t split = compute_units() / tiles;
-        if ((plan.tile == kTileSmall || plan.tile == kTileFlat) && d.K >= 1024) split = small_tile_split(tiles, d.K, cus);
+        // one row of 32 x 128 tiles is bound by the stream of the other operand from HBM: one workgroup per compute
+        // unit, as split = units / tiles says, measured best or within 8 % of it at 4096 ... 16384 columns and steps
+        // (32 x 8192 x 8192: 94 us with the model's 8 parts, 68 with 4); the model below is for the products that
+        // the matrix cores bound
+        const bool one_flat_row = plan.tile == kTileFlat && d.M <= 32;
+        if ((plan.tile == kTileSmall || plan.tile == kTileFlat) && d.K >= 1024 && !one_flat_row)
+            split = small_tile_split(tiles, d.K, cus);
         while (split > 1 && split * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) split /= 2;
         if (split > d.K / kSplitMinK) split = d.K / kSplitMinK;
         if (split > kSplitMax) split = kSplitMax;

@@ -157,7 +157,8 @@ GEMM_PLANS = [
     ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
     ((0, 1, 1000, 333, 777), "wavesplit 32"),                        # configuration 5, ragged: unaligned rows are fine
     ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
-    ((0, 1, 17, 11008, 4096), "mfma flat general split 8"),
+    ((0, 1, 17, 11008, 4096), "mfma flat general split 2"),          # one workgroup per compute unit: 86 tiles x 2
+    ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small general split 8"),
     ((0, 1, 96, 4096, 4096), "mfma flat whole split 8"),             # 65..96 rows: three row tiles of 32, not two of 64
     ((0, 1, 64, 64, 8192), "mfma small whole split 16"),             # one tile, a long reduction
