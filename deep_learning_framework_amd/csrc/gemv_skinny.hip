@@ -86,8 +86,17 @@ gemv_rows_kernel(const SkinnyParams p) {
     if (p.K == 256 * CH) {
         full_chunk(0);   // the common inference width gets loop-free code
     } else {
-        int kc = 0;
-        for (; kc + 256 * CH <= p.K; kc += 256 * CH) full_chunk(kc);
+        // whole chunks, each wave starting at a chunk of its own and wrapping round: with rows a large power of
+        // two apart, waves that all walk their rows from k = 0 keep meeting in the same HBM channels
+        // (8192 x 8192: 50 -> 46 us, 4096 x 16384: 48 -> 44)
+        const int nfull = p.K / (256 * CH);
+        const int first = nfull > 1 ? (int)((blockIdx.x * (kSkinnyThreads / 64) + wave) % nfull) : 0;
+        for (int i = 0; i < nfull; i++) {
+            int c = first + i;
+            if (c >= nfull) c -= nfull;
+            full_chunk(c * 256 * CH);
+        }
+        const int kc = nfull * 256 * CH;
         if (kc < p.K) {
             // last, partial chunk: K % 4 == 0, so a float4 is entirely inside or outside
             const int kbase = kc + 4 * lane;
