@@ -40,15 +40,23 @@ __device__ __forceinline__ float wave_sum(float v) {
 // ---- batch 1: the weight matrix streamed once, x in registers ------------------------------------
 //
 // One wave owns R whole rows of W.  K is walked in chunks of 4096: a lane issues the 16 128-bit
-// loads of each of its rows for the chunk back to back (R*16 KiB in flight per wave), then loads
-// its 16 float4 of x (they hit in L2), then multiplies.  W is read with the non-temporal hint: it
-// is used once and should not displace x from the caches.  No LDS, no barrier.
+// loads of each of its rows for the chunk (R*16 KiB in flight per wave) and its 16 float4 of x (they
+// hit in L2), then multiplies as the loads arrive.  W is read with the non-temporal hint: it is used
+// once and should not displace x from the caches.  No LDS, no barrier.  K == 4096 is a kernel of its
+// own (K4096), so that the common inference width is straight-line code from the entry point.
 
 // amdgpu_waves_per_eu(1, 2): two waves per SIMD are all the grid ever gives a CU, so the register
 // allocator is told not to trade loads in flight for an occupancy it cannot use.
-template <int R>
+template <int R, bool K4096>
 __global__ void __launch_bounds__(kSkinnyThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
-gemv_rows_kernel(const SkinnyParams p) {
+gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t N,
+                 const int K, const int act_acc, float* __restrict__ Y, const float* __restrict__ bias,
+                 float* __restrict__ Y2, const float* __restrict__ leaky_ptr) {
+    // The arguments are scalars in the order of their first use, not a struct: this file is compiled with
+    // kernel-argument preload, so the first 14 dwords (W .. bias) are in SGPRs when a wave starts and the
+    // first loads of W go out without a round trip to the argument buffer.
+    const struct { const float *W, *X; int64_t ldw, N; int K, act, accflag; float *Y, *Y2; const float *bias, *leaky; }
+        p = {W, X, ldw, N, K, act_acc & 0xff, act_acc >> 8, Y, Y2, bias, leaky_ptr};
     constexpr int CH = 16;   // float4 per lane per chunk of 4096 k
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -63,19 +71,26 @@ gemv_rows_kernel(const SkinnyParams p) {
 #pragma unroll
     for (int r = 0; r < R; r++) acc[r] = 0.f;
 
-    // one whole chunk of 4096 k: all loads of W, then x, then the multiplies (straight-line code;
-    // the compiler overlaps the second row's loads with the first row's arithmetic)
+    // One whole chunk of 4096 k.  The order of issue is pinned, because it decides the run time at 4096 x 4096
+    // (us per call, cold): the loads of row 0 paired with those of x, then row 1, every load of the chunk out
+    // before the first wait, the multiplies following the arrivals 10.9 - 11.0; the rows' loads first and x last
+    // (the compiler then holds back the last 12 loads until the first ones return) 11.25; rows then x with all
+    // loads out first 11.50; x first 12.0; the two rows interleaved 11.7; all loads and one wait 12.2.
     auto full_chunk = [&](int kc) {
         const int kbase = kc + 4 * lane;
         f32x4 w[R][CH];
+        f32x4 x[CH];
 #pragma unroll
-        for (int r = 0; r < R; r++)
+        for (int j = 0; j < CH; j++) {
+            w[0][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[0] + kbase + 256 * j));
+            x[j] = *reinterpret_cast<const f32x4*>(p.X + kbase + 256 * j);
+        }
+#pragma unroll
+        for (int r = 1; r < R; r++)
 #pragma unroll
             for (int j = 0; j < CH; j++)
                 w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + kbase + 256 * j));
-        f32x4 x[CH];
-#pragma unroll
-        for (int j = 0; j < CH; j++) x[j] = *reinterpret_cast<const f32x4*>(p.X + kbase + 256 * j);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < R; r++)
 #pragma unroll
@@ -83,8 +98,8 @@ gemv_rows_kernel(const SkinnyParams p) {
                 acc[r] += w[r][j][0] * x[j][0] + w[r][j][1] * x[j][1] + w[r][j][2] * x[j][2] + w[r][j][3] * x[j][3];
     };
 
-    if (p.K == 256 * CH) {
-        full_chunk(0);   // the common inference width gets loop-free code
+    if constexpr (K4096) {
+        full_chunk(0);
     } else {
         // whole chunks, each wave starting at a chunk of its own and wrapping round: with rows a large power of
         // two apart, waves that all walk their rows from k = 0 keep meeting in the same HBM channels
@@ -134,7 +149,13 @@ static int launch_gemv_rows(const SkinnyParams& p, hipStream_t stream) {
     const int64_t rows_per_block = (kSkinnyThreads / 64) * R;
     const int64_t blocks = (p.N + rows_per_block - 1) / rows_per_block;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
-    gemv_rows_kernel<R><<<dim3((unsigned)blocks), dim3(kSkinnyThreads), 0, stream>>>(p);
+    const int act_acc = (p.act & 0xff) | (p.accflag ? 0x100 : 0);
+    if (p.K == 4096)
+        gemv_rows_kernel<R, true><<<dim3((unsigned)blocks), dim3(kSkinnyThreads), 0, stream>>>(
+            p.W, p.X, p.ldw, p.N, p.K, act_acc, p.Y, p.bias, p.Y2, p.leaky);
+    else
+        gemv_rows_kernel<R, false><<<dim3((unsigned)blocks), dim3(kSkinnyThreads), 0, stream>>>(
+            p.W, p.X, p.ldw, p.N, p.K, act_acc, p.Y, p.bias, p.Y2, p.leaky);
     return check_launch("gemv_rows_kernel");
 }
 
