@@ -20,6 +20,27 @@ struct SkinnyParams {
     int act, accflag;
 };
 
+// The arguments only an epilogue reads.  Kernels that stream from HBM take what their first loads need as
+// leading scalar arguments (W, X, ldw, ldx, N, M, K, Y: 14 dwords), which kernel-argument preload puts into
+// SGPRs before a wave starts, and the rest as this struct.
+struct SkinnyTail {
+    float* Y2;
+    const float* bias;
+    const float* leaky;
+    int64_t ldy;
+    int act, accflag;
+};
+
+inline SkinnyTail skinny_tail(const SkinnyParams& p) { return SkinnyTail{p.Y2, p.bias, p.leaky, p.ldy, p.act, p.accflag}; }
+
+__device__ __forceinline__ SkinnyParams skinny_params(const float* W, const float* X, int64_t ldw, int64_t ldx, int64_t N,
+                                                      int M, int K, float* Y, const SkinnyTail& t) {
+    SkinnyParams p;
+    p.W = W; p.X = X; p.Y = Y; p.Y2 = t.Y2; p.bias = t.bias; p.leaky = t.leaky;
+    p.ldw = ldw; p.ldx = ldx; p.ldy = t.ldy; p.N = N; p.M = M; p.K = K; p.act = t.act; p.accflag = t.accflag;
+    return p;
+}
+
 int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream);
 
 // skinny_stream.hip: aligned operands, K split over workgroups (uses the library's scratch memory)

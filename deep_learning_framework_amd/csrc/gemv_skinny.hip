@@ -169,7 +169,10 @@ constexpr int kSliceK = 1024;
 constexpr int kSliceMaxWaves = 4;   // 256 threads: leaves each wave 256 registers
 
 template <int MT, int RB>
-__global__ void __launch_bounds__(64 * kSliceMaxWaves) skinny_slice_kernel(const SkinnyParams p, int waves) {
+__global__ void __launch_bounds__(64 * kSliceMaxWaves) skinny_slice_kernel(
+        const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
+        const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail tail, int waves) {
+    const SkinnyParams p = skinny_params(W, X, ldw, ldx, N, M, K, Y, tail);
     __shared__ float part[MT * RB][kSliceMaxWaves];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -271,7 +274,10 @@ constexpr int kSliceLdsK = 4096;
 constexpr int kSliceLdsGroups = 4;
 
 template <int MT>
-__global__ void __launch_bounds__(64 * kSliceMaxWaves * kSliceLdsGroups) skinny_slice_lds_kernel(const SkinnyParams p) {
+__global__ void __launch_bounds__(64 * kSliceMaxWaves * kSliceLdsGroups) skinny_slice_lds_kernel(
+        const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
+        const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail tail) {
+    const SkinnyParams p = skinny_params(W, X, ldw, ldx, N, M, K, Y, tail);
     constexpr int RB = 4;
     __shared__ __attribute__((aligned(16))) float xs[MT * kSliceLdsK];
     __shared__ float part[kSliceLdsGroups][MT * RB][kSliceMaxWaves];
@@ -371,7 +377,8 @@ static int launch_slice(const SkinnyParams& p, hipStream_t stream) {
         // every wave has a slice, and there are workgroups for a good part of the chip
         const int64_t blocks = (p.N + RB * kSliceLdsGroups - 1) / (RB * kSliceLdsGroups);
         if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
-        skinny_slice_lds_kernel<MT><<<dim3((unsigned)blocks), dim3(64 * kSliceMaxWaves * kSliceLdsGroups), 0, stream>>>(p);
+        skinny_slice_lds_kernel<MT><<<dim3((unsigned)blocks), dim3(64 * kSliceMaxWaves * kSliceLdsGroups), 0, stream>>>(
+            p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, skinny_tail(p));
         return check_launch("skinny_slice_lds_kernel");
     }
     int waves = (p.K + kSliceK - 1) / kSliceK;
@@ -379,7 +386,8 @@ static int launch_slice(const SkinnyParams& p, hipStream_t stream) {
     if (waves > kSliceMaxWaves) waves = kSliceMaxWaves;
     const int64_t blocks = (p.N + RB - 1) / RB;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
-    skinny_slice_kernel<MT, RB><<<dim3((unsigned)blocks), dim3(64 * waves), 0, stream>>>(p, waves);
+    skinny_slice_kernel<MT, RB><<<dim3((unsigned)blocks), dim3(64 * waves), 0, stream>>>(
+        p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, skinny_tail(p), waves);
     return check_launch("skinny_slice_kernel");
 }
 

@@ -41,7 +41,13 @@ struct SkinnyRowsParams {
 };
 
 template <int MT>
-__global__ void __launch_bounds__(kSrThreads) skinny_rows_kernel(const SkinnyRowsParams p) {
+__global__ void __launch_bounds__(kSrThreads)
+skinny_rows_kernel(const float* __restrict__ A, const float* __restrict__ B, const int64_t lda, const int64_t ldb,
+                   const int64_t N, const int M, const int K, const int k_part, const int slices,
+                   float* __restrict__ part) {
+    // scalars, what the loads need first: this file is compiled with kernel-argument preload, so the first 14
+    // dwords are in SGPRs when a wave starts and the stream begins without a fetch of the argument buffer
+    const SkinnyRowsParams p{A, B, part, lda, ldb, N, M, K, k_part, slices};
     __shared__ __attribute__((aligned(16))) float a_lds[MT * kSrMaxPart];
     __shared__ __attribute__((aligned(16))) float red[(kSrWaves / 2) * MT * kSrCols];
 
@@ -145,9 +151,9 @@ int launch_skinny_rows(const GemmDesc& d, hipStream_t stream) {
     p.lda = d.a_rs; p.ldb = d.b_ks; p.N = d.N; p.M = (int)d.M; p.K = (int)d.K;
     p.k_part = (int)k_part; p.slices = (int)slices;
     const dim3 grid((unsigned)(slices * splits)), block(kSrThreads);
-    if (d.M <= 4) skinny_rows_kernel<4><<<grid, block, 0, stream>>>(p);
-    else if (d.M <= 8) skinny_rows_kernel<8><<<grid, block, 0, stream>>>(p);
-    else skinny_rows_kernel<16><<<grid, block, 0, stream>>>(p);
+    if (d.M <= 4) skinny_rows_kernel<4><<<grid, block, 0, stream>>>(p.A, p.B, p.lda, p.ldb, p.N, p.M, p.K, p.k_part, p.slices, p.part);
+    else if (d.M <= 8) skinny_rows_kernel<8><<<grid, block, 0, stream>>>(p.A, p.B, p.lda, p.ldb, p.N, p.M, p.K, p.k_part, p.slices, p.part);
+    else skinny_rows_kernel<16><<<grid, block, 0, stream>>>(p.A, p.B, p.lda, p.ldb, p.N, p.M, p.K, p.k_part, p.slices, p.part);
     KAI_TRY(check_launch("skinny_rows_kernel"));
     SplitReduceParams r{};
     r.part = part; r.C = d.C; r.C2 = d.C2; r.bias = d.bias; r.alpha = d.alpha; r.leaky = d.leaky;

@@ -53,23 +53,12 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
     return o;
 }
 
-// the arguments only the epilogue reads
-struct SkinnyTail {
-    float* Y2;
-    const float* bias;
-    const float* leaky;
-    int64_t ldy;
-    int act, accflag;
-};
-
 // What the first loads need comes as scalars (14 dwords): this file is compiled with kernel-argument preload, so
 // a wave finds them in SGPRs at its start instead of fetching the argument buffer first.
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
-    SkinnyParams p;
-    p.W = W; p.X = X; p.Y = Y; p.Y2 = t.Y2; p.bias = t.bias; p.leaky = t.leaky;
-    p.ldw = ldw; p.ldx = ldx; p.ldy = t.ldy; p.N = N; p.M = M; p.K = K; p.act = t.act; p.accflag = t.accflag;
+    const SkinnyParams p = skinny_params(W, X, ldw, ldx, N, M, K, Y, t);
     __shared__ __attribute__((aligned(16))) float lds_w[kSsWaves][16 * kSsTileStride];
     __shared__ __attribute__((aligned(16))) float lds_x[kSsWaves][16 * kSsTileStride];
 
@@ -186,7 +175,7 @@ bool skinny_stream_applies(const SkinnyParams& p) {
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     const int64_t blocks = (p.N + 15) / 16;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
-    const SkinnyTail t{p.Y2, p.bias, p.leaky, p.ldy, p.act, p.accflag};
+    const SkinnyTail t = skinny_tail(p);
     skinny_stream_kernel<<<dim3((unsigned)blocks), dim3(kSsThreads), 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M,
                                                                                   p.K, p.Y, t);
     return check_launch("skinny_stream_kernel");
