@@ -285,6 +285,8 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
 @pytest.mark.parametrize("m,k,n", [(1, 4096, 4096), (2, 1000, 300), (7, 130, 1024), (16, 4100, 257), (16, 3, 5),
                                    (5, 8192, 256), (9, 68, 300), (13, 1028, 1000), (3, 4096, 1024), (4, 260, 256),
                                    (1, 5000, 300), (2, 4100, 513), (1, 12292, 300), (1, 8192, 1030),
+                                   # batch 1 at K = 4096 (the straight-line kernel) with rows that do not fill the last wave
+                                   (1, 4096, 1027), (1, 4096, 257),
                                    # 2..4 rows with X shared through LDS: K in (3072, 4096], N >= 1024
                                    (3, 3080, 1030), (2, 4096, 1024), (4, 3588, 2050)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
