@@ -33,11 +33,14 @@ int launch_transpose(float* y, const float* x, const int* pn, int64_t axis_size,
                      hipStream_t stream);
 int launch_transpose_bin(float* y, const float* x, int64_t nrow, int64_t ncol, hipStream_t stream);
 
-// VMath::add, lstm_process, gru_process, gru_process_backward (vmath.cu:774-800, 4807-4857, 4946-5080 of the
-// reference): the element-wise steps between the gate products of a recurrent layer
+// VMath::add, lstm_process, lstm_process_backward, gru_process, gru_process_backward (vmath.cu:774-800,
+// 4807-4857, 4899-4943, 4946-5080 of the reference): the element-wise steps between the gate products of a
+// recurrent layer
 int launch_add(float* y, const float* a, const float* b, int64_t n, hipStream_t stream);
 int launch_lstm_process(float* r, float* s, const float* s1, const float* a, int64_t ndat, int64_t nrec,
                         hipStream_t stream);
+int launch_lstm_process_backward(const float* gr, float* gs, float* ga, const float* s_prev, const float* a,
+                                 int64_t ndat, int64_t nrec, hipStream_t stream);
 int launch_gru_process(float* r, const float* ai, const float* ar, int64_t nt, int64_t ndat, int64_t nrec,
                        hipStream_t stream);
 int launch_gru_process_backward(float* gr, float* gai, float* gar, const float* r, const float* ai, const float* ar,

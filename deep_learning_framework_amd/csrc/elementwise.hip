@@ -468,6 +468,47 @@ int launch_lstm_process(float* r, float* s, const float* s1, const float* a, int
     return check_launch("lstm_process_kernel");
 }
 
+// VMath::lstm_process_backward after the reference's device kernel (vmath.cu:4899-4937): one thread per
+// (row, unit) recomputes the four gates from this step's gate sums, writes the four gate-sum gradients
+// nrec apart in ga[ndat, 4*nrec] and replaces gs (gradient of this step's state) by the gradient of the
+// state the step started from.  gr is only read.
+__global__ void __launch_bounds__(kEwThreads)
+    lstm_process_backward_kernel(const float* __restrict__ gr, float* gs, float* __restrict__ ga, const float* s_prev,
+                                 const float* __restrict__ a, int64_t n, int64_t nrec) {
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
+        const int64_t nd = i / nrec, nr = i - nd * nrec;
+        const int64_t apos = nd * 4 * nrec + nr;
+        const float old_state = s_prev ? s_prev[i] : 0.f;
+        const float input_gate = act_sigmoid(a[apos]);
+        const float forget_gate = act_sigmoid(a[apos + nrec]);
+        const float input_block = act_tanh(a[apos + 2 * nrec]);
+        const float output_gate = act_sigmoid(a[apos + 3 * nrec]);
+        const float new_state = old_state * forget_gate + input_block * input_gate;
+        const float g_new_recur = gr[i];
+        const float th = act_tanh(new_state);
+        const float g_output_gate = th * g_new_recur;
+        const float g_tanh_state = output_gate * g_new_recur;
+        const float g_new_state = (1.0f - th * th) * g_tanh_state + gs[i];
+        const float g_forget_gate = old_state * g_new_state;
+        const float g_input_block = input_gate * g_new_state;
+        const float g_input_gate = input_block * g_new_state;
+        ga[apos] = input_gate * (1.0f - input_gate) * g_input_gate;
+        ga[apos + nrec] = forget_gate * (1.0f - forget_gate) * g_forget_gate;
+        ga[apos + 2 * nrec] = (1.0f - input_block * input_block) * g_input_block;
+        ga[apos + 3 * nrec] = output_gate * (1.0f - output_gate) * g_output_gate;
+        gs[i] = forget_gate * g_new_state;
+    }
+}
+
+int launch_lstm_process_backward(const float* gr, float* gs, float* ga, const float* s_prev, const float* a,
+                                 int64_t ndat, int64_t nrec, hipStream_t stream) {
+    const int64_t n = ndat * nrec;
+    if (n <= 0) return KAI_OK;
+    lstm_process_backward_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(gr, gs, ga, s_prev, a, n, nrec);
+    return check_launch("lstm_process_backward_kernel");
+}
+
 struct GruGates {
     float Rt, Zt, Nt, Ht_1, par_n;
 };

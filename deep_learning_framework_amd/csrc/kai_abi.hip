@@ -621,6 +621,16 @@ int kai_lstm_process(int device, float* pr, float* ps, const float* ps1, const f
     return launch_lstm_process(pr, ps, ps1, pa, ndat, nrec, current_stream());
 }
 
+int kai_lstm_process_backward(int device, const float* pgr, float* pgs, float* pga, const float* ps, const float* pa,
+                              int64_t ndat, int64_t nrec, int64_t ninp) {
+    (void)ninp;
+    KAI_REQUIRE_DEVICE(device);
+    KAI_REQUIRE(ndat >= 0 && nrec >= 0, KAI_ERR_INVALID_ARGUMENT, "negative dimension");
+    if (ndat == 0 || nrec == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgr); KAI_REQUIRE_PTR(pgs); KAI_REQUIRE_PTR(pga); KAI_REQUIRE_PTR(pa);
+    return launch_lstm_process_backward(pgr, pgs, pga, ps, pa, ndat, nrec, current_stream());
+}
+
 int kai_gru_process(int device, float* pr, const float* pai, const float* par, int64_t nt, int64_t ntimes, int64_t ndat,
                     int64_t nrec) {
     KAI_REQUIRE_DEVICE(device);

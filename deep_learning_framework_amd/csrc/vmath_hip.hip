@@ -90,6 +90,10 @@ void VMath::add(int device, float* py, float* pa, float* pb, int64 ndat) { raise
 void VMath::lstm_process(int device, float* pr, float* ps, float* ps1, float* pa, int64 ndat, int64 nrec, int64 ninp) {
     raise_on(kai_lstm_process(device, pr, ps, ps1, pa, ndat, nrec, ninp));
 }
+void VMath::lstm_process_backward(int device, float* pgr, float* pgs, float* pga, float* ps, float* pa, int64 ndat,
+                                  int64 nrec, int64 ninp) {
+    raise_on(kai_lstm_process_backward(device, pgr, pgs, pga, ps, pa, ndat, nrec, ninp));
+}
 void VMath::gru_process(int device, float* pr, float* pai, float* par, int64 nt, int64 ntimes, int64 ndat, int64 nrec) {
     raise_on(kai_gru_process(device, pr, pai, par, nt, ntimes, ndat, nrec));
 }

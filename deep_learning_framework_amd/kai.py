@@ -67,6 +67,7 @@ SIGNATURES = {
     "kai_copy": [_INT, _F, _F, _I64],
     "kai_add": [_INT, _F, _F, _F, _I64],
     "kai_lstm_process": [_INT, _F, _F, _F, _F, _I64, _I64, _I64],
+    "kai_lstm_process_backward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64],
     "kai_gru_process": [_INT, _F, _F, _F, _I64, _I64, _I64, _I64],
     "kai_gru_process_backward": [_INT, _F, _F, _F, _F, _F, _F, _I64, _I64, _I64, _I64],
     "kai_lstm_step": [_INT, _F, _F, _F, _F, _F, _F, _F, _F, _I64, _I64],
@@ -339,6 +340,11 @@ class VMath:
     @staticmethod
     def lstm_process(device, pr, ps, ps1, pa, ndat, nrec, ninp):
         _ck(load().kai_lstm_process(device, _addr(pr), _addr(ps), _addr(ps1), _addr(pa), ndat, nrec, ninp))
+
+    @staticmethod
+    def lstm_process_backward(device, pgr, pgs, pga, ps, pa, ndat, nrec, ninp):
+        _ck(load().kai_lstm_process_backward(device, _addr(pgr), _addr(pgs), _addr(pga), _addr(ps), _addr(pa), ndat,
+                                             nrec, ninp))
 
     @staticmethod
     def gru_process(device, pr, pai, par, nt, ntimes, ndat, nrec):

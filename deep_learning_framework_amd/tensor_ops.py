@@ -175,13 +175,17 @@ class Tensor:
         VMath.mix_values(dev, mixed.ptr, probs.ptr, V.ptr, nbat, ntimes, nvec, nhead, npiece)
         VMath.matmul(dev, y.ptr, Ow.ptr, mixed.ptr, nvec, n, nvec, False)
         VMath.add_bias(dev, y.ptr, y.ptr, Ob.ptr, n, nvec)
-        y.saved = {"op": "mh_attention", "key": key, "query": query, "value": value, "Kw": Kw, "Qw": Qw, "Vw": Vw,
+        y.saved = {"op": "mh_attention", "x": x, "key": key, "query": query, "value": value, "Kw": Kw, "Qw": Qw, "Vw": Vw,
                    "Ow": Ow, "K": K, "Q": Q, "V": V, "probs": probs, "mixed": mixed, "head_cnt": nhead,
                    "mask": mask, "coef": hcoef}
         return y
 
-    # vtensor.cpp:3054-3166 (the math calls; gradient registration is the engine's business)
+    # vtensor.cpp:3054-3195 (the math calls; gradient registration is the engine's business)
     def mh_attention_backprop(self, ygrad):
+        """Returns the 16 gradients by name.  ``g["x"]`` is the gradient of the tensor the operator was called on:
+        zero, plus the gradient of each of key / query / value that IS that tensor (self-attention,
+        vtensor.cpp:3168-3195).  The reference's set_zero there passes an element count where bytes are meant
+        and clears a quarter of the buffer; the whole buffer is cleared here."""
         s = self.saved
         nbat, ntimes, nvec = self.shape
         nhead = s["head_cnt"]
@@ -191,7 +195,7 @@ class Tensor:
         T = lambda shape: Tensor(shape, dev)
         g = {name: T((nvec, nvec)) for name in ("Kw", "Qw", "Vw", "Ow")}
         g.update({name: T((nvec,)) for name in ("Kb", "Qb", "Vb", "Ob")})
-        g.update({name: T(self.shape) for name in ("key", "query", "value", "mixed", "K", "Q", "V")})
+        g.update({name: T(self.shape) for name in ("x", "key", "query", "value", "mixed", "K", "Q", "V")})
         g["probs"] = T((nbat, ntimes, ntimes, nhead))
         gy = ygrad.ptr
         VMath.add_bias_backward_b(dev, g["Ob"].ptr, gy, n, nvec, False)
@@ -215,6 +219,11 @@ class Tensor:
         VMath.matmul_backward_x(dev, g["key"].ptr, g["K"].ptr, s["Kw"].ptr, nvec, n, nvec, False)
         VMath.matmul_backward_x(dev, g["query"].ptr, g["Q"].ptr, s["Qw"].ptr, nvec, n, nvec, False)
         VMath.matmul_backward_x(dev, g["value"].ptr, g["V"].ptr, s["Vw"].ptr, nvec, n, nvec, False)
+        xsize = n * nvec
+        VMath.set_zero(dev, g["x"].ptr, xsize * 4)
+        for name in ("key", "query", "value"):
+            if s[name] is s["x"]:
+                VMath.add(dev, g["x"].ptr, g["x"].ptr, g[name].ptr, xsize)
         return g
 
 
@@ -340,14 +349,12 @@ def rnn(x, wi, wr, bi, br, cell_type, rec_size, actfunc="tanh", leaky_alpha=None
     return y, saved
 
 
-def rnn_backprop(saved, ygrad, ytgrad):
-    """vtensor.cpp:2524-2717 for the rnn and gru cells.  ``ygrad [ndat, nrec]`` is used in place as the running
-    gradient of the recurrent output, as there; ``ytgrad [ntimes, ndat, nrec]`` is the per-step gradient.
-    Returns {x, wi, wr[, bi, br]} gradients.  The lstm cell has no backward here: the reference's
-    lstm_process_backward indexes outside its gate-gradient buffer (vmath.cu:4890-4893)."""
+def rnn_backprop(saved, ygrad, ytgrad, use_state=False):
+    """vtensor.cpp:2524-2717.  ``ygrad [ndat, nrec]`` is used in place as the running gradient of the recurrent
+    output (of the cell state for an lstm with ``use_state``), as there; ``ytgrad [ntimes, ndat, nrec]`` is the
+    per-step gradient.  Returns {x, wi, wr[, bi, br]} gradients.  The lstm cell's gradient follows the
+    reference's device kernel (vmath.cu:4899-4937)."""
     cell_type = saved["cell_type"]
-    if cell_type == "lstm":
-        raise KaiError(VERR_UNDEFINED, "lstm backward is not built")
     forward, ngates = saved["forward"], saved["ngates"]
     x, wi, wr = saved["x"], saved["wi"], saved["wr"]
     recurs, iaffines, raffines = saved["recurs"], saved["iaffines"], saved["raffines"]
@@ -370,6 +377,18 @@ def rnn_backprop(saved, ygrad, ytgrad):
         VMath.set_zero(dev, out["bi"].ptr, ngates * nrec * 4)
         VMath.set_zero(dev, out["br"].ptr, ngates * nrec * 4)
     pgr = ygrad.ptr
+    pgs = None
+    states = saved["states"]
+    use_state = use_state and cell_type == "lstm"
+    if cell_type == "lstm":
+        # vtensor.cpp:2614-2631: with use_state the incoming gradient is that of the state and the output's
+        # gradient starts at zero, otherwise the other way round
+        fresh = Tensor(ygrad.shape, dev)
+        VMath.set_zero(dev, fresh.ptr, fresh.total_size() * 4)
+        if use_state:
+            pgs, pgr = ygrad.ptr, fresh.ptr
+        else:
+            pgs = fresh.ptr
     xsize, ysize = ndat * ninp, ndat * nrec
     asize = ngates * ysize
     f4 = 4
@@ -380,9 +399,13 @@ def rnn_backprop(saved, ygrad, ytgrad):
         par = raffines.buf.offset(nt * asize * f4)
         px = x.buf.offset(nt * xsize * f4) if in_seq else x.ptr
         pgx = xgrad.buf.offset(nt * xsize * f4) if in_seq else xgrad.ptr
-        VMath.add(dev, pgr, pgr, ytgrad.buf.offset(nt * ysize * f4), ysize)
+        pg_step = pgs if use_state else pgr
+        VMath.add(dev, pg_step, pg_step, ytgrad.buf.offset(nt * ysize * f4), ysize)
         if cell_type == "rnn":
             VMath.activate_backward_with_y(dev, aigrad.ptr, pgr, pr, ndat, nrec, saved["actfunc"], saved["leaky_alpha"])
+        elif cell_type == "lstm":
+            ps_prev = states.buf.offset((nt - 1 if forward else nt + 1) * ysize * f4) if n < ntimes - 1 else None
+            VMath.lstm_process_backward(dev, pgr, pgs, aigrad.ptr, ps_prev, pai, ndat, nrec, ninp)
         else:
             VMath.gru_process_backward(dev, pgr, aigrad.ptr, argrad.ptr, pr, pai, par, nt, ntimes, ndat, nrec)
         if saved["use_bias"]:

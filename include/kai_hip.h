@@ -222,13 +222,18 @@ int kai_add(int device, float* py, const float* pa, const float* pb, int64_t nda
  * block and output gates; ps = ps1 * f + g * i (ps1 null: 0), pr = tanh(ps) * o.  ninp is unused, as there. */
 int kai_lstm_process(int device, float* pr, float* ps, const float* ps1, const float* pa, int64_t ndat, int64_t nrec,
                      int64_t ninp);
+/* VMath::lstm_process_backward, vmath.cu:4899-4943 (the device kernel; the host loop, vmath.cu:4860-4897, has the
+ * same arithmetic but writes the gate gradients at apos * g + n * nrec, outside the buffer).  pa[ndat, 4*nrec]:
+ * this step's gate sums; ps: the state the step started from (null: 0); pgr: gradient of this step's output
+ * (read only); pgs: gradient of this step's state on entry, of the previous state on return;
+ * pga[ndat, 4*nrec] receives the gate-sum gradients.  ninp is unused, as there. */
+int kai_lstm_process_backward(int device, const float* pgr, float* pgs, float* pga, const float* ps, const float* pa,
+                              int64_t ndat, int64_t nrec, int64_t ninp);
 /* VMath::gru_process, vmath.cu:4946-4996.  pr points at step nt of [ntimes, ndat, nrec] and the previous step is
  * read ndat*nrec floats before it when nt > 0; pai/par[ndat, 3*nrec]: reset, update, candidate. */
 int kai_gru_process(int device, float* pr, const float* pai, const float* par, int64_t nt, int64_t ntimes, int64_t ndat,
                     int64_t nrec);
-/* VMath::gru_process_backward, vmath.cu:4999-5080.  pgr is replaced by the gradient of the previous step's output.
- * VMath::lstm_process_backward (vmath.cu:4860-4943) has no counterpart: its gate-gradient index expression
- * (apos * g + n * nrec) leaves the [ndat, 4*nrec] buffer for nrec > 4. */
+/* VMath::gru_process_backward, vmath.cu:4999-5080.  pgr is replaced by the gradient of the previous step's output. */
 int kai_gru_process_backward(int device, float* pgr, float* pgai, float* pgar, const float* pr, const float* pai,
                              const float* par, int64_t nt, int64_t ntimes, int64_t ndat, int64_t nrec);
 

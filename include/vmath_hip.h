@@ -82,6 +82,8 @@ public:
     static void copy(int device, float* py, float* pa, int64 ndat);
     static void add(int device, float* py, float* pa, float* pb, int64 ndat);
     static void lstm_process(int device, float* pr, float* ps, float* ps1, float* pa, int64 ndat, int64 nrec, int64 ninp);
+    static void lstm_process_backward(int device, float* pgr, float* pgs, float* pga, float* ps, float* pa, int64 ndat,
+                                      int64 nrec, int64 ninp);
     static void gru_process(int device, float* pr, float* pai, float* par, int64 nt, int64 ntimes, int64 ndat, int64 nrec);
     static void gru_process_backward(int device, float* pgr, float* pgai, float* pgar, float* pr, float* pai, float* par,
                                      int64 nt, int64 ntimes, int64 ndat, int64 nrec);

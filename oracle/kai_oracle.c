@@ -578,6 +578,43 @@ int ko_lstm_process(float* pr, float* ps, const float* ps1, const float* pa, int
     return KO_OK;
 }
 
+int ko_lstm_process_backward(const float* pgr, float* pgs, float* pga, const float* ps, const float* pa,
+                             int64_t ndat, int64_t nrec) {
+    /* vmath.cu:4899-4937, the DEVICE twin: gate gradients at pga[apos + g * nrec].  The host twin
+     * (vmath.cu:4860-4897) has the same arithmetic but writes them at pga[apos * g + n * nrec], which
+     * leaves the [ndat, 4*nrec] buffer; the library replaces the device branch, so that is the one
+     * restated.  ps is the state of the step processed BEFORE this one (null: 0), pa the gate sums of
+     * this step, pgr the gradient of this step's output (read only), pgs the gradient of this step's
+     * state on entry and of the previous state on return. */
+    for (int64_t nd = 0, n = 0; nd < ndat; nd++) {
+        for (int64_t nr = 0; nr < nrec; nr++, n++) {
+            int64_t apos = nd * 4 * nrec + nr;
+            float old_state = ps ? ps[n] : 0;
+            float input_gate = ko_sigmoid(pa[apos + 0 * nrec]);
+            float forget_gate = ko_sigmoid(pa[apos + 1 * nrec]);
+            float input_block = ko_tanh(pa[apos + 2 * nrec]);
+            float output_gate = ko_sigmoid(pa[apos + 3 * nrec]);
+            float new_state = old_state * forget_gate + input_block * input_gate;
+            float g_new_recur = pgr[n];
+            float g_output_gate = ko_tanh(new_state) * g_new_recur;
+            float g_tanh_state = output_gate * g_new_recur;
+            float th = ko_tanh(new_state);                       /* _tanh_derv_with_x, vmath.cu:336-339 */
+            float g_new_state = (1.0f - th * th) * g_tanh_state + pgs[n];
+            float g_forget_gate = old_state * g_new_state;
+            float g_old_state = forget_gate * g_new_state;
+            float g_input_block = input_gate * g_new_state;
+            float g_input_gate = input_block * g_new_state;
+            /* _sigmoid_derv_with_y: y * (1 - y); _tanh_derv_with_y: 1 - y * y (vmath.cu:327-347) */
+            pga[apos + 0 * nrec] = input_gate * (1.0f - input_gate) * g_input_gate;
+            pga[apos + 1 * nrec] = forget_gate * (1.0f - forget_gate) * g_forget_gate;
+            pga[apos + 2 * nrec] = (1.0f - input_block * input_block) * g_input_block;
+            pga[apos + 3 * nrec] = output_gate * (1.0f - output_gate) * g_output_gate;
+            pgs[n] = g_old_state;
+        }
+    }
+    return KO_OK;
+}
+
 int ko_gru_process(float* pr, const float* pai, const float* par, int64_t nt, int64_t ndat, int64_t nrec) {
     /* vmath.cu:4946-4965; pr points at time step nt of [ntimes, ndat, nrec], the previous step lies ndat*nrec
      * floats before it; gate order in pai/par[ndat, 3*nrec]: reset, update, candidate */

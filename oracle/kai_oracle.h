@@ -111,12 +111,15 @@ int ko_transpose_bin(float* py, const float* px, int64_t nrow, int64_t ncol);
 /* cosine similarity of every row of x1[nrow1, ncol] with every row of x2[nrow2, ncol] (vmath.cu:6459-6480) */
 int ko_cosinesim(float* py, const float* px1, const float* px2, int64_t nrow1, int64_t nrow2, int64_t ncol);
 
-/* recurrent cells (vmath.cu:732-736, 774-778, 4807-4826, 4946-4965, 4999-5033).  lstm_process_backward
- * (vmath.cu:4860-4897) is not restated: its gate-gradient index expression (apos * g + n * nrec) leaves
- * the [ndat, 4*nrec] buffer for nrec > 4. */
+/* recurrent cells (vmath.cu:732-736, 774-778, 4807-4826, 4899-4937, 4946-4965, 4999-5033).
+ * lstm_process_backward follows the reference's DEVICE kernel (vmath.cu:4899-4937, gate gradients at
+ * apos + g * nrec): the host loop (vmath.cu:4860-4897) has the same arithmetic but its index expression
+ * (apos * g + n * nrec) leaves the [ndat, 4*nrec] buffer. */
 int ko_copy(float* py, const float* pa, int64_t ndat);
 int ko_add(float* py, const float* pa, const float* pb, int64_t ndat);
 int ko_lstm_process(float* pr, float* ps, const float* ps1, const float* pa, int64_t ndat, int64_t nrec);
+int ko_lstm_process_backward(const float* pgr, float* pgs, float* pga, const float* ps, const float* pa,
+                             int64_t ndat, int64_t nrec);
 int ko_gru_process(float* pr, const float* pai, const float* par, int64_t nt, int64_t ndat, int64_t nrec);
 int ko_gru_process_backward(float* pgr, float* pgai, float* pgar, const float* pr, const float* pai,
                             const float* par, int64_t nt, int64_t ndat, int64_t nrec);

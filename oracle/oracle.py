@@ -63,6 +63,7 @@ def lib():
             "ko_copy": [_F, _F, _I64],
             "ko_add": [_F, _F, _F, _I64],
             "ko_lstm_process": [_F, _F, _F, _F, _I64, _I64],
+            "ko_lstm_process_backward": [_F, _F, _F, _F, _F, _I64, _I64],
             "ko_gru_process": [_F, _F, _F, _I64, _I64, _I64],
             "ko_gru_process_backward": [_F, _F, _F, _F, _F, _F, _I64, _I64, _I64],
             "ko_accumulate_grad": [_F, _F, _I64],
@@ -381,6 +382,18 @@ def lstm_process(affine, prev_state=None):
     ps1 = None if prev_state is None else _p(_f32(prev_state))
     _check(lib().ko_lstm_process(_p(r), _p(st), ps1, _p(affine), ndat, nrec))
     return r, st
+
+
+def lstm_process_backward(gr, gs, affine, prev_state=None):
+    """Gradient of one LSTM cell step, the reference's device kernel.  gr, gs [ndat, nrec]: gradients of this
+    step's output and state; affine [ndat, 4*nrec]: this step's gate sums; prev_state: the state the step
+    started from (None: 0).  Returns (gradient of the previous state, gate-sum gradients [ndat, 4*nrec])."""
+    gr, gs, affine = _f32(gr), _f32(gs).copy(), _f32(affine)
+    ndat, nrec = affine.shape[0], affine.shape[1] // 4
+    ga = np.zeros_like(affine)
+    ps = None if prev_state is None else _p(_f32(prev_state))
+    _check(lib().ko_lstm_process_backward(_p(gr), _p(gs), _p(ga), ps, _p(affine), ndat, nrec))
+    return gs, ga
 
 
 def gru_process(recurs, pai, par, nt):

@@ -113,6 +113,12 @@ def next_to_path():
     f["gru_recurs_out"] = ko.gru_process(recurs, ai, ar, 1).copy()
     f["gru_gprev"], f["gru_gai"], f["gru_gar"] = ko.gru_process_backward(gh, f["gru_recurs_out"], ai, ar, 1)
     f["add"] = ko.add(p, g)
+    # lstm cell gradient (drawn after everything above, so the earlier arrays keep their values)
+    lgr = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    lgs = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    f.update(lstm_gr=lgr, lstm_gs=lgs)
+    f["lstm_gprev_state"], f["lstm_gaffine"] = ko.lstm_process_backward(lgr, lgs, a4, st)
+    f["lstm_gprev_state_first"], f["lstm_gaffine_first"] = ko.lstm_process_backward(lgr, lgs, a4, None)
     out = os.path.join(HERE, "next_to_path_small.npz")
     np.savez_compressed(out, **f)
     print("wrote", out, os.path.getsize(out), "bytes,", len(f), "arrays")

@@ -131,6 +131,90 @@ def test_tensor_operator_argument_derivation(monkeypatch):
     assert calls[-1][0] == "matmul_backward_w" and wg.shape == (3, 8) and xg.shape == (6, 5, 8)
 
 
+def test_mh_attention_call_sequence(monkeypatch):
+    """VTensor::mh_attention issues 11 math calls (12 with the mask), its backprop 17 (18) plus the clearing and
+    summing of the operand's own gradient; names, order and the size arguments as in vtensor.cpp:3026-3043 and
+    3142-3195."""
+    from deep_learning_framework_amd import tensor_ops as T
+
+    calls = []
+    counter = [0]
+
+    class FakeBuf:
+        def __init__(self):
+            counter[0] += 1
+            self.ptr = 4096 * counter[0]          # a distinct address per tensor, so the pointers can be told apart
+
+    class Rec:
+        def __getattr__(self, name):
+            return lambda *a: calls.append((name,) + a)
+
+    monkeypatch.setattr(T, "VMath", Rec())
+    monkeypatch.setattr(T, "DeviceBuffer", lambda *a, **k: FakeBuf())
+    monkeypatch.setattr(T.kai, "hyper", lambda v, device=0: ("hyper", None if v is None else round(float(v), 6)))
+    nbat, ntimes, nvec, nhead = 2, 5, 12, 3
+    npiece, n = nvec // nhead, nbat * ntimes
+    mk = lambda *shape: T.Tensor(shape, buf=FakeBuf())
+    x, other = mk(nbat, ntimes, nvec), mk(nbat, ntimes, nvec)
+    Kw, Qw, Vw, Ow = (mk(nvec, nvec) for _ in range(4))
+    Kb, Qb, Vb, Ob = (mk(nvec) for _ in range(4))
+    for mask in (False, True):
+        del calls[:]
+        y = x.mh_attention(x, other, x, Kw, Kb, Qw, Qb, Vw, Vb, Ow, Ob, nhead, mask=mask)
+        sv = y.saved
+        K, Q, V, P, M = (sv[k].ptr for k in ("K", "Q", "V", "probs", "mixed"))
+        coef = ("hyper", round(1 / np.sqrt(npiece), 6))                  # vmodule.cpp:1805
+        want = [("matmul", 0, K, Kw.ptr, x.ptr, nvec, n, nvec, False),
+                ("matmul", 0, Q, Qw.ptr, other.ptr, nvec, n, nvec, False),
+                ("matmul", 0, V, Vw.ptr, x.ptr, nvec, n, nvec, False),
+                ("add_bias", 0, K, K, Kb.ptr, n, nvec),
+                ("add_bias", 0, Q, Q, Qb.ptr, n, nvec),
+                ("add_bias", 0, V, V, Vb.ptr, n, nvec),
+                ("mult_on_heads", 0, P, K, Q, nbat, ntimes, nvec, nhead, npiece, coef)]
+        if mask:
+            want.append(("set_mh_attention_mask", 0, P, nbat, ntimes, nhead, True))
+        want += [("softmax_direct_on_axis", 0, P, n, ntimes, nhead),
+                 ("mix_values", 0, M, P, V, nbat, ntimes, nvec, nhead, npiece),
+                 ("matmul", 0, y.ptr, Ow.ptr, M, nvec, n, nvec, False),
+                 ("add_bias", 0, y.ptr, y.ptr, Ob.ptr, n, nvec)]
+        assert calls == want
+        del calls[:]
+        gy = mk(nbat, ntimes, nvec)
+        g = y.mh_attention_backprop(gy)
+        p = {k: t.ptr for k, t in g.items()}
+        want = [("add_bias_backward_b", 0, p["Ob"], gy.ptr, n, nvec, False),
+                ("matmul_backward_w", 0, p["Ow"], gy.ptr, M, nvec, n, nvec, False),
+                ("matmul_backward_x", 0, p["mixed"], gy.ptr, Ow.ptr, nvec, n, nvec, False),
+                ("mix_values_backward_prop", 0, p["probs"], p["mixed"], V, nbat, ntimes, nvec, nhead, npiece),
+                ("mix_values_backward_value", 0, p["V"], p["mixed"], P, nbat, ntimes, nvec, nhead, npiece),
+                ("softmax_direct_on_axis_backward", 0, p["probs"], P, nbat, ntimes, nhead, coef)]
+        if mask:
+            want.append(("set_mh_attention_mask", 0, p["probs"], nbat, ntimes, nhead, False))
+        want += [("mult_on_heads_backward", 0, p["K"], p["probs"], Q, nbat, ntimes, nvec, nhead, npiece),
+                 ("mult_on_heads_backward", 0, p["Q"], p["probs"], K, nbat, ntimes, nvec, nhead, npiece),
+                 ("add_bias_backward_b", 0, p["Kb"], p["K"], n, nvec, False),
+                 ("add_bias_backward_b", 0, p["Qb"], p["Q"], n, nvec, False),
+                 ("add_bias_backward_b", 0, p["Vb"], p["V"], n, nvec, False),
+                 ("matmul_backward_w", 0, p["Kw"], p["K"], x.ptr, nvec, n, nvec, False),
+                 ("matmul_backward_w", 0, p["Qw"], p["Q"], other.ptr, nvec, n, nvec, False),
+                 ("matmul_backward_w", 0, p["Vw"], p["V"], x.ptr, nvec, n, nvec, False),
+                 ("matmul_backward_x", 0, p["key"], p["K"], Kw.ptr, nvec, n, nvec, False),
+                 ("matmul_backward_x", 0, p["query"], p["Q"], Qw.ptr, nvec, n, nvec, False),
+                 ("matmul_backward_x", 0, p["value"], p["V"], Vw.ptr, nvec, n, nvec, False),
+                 ("set_zero", 0, p["x"], n * nvec * 4),
+                 # key and value are the operand itself, query is another tensor
+                 ("add", 0, p["x"], p["x"], p["key"], n * nvec),
+                 ("add", 0, p["x"], p["x"], p["value"], n * nvec)]
+        assert calls == want
+    with pytest.raises(kai.KaiError) as e:
+        x.mh_attention(x, x, x, Kw, Kb, Qw, Qb, Vw, Vb, Ow, Ob, 5)            # 12 % 5 != 0
+    assert e.value.code == 10003
+    with pytest.raises(kai.KaiError):
+        x.mh_attention(x, mk(nbat, ntimes + 1, nvec), x, Kw, Kb, Qw, Qb, Vw, Vb, Ow, Ob, nhead)
+    with pytest.raises(kai.KaiError):
+        x.mh_attention(x, x, x, mk(nvec, nvec + 1), Kb, Qw, Qb, Vw, Vb, Ow, Ob, nhead)
+
+
 # ---- which kernel a product gets: the dispatcher's rules, from its host-only description ------------------
 
 GEMM_PLANS = [

@@ -132,6 +132,9 @@ def test_oracle_reproduces_the_second_fixture_bit_for_bit():
     assert np.array_equal(ko.transpose_bin(G2["trbin_x"], 13, 7), G2["trbin_y"])
     r, st = ko.lstm_process(G2["lstm_affine"], G2["lstm_prev_state"])
     assert np.array_equal(r, G2["lstm_recur"]) and np.array_equal(st, G2["lstm_state"])
+    for prev, tag in ((G2["lstm_prev_state"], ""), (None, "_first")):
+        gs, ga = ko.lstm_process_backward(G2["lstm_gr"], G2["lstm_gs"], G2["lstm_affine"], prev)
+        assert np.array_equal(gs, G2["lstm_gprev_state" + tag]) and np.array_equal(ga, G2["lstm_gaffine" + tag])
     assert np.array_equal(ko.gru_process(G2["gru_recurs_in"].copy(), G2["gru_ai"], G2["gru_ar"], 1), G2["gru_recurs_out"])
     for got, name in zip(ko.gru_process_backward(G2["gru_gh"], G2["gru_recurs_out"], G2["gru_ai"], G2["gru_ar"], 1),
                          ("gru_gprev", "gru_gai", "gru_gar")):
@@ -191,6 +194,12 @@ def test_hip_path_matches_the_second_fixture():
     assert rel_fro(st.to_numpy((ndat, nrec)), G2["lstm_state"]) <= REL_FRO_TOL
     VMath.lstm_process(0, r, st, None, dev(G2["lstm_affine"]), ndat, nrec, 0)
     assert rel_fro(r.to_numpy((ndat, nrec)), G2["lstm_recur_first"]) <= REL_FRO_TOL
+    for prev, tag in ((G2["lstm_prev_state"], ""), (None, "_first")):
+        gs, ga = dev(G2["lstm_gs"]), DB(G2["lstm_affine"].nbytes)
+        VMath.lstm_process_backward(0, dev(G2["lstm_gr"]), gs, ga, None if prev is None else dev(prev),
+                                    dev(G2["lstm_affine"]), ndat, nrec, 0)
+        assert rel_fro(gs.to_numpy((ndat, nrec)), G2["lstm_gprev_state" + tag]) <= REL_FRO_TOL
+        assert rel_fro(ga.to_numpy(G2["lstm_affine"].shape), G2["lstm_gaffine" + tag]) <= REL_FRO_TOL
     rec = dev(G2["gru_recurs_in"])
     ai, ar = dev(G2["gru_ai"]), dev(G2["gru_ar"])
     VMath.gru_process(0, rec.offset(ndat * nrec * 4), ai, ar, 1, 2, ndat, nrec)

@@ -506,6 +506,131 @@ def test_attention_ops_small(nbat, ntimes, nhead, npiece):
     check(gk.to_numpy((nbat, ntimes, nvec)), ko.mult_on_heads_backward(ref_gs, q, nhead), what="mult_on_heads_backward")
 
 
+# ---- the attention block caller: VTensor::mh_attention and its backprop (vtensor.cpp:2978-3052, 3054-3195) -------
+
+def _oracle_mh_attention(key, query, value, W, nhead, mask, coef):
+    """The 11 (12) math calls of vtensor.cpp:3026-3043 issued against the oracle."""
+    nbat, ntimes, nvec = key.shape
+    n = nbat * ntimes
+    flat = lambda a: a.reshape(n, nvec)
+    K = ko.add_bias(ko.matmul(W["Kw"], flat(key)), W["Kb"]).reshape(key.shape)
+    Q = ko.add_bias(ko.matmul(W["Qw"], flat(query)), W["Qb"]).reshape(key.shape)
+    V = ko.add_bias(ko.matmul(W["Vw"], flat(value)), W["Vb"]).reshape(key.shape)
+    s = ko.mult_on_heads(K, Q, nhead, coef)
+    if mask:
+        s = ko.set_mh_attention_mask(s, True)
+    probs = ko.softmax_direct_on_axis(s, n, ntimes, nhead)
+    mixed = ko.mix_values(probs, V, nhead)
+    y = ko.add_bias(ko.matmul(W["Ow"], flat(mixed)), W["Ob"]).reshape(key.shape)
+    return y, dict(K=K, Q=Q, V=V, probs=probs, mixed=mixed)
+
+
+def _oracle_mh_attention_backprop(gy, key, query, value, W, fw, nhead, mask, coef, same):
+    """The 17 (18) math calls of vtensor.cpp:3142-3166 and the operand's own gradient (3168-3195)."""
+    nbat, ntimes, nvec = key.shape
+    n = nbat * ntimes
+    flat = lambda a: a.reshape(n, nvec)
+    g = {}
+    g["Ob"] = ko.add_bias_backward_b(flat(gy), nvec)
+    g["Ow"] = ko.matmul_backward_w(flat(gy), flat(fw["mixed"]), nvec, nvec)
+    g["mixed"] = ko.matmul_backward_x(flat(gy), W["Ow"]).reshape(key.shape)
+    gp = ko.mix_values_backward_prop(g["mixed"], fw["V"], nhead)
+    g["V"] = ko.mix_values_backward_value(g["mixed"], fw["probs"], nhead)
+    gp = ko.softmax_direct_on_axis_backward(gp, fw["probs"], coef)
+    if mask:
+        gp = ko.set_mh_attention_mask(gp, False)
+    g["probs"] = gp
+    g["K"] = ko.mult_on_heads_backward(gp, fw["Q"], nhead)
+    g["Q"] = ko.mult_on_heads_backward(gp, fw["K"], nhead)
+    for name, src in (("K", key), ("Q", query), ("V", value)):
+        g[name + "b"] = ko.add_bias_backward_b(flat(g[name]), nvec)
+        g[name + "w"] = ko.matmul_backward_w(flat(g[name]), flat(src), nvec, nvec)
+    g["key"] = ko.matmul_backward_x(flat(g["K"]), W["Kw"]).reshape(key.shape)
+    g["query"] = ko.matmul_backward_x(flat(g["Q"]), W["Qw"]).reshape(key.shape)
+    g["value"] = ko.matmul_backward_x(flat(g["V"]), W["Vw"]).reshape(key.shape)
+    gx = np.zeros_like(key)
+    for name in ("key", "query", "value"):
+        if name in same:
+            gx = ko.add(gx, g[name])
+    g["x"] = gx
+    return g
+
+
+@pytest.mark.parametrize("nbat,ntimes,nvec,nhead,mask,same", [
+    (2, 40, 32, 4, False, ("key", "query", "value")),     # self-attention: all three gradients meet in x
+    (2, 40, 32, 4, True, ("key",)),                      # masked; query and value come from other tensors
+    (1, 130, 64, 1, True, ("key", "query", "value")),    # one head, ragged length
+    (3, 64, 96, 8, False, ()),                           # head size 12: the per-head tiled kernels
+    (2, 128, 256, 4, True, ("query", "value")),          # head size 64, four heads per workgroup kernels
+    (1, 33, 20, 5, False, ("value",)),                   # unaligned rows everywhere
+])
+def test_mh_attention_block_and_backprop(nbat, ntimes, nvec, nhead, mask, same):
+    from deep_learning_framework_amd import tensor_ops as T
+    rng = np.random.default_rng(nbat * 1000 + ntimes * 10 + nvec + nhead)
+    tn = T.Tensor.from_numpy
+    act = lambda: rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    x = act()
+    inputs = {name: (x if name in same else act()) for name in ("key", "query", "value")}
+    W = {}
+    for name in ("Kw", "Qw", "Vw", "Ow"):
+        W[name] = (rng.standard_normal((nvec, nvec)) / np.sqrt(nvec)).astype(np.float32)
+    for name in ("Kb", "Qb", "Vb", "Ob"):
+        W[name] = (rng.standard_normal(nvec) * 0.1).astype(np.float32)
+    gy = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    coef = float(1.0 / np.sqrt(nvec / nhead))
+
+    want_y, fw = _oracle_mh_attention(inputs["key"], inputs["query"], inputs["value"], W, nhead, mask, coef)
+    want_g = _oracle_mh_attention_backprop(gy, inputs["key"], inputs["query"], inputs["value"], W, fw, nhead, mask,
+                                           coef, same)
+
+    tx = tn(x)
+    tin = {name: (tx if name in same else tn(inputs[name])) for name in ("key", "query", "value")}
+    tw = {name: tn(a) for name, a in W.items()}
+    y = tx.mh_attention(tin["key"], tin["query"], tin["value"], tw["Kw"], tw["Kb"], tw["Qw"], tw["Qb"], tw["Vw"],
+                        tw["Vb"], tw["Ow"], tw["Ob"], nhead, mask=mask)
+    check(y.numpy(), want_y, what="mh_attention output")
+    for name in ("K", "Q", "V", "probs", "mixed"):
+        check(y.saved[name].numpy(), fw[name], what="mh_attention saved " + name)
+    if mask:
+        upper = np.triu(np.ones((ntimes, ntimes), bool), 1)
+        assert (y.saved["probs"].numpy()[:, upper] == 0).all()       # keys after the query: exactly 0
+    got_g = y.mh_attention_backprop(tn(gy))
+    assert set(got_g) == set(want_g)
+    for name in sorted(want_g):
+        # gradients run through up to eight chained products: the bar of a whole layer
+        check(got_g[name].numpy(), want_g[name], tol=2e-5, what="mh_attention backprop " + name)
+
+
+# the backward ops at the two benchmark mappings of configuration 4 (what bench.py times is what is tested)
+@pytest.mark.parametrize("nbat,nhead,nvec", [(32, 1, 64), (4, 8, 512)])
+def test_cfg4_attention_backward(nbat, nhead, nvec):
+    ntimes, npiece = 512, 64
+    q, k, v = cfg4(nbat, ntimes, nvec)
+    rng = np.random.default_rng(44)
+    gy = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    coef = 1.0 / np.sqrt(npiece)
+    hcoef = kai.hyper(coef)
+    pshape = (nbat, ntimes, ntimes, nhead)
+    ref_p = ko.softmax_direct_on_axis(ko.mult_on_heads(k, q, nhead, coef), nbat * ntimes, ntimes, nhead)
+    dq, dk, dv, dgy, dp = dev(q), dev(k), dev(v), dev(gy), dev(ref_p)
+    gp = DB(ref_p.nbytes)
+    VMath.mix_values_backward_prop(0, gp, dgy, dv, nbat, ntimes, nvec, nhead, npiece)
+    ref_gp = ko.mix_values_backward_prop(gy, v, nhead)
+    check(gp.to_numpy(pshape), ref_gp, what="cfg4 mix_values_backward_prop")
+    gv = DB(v.nbytes)
+    VMath.mix_values_backward_value(0, gv, dgy, dp, nbat, ntimes, nvec, nhead, npiece)
+    check(gv.to_numpy(v.shape), ko.mix_values_backward_value(gy, ref_p, nhead), what="cfg4 mix_values_backward_value")
+    dgp = dev(ref_gp)
+    VMath.softmax_direct_on_axis_backward(0, dgp, dp, nbat, ntimes, nhead, hcoef)
+    ref_gs = ko.softmax_direct_on_axis_backward(ref_gp, ref_p, coef)
+    check(dgp.to_numpy(pshape), ref_gs, what="cfg4 softmax backward")
+    dgs = dev(ref_gs)
+    for src, dsrc, name in ((q, dq, "gK"), (k, dk, "gQ")):
+        g = DB(q.nbytes)
+        VMath.mult_on_heads_backward(0, g, dgs, dsrc, nbat, ntimes, nvec, nhead, npiece)
+        check(g.to_numpy(q.shape), ko.mult_on_heads_backward(ref_gs, src, nhead), what="cfg4 mult_on_heads_backward " + name)
+
+
 # one case per kernel variant: rows in registers (1 head; 2..128 heads, short and long axis), rows through
 # LDS (long axis, odd lengths), one thread per head (more than 128 heads)
 SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8), (3, 20, 128), (2, 9, 129),
@@ -709,6 +834,15 @@ def test_recurrent_cells():
             want_r, want_s = ko.lstm_process(aff, prev)
             check(st.to_numpy((ndat, nrec)), want_s, what="lstm state")
             check(r.to_numpy((ndat, nrec)), want_r, what="lstm recurrent")
+            # the cell's gradient (the reference's device kernel): gate-sum gradients, previous-state gradient
+            gr = rng.standard_normal((ndat, nrec)).astype(np.float32)
+            gs = rng.standard_normal((ndat, nrec)).astype(np.float32)
+            want_gs, want_ga = ko.lstm_process_backward(gr, gs, aff, prev)
+            dgr, dgs, dga = dev(gr), dev(gs), DB(aff.nbytes)
+            VMath.lstm_process_backward(0, dgr, dgs, dga, None if prev is None else dev(prev), dev(aff), ndat, nrec, 7)
+            check(dga.to_numpy(aff.shape), want_ga, what="lstm backward gate gradients")
+            check(dgs.to_numpy(gs.shape), want_gs, what="lstm backward state gradient")
+            np.testing.assert_array_equal(dgr.to_numpy(gr.shape), gr)     # the output's gradient is only read
         ai = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
         ar = rng.standard_normal((ndat, 3 * nrec)).astype(np.float32)
         recurs = np.zeros((3, ndat, nrec), np.float32)
@@ -749,22 +883,32 @@ def _oracle_rnn(x, wi, wr, bi, br, cell, nrec, forward, act="tanh"):
             recurs[nt], states[nt] = ko.lstm_process(ia[nt], states[prev] if n > 0 else None)
         else:
             ko.gru_process(recurs, ia[nt], ra[nt], nt)
-    return recurs, ia, ra
+    return recurs, ia, ra, states
 
 
-def _oracle_rnn_backprop(x, wi, wr, use_bias, cell, recurs, ia, ra, gy, gyt, forward, act="tanh"):
-    """vtensor.cpp:2657-2701 issued against the oracle."""
+def _oracle_rnn_backprop(x, wi, wr, use_bias, cell, recurs, ia, ra, gy, gyt, forward, act="tanh", states=None,
+                         use_state=False):
+    """vtensor.cpp:2614-2631, 2657-2701 issued against the oracle."""
     ntimes, ndat, nrec = gyt.shape
     gx, gwi, gwr = np.zeros_like(x), np.zeros_like(wi), np.zeros_like(wr)
     gbi = np.zeros(wi.shape[0], np.float32)
     gbr = np.zeros(wi.shape[0], np.float32)
     gr = gy.copy()
+    gs = np.zeros_like(gy)
+    if cell == "lstm" and use_state:
+        gs, gr = gy.copy(), np.zeros_like(gy)
     for n in range(ntimes):
         nt = ntimes - n - 1 if forward else n
         prev = nt - 1 if forward else nt + 1
-        gr = ko.add(gr, gyt[nt])
+        if cell == "lstm" and use_state:
+            gs = ko.add(gs, gyt[nt])
+        else:
+            gr = ko.add(gr, gyt[nt])
         if cell == "rnn":
             gai = ko.activate_backward_with_y(gr, recurs[nt], act)
+            gar = gai
+        elif cell == "lstm":
+            gs, gai = ko.lstm_process_backward(gr, gs, ia[nt], states[prev] if n < ntimes - 1 else None)
             gar = gai
         else:
             gr, gai, gar = ko.gru_process_backward(gr, recurs, ia[nt], ra[nt], nt)
@@ -793,7 +937,7 @@ def test_rnn_layer_loop(cell, ntimes, ndat, ninp, nrec, forward, bias):
     wr = (rng.standard_normal((ngates * nrec, nrec)) / np.sqrt(nrec) * 0.5).astype(np.float32)
     bi = (rng.standard_normal(ngates * nrec) * 0.1).astype(np.float32) if bias else None
     br = (rng.standard_normal(ngates * nrec) * 0.1).astype(np.float32) if bias else None
-    recurs, ia, ra = _oracle_rnn(x, wi, wr, bi, br, cell, nrec, forward)
+    recurs, ia, ra, states = _oracle_rnn(x, wi, wr, bi, br, cell, nrec, forward)
     tn = lambda a: None if a is None else T.Tensor.from_numpy(a)
     for batched, fused in ((True, True), (False, False), (True, False)):
         y, saved = T.rnn(tn(x), tn(wi), tn(wr), tn(bi), tn(br), cell, nrec, forward=forward,
@@ -805,15 +949,16 @@ def test_rnn_layer_loop(cell, ntimes, ndat, ninp, nrec, forward, bias):
             check(saved["raffines"].numpy(), ra, what="gru recurrent gate sums (%s)" % mode)
         check(y.numpy(), recurs[-1 if forward else 0], what="%s output (%s)" % (cell, mode))
     if cell == "lstm":
-        with pytest.raises(T.KaiError):
-            T.rnn_backprop(saved, tn(recurs[0]), tn(recurs))
-        return
+        check(saved["states"].numpy(), states, what="lstm cell states")
     gy = rng.standard_normal((ndat, nrec)).astype(np.float32)
     gyt = (rng.standard_normal((ntimes, ndat, nrec)) * 0.5).astype(np.float32)
-    want = _oracle_rnn_backprop(x, wi, wr, bias, cell, recurs, ia, ra, gy, gyt, forward)
-    got = T.rnn_backprop(saved, tn(gy), tn(gyt))
-    for name in got:
-        check(got[name].numpy(), want[name], tol=2e-5, what="%s backprop %s" % (cell, name))
+    for use_state in ((False, True) if cell == "lstm" else (False,)):
+        want = _oracle_rnn_backprop(x, wi, wr, bias, cell, recurs, ia, ra, gy, gyt, forward, states=states,
+                                    use_state=use_state)
+        got = T.rnn_backprop(saved, tn(gy), tn(gyt), use_state=use_state)
+        for name in got:
+            check(got[name].numpy(), want[name], tol=2e-5,
+                  what="%s backprop %s (use_state=%s)" % (cell, name, use_state))
 
 
 # ---- transposes ---------------------------------------------------------------------------------------------------

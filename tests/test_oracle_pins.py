@@ -390,6 +390,59 @@ def test_lstm_cell_equals_textbook_float64():
     assert s[0, 0] == 0.75 and abs(r[0, 0]) < 1e-12
 
 
+def _lstm64(a, prev):
+    """Textbook LSTM cell in float64; gate order input, forget, block, output.  Returns (output, state)."""
+    nrec = a.shape[1] // 4
+    i, f, g, o = (a[:, k * nrec:(k + 1) * nrec] for k in range(4))
+    s = prev * _sig64(f) + np.tanh(g) * _sig64(i)
+    return np.tanh(s) * _sig64(o), s
+
+
+def test_lstm_cell_backward_against_central_differences():
+    # The reference's device kernel (vmath.cu:4899-4937): given gr = dL/d(output) and gs = dL/d(state) of THIS
+    # step it returns dL/d(gate sums) and dL/d(previous state).  L = <output, gr> + <state, gs> in float64.
+    rng = np.random.default_rng(11)
+    ndat, nrec = 3, 5                                 # nrec > 4: the host loop's index expression would leave the buffer
+    a = (rng.standard_normal((ndat, 4 * nrec)) * 1.5).astype(np.float32)
+    s0 = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    gr = rng.standard_normal((ndat, nrec)).astype(np.float32)
+    gs = rng.standard_normal((ndat, nrec)).astype(np.float32)
+
+    def loss(a_, prev_):
+        r, s = _lstm64(a_, prev_)
+        return float((r * gr).sum() + (s * gs).sum())
+
+    got_gs, got_ga = ko.lstm_process_backward(gr, gs, a, s0)
+    eps = 1e-6
+    base = (a.astype(np.float64), s0.astype(np.float64))
+    for which, got in ((0, got_ga), (1, got_gs)):
+        num = np.zeros_like(base[which])
+        for idx in np.ndindex(num.shape):
+            hi = [b.copy() for b in base]
+            lo = [b.copy() for b in base]
+            hi[which][idx] += eps
+            lo[which][idx] -= eps
+            num[idx] = (loss(*hi) - loss(*lo)) / (2 * eps)
+        np.testing.assert_allclose(got, num, rtol=0, atol=2e-6)
+    # no previous state (first processed step): same as a zero state, and its gradient is still forget * g_state
+    z_gs, z_ga = ko.lstm_process_backward(gr, gs, a, None)
+    w_gs, w_ga = ko.lstm_process_backward(gr, gs, a, np.zeros_like(s0))
+    np.testing.assert_array_equal(z_ga, w_ga)
+    np.testing.assert_array_equal(z_gs, w_gs)
+    assert np.all(z_ga[:, nrec:2 * nrec] == 0)        # forget gate's gradient = old_state * ... = 0
+    # gate-order trap: forget gate wide open, the others shut: the state passes through, so does its gradient,
+    # and nothing reaches the gate sums (every sigmoid/tanh derivative is ~0 or multiplied by ~0)
+    a2 = np.full((1, 4), -40.0, np.float32)
+    a2[0, 1] = 40.0
+    p_gs, p_ga = ko.lstm_process_backward(np.array([[0.3]], np.float32), np.array([[0.7]], np.float32), a2,
+                                          np.array([[0.75]], np.float32))
+    assert p_gs[0, 0] == np.float32(0.7) and np.all(np.abs(p_ga) < 1e-12)
+    # the output's gradient is an input only
+    gr_before = gr.copy()
+    ko.lstm_process_backward(gr, gs, a, s0)
+    np.testing.assert_array_equal(gr, gr_before)
+
+
 def test_gru_cell_and_its_backward():
     rng = np.random.default_rng(10)
     ntimes, ndat, nrec = 3, 4, 6
