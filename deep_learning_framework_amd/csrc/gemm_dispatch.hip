@@ -251,9 +251,15 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
     if (heads_pv_applies(d)) return launch_heads_pv(d, stream);
     if (plan.split >= 2) {
         const int64_t split = plan.split;
-        float* part = nullptr;
-        KAI_TRY(workspace(split * d.M * d.N * (int64_t)sizeof(float), &part));
+        float* part = d.scratch;
+        const int64_t part_bytes = split * d.M * d.N * (int64_t)sizeof(float);
+        if (part == nullptr) KAI_TRY(workspace(part_bytes, &part));
+        else if (part_bytes > d.scratch_bytes)
+            return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: this product cuts its reduction into " + std::to_string(split) +
+                        " parts and needs " + std::to_string(part_bytes) + " bytes for their sums; the caller's scratch holds " +
+                        std::to_string(d.scratch_bytes));
         GemmDesc ds = plan.dn;
+        ds.scratch = nullptr; ds.scratch_bytes = 0;
         if (plan.ragged_parts) ds.k_part = plan.k_part;   // K stays the whole length
         else ds.K = plan.k_part;
         ds.nbatch = split; ds.bdiv = 1;

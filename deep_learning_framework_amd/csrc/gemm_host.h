@@ -32,6 +32,10 @@ struct GemmDesc {
     // > 0: the nbatch batches are consecutive parts of k_part reduction steps of ONE product of length K
     // (the last part may be shorter); the batch strides of A and B must then be k_part steps
     int64_t k_part = 0;
+    // where a reduction cut into parts puts its partial sums: null = the library's own scratch (allocated and
+    // grown on demand); otherwise this buffer of scratch_bytes, and a product that needs more is refused
+    float* scratch = nullptr;
+    int64_t scratch_bytes = 0;
 };
 
 // LDS orientation of an operand: reduction index contiguous (KC) or output index contiguous (MC).

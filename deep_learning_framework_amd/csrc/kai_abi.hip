@@ -7,6 +7,7 @@
 #include <cstring>
 #include <cstdlib>
 #include <mutex>
+#include <vector>
 
 #include "elementwise.h"
 #include "gemm_host.h"
@@ -34,31 +35,61 @@ int check_launch(const char* kernel_name) { return check_hip(hipGetLastError(), 
 namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_ws_mutex;
-void* g_ws_ptr[kMaxDevices] = {};
-int64_t g_ws_bytes[kMaxDevices] = {};
+// Per device: the current scratch buffer and the smaller ones it replaced.  A replaced buffer is kept until
+// kai_shutdown: kernels already enqueued (on any stream) and HIP graphs that recorded its address stay valid,
+// and growing needs neither a wait for the device nor a hipFree (which waits, too).  Growth at least doubles
+// the size, so the retired buffers together are smaller than the current one.
+struct DeviceScratch {
+    void* ptr = nullptr;
+    int64_t bytes = 0;
+    std::vector<void*> retired;
+    int64_t retired_bytes = 0;
+    int64_t growths = 0;
+};
+DeviceScratch g_ws[kMaxDevices];
 int g_cu_count[kMaxDevices] = {};
+// bytes at the front of the scratch that an enclosing call of this thread holds (ScratchHold)
+thread_local int64_t tl_ws_held = 0;
+constexpr int64_t kScratchMin = 4ll << 20;
+
+int grow_scratch(DeviceScratch& s, int64_t need) {
+    // an allocation is not allowed while the stream records a graph: the caller sizes the scratch first
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(current_stream(), &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+        return fail(KAI_ERR_GPU, "the library scratch would have to grow to " + std::to_string(need) +
+                                     " bytes while the stream is being captured: run the call once before the "
+                                     "capture or call kai_reserve_scratch");
+    int64_t want = need;
+    if (want < 2 * s.bytes) want = 2 * s.bytes;
+    if (want < kScratchMin) want = kScratchMin;
+    void* fresh = nullptr;
+    KAI_TRY(check_hip(hipMalloc(&fresh, (size_t)want), "hipMalloc(scratch)"));
+    if (s.ptr) {
+        s.retired.push_back(s.ptr);
+        s.retired_bytes += s.bytes;
+    }
+    s.ptr = fresh;
+    s.bytes = want;
+    s.growths++;
+    return KAI_OK;
+}
 }  // namespace
 
 int workspace(int64_t bytes, float** out) {
     int dev = 0;
     KAI_TRY(check_hip(hipGetDevice(&dev), "hipGetDevice"));
     if (dev < 0 || dev >= kMaxDevices) return fail(KAI_ERR_INVALID_ARGUMENT, "workspace: device index out of range");
+    if (bytes < 0) return fail(KAI_ERR_INVALID_ARGUMENT, "workspace: negative size");
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (g_ws_bytes[dev] < bytes) {
-        // earlier users of the smaller buffer are ordered before the free by the device-wide wait
-        if (g_ws_ptr[dev]) {
-            KAI_TRY(check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize"));
-            KAI_TRY(check_hip(hipFree(g_ws_ptr[dev]), "hipFree"));
-            g_ws_ptr[dev] = nullptr;
-            g_ws_bytes[dev] = 0;
-        }
-        const int64_t want = bytes < (4ll << 20) ? (4ll << 20) : bytes;
-        KAI_TRY(check_hip(hipMalloc(&g_ws_ptr[dev], (size_t)want), "hipMalloc(workspace)"));
-        g_ws_bytes[dev] = want;
-    }
-    *out = static_cast<float*>(g_ws_ptr[dev]);
+    DeviceScratch& s = g_ws[dev];
+    const int64_t need = tl_ws_held + bytes;
+    if (s.bytes < need) KAI_TRY(grow_scratch(s, need));
+    *out = reinterpret_cast<float*>(static_cast<char*>(s.ptr) + tl_ws_held);
     return KAI_OK;
 }
+
+ScratchHold::ScratchHold(int64_t bytes) : previous_(tl_ws_held) { tl_ws_held += (bytes + 255) / 256 * 256; }
+ScratchHold::~ScratchHold() { tl_ws_held = previous_; }
 
 int compute_units() {
     int dev = 0;
@@ -77,13 +108,15 @@ static int release_workspaces() {
     if (hipGetDevice(&old) != hipSuccess) old = 0;
     int rc = KAI_OK;
     for (int d = 0; d < kMaxDevices; d++) {
-        if (!g_ws_ptr[d]) continue;
+        DeviceScratch& s = g_ws[d];
+        if (!s.ptr && s.retired.empty()) continue;
         if (hipSetDevice(d) == hipSuccess) {
             (void)hipDeviceSynchronize();
-            if (hipFree(g_ws_ptr[d]) != hipSuccess) rc = KAI_ERR_GPU;
+            if (s.ptr && hipFree(s.ptr) != hipSuccess) rc = KAI_ERR_GPU;
+            for (void* p : s.retired)
+                if (hipFree(p) != hipSuccess) rc = KAI_ERR_GPU;
         }
-        g_ws_ptr[d] = nullptr;
-        g_ws_bytes[d] = 0;
+        s = DeviceScratch();
     }
     (void)hipSetDevice(old);
     return rc;
@@ -122,6 +155,23 @@ int kai_set_stream(void* hip_stream) {
 int kai_shutdown(void) {
     const int rc = release_workspaces();
     if (rc != KAI_OK) return fail(rc, "kai_shutdown: hipFree failed");
+    return KAI_OK;
+}
+
+int kai_reserve_scratch(int64_t bytes) {
+    KAI_REQUIRE(bytes >= 0, KAI_ERR_INVALID_ARGUMENT, "negative size");
+    float* unused = nullptr;
+    return workspace(bytes, &unused);
+}
+
+int kai_scratch_info(int64_t* bytes, int64_t* growths, int64_t* retired_bytes) {
+    int dev = 0;
+    KAI_TRY(check_hip(hipGetDevice(&dev), "hipGetDevice"));
+    KAI_REQUIRE(dev >= 0 && dev < kMaxDevices, KAI_ERR_INVALID_ARGUMENT, "device index out of range");
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (bytes) *bytes = g_ws[dev].bytes;
+    if (growths) *growths = g_ws[dev].growths;
+    if (retired_bytes) *retired_bytes = g_ws[dev].retired_bytes;
     return KAI_OK;
 }
 
@@ -761,8 +811,12 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
         return launch_attention_fused(py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked != 0,
                                       current_stream());
     // any other shape: the separate kernels, probabilities in the library's scratch memory
+    // (the products below may ask for scratch of their own, for partial sums of a reduction cut into parts:
+    // while `held` lives, such requests are placed behind the probabilities)
+    const int64_t pbytes = nbat * ntimes * ntimes * nhead * (int64_t)sizeof(float);
     float* pp = nullptr;
-    KAI_TRY(workspace(nbat * ntimes * ntimes * nhead * (int64_t)sizeof(float), &pp));
+    KAI_TRY(workspace(pbytes, &pp));
+    ScratchHold held(pbytes);
     KAI_TRY(kai_mult_on_heads(device, pp, pK, pQ, nbat, ntimes, nvec, nhead, npiece, hCoef));
     if (masked) KAI_TRY(kai_set_mh_attention_mask(device, pp, nbat, ntimes, nhead, 1));
     KAI_TRY(kai_softmax_direct_on_axis(device, pp, nbat * ntimes, ntimes, nhead));

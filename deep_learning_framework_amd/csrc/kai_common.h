@@ -23,10 +23,27 @@ int check_hip(hipError_t st, const char* what);
 // status of the launch that was just enqueued
 int check_launch(const char* kernel_name);
 
-// Library-owned scratch memory on the CURRENT device (split-K partial sums).  Allocated on first use,
-// grown when a call needs more, released by kai_shutdown.  Calls that use it must be ordered on one
-// stream per device: the engine runs one thread (and the null stream) per device.
+// Library-owned scratch memory on the CURRENT device (partial sums of a reduction cut into parts, row norms,
+// the probabilities of an attention call that runs as separate kernels).  Allocated on first use and released
+// by kai_shutdown.  When a call needs more than there is, a larger buffer is allocated and the old one is
+// kept until kai_shutdown, so growth never waits for the device and pointers handed out earlier (to
+// kernels in flight, to recorded graphs) stay valid.  While a stream capture is active, growth is refused
+// with an error.  Every call returns the front of the same buffer: calls that use it must be ordered on one
+// stream per device (the engine runs one thread and the null stream per device).
 int workspace(int64_t bytes, float** out);
+// While an object of this type lives, workspace() calls of the same thread return memory BEHIND the first
+// `bytes` bytes of the scratch: for a call that keeps data in the scratch across inner calls which may ask
+// for scratch themselves.
+class ScratchHold {
+public:
+    explicit ScratchHold(int64_t bytes);
+    ~ScratchHold();
+    ScratchHold(const ScratchHold&) = delete;
+    ScratchHold& operator=(const ScratchHold&) = delete;
+
+private:
+    int64_t previous_;
+};
 // number of compute units of the current device (cached)
 int compute_units();
 

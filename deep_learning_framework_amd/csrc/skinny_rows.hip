@@ -144,8 +144,12 @@ int launch_skinny_rows(const GemmDesc& d, hipStream_t stream) {
     if (splits > 16) splits = 16;
     const int64_t k_part = ((d.K + splits - 1) / splits + unit - 1) / unit * unit;
     splits = (d.K + k_part - 1) / k_part;
-    float* part = nullptr;
-    KAI_TRY(workspace(splits * d.M * d.N * (int64_t)sizeof(float), &part));
+    float* part = d.scratch;
+    const int64_t part_bytes = splits * d.M * d.N * (int64_t)sizeof(float);
+    if (part == nullptr) KAI_TRY(workspace(part_bytes, &part));
+    else if (part_bytes > d.scratch_bytes)
+        return fail(KAI_ERR_INVALID_ARGUMENT, "skinny rows: the partial sums need " + std::to_string(part_bytes) +
+                    " bytes; the caller's scratch holds " + std::to_string(d.scratch_bytes));
     SkinnyRowsParams p{};
     p.A = d.A; p.B = d.B; p.part = part;
     p.lda = d.a_rs; p.ldb = d.b_ks; p.N = d.N; p.M = (int)d.M; p.K = (int)d.K;

@@ -29,6 +29,8 @@ SIGNATURES = {
     "kai_set_stream": [ctypes.c_void_p],
     "kai_arch_info": [ctypes.c_char_p, ctypes.c_char_p, _INT],
     "kai_shutdown": [],
+    "kai_reserve_scratch": [_I64],
+    "kai_scratch_info": [ctypes.POINTER(_I64), ctypes.POINTER(_I64), ctypes.POINTER(_I64)],
     "kai_mem_alloc": [_INT, _I64, ctypes.POINTER(ctypes.c_void_p)],
     "kai_mem_free": [_INT, ctypes.c_void_p],
     "kai_memcpy_host_to_host": [ctypes.c_void_p, ctypes.c_void_p, _I64],
@@ -200,6 +202,18 @@ def set_stream(stream_handle):
 def shutdown():
     """Release the library's own scratch memory (it is re-created on demand)."""
     _ck(load().kai_shutdown())
+
+
+def reserve_scratch(nbytes):
+    """Size the current device's scratch now, so that later calls allocate nothing."""
+    _ck(load().kai_reserve_scratch(nbytes))
+
+
+def scratch_info():
+    """(bytes, growths since the last shutdown, bytes of replaced buffers still held) of the current device."""
+    b, g, r = _I64(), _I64(), _I64()
+    _ck(load().kai_scratch_info(ctypes.byref(b), ctypes.byref(g), ctypes.byref(r)))
+    return b.value, g.value, r.value
 
 
 def arch_info():

@@ -77,10 +77,23 @@ int kai_device_synchronize(void);
 /* Stream (a hipStream_t, or null for the null stream) that this THREAD's later calls enqueue on.
  * No counterpart in the reference, which only uses the legacy default stream. */
 int kai_set_stream(void* hip_stream);
-/* Releases the scratch memory the library allocated for itself (split-K partial sums; one buffer per
- * device, created on first need).  The library stays usable: the buffer is created again on demand.
- * No counterpart in the reference, whose kernels need no scratch. */
+/* Releases the scratch memory the library allocated for itself (partial sums of reductions cut into parts,
+ * row norms of kai_cosinesim, the probabilities of a kai_attention_forward call that runs as separate
+ * kernels; one buffer per device, created on first need).  Waits for the device first.  The library stays
+ * usable: the buffer is created again on demand.  No counterpart in the reference, whose kernels need no
+ * scratch. */
 int kai_shutdown(void);
+/* Makes the current device's scratch at least `bytes` large now, so that later calls find it and allocate
+ * nothing: for callers that record calls into a HIP graph (a call whose scratch would have to grow while its
+ * stream is being captured fails with KAI_ERR_GPU) or that cannot tolerate an allocation inside a step.  A
+ * product never asks for more than 64 MiB of partial sums; kai_attention_forward outside the fused head sizes
+ * asks for nbat*ntimes*ntimes*nhead floats on top.  Growing never waits for the device: the smaller buffer is
+ * kept until kai_shutdown, so work in flight and recorded graphs stay valid.  No counterpart in the reference. */
+int kai_reserve_scratch(int64_t bytes);
+/* Current size of the current device's scratch, how many times it was allocated or grown since the last
+ * kai_shutdown, and the bytes of replaced buffers still held.  Any pointer may be null.  For tests and
+ * diagnostics; no counterpart in the reference. */
+int kai_scratch_info(int64_t* bytes, int64_t* growths, int64_t* retired_bytes);
 /* Name of the code object's target ("gfx950") and of the current device's architecture. */
 int kai_arch_info(char* built_for, char* device_arch, int buflen);
 

@@ -708,13 +708,88 @@ def test_split_k_scratch_survives_shutdown_and_growth():
         probs = ko.softmax_direct_on_axis(ko.mult_on_heads(k, q, nhead, coef), nbat * T, T, nhead)
         check(o.to_numpy((nbat, T, nhead * npiece)), ko.mix_values(probs, v, nhead), what="attention through the scratch")
 
+    kai.shutdown()
+    assert kai.scratch_info() == (0, 0, 0)
     split_k(64, 64, 4096)
     split_k(256, 512, 4096)
-    attention_with_scratch()
+    assert kai.scratch_info() == (4 << 20, 1, 0)          # first need: 4 MiB, enough for both products
+    attention_with_scratch()                              # 4.5 MiB of probabilities: the buffer grows
+    size, growths, retired = kai.scratch_info()
+    assert size >= 4718592 and growths == 2 and retired == 4 << 20    # the smaller buffer is kept, not freed
     split_k(64, 128, 8192)
+    assert kai.scratch_info()[1] == 2
     kai.shutdown()
+    assert kai.scratch_info() == (0, 0, 0)
     split_k(64, 128, 8192)
     attention_with_scratch()
+    # sizing ahead of time: afterwards nothing grows
+    kai.reserve_scratch(48 << 20)
+    n_growths = kai.scratch_info()[1]
+    split_k(1024, 1024, 8192)
+    attention_with_scratch()
+    assert kai.scratch_info()[1] == n_growths and kai.scratch_info()[0] >= 48 << 20
+
+
+def test_scratch_growth_does_not_wait_for_the_device():
+    # Growth allocates the larger buffer and keeps the old one: no device-wide wait, no free.  Shown by
+    # queueing ~0.1 s of products, then issuing a call that makes the scratch grow: it returns while the queue
+    # is still busy (the wait afterwards takes most of the queued time), and its result is right.
+    import time
+    rng = np.random.default_rng(5)
+    n = 4096
+    a, b, c = dev(rng.standard_normal((n, n)).astype(np.float32)), dev(rng.standard_normal((n, n)).astype(np.float32)), DB(n * n * 4)
+    m, nn, k = 1024, 1024, 8192                        # two parts of 1024 x 1024 sums: 8 MiB
+    assert VMath.gemm_plan(0, 1, m, nn, k).endswith("split 2")
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.uniform(-0.05, 0.05, (nn, k)).astype(np.float32)
+    dx, dw, y = dev(x), dev(w), DB(m * nn * 4)
+    VMath.gemm_f32(0, 0, 0, n, n, n, a, n, b, n, c, n, None, 0, None, False)     # code objects loaded, clocks up
+    kai.shutdown()
+    kai.reserve_scratch(1 << 20)                       # the smallest buffer (4 MiB), which the product below outgrows
+    before = kai.scratch_info()
+    kai.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(100):                               # ~1 ms each
+        VMath.gemm_f32(0, 0, 0, n, n, n, a, n, b, n, c, n, None, 0, None, False)
+    t_queued = time.perf_counter()
+    VMath.matmul(0, y, dw, dx, nn, m, k, False)
+    t_call = time.perf_counter()
+    kai.synchronize()
+    t_done = time.perf_counter()
+    after = kai.scratch_info()
+    print("queueing %.1f ms, growing call %.2f ms, drain %.1f ms, scratch %s -> %s"
+          % ((t_queued - t0) * 1e3, (t_call - t_queued) * 1e3, (t_done - t_call) * 1e3, before, after))
+    assert after[1] == before[1] + 1 and after[0] >= 8 << 20 and after[2] == before[0]
+    rows = list(range(0, m, 32))
+    check(y.to_numpy((m, nn))[rows], ko.matmul_rows(w, x, rows), what="product after growth")
+    if (t_done - t_call) > 0.02:                       # the queue was still busy when the call returned
+        assert (t_call - t_queued) < 0.5 * (t_done - t_call)
+    else:
+        pytest.skip("the queued products had drained before the call: nothing to observe")
+
+
+# the fallback of kai_attention_forward keeps its probabilities in the scratch while its own products cut their
+# reductions into parts and need scratch, too: the partial sums must land behind the probabilities
+@pytest.mark.parametrize("ntimes,npiece,masked", [(1536, 128, False), (1536, 96, True), (2048, 128, True)])
+def test_attention_fallback_with_one_long_head(ntimes, npiece, masked):
+    nbat = nhead = 1
+    nvec = npiece
+    # the product P . V of this geometry is one that cuts its reduction into parts
+    assert int(VMath.gemm_plan(0, 0, ntimes, npiece, ntimes).rsplit(" ", 1)[1]) > 1
+    rng = np.random.default_rng(ntimes + npiece)
+    q, k, v = (rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32) for _ in range(3))
+    coef = 1.0 / np.sqrt(npiece)
+    s = ko.mult_on_heads(k, q, nhead, coef)
+    if masked:
+        s = ko.set_mh_attention_mask(s, True)
+    probs = ko.softmax_direct_on_axis(s, nbat * ntimes, ntimes, nhead)
+    ref = ko.mix_values(probs, v, nhead)
+    kai.shutdown()                                     # start from no scratch: the inner products make it grow
+    o = DB(nbat * ntimes * nvec * 4)
+    VMath.attention_forward(0, o, dev(q), dev(k), dev(v), nbat, ntimes, nvec, nhead, npiece, kai.hyper(coef), masked)
+    check(o.to_numpy((nbat, ntimes, nvec)), ref, what="attention fallback, one head of %d" % npiece)
+    VMath.attention_forward(0, o, dev(q), dev(k), dev(v), nbat, ntimes, nvec, nhead, npiece, kai.hyper(coef), masked)
+    check(o.to_numpy((nbat, ntimes, nvec)), ref, what="attention fallback again, scratch in place")
 
 
 # ---- small products: the reduction cut over the waves of one workgroup ---------------------------------------
