@@ -46,6 +46,7 @@ SIGNATURES = {
     "kai_memcpy_to_device": [_INT, ctypes.c_void_p, ctypes.c_void_p, _I64],
     "kai_get_slice": [_INT, ctypes.c_void_p, ctypes.c_void_p, _I64],
     "kai_matmul": [_INT, _F, _F, _F, _I64, _I64, _I64, _INT],
+    "kai_matmul_noalloc": [_INT, _F, _F, _F, _I64, _I64, _I64, _INT],
     "kai_matmul_backward_x": [_INT, _F, _F, _F, _I64, _I64, _I64, _INT],
     "kai_matmul_backward_w": [_INT, _F, _F, _F, _I64, _I64, _I64, _INT],
     "kai_add_bias": [_INT, _F, _F, _F, _I64, _I64],
@@ -114,6 +115,8 @@ def load():
             fn.restype = _INT
         L.kai_last_error.argtypes = []
         L.kai_last_error.restype = ctypes.c_char_p
+        L.kai_matmul_noalloc_scratch_bytes.argtypes = []
+        L.kai_matmul_noalloc_scratch_bytes.restype = _I64
         _lib = L
     return _lib
 
@@ -229,6 +232,11 @@ class VMath:
     @staticmethod
     def matmul(device, py, pw, px, yvec, ndat, xvec, acc):
         _ck(load().kai_matmul(device, _addr(py), _addr(pw), _addr(px), yvec, ndat, xvec, int(acc)))
+
+    @staticmethod
+    def matmul_noalloc(device, py, pw, px, yvec, ndat, xvec, acc):
+        """kai_matmul without any allocation: partial sums go to a fixed array inside the library."""
+        _ck(load().kai_matmul_noalloc(device, _addr(py), _addr(pw), _addr(px), yvec, ndat, xvec, int(acc)))
 
     @staticmethod
     def matmul_backward_x(device, pgx, pgy, pw, yvec, ndat, xvec, acc):

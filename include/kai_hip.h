@@ -135,6 +135,18 @@ int kai_matmul_backward_x(int device, float* pgx, const float* pgy, const float*
 int kai_matmul_backward_w(int device, float* pgw, const float* pgy, const float* px, int64_t yvec, int64_t ndat,
                           int64_t xvec, int acc);
 
+/* kai_matmul for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same kernels and
+ * the same result as kai_matmul; it calls no hipMalloc / hipFree and never touches the library's heap scratch.
+ * A product whose reduction is cut into parts keeps the partial sums in a fixed 32 MiB array inside the
+ * library's code object (each GPU the library runs on holds its copy until the process ends); a product whose
+ * partial sums would need more (kai_matmul_noalloc_scratch_bytes) is refused with KAI_ERR_INVALID_ARGUMENT and
+ * a message that names both sizes.  All calls on one GPU share that array: calls that overlap on one GPU race
+ * and must be serialised by the caller.  The first call on a device looks up the array's address. */
+int kai_matmul_noalloc(int device, float* py, const float* pw, const float* px, int64_t yvec, int64_t ndat,
+                       int64_t xvec, int acc);
+int64_t kai_matmul_noalloc_scratch_bytes(void);
+
 /* VMath::add_bias, vmath.cu:875-897.  y[r,c] = a[r,c] + b[c]; py may equal pa */
 int kai_add_bias(int device, float* py, const float* pa, const float* pb, int64_t nrow, int64_t ncol);
 /* VMath::add_bias_backward_b, vmath.cu:901-932.  gb[c] (=|+=) sum_r gy[r,c] */
