@@ -38,9 +38,34 @@ def hbm_traffic_from_profile(summary_name):
         return None
 
 
-def cpu_baseline(a_rows, bt, bias, seconds_hint=15.0):
-    """Times the oracle (the reference's host loop restated in C, one thread as in the reference) on
-    a bounded sample of rows of the same 8192^3 product."""
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def usable_cores():
+    """Host threads this process may use: its CPU affinity, capped by OMP_NUM_THREADS where the box sets it."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except AttributeError:
+        n = os.cpu_count() or 1
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    if cap.isdigit() and int(cap) > 0:
+        n = min(n, int(cap))
+    return max(1, n)
+
+
+def cpu_baseline(a_rows, bt, bias, seconds_hint=10.0):
+    """Times the oracle (the reference's host loop restated in C) on a bounded sample of rows of the same
+    8192^3 product: on ONE thread, as the reference's host path runs (`value`), and with the rows spread
+    over all usable cores (`all_cores`; every output element is still summed sequentially, so the results are
+    bit-identical to the single-thread run, which is checked)."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import oracle as ko
     n = bt.shape[0]
@@ -54,11 +79,22 @@ def cpu_baseline(a_rows, bt, bias, seconds_hint=15.0):
     y = ko.activate(ko.add_bias(y, bias), "relu")
     dt = time.perf_counter() - t0
     flops = 2.0 * rows * n * k
+    threads = usable_cores()
+    prow = int(min(a_rows.shape[0], max(threads, rows * min(threads, 8))))
+    t0 = time.perf_counter()
+    yp = ko.matmul_parallel(bt, a_rows[:prow], threads)
+    yp = ko.activate(ko.add_bias(yp, bias), "relu")
+    dtp = time.perf_counter() - t0
     return {
         "value": flops / dt * 1e-12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
         "sample": "%d of %d rows of the same 8192^3 GEMM+bias+ReLU, %.1f s, oracle/kai_oracle.c "
                   "(gcc -O2 -ffp-contract=off), extrapolates to %.0f s for the full product" % (
                       rows, n, dt, dt * n / rows),
+        "all_cores": {"value": 2.0 * prow * n * k / dtp * 1e-12, "unit": "TFLOP/s", "cores": threads,
+                      "sample": "%d rows spread over %d threads, %.1f s, extrapolates to %.0f s" % (
+                          prow, threads, dtp, dtp * n / prow),
+                      "bit_identical_to_one_thread": bool(np.array_equal(yp[:rows], y))},
+        "nproc": os.cpu_count(), "cpu_model": cpu_model(),
     }, y, rows
 
 
@@ -125,6 +161,24 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
         rows.append(r)
 
     relu = kai.ACT["relu"]
+    # the headline product in the ENGINE's operand forms (weights stored [out, in]): forward NT with bias + ReLU in
+    # one launch, the input gradient NN, the weight gradient TN
+    n8 = 8192
+    x8 = torch.rand((n8, n8), device=dev, generator=g) * 2 - 1
+    w8 = torch.rand((n8, n8), device=dev, generator=g) * 2 - 1
+    b8 = torch.randn(n8, device=dev, generator=g)
+    o8 = torch.empty((n8, n8), device=dev)
+    f8 = 2.0 * n8 ** 3
+    row("8192^3 NT  Y = relu(X.W^T + b)  (kai_dense_forward)",
+        gpu_us(lambda: L.kai_dense_forward(0, P(o8), None, P(w8), P(b8), P(x8), I(n8), I(n8), I(n8), relu, None), iters=10),
+        flops=f8)
+    row("8192^3 NT  Y = X.W^T  (kai_matmul)",
+        gpu_us(lambda: L.kai_matmul(0, P(o8), P(w8), P(x8), I(n8), I(n8), I(n8), 0), iters=10), flops=f8)
+    row("8192^3 NN  dX = dY.W  (kai_matmul_backward_x)",
+        gpu_us(lambda: L.kai_matmul_backward_x(0, P(o8), P(x8), P(w8), I(n8), I(n8), I(n8), 0), iters=10), flops=f8)
+    row("8192^3 TN  dW = dY^T.X  (kai_matmul_backward_w)",
+        gpu_us(lambda: L.kai_matmul_backward_w(0, P(o8), P(x8), P(w8), I(n8), I(n8), I(n8), 0), iters=10), flops=f8)
+    del x8, w8, b8, o8
     # cfg1: dense forward 64 x 784 -> 512, fused
     x = torch.randn((64, 784), device=dev, generator=g)
     w = (torch.rand((512, 784), device=dev, generator=g) * 2 - 1) / 28.0
@@ -150,6 +204,12 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
         flops=f, cpu=cpu_us(lambda: ko.matmul_backward_w(gyc, xc, 1024, 1024)))
     row("cfg2 db = colsum(dY)", gpu_us(lambda: L.kai_add_bias_backward_b(0, P(gb), P(gy), I(256), I(1024), 0)),
         nbytes=4.0 * 256 * 1024, cpu=cpu_us(lambda: ko.add_bias_backward_b(gyc, 1024)))
+    pre = torch.randn((256, 1024), device=dev, generator=g)
+    work = torch.empty_like(pre)
+    row("cfg2 dense backward with ReLU: dX, dW, db from dY and the pre-activation (kai_dense_backward)",
+        gpu_us(lambda: L.kai_dense_backward(0, P(gx), P(gw), P(gb), P(work), P(gy), P(w), P(x), P(pre), I(1024), I(256),
+                                            I(1024), relu, None, 0)),
+        flops=2 * f)
     # cfg4: attention, both mappings of 32 batch x heads, seq 512, head dim 64
     for nbat, nhead, nvec in ((32, 1, 64), (4, 8, 512)):
         T, D = 512, 64
@@ -293,7 +353,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="skip the table of the other configurations")
     args = ap.parse_args()
@@ -332,15 +392,19 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # events between the steps as well: the average over the timed region prices the roofline, the per-step
+    # durations give the median
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    ev0.record(stream)
-    for _ in range(args.steps):
+    evs[0].record(stream)
+    for i in range(args.steps):
         step()
-    ev1.record(stream)
+        evs[i + 1].record(stream)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    kernel_ms = ev0.elapsed_time(ev1) / args.steps
+    kernel_ms = evs[0].elapsed_time(evs[-1]) / args.steps
+    step_ms = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
+    kernel_ms_median = step_ms[len(step_ms) // 2] if len(step_ms) % 2 else 0.5 * (step_ms[len(step_ms) // 2 - 1] + step_ms[len(step_ms) // 2])
     flops = 2.0 * n * n * n
     tflops = flops / (wall_ms * 1e-3) * 1e-12
     achieved = flops / (kernel_ms * 1e-3) * 1e-12
@@ -371,20 +435,25 @@ def main():
     argsets = [(0, ctypes.c_void_p(y.data_ptr()), ctypes.c_void_p(w.data_ptr()), ctypes.c_void_p(x.data_ptr()),
                 ctypes.c_int64(nn), ctypes.c_int64(1), ctypes.c_int64(kk), 0) for w in ws]
 
-    def gemv_time(cold, iters=120):
-        for i in range(nbuf):
-            fn(*argsets[i if cold else 0])
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for i in range(iters):
+    def gemv_time(cold, iters=120, repeats=7, warm_launches=60):
+        """Median (and the extremes) over `repeats` measurements of `iters` back-to-back launches each."""
+        for i in range(warm_launches):
             fn(*argsets[i % nbuf if cold else 0])
-        e1.record(stream)
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / iters
+        times = []
+        for _ in range(repeats):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for i in range(iters):
+                fn(*argsets[i % nbuf if cold else 0])
+            e1.record(stream)
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) / iters)
+        times.sort()
+        return times[len(times) // 2], times[0], times[-1]
 
-    cold_ms = gemv_time(True)
-    warm_ms = gemv_time(False)
+    cold_ms, cold_min, cold_max = gemv_time(True)
+    warm_ms, warm_min, warm_max = gemv_time(False)
     gemv_ref = (x.double() @ ws[0].double().T)   # the warm pass ran last, on buffer 0
     gemv_err = float(torch.linalg.norm(y.double() - gemv_ref) / torch.linalg.norm(gemv_ref))
     gemv_gbs = gemv_bytes / (cold_ms * 1e-3) * 1e-9
@@ -400,10 +469,15 @@ def main():
         "rel_fro_err_vs_f64_rows": err,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_FP32_MFMA_TFLOPS, "traffic": hbm_traffic_from_profile("gemm_mfma_kernel_8192_gemm_bias_relu.md"),
-                     "kernel": "gemm_mfma_kernel", "kernel_ms": kernel_ms, "flops_per_launch": flops},
+                     "kernel": "gemm_mfma_kernel", "kernel_ms": kernel_ms, "kernel_ms_median": kernel_ms_median,
+                     "kernel_ms_min_max": [step_ms[0], step_ms[-1]], "flops_per_launch": flops},
         "gemv": {"workload": "batch-1 y = x . W^T, W[4096,4096] fp32 (BASELINE configs[4], M=1), kai_matmul",
                  "value": gemv_gbs, "unit": "GB/s", "us_per_call_cold": cold_ms * 1e3,
-                 "us_per_call_warm": warm_ms * 1e3, "warm_gbs": gemv_bytes / (warm_ms * 1e-3) * 1e-9,
+                 "us_per_call_cold_min_max": [cold_min * 1e3, cold_max * 1e3],
+                 "us_per_call_warm": warm_ms * 1e3, "us_per_call_warm_min_max": [warm_min * 1e3, warm_max * 1e3],
+                 "warm_gbs": gemv_bytes / (warm_ms * 1e-3) * 1e-9,
+                 "timing": "median of 7 measurements of 120 back-to-back launches after 60 warm-up launches; cold = six "
+                           "rotating 64 MiB weight buffers (384 MiB > the 256 MB last-level cache)",
                  "rel_fro_err_vs_f64": gemv_err,
                  "roofline": {"bound": "hbm", "achieved": gemv_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                               "frac": gemv_gbs / PEAK_HBM_GBS, "traffic": hbm_traffic_from_profile("gemv_rows_kernel_4096x4096_batch1.md"),
@@ -411,10 +485,9 @@ def main():
     }
 
     if not args.no_cpu_baseline:
-        a_rows = a[:768].cpu().numpy()
+        a_rows = a[:2048].cpu().numpy()
         bt = np.ascontiguousarray(b.cpu().numpy().T)
         base, y_cpu, nrows = cpu_baseline(a_rows, bt, bias.cpu().numpy())
-        base["host_cores_available"] = os.cpu_count()
         got = c[:nrows].cpu().numpy()
         base["gpu_vs_oracle_rel_fro"] = float(np.linalg.norm((got - y_cpu).astype(np.float64)) /
                                               np.linalg.norm(y_cpu.astype(np.float64)))
