@@ -143,6 +143,13 @@ int launch_skinny_rows(const GemmDesc& d, hipStream_t stream);
 bool heads_pv_applies(const GemmDesc& d);
 int launch_heads_pv(const GemmDesc& d, hipStream_t stream);
 
+// the two products and the bias gradient of a dense layer's backward pass in one launch: dense_backward.hip
+int dense_backward_pair_split(const float* pgx, const float* pgw, const float* pgy, const float* pw, const float* px,
+                              const float* ppre, int64_t yvec, int64_t ndat, int64_t xvec, int act);
+int launch_dense_backward_pair(float* pgx, float* pgw, float* pgb, const float* pgy, const float* pw, const float* px,
+                               const float* ppre, int64_t yvec, int64_t ndat, int64_t xvec, int act,
+                               const float* leaky, bool acc, int split, hipStream_t stream);
+
 // per-layout entry points (one translation unit each, to compile in parallel)
 enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2, kTileFlat = 3 };   // flat: 32 rows x 128 columns
 int launch_gemm_kc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);

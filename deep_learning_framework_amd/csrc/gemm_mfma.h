@@ -93,6 +93,11 @@ struct GemmParams {
     // EDGE kernels only: when > 0 the batch index also cuts the reduction: batch z covers the
     // k_part steps from z*k_part on (fewer in the last batch), K being the whole length
     int k_part;
+    // AMASK bodies only: the A operand is the output gradient of a dense layer and A2, laid out like A, its
+    // pre-activation: the product uses A(m,k) * f'(A2(m,k)) with f = relu (a_mask 1) or leaky relu (a_mask 2,
+    // slope *leaky, 0 if null); a_mask 0 uses A as it is
+    const float* A2;
+    int a_mask;
 };
 
 constexpr int kLdsPad = 4;
@@ -557,9 +562,19 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 // ROWSUM (PIPE 0 only): the workgroups of the first tile column also sum every row of their A tile
 // over K, one thread per row reading the tile from LDS, k ascending across tiles: a fixed order
 // that is the order of a sequential loop.
-template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
-          int DEPTH = 1, bool ROWSUM = false>
-__global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const GemmParams p) {
+//
+// AMASK (PIPE 0, whole tiles only): the A tile is multiplied element by element with the derivative of
+// relu / leaky relu at a second tensor A2 of the same layout on its way to LDS (GemmParams::a_mask): the
+// backward products of a dense layer read the output gradient and the pre-activation directly.
+//
+// The body is a device function over (workgroup id, batch index, the two LDS tile pairs) so that one launch
+// can hold the workgroups of two different products (dense_backward.hip); gemm_mfma_kernel is one product.
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE, int DEPTH,
+          bool ROWSUM, bool AMASK>
+__device__ __forceinline__ void gemm_tile_body(
+    const GemmParams& p, const int bid, const int z,
+    float (*lds_a)[TileShape<A_KC, WM * NBM * 32, BK>::kFloats],
+    float (*lds_b)[TileShape<B_KC, WN * NBN * 32, BK>::kFloats]) {
     constexpr int NT = 64 * WM * WN;
     constexpr int BM = WM * NBM * 32;
     constexpr int BN = WN * NBN * 32;
@@ -569,9 +584,7 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     constexpr int NCHB = TB::kChunks / NT;
     static_assert(TA::kChunks % NT == 0 && TB::kChunks % NT == 0, "tile must divide over the threads");
     static_assert(BK % 8 == 0, "BK must hold whole groups of 8 k");
-
-    __shared__ __attribute__((aligned(16))) float lds_a[2][TA::kFloats];
-    __shared__ __attribute__((aligned(16))) float lds_b[2][TB::kFloats];
+    static_assert(!AMASK || (PIPE == 0 && !EDGE), "the masked A operand exists for whole tiles on the simple schedule");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -582,11 +595,10 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     const int wn0 = (wave % WN) * (NBN * 32);
 
     int tm, tn;
-    tile_of_block(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    tile_of_block(bid, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
     const int m0 = tm * BM;
     const int n0 = tn * BN;
 
-    const int z = blockIdx.z;
     const int zq = z / p.bdiv, zr = z % p.bdiv;
     const float* __restrict__ Ab = p.A + zq * p.a_bs0 + zr * p.a_bs1 + (int64_t)m0 * p.a_rs;
     const float* __restrict__ Bb = p.B + zq * p.b_bs0 + zr * p.b_bs1 + (int64_t)n0 * p.b_rs;
@@ -615,6 +627,7 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     const bool do_rowsum = ROWSUM && p.rowsum != nullptr && tn == 0 && z == 0 && tid < BM;
     float rowsum = 0.f;
     f32x4 rax[DEPTH][NCHA], rbx[DEPTH][NCHB];
+    f32x4 rax2[AMASK ? DEPTH : 1][NCHA];   // AMASK: the pre-activation tile that belongs to rax
     f32x4(&ra)[NCHA] = rax[0];
     f32x4(&rb)[NCHB] = rbx[0];
     // reduction length of this workgroup
@@ -658,6 +671,11 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     const __amdgpu_buffer_rsrc_t rsrc_b =
         RAGGED_PIPE ? edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Bb)), p.b_rs, p.b_ks, p.N - n0, p.K, 0)
                     : __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Bb), 0, (int)0xFFFFFFFFu, 0x00020000);
+    // AMASK: the second tensor behind the A operand, addressed exactly like A
+    const bool a_masked = AMASK && p.a_mask != 0;
+    const __amdgpu_buffer_rsrc_t rsrc_a2 = __builtin_amdgcn_make_buffer_rsrc(
+        uniform_ptr(a_masked ? p.A2 + (Ab - p.A) : Ab), 0, (int)0xFFFFFFFFu, 0x00020000);
+    const float a_mask_slope = (AMASK && p.a_mask == 2 && p.leaky) ? *p.leaky : 0.f;
 
     if (PIPE == 0) {
         // The whole loop exists once per combination of 128-bit / element-wise loads of A and B.  The
@@ -676,6 +694,26 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
                 a_base = reinterpret_cast<uint64_t>(uniform_ptr(Ab));
                 b_base = reinterpret_cast<uint64_t>(uniform_ptr(Bb));
             }
+            // AMASK: da2 receives the pre-activation tile that goes with da; amask_tile turns da into
+            // da * f'(da2) when the tile leaves the staging registers
+            auto load_a2 = [&](int kt, f32x4(&da2)[NCHA]) {
+                if constexpr (AMASK) {
+                    const int k0 = min(kt, nkt - 1) * BK;
+#pragma unroll
+                    for (int i = 0; i < NCHA; i++)
+                        load_tile_chunk_buf<A_KC, BM, BK, NT>(da2, rsrc_a2, k0 * (int)p.a_ks * 4, (int)a_ld * 4, (int)toff_a * 4, i);
+                }
+            };
+            auto amask_tile = [&](f32x4(&da)[NCHA], const f32x4(&da2)[NCHA]) {
+                if constexpr (AMASK) {
+                    if (a_masked) {   // uniform
+#pragma unroll
+                        for (int i = 0; i < NCHA; i++)
+#pragma unroll
+                            for (int j = 0; j < 4; j++) da[i][j] = ((da2[i][j] > 0) ? 1.0f : a_mask_slope) * da[i][j];
+                    }
+                }
+            };
             auto load_into = [&](int kt, f32x4(&da)[NCHA], f32x4(&db)[NCHB]) {
                 const int ktc = min(kt, nkt - 1);
                 const int k0 = ktc * BK;
@@ -709,11 +747,16 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
             static_for<0, DEPTH>([&](auto dc) {
                 constexpr int d = decltype(dc)::value;
                 load_into(d, rax[d], rbx[d]);
+                load_a2(d, rax2[AMASK ? d : 0]);
             });
             mask_tile(0, ra, rb);
+            amask_tile(ra, rax2[0]);
             store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
             store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
-            if (DEPTH > 1) load_into(DEPTH, ra, rb);
+            if (DEPTH > 1) {
+                load_into(DEPTH, ra, rb);
+                load_a2(DEPTH, rax2[0]);
+            }
             __syncthreads();
 
             // At the top of tile kt: LDS[kt & 1] holds tile kt; slot (kt + j) % DEPTH holds tile kt + j for
@@ -723,7 +766,10 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
                 constexpr int d = decltype(dc)::value;
                 constexpr int nslot = (d + 1) % DEPTH;
                 const int cur = kt & 1;
-                if (DEPTH == 1) load_into(kt + 1, ra, rb);
+                if (DEPTH == 1) {
+                    load_into(kt + 1, ra, rb);
+                    load_a2(kt + 1, rax2[0]);
+                }
                 // With DEPTH > 1 the next tile has been in registers for a while: it goes to the free LDS
                 // buffer first, so that the store's latency runs under this tile's MFMAs instead of between
                 // them and the barrier.  (Every wave left that buffer before the last barrier.)  In the main
@@ -732,10 +778,14 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
                 auto store_next = [&]() {
                     if (!last_tiles || kt + 1 < nkt) {
                         mask_tile(kt + 1, rax[nslot], rbx[nslot]);
+                        amask_tile(rax[nslot], rax2[AMASK ? nslot : 0]);
                         store_tile_lds<A_KC, BM, BK, NT>(lds_a[cur ^ 1], rax[nslot], tid);
                         store_tile_lds<B_KC, BN, BK, NT>(lds_b[cur ^ 1], rbx[nslot], tid);
                     }
-                    if (DEPTH > 1) load_into(kt + 1 + DEPTH, rax[nslot], rbx[nslot]);
+                    if (DEPTH > 1) {
+                        load_into(kt + 1 + DEPTH, rax[nslot], rbx[nslot]);
+                        load_a2(kt + 1 + DEPTH, rax2[AMASK ? nslot : 0]);
+                    }
                 };
                 if (DEPTH > 1) store_next();
                 const float* la = lds_a[cur];
@@ -929,6 +979,15 @@ __global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const Gem
     const float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
     const float leaky = p.leaky ? *p.leaky : 0.f;
     gemm_epilogue<NBM, NBN, A_KC, B_KC>(p, acc, m0, n0, c_off, wm0, wn0, l32, half, alpha, leaky);
+}
+
+template <int WM, int WN, int NBM, int NBN, int BK, bool A_KC, bool B_KC, bool EDGE, int PIPE = 0, int MINW = 1,
+          int DEPTH = 1, bool ROWSUM = false>
+__global__ void __launch_bounds__(64 * WM * WN, MINW) gemm_mfma_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) float lds_a[2][TileShape<A_KC, WM * NBM * 32, BK>::kFloats];
+    __shared__ __attribute__((aligned(16))) float lds_b[2][TileShape<B_KC, WN * NBN * 32, BK>::kFloats];
+    gemm_tile_body<WM, WN, NBM, NBN, BK, A_KC, B_KC, EDGE, PIPE, DEPTH, ROWSUM, false>(p, blockIdx.x, blockIdx.z, lds_a,
+                                                                                       lds_b);
 }
 
 }  // namespace kai

@@ -591,18 +591,36 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
     KAI_REQUIRE_DIM(yvec); KAI_REQUIRE_DIM(ndat); KAI_REQUIRE_DIM(xvec);
     KAI_REQUIRE(act_is_elementwise(actFunc), KAI_ERR_CONDITIONAL_STATEMENT, "activation code must be 0..8");
     KAI_REQUIRE_PTR(pgy);
+    if (pgx) KAI_REQUIRE_PTR(pw);
+    if (pgw && yvec > 0 && xvec > 0) KAI_REQUIRE_PTR(px);
+    const bool has_act = actFunc != KAI_ACT_NONE && ppre != nullptr;
+    // a mini-batch step's sizes: both products, the activation's derivative and the bias gradient in ONE
+    // launch (dense_backward.hip), plus the sum of the parts when gx's reduction is cut
+    const int pair_split = dense_backward_pair_split(pgx, pgw, pgy, pw, px, has_act ? ppre : nullptr, yvec, ndat, xvec,
+                                                     has_act ? actFunc : KAI_ACT_NONE);
+    if (pair_split > 0)
+        return launch_dense_backward_pair(pgx, pgw, pgb, pgy, pw, px, has_act ? ppre : nullptr, yvec, ndat, xvec,
+                                          has_act ? actFunc : KAI_ACT_NONE, hLeakyAlpha, acc != 0, pair_split,
+                                          current_stream());
+    // otherwise the separate calls.  ga = gy * f'(pre) goes to the caller's work buffer, or, without one, to
+    // the library scratch (the products below may ask for scratch of their own: it is placed behind ga)
     const float* ga = pgy;
-    if (actFunc != KAI_ACT_NONE && ppre != nullptr) {
-        KAI_REQUIRE(pga_work != nullptr, KAI_ERR_INVALID_POINTER, "pga_work is required when an activation is applied");
-        KAI_TRY(launch_activate_backward(pga_work, pgy, ppre, ndat * yvec, actFunc, hLeakyAlpha, current_stream()));
-        ga = pga_work;
+    int64_t held_bytes = 0;
+    if (has_act && ndat > 0 && yvec > 0) {
+        float* work = pga_work;
+        if (work == nullptr) {
+            held_bytes = ndat * yvec * (int64_t)sizeof(float);
+            KAI_TRY(workspace(held_bytes, &work));
+        }
+        KAI_TRY(launch_activate_backward(work, pgy, ppre, ndat * yvec, actFunc, hLeakyAlpha, current_stream()));
+        ga = work;
     }
+    ScratchHold held(held_bytes);
     // gw[yvec,xvec] = ga^T . x reads every element of ga; where that product runs on the medium or small
     // tile its first tile column also produces gb = column sums of ga, in the order of a sequential loop
     GemmDesc dw;
     bool fused_gb = false;
     if (pgw && yvec > 0 && xvec > 0) {
-        KAI_REQUIRE_PTR(px);
         dw.A = ga; dw.B = px; dw.C = pgw;
         dw.M = yvec; dw.N = xvec; dw.K = ndat;
         dw.a_rs = 1; dw.a_ks = yvec; dw.b_rs = 1; dw.b_ks = xvec; dw.c_rs = xvec; dw.c_cs = 1;
@@ -614,10 +632,7 @@ int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pg
         }
     }
     if (pgb && !fused_gb) KAI_TRY(kai_add_bias_backward_b(device, pgb, ga, ndat, yvec, acc));
-    if (pgx) {
-        KAI_REQUIRE_PTR(pw);
-        KAI_TRY(kai_matmul_backward_x(device, pgx, ga, pw, yvec, ndat, xvec, acc));
-    }
+    if (pgx) KAI_TRY(kai_matmul_backward_x(device, pgx, ga, pw, yvec, ndat, xvec, acc));
     if (pgw && yvec > 0 && xvec > 0) KAI_TRY(launch_gemm(dw, current_stream()));
     return KAI_OK;
 }

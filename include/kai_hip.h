@@ -220,9 +220,13 @@ int kai_dense_forward(int device, float* py, float* ppre, const float* pw, const
                       int64_t yvec, int64_t ndat, int64_t xvec, int actFunc, const float* hLeakyAlpha);
 
 /* Backward of the same layer: ga = activate_backward(gy, ppre) (skipped when ppre is null or
- * actFunc == 0), then gb = colsum(ga), gx = ga . w, gw = ga^T . x.  Any of pgx, pgw, pgb may be
- * null.  pga_work is a caller buffer of ndat*yvec floats for ga (required when an activation is
- * applied; may equal pgy to overwrite it). */
+ * actFunc == 0), then gb = colsum(ga), gx = ga . w, gw = ga^T . x: the calls of VTensor::activate_backprop,
+ * add_backprop and matmul_backprop (vtensor.cpp:5697-5718, 3470-3479, 1337-1375).  Any of pgx, pgw, pgb may
+ * be null.  For none / relu / leaky relu, whole 64 x 64 x 32 tiles, 16-byte aligned operands and the sizes of a
+ * mini-batch step (both products together at most four workgroups per compute unit) everything runs in ONE
+ * launch, ga never written anywhere (plus a second launch that sums the parts of gx when its reduction is cut);
+ * other shapes run the separate kernels with ga in pga_work, a caller buffer of ndat*yvec floats (may equal pgy
+ * to overwrite it) or, when pga_work is null, in the library's scratch memory. */
 int kai_dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pga_work, const float* pgy,
                        const float* pw, const float* px, const float* ppre, int64_t yvec, int64_t ndat,
                        int64_t xvec, int actFunc, const float* hLeakyAlpha, int acc);

@@ -129,6 +129,58 @@ def test_dense_backward_bias_gradient_fused_or_not(ndat, yvec, xvec, acc):
     check(gb.to_numpy((yvec,)), ko.add_bias_backward_b(gy, yvec, **a), what="db")
 
 
+# The whole backward of a dense layer through kai_dense_backward with an activation and NO work buffer: shapes that
+# run as one launch (both products, the derivative of relu / leaky relu on the loads, the bias gradient from the
+# staged tiles; gx's reduction whole or cut into parts) and shapes that run the separate kernels with ga in the
+# library scratch.  The bias gradient sums in the order of a sequential loop: bit-identical to the oracle.
+@pytest.mark.parametrize("ndat,yvec,xvec,act,acc,one_launch", [
+    (256, 1024, 1024, "relu", False, True),      # configuration 2: gx cut into 4 parts of 256 steps
+    (256, 1024, 1024, "leaky", True, True),
+    (64, 512, 128, "relu", True, True),          # gx cut into 4 parts of 128
+    (128, 256, 320, "none", False, True),        # two parts of 128
+    (512, 512, 512, "leaky", False, True),       # no cut: a part would be shorter than gw's reduction
+    (1024, 1024, 1024, "relu", False, True),     # 512 workgroups, no cut
+    (64, 2048, 64, "relu", True, True),          # one tile of gx, 16 parts
+    (192, 1024, 1024, "relu", False, False),      # separate kernels from here on: 192 is no whole number of 64s
+    (100, 130, 70, "leaky", True, False),
+    (2048, 2048, 1024, "relu", False, False),     # too many workgroups for the paired launch
+    (256, 1024, 1024, "gelu", False, False),      # a derivative that is no select
+])
+def test_dense_backward_with_activation_and_no_work_buffer(ndat, yvec, xvec, act, acc, one_launch):
+    rng = np.random.default_rng(ndat + 3 * yvec + 7 * xvec + len(act))
+    x = rng.standard_normal((ndat, xvec)).astype(np.float32)
+    w = rng.uniform(-0.1, 0.1, (yvec, xvec)).astype(np.float32)
+    pre = rng.standard_normal((ndat, yvec)).astype(np.float32)
+    pre[0, :7] = [0.0, -0.0, np.nan, np.inf, -np.inf, 1e-30, -1e-30][:min(7, yvec)]
+    gy = rng.standard_normal((ndat, yvec)).astype(np.float32)
+    gx0 = rng.standard_normal((ndat, xvec)).astype(np.float32)
+    gw0 = rng.standard_normal((yvec, xvec)).astype(np.float32)
+    gb0 = rng.standard_normal(yvec).astype(np.float32)
+    alpha = 0.1 if act == "leaky" else None
+    if act == "gelu":
+        pre[0, 2:5] = 0.5                                   # keep the transcendental derivative finite
+    ga = gy if act == "none" else ko.activate_backward(gy, pre, act, alpha)
+    a = lambda base: dict(acc_into=base) if acc else {}
+    want_gx = ko.matmul_backward_x(ga, w, **a(gx0))
+    want_gw = ko.matmul_backward_w(ga, x, yvec, xvec, **a(gw0))
+    want_gb = ko.add_bias_backward_b(ga, yvec, **a(gb0))
+    gx, gw, gb = dev(gx0), dev(gw0), dev(gb0)
+    dgy, dpre = dev(gy), dev(pre)
+    VMath.dense_backward(0, gx, gw, gb, None, dgy, dev(w), dev(x), dpre, yvec, ndat, xvec, kai.ACT[act], kai.hyper(alpha), acc)
+    what = "dense backward %dx%dx%d %s acc=%s " % (ndat, yvec, xvec, act, acc)
+    check(gx.to_numpy((ndat, xvec)), want_gx, what=what + "dX")
+    check(gw.to_numpy((yvec, xvec)), want_gw, what=what + "dW")
+    got_gb = gb.to_numpy((yvec,))
+    check(got_gb, want_gb, what=what + "db")
+    if one_launch:      # summed in the order of a sequential loop (the separate column-sum kernel folds in a tree)
+        np.testing.assert_array_equal(got_gb, want_gb, err_msg=what + "db bit for bit")
+    np.testing.assert_array_equal(dgy.to_numpy(gy.shape), gy)        # the inputs are read only
+    # only some of the outputs requested (separate kernels; same values)
+    gx2 = dev(gx0)
+    VMath.dense_backward(0, gx2, None, None, None, dgy, dev(w), dev(x), dpre, yvec, ndat, xvec, kai.ACT[act], kai.hyper(alpha), acc)
+    check(gx2.to_numpy((ndat, xvec)), want_gx, what=what + "dX alone")
+
+
 # ---- configuration 3: 8192^3 GEMM + bias + ReLU -------------------------------------------------------------
 
 def test_cfg3_large_gemm_bias_relu_row_sample():
