@@ -396,16 +396,19 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         v = cheap_act(v);
     };
 
+    // Row r of a lane's 16 accumulator rows lies dr(r) rows below its row 0, a compile-time number, so a row's
+    // offset in C is the lane's 64-bit offset of row 0 plus a wave-uniform product dr(r) * c_rs: no per-row
+    // address is kept in vector registers (sixteen 64-bit offsets next to 128 accumulators did not fit).
+    auto dr = [](int r) constexpr -> int { return (A_KC ? 1 : NBM) * (8 * (r >> 2) + (r & 3)); };
     static_for<0, NBM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        int rows[16];
-        int64_t rowbase[16], rowbase_c[16];
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            rows[r] = row_of(i, r);
-            rowbase[r] = (int64_t)rows[r] * p.c_rs;
-            rowbase_c[r] = (int64_t)(rows[r] < p.M ? rows[r] : p.M - 1) * p.c_rs;
-        }
+        const int row0 = row_of(i, 0);
+        const int64_t base0 = (int64_t)row0 * p.c_rs;
+        // where a load must not leave the matrix: rows past the end read the lane's row 0, or the last row
+        const int64_t base0_c = (int64_t)(row0 < p.M ? row0 : p.M - 1) * p.c_rs;
+        auto row_ok = [&](int r) -> bool { return row0 + dr(r) < p.M; };
+        auto rowoff = [&](int r) -> int64_t { return base0 + (int64_t)dr(r) * p.c_rs; };
+        auto rowoff_c = [&](int r) -> int64_t { return row_ok(r) ? rowoff(r) : base0_c; };
         if (vec_store) {
             // the NBN columns of a lane are adjacent in memory: one store of NBN floats per row
             constexpr int VW = (NBN == 2 || NBN == 4) ? NBN : 4;
@@ -428,7 +431,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             if (accf) {
                 vecw cin[16];
 #pragma unroll
-                for (int r = 0; r < 16; r++) cin[r] = *reinterpret_cast<const vecw*>(C + rowbase_c[r] + colc);
+                for (int r = 0; r < 16; r++) cin[r] = *reinterpret_cast<const vecw*>(C + rowoff_c(r) + colc);
 #pragma unroll
                 for (int r = 0; r < 16; r++) o[r] += cin[r];
             }
@@ -440,7 +443,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             if (C2) {
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    if (rows[r] < p.M && col_ok) *reinterpret_cast<vecw*>(C2 + rowbase[r] + col) = o[r];
+                    if (row_ok(r) && col_ok) *reinterpret_cast<vecw*>(C2 + rowoff(r) + col) = o[r];
             }
             if (act != kActNone) {
 #pragma unroll
@@ -454,7 +457,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             }
 #pragma unroll
             for (int r = 0; r < 16; r++)
-                if (rows[r] < p.M && col_ok) *reinterpret_cast<vecw*>(C + rowbase[r] + col) = o[r];
+                if (row_ok(r) && col_ok) *reinterpret_cast<vecw*>(C + rowoff(r) + col) = o[r];
         } else {
             float v[NBN][16];
             int cols[NBN];
@@ -483,7 +486,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 #pragma unroll
                 for (int j = 0; j < NBN; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) cin[j][r] = C[rowbase_c[r] + coloff_c[j]];
+                    for (int r = 0; r < 16; r++) cin[j][r] = C[rowoff_c(r) + coloff_c[j]];
 #pragma unroll
                 for (int j = 0; j < NBN; j++)
 #pragma unroll
@@ -502,7 +505,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                 for (int j = 0; j < NBN; j++)
 #pragma unroll
                     for (int r = 0; r < 16; r++)
-                        if (rows[r] < p.M && cols[j] < p.N) C2[rowbase[r] + coloff[j]] = v[j][r];
+                        if (row_ok(r) && cols[j] < p.N) C2[rowoff(r) + coloff[j]] = v[j][r];
             }
             if (act != kActNone) {
 #pragma unroll
@@ -514,7 +517,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             for (int j = 0; j < NBN; j++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    if (rows[r] < p.M && cols[j] < p.N) C[rowbase[r] + coloff[j]] = v[j][r];
+                    if (row_ok(r) && cols[j] < p.N) C[rowoff(r) + coloff[j]] = v[j][r];
         }
     });
 
