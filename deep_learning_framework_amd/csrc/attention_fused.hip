@@ -256,7 +256,10 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
 
 bool attention_fused_applies(const float* q, const float* k, const float* v, const float* o, int64_t ntimes,
                              int64_t nvec, int64_t nhead, int64_t npiece) {
-    return (npiece == 16 || npiece == 32 || npiece == 64) && nvec % 4 == 0 && ntimes >= 1 && ntimes <= kMaxDim &&
+    // the kernel writes its output with the row stride of the inputs; the output of the separate calls is
+    // [nbat, ntimes, nhead, npiece], which is the same thing only when the heads fill the vector
+    return nhead * npiece == nvec &&
+           (npiece == 16 || npiece == 32 || npiece == 64) && nvec % 4 == 0 && ntimes >= 1 && ntimes <= kMaxDim &&
            ntimes * nvec * 4 < (1ll << 31) &&
            nhead >= 1 && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o);
 }

@@ -714,6 +714,24 @@ def test_attention_forward_fused(nbat, ntimes, nhead, npiece, masked):
     check(o.to_numpy((nbat, ntimes, nvec)), ref, what="fused attention")
 
 
+def test_attention_forward_when_the_heads_do_not_fill_the_vector():
+    # nhead * npiece < nvec: the engine never does this, the interface allows it.  The output is the compact
+    # [nbat, ntimes, nhead, npiece] of mix_values whatever the head size (the one-launch kernel steps aside).
+    nbat, ntimes, nvec, nhead = 2, 70, 80, 2
+    for npiece in (32, 24):
+        rng = np.random.default_rng(npiece)
+        q, k, v = (rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32) for _ in range(3))
+        coef = 1.0 / np.sqrt(npiece)
+        used = slice(0, nhead * npiece)
+        # the oracle on the used part of the vectors, packed: same values, compact layout
+        qc, kc, vc = (np.ascontiguousarray(t[:, :, used]) for t in (q, k, v))
+        probs = ko.softmax_direct_on_axis(ko.mult_on_heads(kc, qc, nhead, coef), nbat * ntimes, ntimes, nhead)
+        ref = ko.mix_values(probs, vc, nhead)
+        o = DB(nbat * ntimes * nhead * npiece * 4)
+        VMath.attention_forward(0, o, dev(q), dev(k), dev(v), nbat, ntimes, nvec, nhead, npiece, kai.hyper(coef), False)
+        check(o.to_numpy((nbat, ntimes, nhead * npiece)), ref, what="attention, heads of %d in vectors of %d" % (npiece, nvec))
+
+
 @pytest.mark.parametrize("nrow,nvec,ncol", SOFTMAX_AXIS_SHAPES)
 def test_softmax_axis_layouts(nrow, nvec, ncol):
     rng = np.random.default_rng(nrow + nvec + ncol)
