@@ -687,7 +687,9 @@ def test_cfg4_attention_backward(nbat, nhead, nvec):
 # LDS (long axis, odd lengths), one thread per head (more than 128 heads)
 SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8), (3, 20, 128), (2, 9, 129),
                        (2, 5, 300), (300, 512, 1), (3, 2048, 1), (2, 2052, 1), (2, 700, 8), (1, 2000, 8),
-                       (2, 1030, 2), (40, 64, 16)]
+                       (2, 1030, 2), (40, 64, 16),
+                       # many rows with 4, 8, 16 or 128 heads: a whole head-interleaved row per wave
+                       (1100, 33, 8), (2048, 512, 8), (1030, 100, 4), (1200, 30, 128), (1024, 1024, 4), (1500, 7, 16)]
 
 
 # fused forward attention against the oracle's four separate steps: both cfg4 mappings, ragged lengths, the three
@@ -741,7 +743,7 @@ def test_softmax_axis_layouts(nrow, nvec, ncol):
     check(d.to_numpy(s.shape), ko.softmax_direct_on_axis(s, nrow, nvec, ncol), what="softmax axis")
 
 
-@pytest.mark.parametrize("nbat,ntimes,nhead", [(3, 512, 1), (1, 512, 8), (2, 700, 8), (1, 2000, 4), (1, 300, 130),
+@pytest.mark.parametrize("nbat,ntimes,nhead", [(3, 512, 1), (1, 512, 8), (2, 700, 8), (1, 2000, 4), (1, 300, 130), (3, 400, 4), (9, 130, 16),
                                                (2, 2052, 1)])
 def test_softmax_axis_backward_layouts(nbat, ntimes, nhead):
     rng = np.random.default_rng(nbat + ntimes + nhead)
