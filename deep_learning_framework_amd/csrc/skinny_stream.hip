@@ -55,6 +55,14 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 
 // What the first loads need comes as scalars (14 dwords): this file is compiled with kernel-argument preload, so
 // a wave finds them in SGPRs at its start instead of fetching the argument buffer first.
+//
+// WHOLE: N is a multiple of 16 and K of 32 (every tile of W lies inside the matrix).  The tiles then come through
+// buffer loads: a resource over this workgroup's 16 rows of W and one over the M rows of X, a constant byte
+// offset per lane and a scalar offset per tile.  Nothing is clamped or masked (a row of X past M lies behind the
+// end of its resource and reads as zero), so a tile costs no vector instruction besides its LDS accesses and
+// MFMAs: in the general variant the clamps, 64-bit addresses and masks of a tile were more issue cycles than its
+// eight MFMAs.
+template <bool WHOLE>
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
@@ -81,7 +89,32 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     // One tile = 16 rows x kSsTileK k of W and of X, kSsLoadsPerTile 128-bit loads per lane each.  Addresses past
     // K are clamped into the row (every load is unconditional); what they return is zeroed on the way to LDS.
+    // WHOLE: resources and per-lane offsets (bytes)
+    auto uniform_ptr = [](const float* q) -> float* {
+        const uint64_t a = reinterpret_cast<uint64_t>(q);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
+    };
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        uniform_ptr(p.W + n0 * p.ldw), 0, (int)(((int64_t)15 * p.ldw + p.K) * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+        uniform_ptr(p.X), 0, (int)(((int64_t)(p.M - 1) * p.ldx + p.K) * 4), 0x00020000);
+    int woff[kSsLoadsPerTile], xoff[kSsLoadsPerTile];
+#pragma unroll
+    for (int j = 0; j < kSsLoadsPerTile; j++) {
+        woff[j] = (int)(((int64_t)(kSsRowsPerLoad * j + lrow) * p.ldw + lk) * 4);
+        // a row past M must land behind the end of the resource whatever ldx is: the last row's end is the limit
+        const int m = kSsRowsPerLoad * j + lrow;
+        xoff[j] = m < p.M ? (int)(((int64_t)m * p.ldx + lk) * 4) : 0x7FFFFFF0;
+    }
     auto load_w = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
+        if constexpr (WHOLE) {
+#pragma unroll
+            for (int j = 0; j < kSsLoadsPerTile; j++)   // aux 2: non-temporal, as the general variant's loads
+                dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff[j], kt * 4, 2));
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < kSsLoadsPerTile; j++) {
             const int64_t n = n0 + kSsRowsPerLoad * j + lrow;
@@ -90,6 +123,13 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         }
     };
     auto load_x = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
+        if constexpr (WHOLE) {
+#pragma unroll
+            for (int j = 0; j < kSsLoadsPerTile; j++)
+                if (kSsRowsPerLoad * j < p.M)   // uniform
+                    dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, xoff[j], kt * 4, 0));
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < kSsLoadsPerTile; j++) {
             if (kSsRowsPerLoad * j < p.M) {   // uniform: these rows hold a row of X
@@ -103,9 +143,11 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
 #pragma unroll
             for (int j = 0; j < kSsLoadsPerTile; j++) {
                 const int row = kSsRowsPerLoad * j + lrow;
-                *reinterpret_cast<f32x4*>(tw + row * kSsTileStride + lk) = keep_if(w[j], n0 + row < p.N && kt + lk < p.K);
+                *reinterpret_cast<f32x4*>(tw + row * kSsTileStride + lk) =
+                    WHOLE ? w[j] : keep_if(w[j], n0 + row < p.N && kt + lk < p.K);
                 if (kSsRowsPerLoad * j < p.M)
-                    *reinterpret_cast<f32x4*>(tx + row * kSsTileStride + lk) = keep_if(x[j], row < p.M && kt + lk < p.K);
+                    *reinterpret_cast<f32x4*>(tx + row * kSsTileStride + lk) =
+                        WHOLE ? x[j] : keep_if(x[j], row < p.M && kt + lk < p.K);
             }
             __builtin_amdgcn_wave_barrier();   // LDS serves a wave's accesses in order; the compiler must too
 #pragma unroll
@@ -176,8 +218,15 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     const int64_t blocks = (p.N + 15) / 16;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
     const SkinnyTail t = skinny_tail(p);
-    skinny_stream_kernel<<<dim3((unsigned)blocks), dim3(kSsThreads), 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M,
-                                                                                  p.K, p.Y, t);
+    // whole tiles, and byte offsets inside a workgroup's 16 rows of W and inside X that fit 31 bits
+    const bool whole = p.N % 16 == 0 && p.K % kSsTileK == 0 && (15 * p.ldw + p.K) * 4 < (1ll << 31) &&
+                       ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
+    if (whole)
+        skinny_stream_kernel<true><<<dim3((unsigned)blocks), dim3(kSsThreads), 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N,
+                                                                                          p.M, p.K, p.Y, t);
+    else
+        skinny_stream_kernel<false><<<dim3((unsigned)blocks), dim3(kSsThreads), 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N,
+                                                                                           p.M, p.K, p.Y, t);
     return check_launch("skinny_stream_kernel");
 }
 
