@@ -166,3 +166,79 @@ def test_attention_random_geometries():
         assert rel_fro(gp.to_numpy(ps), ref_gp) <= REL_FRO_TOL, what + "gP"
         VMath.mult_on_heads_backward(0, g, dev(ref_gp), dev(k), nbat, T, nvec, nhead, npiece)
         assert rel_fro(g.to_numpy((nbat, T, nvec)), ko.mult_on_heads_backward(ref_gp, k, nhead)) <= REL_FRO_TOL, what + "gQ"
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_dense_backward_random_shapes(seed):
+    """kai_dense_backward over random layer sizes, activations, acc and subsets of the outputs: multiples of 64 (the
+    one-launch kernel, with gx's reduction whole or cut) mixed with ragged sizes (the separate kernels)."""
+    kai, DB, VMath = _kai()
+    rng = np.random.default_rng(seed)
+    sizes = [64, 64, 128, 192, 256, 320, 512, 576, 1024, 100, 37, 130, 1000]
+    for it in range(14):
+        ndat, yvec, xvec = (int(rng.choice(sizes)) for _ in range(3))
+        while ndat * yvec * xvec > 6e7:                       # keeps the oracle's scalar loops to a second
+            if yvec > 64:
+                yvec //= 2
+            elif ndat > 64:
+                ndat //= 2
+            else:
+                xvec //= 2
+        act = str(rng.choice(["none", "relu", "leaky", "relu", "sigmoid"]))
+        acc = bool(rng.integers(0, 2))
+        alpha = float(rng.choice([0.1, 0.3])) if act == "leaky" else None
+        x = rng.standard_normal((ndat, xvec)).astype(np.float32)
+        w = rng.uniform(-0.1, 0.1, (yvec, xvec)).astype(np.float32)
+        pre = rng.standard_normal((ndat, yvec)).astype(np.float32)
+        gy = rng.standard_normal((ndat, yvec)).astype(np.float32)
+        gx0, gw0, gb0 = (rng.standard_normal(s).astype(np.float32) for s in ((ndat, xvec), (yvec, xvec), (yvec,)))
+        ga = gy if act == "none" else ko.activate_backward(gy, pre, act, alpha)
+        a = lambda base: dict(acc_into=base) if acc else {}
+        want = {"gx": ko.matmul_backward_x(ga, w, **a(gx0)), "gw": ko.matmul_backward_w(ga, x, yvec, xvec, **a(gw0)),
+                "gb": ko.add_bias_backward_b(ga, yvec, **a(gb0))}
+        ask = {"gx": True, "gw": True, "gb": bool(rng.integers(0, 4))} if it % 3 else \
+              {k: bool(rng.integers(0, 2)) for k in ("gx", "gw", "gb")}
+        bufs = {"gx": DB.from_numpy(gx0), "gw": DB.from_numpy(gw0), "gb": DB.from_numpy(gb0)}
+        work = DB(ndat * yvec * 4) if rng.integers(0, 2) else None
+        VMath.dense_backward(0, bufs["gx"] if ask["gx"] else None, bufs["gw"] if ask["gw"] else None,
+                             bufs["gb"] if ask["gb"] else None, work, DB.from_numpy(gy), DB.from_numpy(w), DB.from_numpy(x),
+                             DB.from_numpy(pre), yvec, ndat, xvec, kai.ACT[act], kai.hyper(alpha), acc)
+        what = "seed %d case %d: %dx%dx%d %s acc=%s ask=%s work=%s" % (seed, it, ndat, yvec, xvec, act, acc, ask, work is not None)
+        for name, shape, start in (("gx", (ndat, xvec), gx0), ("gw", (yvec, xvec), gw0), ("gb", (yvec,), gb0)):
+            got = bufs[name].to_numpy(shape)
+            if ask[name]:
+                assert np.isfinite(got).all(), what + " " + name
+                assert rel_fro(got, want[name]) <= REL_FRO_TOL, "%s %s: %.3e" % (what, name, rel_fro(got, want[name]))
+            else:
+                np.testing.assert_array_equal(got, start, err_msg=what + " " + name + " must stay untouched")
+
+
+def test_skinny_whole_tile_shapes_random():
+    """At most 16 rows against weight matrices whose sides are whole tiles of the streaming kernel (N % 16 == 0,
+    K % 32 == 0) and just beside them, with padded rows, bias, activation and acc."""
+    kai, DB, VMath = _kai()
+    rng = np.random.default_rng(31)
+    for it in range(16):
+        m = int(rng.integers(1, 17))
+        n = int(rng.choice([256, 272, 1024, 4096, 4112, 1000]))
+        k = int(rng.choice([64, 96, 512, 1056, 4096, 4128, 1000]))
+        padw, padx = int(rng.choice([0, 0, 4, 32])), int(rng.choice([0, 0, 4]))
+        w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        wp = np.full((n, k + padw), np.nan, np.float32); wp[:, :k] = w
+        xp = np.full((m, k + padx), np.nan, np.float32); xp[:, :k] = x
+        bias = rng.standard_normal(n).astype(np.float32)
+        y0 = rng.standard_normal((m, n)).astype(np.float32)
+        acc, use_bias, act = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), str(rng.choice(["none", "relu", "tanh"]))
+        y = DB.from_numpy(y0)
+        # B stored [N, K] (transB), lda / ldb carry the padding
+        VMath.gemm_f32(0, 0, 1, m, n, k, DB.from_numpy(xp), k + padx, DB.from_numpy(wp), k + padw, y, n,
+                       DB.from_numpy(bias) if use_bias else None, kai.ACT[act], None, acc)
+        ref = ko.matmul(w, x, acc_into=y0 if acc else None)
+        if use_bias:
+            ref = ko.add_bias(ref, bias)
+        ref = ko.activate(ref, act)
+        got = y.to_numpy((m, n))
+        what = "case %d: %dx%dx%d pad %d/%d acc=%s bias=%s %s" % (it, m, n, k, padw, padx, acc, use_bias, act)
+        assert np.isfinite(got).all(), what
+        assert rel_fro(got, ref) <= REL_FRO_TOL, "%s: %.3e" % (what, rel_fro(got, ref))
