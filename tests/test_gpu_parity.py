@@ -209,6 +209,36 @@ def test_cfg3_large_gemm_bias_relu_row_sample():
     assert abs((got > 0).mean() - 0.5) < 0.01
 
 
+def test_cfg3_size_backward_products_sampled_and_adjoint():
+    """The backward pair at the size of configuration 3 (8192^3, the engine's NN and TN forms): sampled rows of dX
+    and sampled rows of dW against the oracle, and the adjoint identities <dY, X.W^T> = <dY.W, X> = <dY^T.X, W>
+    over the whole matrices (float64 sums), which tie the three products together at a size the oracle cannot
+    compute in full."""
+    n = 8192
+    rng = np.random.default_rng(33)
+    x = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    w = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    gy = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    dx, dw, dgy = dev(x), dev(w), dev(gy)
+    out = DB(n * n * 4)
+    VMath.matmul(0, out, dw, dx, n, n, n, False)
+    y = out.to_numpy((n, n))
+    VMath.matmul_backward_x(0, out, dgy, dw, n, n, n, False)
+    gx = out.to_numpy((n, n))
+    VMath.matmul_backward_w(0, out, dgy, dx, n, n, n, False)
+    gw = out.to_numpy((n, n))
+    rows = np.array([0, 4095, 4096, 8191] + list(rng.integers(0, n, 4)))
+    # dX rows are independent: gx[r] = gy[r] . w
+    check(gx[rows], ko.matmul_backward_x(gy[rows], w), what="8192^3 dX sampled rows")
+    # dW rows belong to columns of gy: gw[c] = sum_m gy[m, c] * x[m]
+    check(gw[rows], ko.matmul_backward_w(np.ascontiguousarray(gy[:, rows]), x, len(rows), n), what="8192^3 dW sampled rows")
+    check(y[rows], ko.matmul_rows(w, x, rows), what="8192^3 Y sampled rows")
+    dot = lambda a, b: float(np.einsum("ij,ij->", a, b, dtype=np.float64))
+    s_y, s_x, s_w = dot(gy, y), dot(gx, x), dot(gw, w)
+    scale = np.sqrt(dot(gy, gy) * dot(y, y))
+    assert abs(s_y - s_x) <= 1e-5 * scale and abs(s_y - s_w) <= 1e-5 * scale, (s_y, s_x, s_w, scale)
+
+
 # ---- configuration 4: attention batched matmul ---------------------------------------------------------------
 
 @pytest.mark.parametrize("nbat,nhead,nvec", [(32, 1, 64), (4, 8, 512)])
