@@ -110,9 +110,12 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     }
     auto load_w = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
         if constexpr (WHOLE) {
+            // a tile past the end of K (a wave's last slice may be short) re-reads the last whole tile instead of
+            // counting on the range check for the scalar part of the address; it is never consumed
+            const int kc = min(kt, p.K - kSsTileK) * 4;
 #pragma unroll
             for (int j = 0; j < kSsLoadsPerTile; j++)   // aux 2: non-temporal, as the general variant's loads
-                dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff[j], kt * 4, 2));
+                dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff[j], kc, 2));
             return;
         }
 #pragma unroll
@@ -124,10 +127,11 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     };
     auto load_x = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
         if constexpr (WHOLE) {
+            const int kc = min(kt, p.K - kSsTileK) * 4;
 #pragma unroll
             for (int j = 0; j < kSsLoadsPerTile; j++)
                 if (kSsRowsPerLoad * j < p.M)   // uniform
-                    dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, xoff[j], kt * 4, 0));
+                    dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, xoff[j], kc, 0));
             return;
         }
 #pragma unroll
