@@ -511,8 +511,10 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
         if (p.M == 1) return launch_gemv_rows(p, stream);
         // 3 and 4 rows: the streaming kernel once its workgroups (16 rows of W each) cover the chip (measured at
         // 4096 x 4096: 12.6 against 16.0 us, 11008 x 4096: 30 against 40; at 2048 x 8192, 128 workgroups:
-        // 19.8 against 15.3); 2 rows run as fast either way
-        if (p.M >= 3 && p.N >= 16 * (int64_t)compute_units() && skinny_stream_applies(p))
+        // 19.8 against 15.3); 2 rows: the streaming kernel where its slices are written out (K a multiple of 4096:
+        // 12.3 against 12.45 us at 4096 x 4096, 29.0 against 30.5 at 11008 x 4096), the slice kernel otherwise
+        // (4096 x 11008: 30.7 against 33.3)
+        if ((p.M >= 3 || p.K % 4096 == 0) && p.N >= 16 * (int64_t)compute_units() && skinny_stream_applies(p))
             return launch_skinny_stream(p, stream);
         if (p.M == 2) return launch_slice<2>(p, stream);
         if (p.M <= 4) return launch_slice<4>(p, stream);

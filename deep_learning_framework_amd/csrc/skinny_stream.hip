@@ -2,8 +2,8 @@
 //
 //   y[m,n] (=|+=) act( sum_k x[m,k] * w[n,k] + bias[n] ),   m < M <= 16
 //
-// A workgroup of eight waves owns 16 rows of W and all of K; wave w owns the slices of 512 reduction
-// steps number w, w+8, ...  Everything up to the final sum is private to a wave, so there is no
+// A workgroup of eight waves owns 16 rows of W and all of K; wave w owns a contiguous eighth of the tiles of
+// 32 reduction steps.  Everything up to the final sum is private to a wave, so there is no
 // barrier in the stream: a wave loads its slice tile by tile (16 x 32 of W and of X, one 128-byte
 // line per row and load; rows of X beyond M are not loaded), two tiles ahead of the tile it is
 // working on, and passes both through its own LDS tiles into the operand layout of
@@ -25,9 +25,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kSsWaves = 8;
 constexpr int kSsThreads = 64 * kSsWaves;
-constexpr int kSsSlice = 512;                 // reduction steps per wave and pass of the pipeline
 constexpr int kSsTileK = 32;                  // k per staged tile: one 128-byte line per row
-constexpr int kSsTiles = kSsSlice / kSsTileK; // tiles per slice
 constexpr int kSsRing = 3;                    // tiles of a wave in registers: one at work, the others on their way
 constexpr int kSsLanesPerRow = kSsTileK / 4;
 constexpr int kSsRowsPerLoad = 64 / kSsLanesPerRow;
@@ -62,7 +60,11 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // end of its resource and reads as zero), so a tile costs no vector instruction besides its LDS accesses and
 // MFMAs: in the general variant the clamps, 64-bit addresses and masks of a tile were more issue cycles than its
 // eight MFMAs.
-template <bool WHOLE>
+//
+// SLICES: K is a multiple of 8 x 512, so every wave owns the same number of slices of 512 steps and the tile loop
+// of a slice is written out (16 tiles, every wait counted exactly by the compiler): 12.2 us at M = 4 against
+// 12.9 us for the rolled loop that other lengths use.
+template <bool WHOLE, bool SLICES>
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
@@ -164,28 +166,66 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
             __builtin_amdgcn_wave_barrier();
         }
     };
-    // Software pipeline over the tiles of a slice: a ring of kSsRing tiles per wave, the loads of tile t + kSsRing
-    // issued as soon as tile t has left its registers, so the stream of a wave goes on while the wave passes a
-    // tile through LDS and the matrix core.  A deeper ring does not help: a wave that asks for more than the
-    // compute unit's memory pipeline takes at once stalls at the issue of its loads, in front of the tile that
-    // has long arrived.
-    for (int k0 = wave * kSsSlice; k0 < p.K; k0 += kSsWaves * kSsSlice) {
+    if constexpr (SLICES) {
+        // wave w owns the slices of 512 steps number w, w + 8, ...; per slice a ring of kSsRing tiles, the loads of
+        // tile t + kSsRing issued as soon as tile t has left its registers
+        constexpr int kSlice = 512, kTiles = kSlice / kSsTileK;
+        for (int k0 = wave * kSlice; k0 < p.K; k0 += kSsWaves * kSlice) {
+            f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kSsLoadsPerTile];
+            ss_static_for<0, kSsRing>([&](auto tc) {
+                constexpr int t = decltype(tc)::value;
+                load_w(w[t], k0 + t * kSsTileK);
+                load_x(x[t], k0 + t * kSsTileK);
+            });
+            ss_static_for<0, kTiles>([&](auto tc) {
+                constexpr int t = decltype(tc)::value;
+                constexpr int slot = t % kSsRing;
+                __builtin_amdgcn_sched_barrier(0);
+                consume(w[slot], x[slot], k0 + t * kSsTileK);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (t + kSsRing < kTiles) {
+                    load_w(w[slot], k0 + (t + kSsRing) * kSsTileK);
+                    load_x(x[slot], k0 + (t + kSsRing) * kSsTileK);
+                }
+            });
+        }
+    } else {
+        // Software pipeline over a wave's tiles: the tiles of K are dealt out evenly, wave w takes a contiguous run
+        // (one or two tiles' difference between waves whatever K is; fixed slices of 512 left some waves with three
+        // slices and others with two at K = 11008).  A ring of kSsRing tiles per wave, the loads of tile t + kSsRing
+        // issued as soon as tile t has left its registers, so the stream of a wave goes on while the wave passes a
+        // tile through LDS and the matrix core.  A deeper ring does not help: a wave that asks for more than the
+        // compute unit's memory pipeline takes at once stalls at the issue of its loads, in front of the tile that
+        // has long arrived.
+        const int tiles_total = (p.K + kSsTileK - 1) / kSsTileK;
+        const int tiles_base = tiles_total / kSsWaves, tiles_rem = tiles_total % kSsWaves;
+        const int t_count = tiles_base + (wave < tiles_rem ? 1 : 0);
+        const int k_begin = (wave * tiles_base + min(wave, tiles_rem)) * kSsTileK;
         f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kSsLoadsPerTile];
         ss_static_for<0, kSsRing>([&](auto tc) {
             constexpr int t = decltype(tc)::value;
-            load_w(w[t], k0 + t * kSsTileK);
-            load_x(x[t], k0 + t * kSsTileK);
+            load_w(w[t], k_begin + t * kSsTileK);
+            load_x(x[t], k_begin + t * kSsTileK);
         });
-        ss_static_for<0, kSsTiles>([&](auto tc) {
-            constexpr int t = decltype(tc)::value;
-            constexpr int slot = t % kSsRing;
-            __builtin_amdgcn_sched_barrier(0);
-            consume(w[slot], x[slot], k0 + t * kSsTileK);
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (t + kSsRing < kSsTiles) {
-                load_w(w[slot], k0 + (t + kSsRing) * kSsTileK);
-                load_x(x[slot], k0 + (t + kSsRing) * kSsTileK);
-            }
+        // Whole rounds of the ring that every wave of the workgroup has: no condition inside the loop, so the
+        // compiler counts the loads in flight exactly across the back edge (with a condition around a tile it
+        // waited for every load once per round: 12.2 -> 14.4 us at M = 4).  At most kSsRing tiles follow.
+        const int rounds = tiles_base / kSsRing;
+        for (int r = 0; r < rounds; r++) {
+            ss_static_for<0, kSsRing>([&](auto sc) {
+                constexpr int slot = decltype(sc)::value;
+                const int kt = k_begin + (r * kSsRing + slot) * kSsTileK;
+                __builtin_amdgcn_sched_barrier(0);
+                consume(w[slot], x[slot], kt);
+                __builtin_amdgcn_sched_barrier(0);
+                load_w(w[slot], kt + kSsRing * kSsTileK);   // past the wave's run: surplus, clamped, never consumed
+                load_x(x[slot], kt + kSsRing * kSsTileK);
+            });
+        }
+        ss_static_for<0, kSsRing>([&](auto sc) {
+            constexpr int slot = decltype(sc)::value;
+            const int t = rounds * kSsRing + slot;
+            if (t < t_count) consume(w[slot], x[slot], k_begin + t * kSsTileK);   // uniform
         });
     }
 
@@ -225,12 +265,11 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     // whole tiles, and byte offsets inside a workgroup's 16 rows of W and inside X that fit 31 bits
     const bool whole = p.N % 16 == 0 && p.K % kSsTileK == 0 && (15 * p.ldw + p.K) * 4 < (1ll << 31) &&
                        ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
-    if (whole)
-        skinny_stream_kernel<true><<<dim3((unsigned)blocks), dim3(kSsThreads), 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N,
-                                                                                          p.M, p.K, p.Y, t);
-    else
-        skinny_stream_kernel<false><<<dim3((unsigned)blocks), dim3(kSsThreads), 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N,
-                                                                                           p.M, p.K, p.Y, t);
+    const bool slices = p.K % (kSsWaves * 512) == 0;
+    const dim3 grid((unsigned)blocks), block(kSsThreads);
+    if (whole && slices) skinny_stream_kernel<true, true><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (whole) skinny_stream_kernel<true, false><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else skinny_stream_kernel<false, false><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     return check_launch("skinny_stream_kernel");
 }
 
