@@ -686,10 +686,15 @@ __global__ void __launch_bounds__(kEwThreads) splitk_reduce_kernel(SplitReducePa
     }
 }
 
+// one thread per output element (or four of them): the grid covers the output, it is not capped like the
+// grids of the kernels above, which loop
 template <int NMAX>
 static int launch_splitk_reduce_n(const SplitReduceParams& p, bool vec, int64_t total, hipStream_t stream) {
-    if (vec) splitk_reduce_kernel<true, NMAX><<<blocks_for(total / 4), kEwThreads, 0, stream>>>(p);
-    else splitk_reduce_kernel<false, NMAX><<<blocks_for(total), kEwThreads, 0, stream>>>(p);
+    const int64_t items = vec ? total / 4 : total;
+    const int64_t blocks = (items + kEwThreads - 1) / kEwThreads;
+    if (blocks > 0x7fffffffll) return fail(KAI_ERR_INVALID_ARGUMENT, "split-K: output too large for one grid");
+    if (vec) splitk_reduce_kernel<true, NMAX><<<(unsigned)blocks, kEwThreads, 0, stream>>>(p);
+    else splitk_reduce_kernel<false, NMAX><<<(unsigned)blocks, kEwThreads, 0, stream>>>(p);
     return check_launch("splitk_reduce_kernel");
 }
 

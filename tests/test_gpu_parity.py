@@ -832,6 +832,35 @@ def test_split_k_scratch_survives_shutdown_and_growth():
     assert kai.scratch_info()[1] == n_growths and kai.scratch_info()[0] >= 48 << 20
 
 
+# products cut along K whose outputs are larger than one capped element-wise grid covers (4096 workgroups x 256
+# threads: 4 Mi outputs with 128-bit accesses, 1 Mi without): the pass that sums the parts covers all of them
+@pytest.mark.parametrize("m,n,k,bias_act", [(1152, 4096, 4096, False), (1280, 5120, 5120, True), (2047, 2049, 2051, False),
+                                            (1100, 1023, 3000, True)])
+def test_split_k_with_a_large_output(m, n, k, bias_act):
+    plan = VMath.gemm_plan(0, 1, m, n, k)
+    assert int(plan.rsplit(" ", 1)[1]) > 1, plan
+    rng = np.random.default_rng(m + n + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    y = DB(m * n * 4)
+    VMath.fill_float(0, y, m * n, 123.0)
+    if bias_act:
+        VMath.dense_forward(0, y, None, dev(w), dev(b), dev(x), n, m, k, kai.ACT["relu"], None)
+    else:
+        VMath.matmul(0, y, dev(w), dev(x), n, m, k, False)
+    got = y.to_numpy((m, n))
+    # sampled rows against the oracle (first, last and a spread in between), the whole output against float64
+    rows = sorted(set([0, 1, m // 2, m - 2, m - 1] + list(range(0, m, max(1, m // 24)))))
+    ref_rows = ko.matmul_rows(w, x, rows)
+    ref_all = x.astype(np.float64) @ w.astype(np.float64).T
+    if bias_act:
+        ref_rows = ko.activate(ko.add_bias(ref_rows, b), "relu")
+        ref_all = np.maximum(ref_all + b, 0.0)
+    check(got[rows], ref_rows, what="split-K %dx%dx%d sampled rows" % (m, n, k))
+    check(got, ref_all.astype(np.float32), what="split-K %dx%dx%d whole output" % (m, n, k))
+
+
 def test_scratch_growth_does_not_wait_for_the_device():
     # Growth allocates the larger buffer and keeps the old one: no device-wide wait, no free.  Shown by
     # queueing ~0.1 s of products, then issuing a call that makes the scratch grow: it returns while the queue
@@ -840,11 +869,12 @@ def test_scratch_growth_does_not_wait_for_the_device():
     rng = np.random.default_rng(5)
     n = 4096
     a, b, c = dev(rng.standard_normal((n, n)).astype(np.float32)), dev(rng.standard_normal((n, n)).astype(np.float32)), DB(n * n * 4)
-    m, nn, k = 1024, 1024, 8192                        # two parts of 1024 x 1024 sums: 8 MiB
-    assert VMath.gemm_plan(0, 1, m, nn, k).endswith("split 2")
-    x = rng.standard_normal((m, k)).astype(np.float32)
-    w = rng.uniform(-0.05, 0.05, (nn, k)).astype(np.float32)
-    dx, dw, y = dev(x), dev(w), DB(m * nn * 4)
+    m, nn, k = 1024, 1024, 4096                        # gx = gy . w, cut into parts: 8 MiB of partial sums
+    plan = VMath.gemm_plan(0, 0, m, nn, k)
+    assert int(plan.rsplit(" ", 1)[1]) * m * nn * 4 >= 8 << 20, plan
+    gy = rng.standard_normal((m, k)).astype(np.float32)
+    w = rng.uniform(-0.05, 0.05, (k, nn)).astype(np.float32)
+    dgy, dw, y = dev(gy), dev(w), DB(m * nn * 4)
     VMath.gemm_f32(0, 0, 0, n, n, n, a, n, b, n, c, n, None, 0, None, False)     # code objects loaded, clocks up
     kai.shutdown()
     kai.reserve_scratch(1 << 20)                       # the smallest buffer (4 MiB), which the product below outgrows
@@ -854,7 +884,7 @@ def test_scratch_growth_does_not_wait_for_the_device():
     for _ in range(100):                               # ~1 ms each
         VMath.gemm_f32(0, 0, 0, n, n, n, a, n, b, n, c, n, None, 0, None, False)
     t_queued = time.perf_counter()
-    VMath.matmul(0, y, dw, dx, nn, m, k, False)
+    VMath.matmul_backward_x(0, y, dgy, dw, k, m, nn, False)
     t_call = time.perf_counter()
     kai.synchronize()
     t_done = time.perf_counter()
@@ -863,7 +893,7 @@ def test_scratch_growth_does_not_wait_for_the_device():
           % ((t_queued - t0) * 1e3, (t_call - t_queued) * 1e3, (t_done - t_call) * 1e3, before, after))
     assert after[1] == before[1] + 1 and after[0] >= 8 << 20 and after[2] == before[0]
     rows = list(range(0, m, 32))
-    check(y.to_numpy((m, nn))[rows], ko.matmul_rows(w, x, rows), what="product after growth")
+    check(y.to_numpy((m, nn))[rows], ko.matmul_backward_x(gy[rows], w), what="product after growth")
     if (t_done - t_call) > 0.02:                       # the queue was still busy when the call returned
         assert (t_call - t_queued) < 0.5 * (t_done - t_call)
     else:
