@@ -81,6 +81,31 @@ int64_t small_tile_split(int64_t tiles, int64_t K, int64_t cus) {
     return best;
 }
 
+// Expected duration in microseconds of a single product of whole tiles on `tile` (small, wide or medium) with
+// the reduction cut into s equal parts, fitted to a sweep of 380 shapes (M 64..2048, N and K 512..4096, the
+// three operand forms, every tile and part count; the choice made from it is within 1 % of the best measured
+// one on average, 8 % at worst).  A workgroup takes a fixed time per 32 reduction steps whatever shares its
+// compute unit -- small 0.48 us on the pipelined schedule (both operands K-contiguous), 0.62 / 0.555 / 0.53 with
+// one / two / more workgroups per unit on the simple one, wide 0.95, medium 1.8 (two resident at most) -- so the
+// kernel takes rounds x steps x that, plus 3.5 us of launch, first loads and epilogue; the parts cost a second
+// launch (3.5 us + 0.1 per part) and their traffic (each part written and read once, at about 6 TB/s).
+double tiled_cost(int tile, bool both_kc, int64_t M, int64_t N, int64_t K, int64_t s, int64_t cus) {
+    const int64_t bm = tile == kTileMedium ? 128 : 64, bn = tile == kTileSmall ? 64 : 128;
+    const int64_t groups = (M / bm) * (N / bn) * s;
+    const int64_t per_cu = (groups + cus - 1) / cus;
+    const double steps = (double)K / (double)s / 32.0;
+    double t;
+    if (tile == kTileMedium) {
+        const double one = both_kc ? 1.79 : 1.86;
+        t = per_cu == 1 ? steps * one : steps * 1.02 * one * (double)(2 * (per_cu / 2)) + steps * one * (double)(per_cu % 2);
+    } else if (tile == kTileWide) {
+        t = (double)per_cu * steps * (both_kc ? 0.95 : 0.96);
+    } else {
+        t = (double)per_cu * steps * (both_kc ? 0.48 : per_cu == 1 ? 0.62 : per_cu == 2 ? 0.555 : 0.53);
+    }
+    return t + 3.5 + (s > 1 ? 3.5 + 0.1 * (double)s + (double)(2 * s + 1) * (double)(M * N) * 4.0 / 6.0e6 : 0.0);
+}
+
 GemmPlan plan_gemm(const GemmDesc& d) {
     GemmPlan plan;
     // skinny: y = x . w^T with both operands K-contiguous, a contiguous output row, no scaling
@@ -130,11 +155,42 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         if (best > 0 && best <= limit) plan.wavesplit_edge = take16 ? 16 : 32;
     }
 
+    // A single product of whole 64-wide tiles: tile and number of parts together, from the model above.  (The
+    // kernels of the wide tile and of the pipelined small tile exist for whole tiles only; everything else keeps
+    // the rules above and below.)
+    bool modelled = false;
+    if (!plan.skinny && !plan.wavesplit_edge && d.nbatch == 1 && (plan.tile == kTileSmall || plan.tile == kTileMedium) &&
+        d.M % 64 == 0 && d.N % 64 == 0 && d.K % 32 == 0 && !skinny_rows_applies(dn) && !shortk_nt_applies(dn)) {
+        const GemmParams pp = make_params(dn, plan.a_kc, plan.b_kc);
+        if (fits_without_edges(pp, plan.a_kc, plan.b_kc, 64, 64, 32) && fits_buffer_offsets(pp, plan.a_kc, plan.b_kc, 128, 128)) {
+            const bool both_kc = plan.a_kc && plan.b_kc;
+            double best = 0.0;
+            for (const int tile : {(int)kTileMedium, (int)kTileWide, (int)kTileSmall}) {   // on a tie the larger tile
+                if (tile != kTileSmall && d.N % 128 != 0) continue;
+                if (tile == kTileMedium && d.M % 128 != 0) continue;
+                for (int64_t sp = 1; sp <= kSplitMax; sp *= 2) {
+                    if (sp > 1 && (d.K < kSplitFromK || d.K % (32 * sp) != 0 || d.K / sp < 256 ||
+                                   sp * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax))
+                        break;
+                    const double c = tiled_cost(tile, both_kc, d.M, d.N, d.K, sp, cus);
+                    if (!modelled || c < 0.98 * best) {
+                        modelled = true;
+                        best = c;
+                        plan.tile = tile;
+                        plan.split = sp;
+                        plan.k_part = sp > 1 ? d.K / sp : 0;
+                        plan.ragged_parts = false;
+                    }
+                }
+            }
+        }
+    }
+
     // Split-K: a single product whose output tiles leave most compute units idle is cut along K
     // into `split` equal parts that run as the batch dimension of the same kernel and write raw
     // partial products to the library's scratch; a second launch sums them in a fixed order and
     // applies the epilogue.
-    if (!plan.skinny && d.nbatch == 1 && d.K >= kSplitFromK) {
+    if (!modelled && !plan.skinny && d.nbatch == 1 && d.K >= kSplitFromK) {
         const int64_t edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
         const int64_t tiles = plan.tile == kTileFlat ? ((d.M + 31) / 32) * ((d.N + 127) / 128) : tiles_of(d.M, d.N, 1, edge);
         int64_t split = compute_units() / tiles;
@@ -177,7 +233,7 @@ bool gemm_fuses_rowsum(const GemmDesc& d) {
     if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
     const GemmPlan plan = plan_gemm(d);
     return !plan.skinny && !plan.wavesplit_edge && !skinny_rows_applies(plan.dn) && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge &&
-           plan.tile != kTileFlat && plan.split == 1;
+           plan.tile != kTileFlat && plan.tile != kTileWide && plan.split == 1;
 }
 
 // What launch_gemm would do with this product, as text: the kernel family and, for the tiled kernel, tile,
@@ -204,19 +260,23 @@ std::string describe_gemm(const GemmDesc& d) {
     }
     const GemmParams p = make_params(dt, a_kc, b_kc);
     const int edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
+    const bool wide = plan.tile == kTileWide && fits_without_edges(p, a_kc, b_kc, 64, 128, 32) &&
+                      fits_buffer_offsets(p, a_kc, b_kc, 64, 128);   // else the small tile runs
     const char* tile = plan.tile == kTileLarge ? "large" : plan.tile == kTileMedium ? "medium" :
-                       plan.tile == kTileFlat ? "flat" : "small";
+                       plan.tile == kTileFlat ? "flat" : wide ? "wide" : "small";
     const char* variant = "general";
-    if (plan.tile == kTileFlat) {
+    if (wide) {
+        variant = "whole pipelined";
+    } else if (plan.tile == kTileFlat) {
         if (fits_without_edges(p, a_kc, b_kc, 32, 128, 32) && fits_buffer_offsets(p, a_kc, b_kc, 32, 128)) variant = "whole";
-    } else if (plan.tile != kTileSmall) {
+    } else if (plan.tile == kTileLarge || plan.tile == kTileMedium) {
         const int bk = plan.tile == kTileLarge ? 16 : 32;
         if (fits_without_edges(p, a_kc, b_kc, edge, edge, bk) && fits_buffer_offsets(p, a_kc, b_kc, edge, edge))
             variant = "whole pipelined";
         else if (fits_ragged_pipe(p, a_kc, b_kc, edge, edge)) variant = "ragged pipelined";
     } else if ((fits_without_edges(p, a_kc, b_kc, 64, 64, 32) || fits_without_edges(p, a_kc, b_kc, 64, 64, 16)) &&
                fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
-        variant = "whole";
+        variant = a_kc && b_kc && fits_without_edges(p, a_kc, b_kc, 64, 64, 32) ? "whole pipelined" : "whole";
     }
     return std::string("mfma ") + tile + " " + variant + " split " + std::to_string(plan.split);
 }

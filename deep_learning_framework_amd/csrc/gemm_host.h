@@ -151,7 +151,8 @@ int launch_dense_backward_pair(float* pgx, float* pgw, float* pgb, const float* 
                                const float* leaky, bool acc, int split, hipStream_t stream);
 
 // per-layout entry points (one translation unit each, to compile in parallel)
-enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2, kTileFlat = 3 };   // flat: 32 rows x 128 columns
+// flat: 32 rows x 128 columns; wide: 64 rows x 128 columns (whole tiles only, else the small tile runs)
+enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2, kTileFlat = 3, kTileWide = 4 };
 int launch_gemm_kc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
 int launch_gemm_kc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
 int launch_gemm_mc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);

@@ -5,10 +5,12 @@
 //   large  256x256 tile, 8 waves of 128x64 (2 waves per SIMD)  -- big, compute-bound products
 //   medium 128x128 tile, 4 waves of 64x64, 2 workgroups per CU -- fills the chip at mid sizes
 //   small   64x64  tile, 4 waves of 32x32                      -- small or very ragged products
+//   wide    64x128 tile, 4 waves of 32x64                      -- whole tiles, fewer workgroups than the small tile
 //   flat    32x128 tile, 4 waves of 32x32 side by side         -- at most 32 rows against many columns
 // On the two bigger tiles, operands that allow 128-bit loads run the pipelined kernel: predicate-free
 // when the shape is a whole multiple of the tile, else with range-checked buffer resources and one
-// masked K-tile at the end.  Everything else runs the general kernel with the simple schedule.
+// masked K-tile at the end.  The wide tile and, for two K-contiguous operands, whole small tiles run the
+// pipelined kernel too.  Everything else runs the general kernel with the simple schedule.
 #pragma once
 
 #include "gemm_host.h"
@@ -48,7 +50,18 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
         if (fits_without_edges(p, A_KC, B_KC, 32, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 32, 128))
             return launch_gemm_config<1, 4, 1, 1, 32, A_KC, B_KC, false, 0, 2, 4>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<1, 4, 1, 1, 32, A_KC, B_KC, true, 0, 1, 4>(p, nbatch, kGroupM, stream);
+    case kTileWide:
+        if (fits_without_edges(p, A_KC, B_KC, 64, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 128))
+            return launch_gemm_config<2, 2, 1, 2, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
+        [[fallthrough]];
     default:
+        // Both operands K-contiguous, whole tiles: the pipelined schedule (fragment reads and LDS stores dealt
+        // between the MFMAs) runs a 32-step tile in 0.48 us whether the workgroup has the compute unit to itself
+        // or not, the simple schedule below in 0.53-0.70 (1024^3: 22.6 -> 18.9 us, 512 x 2048 x 2048: 41.0 -> 34.2,
+        // 64 x 4096 x 4096: 27.2 -> 22.8).  With an operand that is not K-contiguous it gains nothing (its
+        // fragments take four LDS reads instead of one), so those keep the simple schedule.
+        if (A_KC && B_KC && fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
+            return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
         // a 64x64x16 tile computes for ~0.25 us, a global load takes ~1-2 us: 128 reduction steps in flight
         // (measured with whole tiles of 32 steps against 16 and 64: 15.5 / 16.9 / 16.0 us for 256x1024x1024)
         if (fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))

@@ -230,7 +230,7 @@ GEMM_PLANS = [
     ((0, 1, 4096, 4096, 4096), "mfma large whole pipelined split 1"),   # exactly one round of large tiles
     ((0, 1, 3072, 4096, 4096), "mfma medium whole pipelined split 1"),  # 192 large tiles leave a quarter of the chip idle
     ((0, 1, 2048, 2048, 2048), "mfma medium whole pipelined split 1"),
-    ((0, 1, 1024, 2048, 512), "mfma small whole split 1"),           # 128 medium tiles on 256 units: the finer tile
+    ((0, 1, 1024, 2048, 512), "mfma wide whole pipelined split 1"),           # 128 medium tiles on 256 units: the finer tile
     ((0, 1, 1, 4096, 4096), "skinny"),                               # configuration 5
     ((0, 1, 4, 4096, 4096), "skinny"),
     ((0, 1, 16, 4096, 4096), "skinny"),
@@ -245,11 +245,11 @@ GEMM_PLANS = [
     ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small general split 8"),
     ((0, 1, 96, 4096, 4096), "mfma flat whole split 8"),             # 65..96 rows: three row tiles of 32, not two of 64
-    ((0, 1, 64, 64, 8192), "mfma small whole split 16"),             # one tile, a long reduction
-    ((0, 1, 768, 768, 4096), "mfma small whole split 8"),            # K cut to fill the rounds
-    ((0, 1, 1024, 1024, 8192), "mfma small whole split 2"),          # K cut to bring a second workgroup onto each unit
-    ((0, 1, 1024, 1024, 1024), "mfma small whole split 1"),
-    ((0, 1, 128, 128, 4096), "mfma small whole split 8"),            # too long for the one-launch kernel
+    ((0, 1, 64, 64, 8192), "mfma small whole pipelined split 16"),             # one tile, a long reduction
+    ((0, 1, 768, 768, 4096), "mfma small whole pipelined split 8"),            # K cut to fill the rounds
+    ((0, 1, 1024, 1024, 8192), "mfma medium whole pipelined split 4"),          # K cut to bring a second workgroup onto each unit
+    ((0, 1, 1024, 1024, 1024), "mfma small whole pipelined split 1"),
+    ((0, 1, 128, 128, 4096), "mfma small whole pipelined split 16"),            # too long for the one-launch kernel
     ((0, 1, 0, 5, 5), "nothing"),
 ]
 
