@@ -81,29 +81,37 @@ int64_t small_tile_split(int64_t tiles, int64_t K, int64_t cus) {
     return best;
 }
 
-// Expected duration in microseconds of a single product of whole tiles on `tile` (small, wide or medium) with
-// the reduction cut into s equal parts, fitted to a sweep of 380 shapes (M 64..2048, N and K 512..4096, the
-// three operand forms, every tile and part count; the choice made from it is within 1 % of the best measured
-// one on average, 8 % at worst).  A workgroup takes a fixed time per 32 reduction steps whatever shares its
-// compute unit -- small 0.48 us on the pipelined schedule (both operands K-contiguous), 0.62 / 0.555 / 0.53 with
-// one / two / more workgroups per unit on the simple one, wide 0.95, medium 1.8 (two resident at most) -- so the
-// kernel takes rounds x steps x that, plus 3.5 us of launch, first loads and epilogue; the parts cost a second
-// launch (3.5 us + 0.1 per part) and their traffic (each part written and read once, at about 6 TB/s).
-double tiled_cost(int tile, bool both_kc, int64_t M, int64_t N, int64_t K, int64_t s, int64_t cus) {
+// Expected duration in microseconds of a single product on `tile` (small, wide or medium) with the reduction cut
+// into `parts` parts of `k_len` steps, fitted to sweeps of 380 whole-tile and 75 ragged shapes (M 40..3000, N and K
+// 250..11008, the three operand forms, every tile and part count; the choice made from it is within 1 % of the
+// best measured one on average, 8 % at worst).  A workgroup takes a fixed time per 32 reduction steps whatever
+// shares its compute unit -- small 0.48 us on the pipelined schedule (both operands K-contiguous), 0.62 / 0.555 /
+// 0.53 / 0.49 with one / two / three / more workgroups per unit on the simple one, wide 0.95, medium 1.8 (two
+// resident at most);
+// edge tiles cost the pipelined kernels a twentieth more and the simple one a quarter -- so the kernel takes
+// rounds x steps x that, plus 3.5 us of launch, first loads and epilogue; the parts cost a second launch
+// (3.5 us + 0.1 per part) and their traffic (each part written and read once, at about 6 TB/s).
+double tiled_cost(int tile, bool both_kc, bool pipelined, bool whole, int64_t M, int64_t N, int64_t k_len, int64_t parts,
+                  int64_t cus) {
     const int64_t bm = tile == kTileMedium ? 128 : 64, bn = tile == kTileSmall ? 64 : 128;
-    const int64_t groups = (M / bm) * (N / bn) * s;
+    const int64_t groups = ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * parts;
     const int64_t per_cu = (groups + cus - 1) / cus;
-    const double steps = (double)K / (double)s / 32.0;
+    const double steps = (double)k_len / 32.0;
     double t;
     if (tile == kTileMedium) {
-        const double one = both_kc ? 1.79 : 1.86;
+        const double one = (both_kc ? 1.79 : 1.86) * (whole ? 1.0 : 1.05);
         t = per_cu == 1 ? steps * one : steps * 1.02 * one * (double)(2 * (per_cu / 2)) + steps * one * (double)(per_cu % 2);
     } else if (tile == kTileWide) {
-        t = (double)per_cu * steps * (both_kc ? 0.95 : 0.96);
+        t = (double)per_cu * steps * (both_kc ? 0.95 : 0.96) * (whole ? 1.0 : 1.05);
+    } else if (pipelined) {
+        t = (double)per_cu * steps * 0.48;
     } else {
-        t = (double)per_cu * steps * (both_kc ? 0.48 : per_cu == 1 ? 0.62 : per_cu == 2 ? 0.555 : 0.53);
+        t = (double)per_cu * steps * (per_cu == 1 ? 0.62 : per_cu == 2 ? 0.555 : per_cu == 3 ? 0.53 : 0.49) * (whole ? 1.0 : 1.25);
     }
-    return t + 3.5 + (s > 1 ? 3.5 + 0.1 * (double)s + (double)(2 * s + 1) * (double)(M * N) * 4.0 / 6.0e6 : 0.0);
+    // the pipelined kernels run the steps after the last whole tile of 32 as a tile of their own, loaded, masked
+    // and multiplied with nothing else in flight
+    if (pipelined && k_len % 32 != 0) t += 1.5 * (double)per_cu;
+    return t + 3.5 + (parts > 1 ? 3.5 + 0.1 * (double)parts + (double)(2 * parts + 1) * (double)(M * N) * 4.0 / 6.0e6 : 0.0);
 }
 
 GemmPlan plan_gemm(const GemmDesc& d) {
@@ -155,31 +163,44 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         if (best > 0 && best <= limit) plan.wavesplit_edge = take16 ? 16 : 32;
     }
 
-    // A single product of whole 64-wide tiles: tile and number of parts together, from the model above.  (The
-    // kernels of the wide tile and of the pipelined small tile exist for whole tiles only; everything else keeps
-    // the rules above and below.)
+    // A single product of more than 32 rows whose operands the pipelined kernels can load (unit strides): tile and
+    // number of parts together, from the model above.  Everything else keeps the rules above and below.
     bool modelled = false;
-    if (!plan.skinny && !plan.wavesplit_edge && d.nbatch == 1 && (plan.tile == kTileSmall || plan.tile == kTileMedium) &&
-        d.M % 64 == 0 && d.N % 64 == 0 && d.K % 32 == 0 && !skinny_rows_applies(dn) && !shortk_nt_applies(dn)) {
+    // (The 32 x 128 tile keeps 65..96 rows where it wastes nothing or both operands are K-contiguous: 96 x 4096 x 4096
+    // 36 us against 37-39 with the tiles below, but 72 x 4096 x 11008 with a [K, N] matrix 101 -> 90.)
+    const bool keep_flat = plan.tile == kTileFlat && (d.M <= 32 || d.M % 32 == 0 || (plan.a_kc && plan.b_kc));
+    if (!plan.skinny && !plan.wavesplit_edge && d.nbatch == 1 && plan.tile != kTileLarge && !keep_flat && d.M > 32 &&
+        d.N >= 64 && d.K >= 32 && !skinny_rows_applies(dn) && !shortk_nt_applies(dn)) {
         const GemmParams pp = make_params(dn, plan.a_kc, plan.b_kc);
-        if (fits_without_edges(pp, plan.a_kc, plan.b_kc, 64, 64, 32) && fits_buffer_offsets(pp, plan.a_kc, plan.b_kc, 128, 128)) {
-            const bool both_kc = plan.a_kc && plan.b_kc;
+        const bool both_kc = plan.a_kc && plan.b_kc;
+        const bool vec = pp.a_vec && pp.b_vec && fits_buffer_offsets(pp, plan.a_kc, plan.b_kc, 128, 128);
+        if (vec || fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, 128, 128)) {
             double best = 0.0;
             for (const int tile : {(int)kTileMedium, (int)kTileWide, (int)kTileSmall}) {   // on a tie the larger tile
-                if (tile != kTileSmall && d.N % 128 != 0) continue;
-                if (tile == kTileMedium && d.M % 128 != 0) continue;
-                for (int64_t sp = 1; sp <= kSplitMax; sp *= 2) {
-                    if (sp > 1 && (d.K < kSplitFromK || d.K % (32 * sp) != 0 || d.K / sp < 256 ||
-                                   sp * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax))
-                        break;
-                    const double c = tiled_cost(tile, both_kc, d.M, d.N, d.K, sp, cus);
+                const int64_t bm = tile == kTileMedium ? 128 : 64, bn = tile == kTileSmall ? 64 : 128;
+                if (d.M <= bm / 2 || d.N <= bn / 2) continue;   // more than half of a lone tile would be padding
+                for (int64_t sp = 1; sp <= kSplitMax; sp++) {
+                    int64_t k_len = d.K;
+                    bool equal = true;
+                    if (sp > 1) {
+                        if (d.K < kSplitFromK || sp * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) break;
+                        equal = d.K % (16 * sp) == 0;
+                        k_len = equal ? d.K / sp : ((d.K + sp - 1) / sp + 15) / 16 * 16;
+                        // parts of at least 256 steps, 512 for the larger tiles (their first tile takes longer to arrive)
+                        if (k_len < (tile == kTileSmall ? 256 : 512)) break;
+                        if ((d.K + k_len - 1) / k_len != sp) continue;   // this part length needs fewer parts
+                    }
+                    const bool whole = vec && equal && d.M % bm == 0 && d.N % bn == 0 && k_len % 32 == 0;
+                    const bool pipelined = tile != kTileSmall || both_kc;
+                    if (!whole && pipelined && !fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, (int)bm, (int)bn)) continue;
+                    const double c = tiled_cost(tile, both_kc, pipelined, whole, d.M, d.N, k_len, sp, cus);
                     if (!modelled || c < 0.98 * best) {
                         modelled = true;
                         best = c;
                         plan.tile = tile;
                         plan.split = sp;
-                        plan.k_part = sp > 1 ? d.K / sp : 0;
-                        plan.ragged_parts = false;
+                        plan.k_part = sp > 1 ? k_len : 0;
+                        plan.ragged_parts = !equal;
                     }
                 }
             }
@@ -260,13 +281,15 @@ std::string describe_gemm(const GemmDesc& d) {
     }
     const GemmParams p = make_params(dt, a_kc, b_kc);
     const int edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
-    const bool wide = plan.tile == kTileWide && fits_without_edges(p, a_kc, b_kc, 64, 128, 32) &&
-                      fits_buffer_offsets(p, a_kc, b_kc, 64, 128);   // else the small tile runs
+    // the same tests, in the same order, as launch_gemm_layout makes
+    const bool wide_whole = plan.tile == kTileWide && fits_without_edges(p, a_kc, b_kc, 64, 128, 32) &&
+                            fits_buffer_offsets(p, a_kc, b_kc, 64, 128);
+    const bool wide = wide_whole || (plan.tile == kTileWide && fits_ragged_pipe(p, a_kc, b_kc, 64, 128));   // else the small tile runs
     const char* tile = plan.tile == kTileLarge ? "large" : plan.tile == kTileMedium ? "medium" :
                        plan.tile == kTileFlat ? "flat" : wide ? "wide" : "small";
     const char* variant = "general";
     if (wide) {
-        variant = "whole pipelined";
+        variant = wide_whole ? "whole pipelined" : "ragged pipelined";
     } else if (plan.tile == kTileFlat) {
         if (fits_without_edges(p, a_kc, b_kc, 32, 128, 32) && fits_buffer_offsets(p, a_kc, b_kc, 32, 128)) variant = "whole";
     } else if (plan.tile == kTileLarge || plan.tile == kTileMedium) {
@@ -274,9 +297,13 @@ std::string describe_gemm(const GemmDesc& d) {
         if (fits_without_edges(p, a_kc, b_kc, edge, edge, bk) && fits_buffer_offsets(p, a_kc, b_kc, edge, edge))
             variant = "whole pipelined";
         else if (fits_ragged_pipe(p, a_kc, b_kc, edge, edge)) variant = "ragged pipelined";
+    } else if (a_kc && b_kc && fits_without_edges(p, a_kc, b_kc, 64, 64, 32) && fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
+        variant = "whole pipelined";
+    } else if (a_kc && b_kc && fits_ragged_pipe(p, a_kc, b_kc, 64, 64)) {
+        variant = "ragged pipelined";
     } else if ((fits_without_edges(p, a_kc, b_kc, 64, 64, 32) || fits_without_edges(p, a_kc, b_kc, 64, 64, 16)) &&
                fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
-        variant = a_kc && b_kc && fits_without_edges(p, a_kc, b_kc, 64, 64, 32) ? "whole pipelined" : "whole";
+        variant = "whole";
     }
     return std::string("mfma ") + tile + " " + variant + " split " + std::to_string(plan.split);
 }

@@ -85,11 +85,11 @@ inline bool fits_buffer_offsets(const GemmParams& p, bool a_kc, bool b_kc, int B
 
 // true when the pipelined kernel's general variant may run the problem: both operands have a unit stride (its
 // buffer loads fetch 128 bits at any 4-byte aligned address; M, N, K and the leading dimensions are arbitrary:
-// rows past the end are never stored, the last partial K-tile is masked) and the reduction is not cut over
-// the batch index
+// rows past the end are never stored, the last partial K-tile is masked; a reduction cut over the batch index
+// into parts of k_part steps is fine, too)
 inline bool fits_ragged_pipe(const GemmParams& p, bool a_kc, bool b_kc, int BM, int BN) {
     const int64_t a_ld = a_kc ? p.a_rs : p.a_ks, b_ld = b_kc ? p.b_rs : p.b_ks;
-    return p.k_part == 0 && p.a_cont && p.b_cont && p.K > 0 && a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30) &&
+    return p.a_cont && p.b_cont && p.K > 0 && a_ld * BM < (1ll << 30) && b_ld * BN < (1ll << 30) &&
            fits_buffer_offsets(p, a_kc, b_kc, BM, BN);
 }
 

@@ -53,6 +53,8 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
     case kTileWide:
         if (fits_without_edges(p, A_KC, B_KC, 64, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 128))
             return launch_gemm_config<2, 2, 1, 2, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
+        if (fits_ragged_pipe(p, A_KC, B_KC, 64, 128))
+            return launch_gemm_config<2, 2, 1, 2, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
         [[fallthrough]];
     default:
         // Both operands K-contiguous, whole tiles: the pipelined schedule (fragment reads and LDS stores dealt
@@ -62,6 +64,8 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
         // fragments take four LDS reads instead of one), so those keep the simple schedule.
         if (A_KC && B_KC && fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
             return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
+        if (A_KC && B_KC && fits_ragged_pipe(p, A_KC, B_KC, 64, 64))
+            return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
         // a 64x64x16 tile computes for ~0.25 us, a global load takes ~1-2 us: 128 reduction steps in flight
         // (measured with whole tiles of 32 steps against 16 and 64: 15.5 / 16.9 / 16.0 us for 256x1024x1024)
         if (fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))

@@ -635,6 +635,8 @@ __device__ __forceinline__ void gemm_tile_body(
     f32x4(&rb)[NCHB] = rbx[0];
     // reduction length of this workgroup
     const int Kz = (EDGE && p.k_part > 0) ? min(p.k_part, p.K - z * p.k_part) : p.K;
+    // steps from this workgroup's first one to the end of the operand (the bound of its buffer resources)
+    const int Krem = (EDGE && p.k_part > 0) ? p.K - z * p.k_part : p.K;
     const int nkt = (Kz + BK - 1) / BK;
 
     constexpr int NKG = BK / 8;
@@ -669,10 +671,10 @@ __device__ __forceinline__ void gemm_tile_body(
     // predicate, and the rest of K follows as one masked tile.
     constexpr bool RAGGED_PIPE = EDGE && PIPE == 1;
     const __amdgpu_buffer_rsrc_t rsrc_a =
-        RAGGED_PIPE ? edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Ab)), p.a_rs, p.a_ks, p.M - m0, p.K, 0)
+        RAGGED_PIPE ? edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Ab)), p.a_rs, p.a_ks, p.M - m0, Krem, 0)
                     : __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Ab), 0, (int)0xFFFFFFFFu, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b =
-        RAGGED_PIPE ? edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Bb)), p.b_rs, p.b_ks, p.N - n0, p.K, 0)
+        RAGGED_PIPE ? edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Bb)), p.b_rs, p.b_ks, p.N - n0, Krem, 0)
                     : __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(Bb), 0, (int)0xFFFFFFFFu, 0x00020000);
     // AMASK: the second tensor behind the A operand, addressed exactly like A
     const bool a_masked = AMASK && p.a_mask != 0;
@@ -839,7 +841,7 @@ __device__ __forceinline__ void gemm_tile_body(
         static_assert(PIPE == 0 || NKG % 2 == 0, "the pipelined schedule needs an even number of groups per tile");
         // whole K-tiles of the pipelined loop; a general shape's last, partial tile follows it
         const int nkt_all = nkt;
-        const int nkt = RAGGED_PIPE ? p.K / BK : nkt_all;
+        const int nkt = RAGGED_PIPE ? Kz / BK : nkt_all;
         constexpr int kReadsA = A_KC ? NBM : 4;
         constexpr int kReads = kReadsA + (B_KC ? NBN : 4);   // LDS reads per group
         constexpr int kWrites = NCHA + NCHB;                  // LDS stores per tile and thread
@@ -948,15 +950,15 @@ __device__ __forceinline__ void gemm_tile_body(
             for (int kg = 0; kg < NKG; kg++) group(kg & 1, (kg + 1) & 1, kg + 1 < NKG, cur, kg + 1, false, 0, false, 0);
         }
         if constexpr (RAGGED_PIPE) {
-            const int k0 = nkt * BK, k_left = p.K - k0;
+            const int k0 = nkt * BK, k_left = Kz - k0;
             if (k_left > 0) {   // uniform
                 int voa[NCHA][4], vob[NCHB][4];
                 edge_offsets<A_KC, BM, BK, NT, false>(voa, p.a_rs, p.a_ks, tid);
                 edge_offsets<B_KC, BN, BK, NT, false>(vob, p.b_rs, p.b_ks, tid);
                 load_tile_edge_buf<NCHA, false>(
-                    ra, edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Ab)), p.a_rs, p.a_ks, p.M - m0, p.K, k0), voa);
+                    ra, edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Ab)), p.a_rs, p.a_ks, p.M - m0, Krem, k0), voa);
                 load_tile_edge_buf<NCHB, false>(
-                    rb, edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Bb)), p.b_rs, p.b_ks, p.N - n0, p.K, k0), vob);
+                    rb, edge_resource(reinterpret_cast<uint64_t>(uniform_ptr(Bb)), p.b_rs, p.b_ks, p.N - n0, Krem, k0), vob);
                 mask_tile_edge<A_KC, BM, BK, NT>(ra, rows_a, k_left, tid);
                 mask_tile_edge<B_KC, BN, BK, NT>(rb, rows_b, k_left, tid);
                 __syncthreads();   // every wave has read its last fragments of the whole tiles

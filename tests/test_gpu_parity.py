@@ -309,7 +309,11 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (17, 33, 9), (64, 64, 64), (65, 63, 66), (100, 3
           (32, 2048, 2304), (20, 1030, 2100),
           # short reductions: the tiled kernel below 4M outputs, the panel-resident kernel (K-contiguous form)
           # above: odd K, ragged rows and columns
-          (200, 130, 61), (513, 700, 64), (64, 1000, 8), (2050, 2100, 61), (2048, 2048, 64), (4100, 1030, 24)]
+          (200, 130, 61), (513, 700, 64), (64, 1000, 8), (2050, 2100, 61), (2048, 2048, 64), (4100, 1030, 24),
+          # tile and number of parts from the cost model: the pipelined 64 x 64, 64 x 128 and 128 x 128 tiles, whole and
+          # with edges, the reduction in equal parts and in parts with a shorter last one
+          (300, 200, 5003), (130, 260, 3001), (192, 384, 2048), (100, 1000, 4100), (640, 512, 1024), (333, 444, 2222),
+          (64, 128, 31), (65, 129, 33), (500, 1000, 1000)]
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -834,7 +838,7 @@ def test_split_k_scratch_survives_shutdown_and_growth():
 
 # products cut along K whose outputs are larger than one capped element-wise grid covers (4096 workgroups x 256
 # threads: 4 Mi outputs with 128-bit accesses, 1 Mi without): the pass that sums the parts covers all of them
-@pytest.mark.parametrize("m,n,k,bias_act", [(1152, 4096, 4096, False), (1280, 5120, 5120, True), (2047, 2049, 2051, False),
+@pytest.mark.parametrize("m,n,k,bias_act", [(1152, 4096, 4096, False), (1280, 5120, 5120, True), (1030, 1031, 8000, False), (1025, 1027, 6001, True),
                                             (1100, 1023, 3000, True)])
 def test_split_k_with_a_large_output(m, n, k, bias_act):
     plan = VMath.gemm_plan(0, 1, m, n, k)
