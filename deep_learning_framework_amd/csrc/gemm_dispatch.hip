@@ -47,7 +47,7 @@ struct GemmPlan {
 // (a fixed cost, then the larger of the stream of operand bytes through the compute units' address units and
 // one wave's chain of rounds along K; an operand that is not K-contiguous adds about an eighth), or a negative
 // value outside the measured range.
-double wavesplit_estimate(const GemmDesc& d, int T) {
+double wavesplit_estimate(const GemmDesc& d, int T, bool rounds_counted = false) {
     const int64_t wgs = ((d.M + T - 1) / T) * ((d.N + T - 1) / T);
     const double K = (double)d.K;
     const double forms = 1.0 + 0.12 * ((d.a_ks != 1) + (d.b_ks != 1));
@@ -56,7 +56,14 @@ double wavesplit_estimate(const GemmDesc& d, int T) {
         return (3.8 + std::max(1.3e-5 * (double)wgs * K, 3.1e-3 * std::max(0.0, K - 256.0))) * forms;
     }
     if (d.K > 1024 || wgs > 512 || (d.K < 256 && wgs > 256)) return -1.0;
-    return (4.0 + std::max(2.7e-5 * (double)wgs * K, 6.45e-3 * K)) * forms;
+    if (!rounds_counted) return (4.0 + std::max(2.7e-5 * (double)wgs * K, 6.45e-3 * K)) * forms;
+    // The workgroups of 16 waves run one per compute unit at a time: beyond that many a second round follows
+    // (512 x 1024 x 256: 11.6 us against 6.5 for 512 x 512 x 256).  This closer figure is the one compared with
+    // the tiled kernels' expected time.
+    const int64_t cus = compute_units();
+    const double rounds = (double)((wgs + cus - 1) / cus);
+    const double one = std::max(2.7e-5 * (double)std::min(wgs, cus) * K, 6.45e-3 * K);
+    return (4.0 + rounds * one + 3.0 * (rounds - 1.0)) * forms;
 }
 
 // Number of parts for a long reduction on the 64x64 tile.  A compute unit that holds one workgroup spends
@@ -155,12 +162,19 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // kernel (plus, for long K, its second launch) could: measured, it wins wherever its estimate stays below
     // ~12.5 us (64x512x784 9.8 -> 4.9 us, 256x1024x1024 14.3 -> 11.0, its backward_x form 14.3 -> 12.4,
     // 300^3 11.1 -> 4.9), and against the skinny kernels for 5..16 rows below ~7 us (16x1024x1024 7.8 -> 5.9).
+    // (and where the cost model below expects no less of the tiled kernels: 1000 x 333 x 777 19.4 -> 14.6 us,
+    // 512 x 1024 x 256 11.6 -> 7.0)
+    int ws_edge = 0;
+    double ws_cost = 0.0;
     if (wavesplit_applies(dn)) {
         const double e16 = wavesplit_estimate(dn, 16), e32 = wavesplit_estimate(dn, 32);
         const bool take16 = e16 > 0 && (e32 < 0 || e16 <= e32);
         const double best = take16 ? e16 : e32;
         const double limit = plan.skinny ? (d.M <= 4 ? 0.0 : 7.0) : 12.5;
-        if (best > 0 && best <= limit) plan.wavesplit_edge = take16 ? 16 : 32;
+        if (best > 0 && best <= limit) {
+            ws_edge = take16 ? 16 : 32;
+            ws_cost = take16 ? best : wavesplit_estimate(dn, 32, true);
+        }
     }
 
     // A single product of more than 32 rows whose operands the pipelined kernels can load (unit strides): tile and
@@ -169,7 +183,8 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // (The 32 x 128 tile keeps 65..96 rows where it wastes nothing or both operands are K-contiguous: 96 x 4096 x 4096
     // 36 us against 37-39 with the tiles below, but 72 x 4096 x 11008 with a [K, N] matrix 101 -> 90.)
     const bool keep_flat = plan.tile == kTileFlat && (d.M <= 32 || d.M % 32 == 0 || (plan.a_kc && plan.b_kc));
-    if (!plan.skinny && !plan.wavesplit_edge && d.nbatch == 1 && plan.tile != kTileLarge && !keep_flat && d.M > 32 &&
+    double tiles_cost = 0.0;
+    if (!plan.skinny && d.nbatch == 1 && plan.tile != kTileLarge && !keep_flat && d.M > 32 &&
         d.N >= 64 && d.K >= 32 && !skinny_rows_applies(dn) && !shortk_nt_applies(dn)) {
         const GemmParams pp = make_params(dn, plan.a_kc, plan.b_kc);
         const bool both_kc = plan.a_kc && plan.b_kc;
@@ -196,7 +211,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
                     const double c = tiled_cost(tile, both_kc, pipelined, whole, d.M, d.N, k_len, sp, cus);
                     if (!modelled || c < 0.98 * best) {
                         modelled = true;
-                        best = c;
+                        best = tiles_cost = c;
                         plan.tile = tile;
                         plan.split = sp;
                         plan.k_part = sp > 1 ? k_len : 0;
@@ -205,6 +220,18 @@ GemmPlan plan_gemm(const GemmDesc& d) {
                 }
             }
         }
+    }
+
+    // (the model is trusted against the one-launch kernel for the pipelined kernels only; for the simple schedule
+    // with K parts it is too optimistic at these sizes: 256 x 1024 x 777 with a [K, N] operand 13.6 us for its
+    // choice against 10.4)
+    const bool tiles_pipelined = modelled && (plan.tile != kTileSmall || (plan.a_kc && plan.b_kc));
+    if (ws_edge && !(tiles_pipelined && tiles_cost < 0.95 * ws_cost)) {
+        plan.wavesplit_edge = ws_edge;
+        modelled = false;
+        plan.split = 1;
+        plan.k_part = 0;
+        plan.ragged_parts = false;
     }
 
     // Split-K: a single product whose output tiles leave most compute units idle is cut along K

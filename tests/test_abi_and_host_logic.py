@@ -239,7 +239,7 @@ GEMM_PLANS = [
     ((0, 0, 17, 4096, 4096), "mfma flat general split 8"),
     ((0, 1, 16, 1024, 1024), "wavesplit 16"),                        # 5..16 rows against a small weight matrix
     ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
-    ((0, 1, 1000, 333, 777), "wavesplit 32"),                        # configuration 5, ragged: unaligned rows are fine
+    ((0, 1, 1000, 333, 777), "mfma small ragged pipelined split 2"),   # configuration 5, ragged: two rounds of the one-launch kernel would take longer
     ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
     ((0, 1, 17, 11008, 4096), "mfma flat general split 2"),          # one workgroup per compute unit: 86 tiles x 2
     ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
