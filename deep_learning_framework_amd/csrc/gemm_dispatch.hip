@@ -319,6 +319,7 @@ std::string describe_gemm(const GemmDesc& d) {
         variant = wide_whole ? "whole pipelined" : "ragged pipelined";
     } else if (plan.tile == kTileFlat) {
         if (fits_without_edges(p, a_kc, b_kc, 32, 128, 32) && fits_buffer_offsets(p, a_kc, b_kc, 32, 128)) variant = "whole";
+        else if (fits_ragged_pipe(p, a_kc, b_kc, 32, 128)) variant = "ragged pipelined";
     } else if (plan.tile == kTileLarge || plan.tile == kTileMedium) {
         const int bk = plan.tile == kTileLarge ? 16 : 32;
         if (fits_without_edges(p, a_kc, b_kc, edge, edge, bk) && fits_buffer_offsets(p, a_kc, b_kc, edge, edge))

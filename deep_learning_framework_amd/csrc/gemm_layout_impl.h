@@ -49,6 +49,11 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
         // by side, so that the matrix cores do not spend half their time on rows that do not exist
         if (fits_without_edges(p, A_KC, B_KC, 32, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 32, 128))
             return launch_gemm_config<1, 4, 1, 1, 32, A_KC, B_KC, false, 0, 2, 4>(p, nbatch, kGroupM, stream);
+        // with edges the pipelined schedule is the faster one (80 x 4096 x 4096: 41.2 -> 36.6 us, 72 x 4096 x 11008:
+        // 88.6 -> 79.9, 17 and 24 rows 22.9 -> 22.4); whole tiles lose with it (32 x 11008 x 4096: 50 -> 65: the
+        // stream of the other operand wants the four tiles in flight that the simple schedule keeps)
+        if (fits_ragged_pipe(p, A_KC, B_KC, 32, 128))
+            return launch_gemm_config<1, 4, 1, 1, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
         return launch_gemm_config<1, 4, 1, 1, 32, A_KC, B_KC, true, 0, 1, 4>(p, nbatch, kGroupM, stream);
     case kTileWide:
         if (fits_without_edges(p, A_KC, B_KC, 64, 128, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 128))

@@ -236,12 +236,12 @@ GEMM_PLANS = [
     ((0, 1, 16, 4096, 4096), "skinny"),
     ((0, 0, 4, 4096, 4096), "skinny rows"),                          # backward_x at a small batch: b stored [K, N]
     ((0, 0, 16, 11008, 4096), "skinny rows"),
-    ((0, 0, 17, 4096, 4096), "mfma flat general split 8"),
+    ((0, 0, 17, 4096, 4096), "mfma flat ragged pipelined split 8"),
     ((0, 1, 16, 1024, 1024), "wavesplit 16"),                        # 5..16 rows against a small weight matrix
     ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
     ((0, 1, 1000, 333, 777), "mfma small ragged pipelined split 2"),   # configuration 5, ragged: two rounds of the one-launch kernel would take longer
     ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
-    ((0, 1, 17, 11008, 4096), "mfma flat general split 2"),          # one workgroup per compute unit: 86 tiles x 2
+    ((0, 1, 17, 11008, 4096), "mfma flat ragged pipelined split 2"),          # one workgroup per compute unit: 86 tiles x 2
     ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined split 4"),   # 33..64 rows: one row of 64-row tiles with edges
     ((0, 1, 96, 4096, 4096), "mfma flat whole split 8"),             # 65..96 rows: three row tiles of 32, not two of 64
@@ -258,7 +258,7 @@ GEMM_PLANS = [
     ((0, 0, 1000, 1000, 1000), "mfma wide ragged pipelined split 2"),
     ((0, 1, 600, 600, 6000), "mfma medium ragged pipelined split 10"),  # 25 medium tiles x 10 parts: parts need not be a power of two
     ((0, 0, 72, 4096, 11008), "mfma medium ragged pipelined split 8"),  # 65..96 rows that are no multiple of 32, [K, N] operand
-    ((0, 1, 72, 4096, 11008), "mfma flat general split 8"),
+    ((0, 1, 72, 4096, 11008), "mfma flat ragged pipelined split 8"),
     ((0, 1, 0, 5, 5), "nothing"),
 ]
 
