@@ -92,14 +92,13 @@ int64_t small_tile_split(int64_t tiles, int64_t K, int64_t cus) {
 // into `parts` parts of `k_len` steps, fitted to sweeps of 380 whole-tile and 75 ragged shapes (M 40..3000, N and K
 // 250..11008, the three operand forms, every tile and part count; the choice made from it is within 1 % of the
 // best measured one on average, 8 % at worst).  A workgroup takes a fixed time per 32 reduction steps whatever
-// shares its compute unit -- small 0.48 us on the pipelined schedule (both operands K-contiguous), 0.62 / 0.555 /
-// 0.53 / 0.49 with one / two / three / more workgroups per unit on the simple one, wide 0.95, medium 1.8 (two
-// resident at most);
-// edge tiles cost the pipelined kernels a twentieth more and the simple one a quarter -- so the kernel takes
+// shares its compute unit -- small 0.48 us with both operands K-contiguous, else 0.57 / 0.54 / 0.52 with one / two /
+// three workgroups per unit and 0.49 with more (the simple schedule), wide 0.95, medium 1.8 (two resident at
+// most); edge tiles cost a twentieth more -- so the kernel takes
 // rounds x steps x that, plus 3.5 us of launch, first loads and epilogue; the parts cost a second launch
 // (3.5 us + 0.1 per part) and their traffic (each part written and read once, at about 6 TB/s).
-double tiled_cost(int tile, bool both_kc, bool pipelined, bool whole, int64_t M, int64_t N, int64_t k_len, int64_t parts,
-                  int64_t cus) {
+double tiled_cost(int tile, bool both_kc, bool whole, int64_t M, int64_t N, int64_t k_len, int64_t parts, int64_t cus) {
+    bool pipelined = true;
     const int64_t bm = tile == kTileMedium ? 128 : 64, bn = tile == kTileSmall ? 64 : 128;
     const int64_t groups = ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * parts;
     const int64_t per_cu = (groups + cus - 1) / cus;
@@ -110,10 +109,13 @@ double tiled_cost(int tile, bool both_kc, bool pipelined, bool whole, int64_t M,
         t = per_cu == 1 ? steps * one : steps * 1.02 * one * (double)(2 * (per_cu / 2)) + steps * one * (double)(per_cu % 2);
     } else if (tile == kTileWide) {
         t = (double)per_cu * steps * (both_kc ? 0.95 : 0.96) * (whole ? 1.0 : 1.05);
-    } else if (pipelined) {
+    } else if (both_kc) {
         t = (double)per_cu * steps * 0.48;
+    } else if (whole && per_cu >= 4) {
+        pipelined = false;   // the simple schedule
+        t = (double)per_cu * steps * 0.49;
     } else {
-        t = (double)per_cu * steps * (per_cu == 1 ? 0.62 : per_cu == 2 ? 0.555 : per_cu == 3 ? 0.53 : 0.49) * (whole ? 1.0 : 1.25);
+        t = (double)per_cu * steps * (per_cu == 1 ? 0.57 : per_cu == 2 ? 0.54 : 0.52) * (whole ? 1.0 : 1.05);
     }
     // the pipelined kernels run the steps after the last whole tile of 32 as a tile of their own, loaded, masked
     // and multiplied with nothing else in flight
@@ -206,9 +208,8 @@ GemmPlan plan_gemm(const GemmDesc& d) {
                         if ((d.K + k_len - 1) / k_len != sp) continue;   // this part length needs fewer parts
                     }
                     const bool whole = vec && equal && d.M % bm == 0 && d.N % bn == 0 && k_len % 32 == 0;
-                    const bool pipelined = tile != kTileSmall || both_kc;
-                    if (!whole && pipelined && !fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, (int)bm, (int)bn)) continue;
-                    const double c = tiled_cost(tile, both_kc, pipelined, whole, d.M, d.N, k_len, sp, cus);
+                    if (!whole && !fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, (int)bm, (int)bn)) continue;
+                    const double c = tiled_cost(tile, both_kc, whole, d.M, d.N, k_len, sp, cus);
                     if (!modelled || c < 0.98 * best) {
                         modelled = true;
                         best = tiles_cost = c;
@@ -325,12 +326,12 @@ std::string describe_gemm(const GemmDesc& d) {
         if (fits_without_edges(p, a_kc, b_kc, edge, edge, bk) && fits_buffer_offsets(p, a_kc, b_kc, edge, edge))
             variant = "whole pipelined";
         else if (fits_ragged_pipe(p, a_kc, b_kc, edge, edge)) variant = "ragged pipelined";
-    } else if (a_kc && b_kc && fits_without_edges(p, a_kc, b_kc, 64, 64, 32) && fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
-        variant = "whole pipelined";
-    } else if (a_kc && b_kc && fits_ragged_pipe(p, a_kc, b_kc, 64, 64)) {
+    } else if (fits_without_edges(p, a_kc, b_kc, 64, 64, 32) && fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
+        const int64_t groups = ((dt.M + 63) / 64) * ((dt.N + 63) / 64) * (dt.nbatch > 0 ? dt.nbatch : 1);
+        variant = (a_kc && b_kc) || groups <= 3 * (int64_t)compute_units() ? "whole pipelined" : "whole";
+    } else if (fits_ragged_pipe(p, a_kc, b_kc, 64, 64)) {
         variant = "ragged pipelined";
-    } else if ((fits_without_edges(p, a_kc, b_kc, 64, 64, 32) || fits_without_edges(p, a_kc, b_kc, 64, 64, 16)) &&
-               fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
+    } else if (fits_without_edges(p, a_kc, b_kc, 64, 64, 16) && fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
         variant = "whole";
     }
     return std::string("mfma ") + tile + " " + variant + " split " + std::to_string(plan.split);

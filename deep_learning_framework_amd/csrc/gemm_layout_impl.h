@@ -62,19 +62,26 @@ int launch_gemm_layout(const GemmParams& p, int64_t nbatch, int tile, hipStream_
             return launch_gemm_config<2, 2, 1, 2, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
         [[fallthrough]];
     default:
-        // Both operands K-contiguous, whole tiles: the pipelined schedule (fragment reads and LDS stores dealt
-        // between the MFMAs) runs a 32-step tile in 0.48 us whether the workgroup has the compute unit to itself
-        // or not, the simple schedule below in 0.53-0.70 (1024^3: 22.6 -> 18.9 us, 512 x 2048 x 2048: 41.0 -> 34.2,
-        // 64 x 4096 x 4096: 27.2 -> 22.8).  With an operand that is not K-contiguous it gains nothing (its
-        // fragments take four LDS reads instead of one), so those keep the simple schedule.
-        if (A_KC && B_KC && fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
-            return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
-        if (A_KC && B_KC && fits_ragged_pipe(p, A_KC, B_KC, 64, 64))
-            return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
+        // The pipelined schedule (fragment reads and LDS stores dealt between the MFMAs).  Both operands
+        // K-contiguous: a 32-step tile takes 0.48 us whether the workgroup has the compute unit to itself or not,
+        // the simple schedule below 0.53-0.70 (1024^3: 22.6 -> 18.9 us, 512 x 2048 x 2048: 41.0 -> 34.2,
+        // 64 x 4096 x 4096: 27.2 -> 22.8).  An operand that is not K-contiguous takes four LDS reads per fragment
+        // instead of one: the pipelined schedule still wins while at most three workgroups share a unit
+        // (1024^3 23.7 -> 21.8, 128 x 2048 x 2048 18.0 -> 16.5) and loses beyond (3072^3: 420 -> 432).
+        {
+            const int64_t small_tiles = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64) * nbatch;
+            const bool pipelined = (A_KC && B_KC) || small_tiles <= 3 * (int64_t)compute_units();
+            if (pipelined && fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
+                return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, false, 1, 2>(p, nbatch, kGroupM, stream);
+        }
         // a 64x64x16 tile computes for ~0.25 us, a global load takes ~1-2 us: 128 reduction steps in flight
         // (measured with whole tiles of 32 steps against 16 and 64: 15.5 / 16.9 / 16.0 us for 256x1024x1024)
         if (fits_without_edges(p, A_KC, B_KC, 64, 64, 32) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
             return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, false, 0, 2, 4>(p, nbatch, kGroupM, stream);
+        // shapes with edges: the pipelined schedule in every operand form (777^3 with a [K, N] operand 24.2 -> 19.1 us,
+        // 200 x 200 x 8192 20.5 -> 16.5)
+        if (fits_ragged_pipe(p, A_KC, B_KC, 64, 64))
+            return launch_gemm_config<2, 2, 1, 1, 32, A_KC, B_KC, true, 1, 2>(p, nbatch, kGroupM, stream);
         if (fits_without_edges(p, A_KC, B_KC, 64, 64, 16) && fits_buffer_offsets(p, A_KC, B_KC, 64, 64))
             return launch_gemm_config<2, 2, 1, 1, 16, A_KC, B_KC, false, 0, 2, 8>(p, nbatch, kGroupM, stream);
         // 32-step tiles halve the number of rounds; with an operand that is strided in both directions (one

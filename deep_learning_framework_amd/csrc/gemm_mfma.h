@@ -896,9 +896,12 @@ __device__ __forceinline__ void gemm_tile_body(
                         else load_tile_chunk_buf<B_KC, BN, BK, NT>(rb, rsrc_b, gb_off, (int)b_ld * 4, (int)toff_b * 4, sl - NCHA);
                     }
                     __builtin_amdgcn_sched_barrier(0);
+                    // fewer MFMAs than slots (one block per wave and an operand whose fragments take four reads):
+                    // they are spread evenly over the slots instead
+                    const int cnt = per > 0 ? per : ((sl + 1) * kMfma) / slots - (sl * kMfma) / slots;
 #pragma unroll
                     for (int u = 0; u < kMfma; u++) {
-                        if (u < per) {
+                        if (u < cnt) {
                             const int t = q / (NBM * NBN), i = (q / NBN) % NBM, j = q % NBN;
                             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[use].get(i, t), fb[use].get(j, t),
                                                                             acc[i][j], 0, 0, 0);

@@ -222,7 +222,7 @@ GEMM_PLANS = [
     ((0, 1, 64, 512, 784), "wavesplit 16"),                          # configuration 1: one launch, 16 x 16 blocks
     ((0, 1, 256, 1024, 1024), "wavesplit 32"),                       # configuration 2 forward
     ((0, 0, 256, 1024, 1024), "wavesplit 32"),                       # configuration 2 dX: one operand not K-contiguous
-    ((1, 0, 1024, 1024, 256), "mfma small whole split 1"),           # configuration 2 dW: 256 tiles of 64 x 64
+    ((1, 0, 1024, 1024, 256), "mfma small whole pipelined split 1"),           # configuration 2 dW: 256 tiles of 64 x 64
     ((0, 0, 8192, 8192, 8192), "mfma large whole pipelined split 1"),  # the headline product
     ((0, 1, 8192, 8192, 8192), "mfma large whole pipelined split 1"),
     ((0, 0, 8191, 8191, 8191), "mfma large ragged pipelined split 1"),  # odd sizes keep the pipelined loop
@@ -255,7 +255,7 @@ GEMM_PLANS = [
     ((0, 1, 512, 4096, 4096), "mfma wide whole pipelined split 1"),
     ((0, 1, 256, 4096, 4096), "mfma small whole pipelined split 1"),  # both K-contiguous: one small tile per unit
     ((0, 1, 1000, 1000, 1000), "mfma small ragged pipelined split 1"),
-    ((0, 0, 1000, 1000, 1000), "mfma wide ragged pipelined split 2"),
+    ((0, 0, 1000, 1000, 1000), "mfma small ragged pipelined split 1"),
     ((0, 1, 600, 600, 6000), "mfma medium ragged pipelined split 10"),  # 25 medium tiles x 10 parts: parts need not be a power of two
     ((0, 0, 72, 4096, 11008), "mfma medium ragged pipelined split 8"),  # 65..96 rows that are no multiple of 32, [K, N] operand
     ((0, 1, 72, 4096, 11008), "mfma flat ragged pipelined split 8"),
