@@ -625,7 +625,7 @@ __device__ __forceinline__ void gemm_tile_body(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    static_assert(DEPTH >= 1 && (PIPE == 0 || DEPTH == 1), "deep register staging belongs to the PIPE 0 schedule");
+    static_assert(DEPTH >= 1, "at least one tile is staged in registers");
     static_assert(!ROWSUM || (PIPE == 0 && BM <= NT), "row sums: PIPE 0 schedule, one thread per tile row");
     const bool do_rowsum = ROWSUM && p.rowsum != nullptr && tn == 0 && z == 0 && tid < BM;
     float rowsum = 0.f;
@@ -872,7 +872,11 @@ __device__ __forceinline__ void gemm_tile_body(
         // tile buffer `rbuf`, group `rkg`) and, when `store` is set, by the s-th LDS store of the
         // staged next tile (into buffer `wbuf`).  Scheduling fences pin that interleaving, so the
         // waves of a workgroup never hit LDS in one burst and no MFMA waits for an LDS round trip.
-        auto group = [&](int use, int fill, bool read, int rbuf, int rkg, bool store, int wbuf, bool gload, int gkt) {
+        auto group = [&](int use, int fill, bool read, int rbuf, int rkg, bool store, int wbuf, bool gload, int gkt,
+                         auto setc) {
+            constexpr int set = decltype(setc)::value;   // the staging registers that `store` empties / `gload` fills
+            f32x4(&ra)[NCHA] = rax[set];
+            f32x4(&rb)[NCHB] = rbx[set];
             const int memops = (store || gload) ? kWrites : 0;
             const int slots = (read ? kReads : 0) > memops ? (read ? kReads : 0) : memops;
             const int ga_off = gkt * BK * (int)p.a_ks * 4, gb_off = gkt * BK * (int)p.b_ks * 4;   // bytes, uniform
@@ -927,30 +931,79 @@ __device__ __forceinline__ void gemm_tile_body(
         // them into the free LDS buffer, one store per slot; the last group refills them with tile
         // kt+2, one global load per slot, so that the waves of a workgroup never queue all their
         // loads on the address unit at once and every load has most of a tile to land.
-        if (nkt > 1) load_whole(1);
+        constexpr std::integral_constant<int, 0> set0{};
+        if constexpr (DEPTH == 1) {
+            if (nkt > 1) load_whole(1);
+        } else if (nkt > 0) {
+            // DEPTH > 1: tile t waits in staging set t % DEPTH, requested DEPTH tiles before its turn -- the
+            // workgroups that have a compute unit to themselves and stream an operand from HBM need that much
+            // (a load has a tile's time to land otherwise: 0.4 us for the 64x64 tile).  Tiles 1 .. DEPTH now
+            // (tile DEPTH into set 0, which tile 0 has left); past the end: the last tile again, never stored.
+            static_for<1, DEPTH + 1>([&](auto dc) {
+                constexpr int d = decltype(dc)::value;
+                const int kt = min(d, nkt - 1);
+#pragma unroll
+                for (int i = 0; i < NCHA; i++)
+                    load_tile_chunk_buf<A_KC, BM, BK, NT>(rax[d % DEPTH], rsrc_a, kt * BK * (int)p.a_ks * 4, (int)a_ld * 4, (int)toff_a * 4, i);
+#pragma unroll
+                for (int i = 0; i < NCHB; i++)
+                    load_tile_chunk_buf<B_KC, BN, BK, NT>(rbx[d % DEPTH], rsrc_b, kt * BK * (int)p.b_ks * 4, (int)b_ld * 4, (int)toff_b * 4, i);
+            });
+        }
         if (nkt > 0) {
             read_frag<A_KC, NBM, BM, BK>(fa[0], lds_a[0], wm0, 0, l32, half);
             read_frag<B_KC, NBN, BN, BK>(fb[0], lds_b[0], wn0, 0, l32, half);
         }
-        for (int kt = 0; kt + 1 < nkt; kt++) {
-            const int cur = kt & 1;
-            const int gkt = min(kt + 2, nkt - 1);   // clamped: the surplus load of the last round is never stored
+        if constexpr (DEPTH == 1) {
+            for (int kt = 0; kt + 1 < nkt; kt++) {
+                const int cur = kt & 1;
+                const int gkt = min(kt + 2, nkt - 1);   // clamped: the surplus load of the last round is never stored
 #pragma unroll
-            for (int kg = 0; kg < NKG; kg++) {
-                if (kg + 1 < NKG) {
-                    group(kg & 1, (kg + 1) & 1, true, cur, kg + 1, kg == NKG - 2, cur ^ 1, false, 0);
-                } else {
-                    // last group: everyone's stores are in LDS after the barrier; its MFMAs (operands
-                    // already in registers) cover the first fragment reads of the next tile
-                    __syncthreads();
-                    group(kg & 1, (kg + 1) & 1, true, cur ^ 1, 0, false, 0, true, gkt);
+                for (int kg = 0; kg < NKG; kg++) {
+                    if (kg + 1 < NKG) {
+                        group(kg & 1, (kg + 1) & 1, true, cur, kg + 1, kg == NKG - 2, cur ^ 1, false, 0, set0);
+                    } else {
+                        // last group: everyone's stores are in LDS after the barrier; its MFMAs (operands
+                        // already in registers) cover the first fragment reads of the next tile
+                        __syncthreads();
+                        group(kg & 1, (kg + 1) & 1, true, cur ^ 1, 0, false, 0, true, gkt, set0);
+                    }
                 }
             }
+        } else {
+            static_assert(DEPTH % 2 == 0, "an even number of staging sets keeps the LDS buffer of a tile a constant");
+            // tile kt (in LDS buffer `curc`): group NKG-2 moves tile kt+1 from staging set `setc` into the other LDS
+            // buffer, the last group refills that set with tile kt+1+DEPTH
+            auto tile_round = [&](int kt, auto setc, auto curc) {
+                constexpr int cur = decltype(curc)::value;
+                const int gkt = min(kt + 1 + DEPTH, nkt - 1);   // clamped: a surplus load is never stored
+#pragma unroll
+                for (int kg = 0; kg < NKG; kg++) {
+                    if (kg + 1 < NKG) {
+                        group(kg & 1, (kg + 1) & 1, true, cur, kg + 1, kg == NKG - 2, cur ^ 1, false, 0, setc);
+                    } else {
+                        __syncthreads();
+                        group(kg & 1, (kg + 1) & 1, true, cur ^ 1, 0, false, 0, true, gkt, setc);
+                    }
+                }
+            };
+            // whole rounds over the staging sets without a condition inside, then a guarded remainder
+            int kt0 = 0;
+            for (; kt0 + DEPTH < nkt; kt0 += DEPTH)
+                static_for<0, DEPTH>([&](auto dc) {
+                    constexpr int d = decltype(dc)::value;
+                    tile_round(kt0 + d, std::integral_constant<int, (d + 1) % DEPTH>{}, std::integral_constant<int, d & 1>{});
+                });
+            static_for<0, DEPTH>([&](auto dc) {
+                constexpr int d = decltype(dc)::value;
+                if (kt0 + d + 1 < nkt)   // uniform
+                    tile_round(kt0 + d, std::integral_constant<int, (d + 1) % DEPTH>{}, std::integral_constant<int, d & 1>{});
+            });
         }
         if (nkt > 0) {
             const int cur = (nkt - 1) & 1;
 #pragma unroll
-            for (int kg = 0; kg < NKG; kg++) group(kg & 1, (kg + 1) & 1, kg + 1 < NKG, cur, kg + 1, false, 0, false, 0);
+            for (int kg = 0; kg < NKG; kg++) group(kg & 1, (kg + 1) & 1, kg + 1 < NKG, cur, kg + 1, false, 0, false, 0, set0);
         }
         if constexpr (RAGGED_PIPE) {
             const int k0 = nkt * BK, k_left = Kz - k0;
