@@ -97,8 +97,7 @@ int64_t small_tile_split(int64_t tiles, int64_t K, int64_t cus) {
 // most); edge tiles cost a twentieth more -- so the kernel takes
 // rounds x steps x that, plus 3.5 us of launch, first loads and epilogue; the parts cost a second launch
 // (3.5 us + 0.1 per part) and their traffic (each part written and read once, at about 6 TB/s).
-double tiled_cost(int tile, bool both_kc, bool whole, bool streamed, int64_t M, int64_t N, int64_t k_len, int64_t parts,
-                  int64_t cus) {
+double tiled_cost(int tile, bool both_kc, bool whole, int64_t M, int64_t N, int64_t k_len, int64_t parts, int64_t cus) {
     bool pipelined = true;
     const int64_t bm = tile == kTileMedium ? 128 : 64, bn = tile == kTileSmall ? 64 : 128;
     const int64_t groups = ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * parts;
@@ -115,12 +114,6 @@ double tiled_cost(int tile, bool both_kc, bool whole, bool streamed, int64_t M, 
         t = (double)per_cu * steps * 0.49;
     } else {
         double c = both_kc ? 0.48 : (per_cu == 1 ? 0.57 : per_cu == 2 ? 0.54 : 0.52) * (whole ? 1.0 : 1.05);
-        // The pipelined kernels request a tile two steps before its turn.  A workgroup that has the compute unit to
-        // itself and streams an operand from HBM (one too large to be expected in the last-level cache) then waits
-        // for every tile: 0.73 us per step (64 x 4096 x 4096 with the 64 MiB matrix from HBM: 32.4 us in 4 parts of
-        // K, one workgroup per unit, against 27.1 in 8 parts, two per unit; from the cache 22.8 against 24.2).
-        if (streamed && per_cu == 1 && c < 0.73) c = 0.73;
-        if (streamed && per_cu == 2 && c < 0.55) c = 0.55;   // two per unit: a little of the same
         t = (double)per_cu * steps * c;
     }
     // the pipelined kernels run the steps after the last whole tile of 32 as a tile of their own, loaded, masked
@@ -196,8 +189,6 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         d.N >= 64 && d.K >= 32 && !skinny_rows_applies(dn) && !shortk_nt_applies(dn)) {
         const GemmParams pp = make_params(dn, plan.a_kc, plan.b_kc);
         const bool both_kc = plan.a_kc && plan.b_kc;
-        // an operand of 32 MiB or more is taken to come from HBM, not from the 256 MiB last-level cache
-        const bool streamed = std::max(d.M, d.N) * d.K * (int64_t)sizeof(float) >= (32ll << 20);
         const bool vec = pp.a_vec && pp.b_vec && fits_buffer_offsets(pp, plan.a_kc, plan.b_kc, 128, 128);
         if (vec || fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, 128, 128)) {
             double best = 0.0;
@@ -217,7 +208,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
                     }
                     const bool whole = vec && equal && d.M % bm == 0 && d.N % bn == 0 && k_len % 32 == 0;
                     if (!whole && !fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, (int)bm, (int)bn)) continue;
-                    const double c = tiled_cost(tile, both_kc, whole, streamed, d.M, d.N, k_len, sp, cus);
+                    const double c = tiled_cost(tile, both_kc, whole, d.M, d.N, k_len, sp, cus);
                     if (!modelled || c < 0.98 * best) {
                         modelled = true;
                         best = tiles_cost = c;

@@ -243,7 +243,7 @@ GEMM_PLANS = [
     ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
     ((0, 1, 17, 11008, 4096), "mfma flat ragged pipelined split 2"),          # one workgroup per compute unit: 86 tiles x 2
     ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
-    ((0, 1, 48, 4096, 4096), "mfma wide ragged pipelined split 8"),   # 33..64 rows against a matrix that streams from HBM: 32 wide tiles x 8 parts, one per unit
+    ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
     ((0, 1, 96, 4096, 4096), "mfma flat whole split 8"),             # 65..96 rows: three row tiles of 32, not two of 64
     ((0, 1, 64, 64, 8192), "mfma small whole pipelined split 16"),             # one tile, a long reduction
     ((0, 1, 768, 768, 4096), "mfma medium ragged pipelined split 7"),   # 36 medium tiles x 7 parts of 592 steps: one workgroup per unit
@@ -253,7 +253,7 @@ GEMM_PLANS = [
     ((0, 0, 512, 4096, 4096), "mfma wide whole pipelined split 1"),   # a [K, N] operand: the 64 x 128 tile, one per unit
     ((1, 0, 512, 4096, 4096), "mfma wide whole pipelined split 1"),
     ((0, 1, 512, 4096, 4096), "mfma wide whole pipelined split 1"),
-    ((0, 1, 256, 4096, 4096), "mfma medium whole pipelined split 4"),   # a 64 MiB operand is taken to stream from HBM: not one small tile per unit, which would wait for every tile
+    ((0, 1, 256, 4096, 4096), "mfma small whole pipelined split 1"),   # 256 small tiles, one per unit, four tiles of K on their way each
     ((0, 1, 1000, 1000, 1000), "mfma small ragged pipelined split 1"),
     ((0, 0, 1000, 1000, 1000), "mfma small ragged pipelined split 1"),
     ((0, 1, 600, 600, 6000), "mfma medium ragged pipelined split 10"),  # 25 medium tiles x 10 parts: parts need not be a power of two
