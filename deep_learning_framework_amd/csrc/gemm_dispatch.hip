@@ -307,33 +307,13 @@ std::string describe_gemm(const GemmDesc& d) {
         dt.c_rs = d.N; dt.c_cs = 1;
     }
     const GemmParams p = make_params(dt, a_kc, b_kc);
-    const int edge = plan.tile == kTileLarge ? 256 : plan.tile == kTileMedium ? 128 : 64;
-    // the same tests, in the same order, as launch_gemm_layout makes
-    const bool wide_whole = plan.tile == kTileWide && fits_without_edges(p, a_kc, b_kc, 64, 128, 32) &&
-                            fits_buffer_offsets(p, a_kc, b_kc, 64, 128);
-    const bool wide = wide_whole || (plan.tile == kTileWide && fits_ragged_pipe(p, a_kc, b_kc, 64, 128));   // else the small tile runs
-    const char* tile = plan.tile == kTileLarge ? "large" : plan.tile == kTileMedium ? "medium" :
-                       plan.tile == kTileFlat ? "flat" : wide ? "wide" : "small";
-    const char* variant = "general";
-    if (wide) {
-        variant = wide_whole ? "whole pipelined" : "ragged pipelined";
-    } else if (plan.tile == kTileFlat) {
-        if (fits_without_edges(p, a_kc, b_kc, 32, 128, 32) && fits_buffer_offsets(p, a_kc, b_kc, 32, 128)) variant = "whole";
-        else if (fits_ragged_pipe(p, a_kc, b_kc, 32, 128)) variant = "ragged pipelined";
-    } else if (plan.tile == kTileLarge || plan.tile == kTileMedium) {
-        const int bk = plan.tile == kTileLarge ? 16 : 32;
-        if (fits_without_edges(p, a_kc, b_kc, edge, edge, bk) && fits_buffer_offsets(p, a_kc, b_kc, edge, edge))
-            variant = "whole pipelined";
-        else if (fits_ragged_pipe(p, a_kc, b_kc, edge, edge)) variant = "ragged pipelined";
-    } else if (fits_without_edges(p, a_kc, b_kc, 64, 64, 32) && fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
-        const int64_t groups = ((dt.M + 63) / 64) * ((dt.N + 63) / 64) * (dt.nbatch > 0 ? dt.nbatch : 1);
-        variant = (a_kc && b_kc) || groups <= 3 * (int64_t)compute_units() ? "whole pipelined" : "whole";
-    } else if (fits_ragged_pipe(p, a_kc, b_kc, 64, 64)) {
-        variant = "ragged pipelined";
-    } else if (fits_without_edges(p, a_kc, b_kc, 64, 64, 16) && fits_buffer_offsets(p, a_kc, b_kc, 64, 64)) {
-        variant = "whole";
-    }
-    return std::string("mfma ") + tile + " " + variant + " split " + std::to_string(plan.split);
+    const GemmVariant v = pick_gemm_variant(p, a_kc, b_kc, dt.nbatch > 0 ? dt.nbatch : 1, plan.tile);
+    static const char* const tiles[] = {"large", "medium", "small", "flat", "wide"};
+    static const char* const kinds[] = {"general", "whole", "whole pipelined", "ragged pipelined"};
+    std::string text = std::string("mfma ") + tiles[v.tile] + " " + kinds[v.kind];
+    if ((v.kind == kKindWholePipelined || v.kind == kKindRaggedPipelined) && v.depth > 1)
+        text += " staged " + std::to_string(v.depth);
+    return text + " split " + std::to_string(plan.split);
 }
 
 int launch_gemm(const GemmDesc& d, hipStream_t stream) {

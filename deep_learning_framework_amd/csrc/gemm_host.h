@@ -151,8 +151,110 @@ int launch_dense_backward_pair(float* pgx, float* pgw, float* pgb, const float* 
                                const float* leaky, bool acc, int split, hipStream_t stream);
 
 // per-layout entry points (one translation unit each, to compile in parallel)
-// flat: 32 rows x 128 columns; wide: 64 rows x 128 columns (whole tiles only, else the small tile runs)
+// flat: 32 rows x 128 columns; wide: 64 rows x 128 columns (pipelined kernels only, else the small tile runs)
 enum GemmTile { kTileLarge = 0, kTileMedium = 1, kTileSmall = 2, kTileFlat = 3, kTileWide = 4 };
+
+// Which kernel of a tile runs a product.  whole: predicate-free (the shape is a whole multiple of the tile, 128-bit
+// loads); ragged pipelined: range-checked buffer resources and one masked K-tile at the end; general: any strides.
+enum GemmKind { kKindGeneral = 0, kKindWhole = 1, kKindWholePipelined = 2, kKindRaggedPipelined = 3 };
+struct GemmVariant {
+    int tile;    // the tile that runs (the wide tile gives way to the small one where it has no kernel)
+    int kind;
+    int bk;      // reduction steps per tile
+    int depth;   // tiles on their way in registers (pipelined kernels: 1, 2 or 4; the others: their fixed ring)
+};
+
+// How many tiles the pipelined kernels keep on their way in registers (their DEPTH).  A load has that many tiles'
+// time to land; one tile's time is little for a workgroup that has a compute unit to itself, and too little when
+// the operand comes from HBM or the last-level cache instead of L2 (64 x 4096 x 4096 with the matrix from HBM,
+// one 64x64 workgroup per unit: 0.73 us per tile against 0.48; 512 x 4096 x 4096 on the wide tile: 139 -> 120 us
+// with four tiles in flight).  Measured over 1..8 workgroups per unit x 4..128 tiles per workgroup, both operand
+// forms, operands in L2: below 16 tiles the requests for tiles that do not exist cost 2-9 %; the small tile gains
+// 1-9 % with four tiles up to four workgroups per unit and loses 8-13 % with six or eight; the wide tile gains
+// 1-5 % with two tiles up to three workgroups per unit (and loses 14 % at four with a [K, N] operand); the two
+// big tiles gain 1-5 % with two on long reductions.
+inline int staging_depth(int tile, const GemmParams& p, int64_t groups, int64_t nbatch, int bk) {
+    const int64_t k_len = p.k_part > 0 ? p.k_part : p.K;
+    const int64_t tiles_k = k_len / bk;
+    const int64_t cus = compute_units();
+    const bool streamed = (int64_t)(p.M > p.N ? p.M : p.N) * k_len * nbatch * 4 >= (32ll << 20);
+    switch (tile) {
+    case kTileSmall:
+        return (tiles_k >= 32 && groups <= 4 * cus) || (tiles_k >= 16 && groups <= 2 * cus) ? 4 : 1;
+    case kTileWide:
+        if (streamed && tiles_k >= 32 && groups <= 2 * cus) return 4;
+        return tiles_k >= 16 && groups <= 3 * cus ? 2 : 1;
+    case kTileMedium:
+        return tiles_k >= 32 && groups <= 2 * cus ? 2 : 1;
+    default:   // large (256 x 256 x 16), flat with edges
+        return tiles_k >= 32 ? 2 : 1;
+    }
+}
+
+// The kernel that launch_gemm_layout starts for a tile choice (host arithmetic only).
+inline GemmVariant pick_gemm_variant(const GemmParams& p, bool a_kc, bool b_kc, int64_t nbatch, int tile) {
+    auto whole = [&](int bm, int bn, int bk) {
+        return fits_without_edges(p, a_kc, b_kc, bm, bn, bk) && fits_buffer_offsets(p, a_kc, b_kc, bm, bn);
+    };
+    auto groups = [&](int bm, int bn) { return (int64_t)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * nbatch; };
+    switch (tile) {
+    case kTileLarge:
+        if (whole(256, 256, 16)) return {tile, kKindWholePipelined, 16, staging_depth(tile, p, 0, nbatch, 16)};
+        if (fits_ragged_pipe(p, a_kc, b_kc, 256, 256))
+            return {tile, kKindRaggedPipelined, 16, staging_depth(tile, p, 0, nbatch, 16)};
+        return {tile, kKindGeneral, 16, 1};
+    case kTileMedium:
+        if (whole(128, 128, 32))
+            return {tile, kKindWholePipelined, 32, staging_depth(tile, p, groups(128, 128), nbatch, 32)};
+        if (fits_ragged_pipe(p, a_kc, b_kc, 128, 128))
+            return {tile, kKindRaggedPipelined, 32, staging_depth(tile, p, groups(128, 128), nbatch, 32)};
+        return {tile, kKindGeneral, 16, 1};
+    case kTileFlat:
+        // at most 32 rows against many columns (a batch of 17..32 rows against a weight matrix): four waves side
+        // by side, so that the matrix cores do not spend half their time on rows that do not exist.  With edges
+        // the pipelined schedule is the faster one (80 x 4096 x 4096: 41.2 -> 36.6 us, 72 x 4096 x 11008:
+        // 88.6 -> 79.9, 17 and 24 rows 22.9 -> 22.4); whole tiles lose with it (32 x 11008 x 4096: 50 -> 65: the
+        // stream of the other operand wants the four tiles in flight that the simple schedule keeps)
+        if (whole(32, 128, 32)) return {tile, kKindWhole, 32, 4};
+        if (fits_ragged_pipe(p, a_kc, b_kc, 32, 128))
+            return {tile, kKindRaggedPipelined, 32, staging_depth(tile, p, 0, nbatch, 32)};
+        return {tile, kKindGeneral, 32, 4};
+    case kTileWide:
+        if (whole(64, 128, 32))
+            return {tile, kKindWholePipelined, 32, staging_depth(tile, p, groups(64, 128), nbatch, 32)};
+        if (fits_ragged_pipe(p, a_kc, b_kc, 64, 128))
+            return {tile, kKindRaggedPipelined, 32, staging_depth(tile, p, groups(64, 128), nbatch, 32) >= 2 ? 2 : 1};
+        [[fallthrough]];
+    default: {
+        // The pipelined schedule (fragment reads and LDS stores dealt between the MFMAs).  Both operands
+        // K-contiguous: a 32-step tile takes 0.48 us whether the workgroup has the compute unit to itself or not,
+        // the simple schedule 0.53-0.70 (1024^3: 22.6 -> 18.9 us, 512 x 2048 x 2048: 41.0 -> 34.2,
+        // 64 x 4096 x 4096: 27.2 -> 22.8).  An operand that is not K-contiguous takes four LDS reads per fragment
+        // instead of one: the pipelined schedule still wins while at most three workgroups share a unit
+        // (1024^3 23.7 -> 21.8, 128 x 2048 x 2048 18.0 -> 16.5) and loses beyond (3072^3: 420 -> 432).
+        const int64_t small_tiles = groups(64, 64);
+        const bool pipelined = (a_kc && b_kc) || small_tiles <= 3 * (int64_t)compute_units();
+        if (whole(64, 64, 32)) {
+            if (pipelined) return {kTileSmall, kKindWholePipelined, 32, staging_depth(kTileSmall, p, small_tiles, nbatch, 32)};
+            // a 64x64x16 tile computes for ~0.25 us, a global load takes ~1-2 us: 128 reduction steps in flight
+            // (measured with whole tiles of 32 steps against 16 and 64: 15.5 / 16.9 / 16.0 us for 256x1024x1024)
+            return {kTileSmall, kKindWhole, 32, 4};
+        }
+        // shapes with edges: the pipelined schedule in every operand form (777^3 with a [K, N] operand
+        // 24.2 -> 19.1 us, 200 x 200 x 8192 20.5 -> 16.5)
+        if (fits_ragged_pipe(p, a_kc, b_kc, 64, 64))
+            return {kTileSmall, kKindRaggedPipelined, 32, staging_depth(kTileSmall, p, small_tiles, nbatch, 32)};
+        if (whole(64, 64, 16)) return {kTileSmall, kKindWhole, 16, 8};
+        // 32-step tiles halve the number of rounds; with an operand that is strided in both directions (one
+        // head of an interleaved tensor) the element-wise loads of a tile cost more than the round saves
+        // (measured: 1000x777x333 28.8 -> 26.7 us, head-strided 512x512x64 26 -> 32 us)
+        if (p.K >= 128 && (p.a_ks == 1 || p.a_rs == 1) && (p.b_ks == 1 || p.b_rs == 1))
+            return {kTileSmall, kKindGeneral, 32, 4};
+        return {kTileSmall, kKindGeneral, 16, 4};
+    }
+    }
+}
+
 int launch_gemm_kc_kc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
 int launch_gemm_kc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);
 int launch_gemm_mc_mc(const GemmParams& p, int64_t nbatch, int tile, hipStream_t stream);

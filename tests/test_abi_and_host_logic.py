@@ -223,14 +223,14 @@ GEMM_PLANS = [
     ((0, 1, 256, 1024, 1024), "wavesplit 32"),                       # configuration 2 forward
     ((0, 0, 256, 1024, 1024), "wavesplit 32"),                       # configuration 2 dX: one operand not K-contiguous
     ((1, 0, 1024, 1024, 256), "mfma small whole pipelined split 1"),           # configuration 2 dW: 256 tiles of 64 x 64
-    ((0, 0, 8192, 8192, 8192), "mfma large whole pipelined split 1"),  # the headline product
-    ((0, 1, 8192, 8192, 8192), "mfma large whole pipelined split 1"),
-    ((0, 0, 8191, 8191, 8191), "mfma large ragged pipelined split 1"),  # odd sizes keep the pipelined loop
+    ((0, 0, 8192, 8192, 8192), "mfma large whole pipelined staged 2 split 1"),  # the headline product
+    ((0, 1, 8192, 8192, 8192), "mfma large whole pipelined staged 2 split 1"),
+    ((0, 0, 8191, 8191, 8191), "mfma large ragged pipelined staged 2 split 1"),  # odd sizes keep the pipelined loop
     ((0, 1, 4100, 4100, 4100), "mfma small ragged pipelined split 1"),   # edges in every dimension: 4225 small tiles (17 rounds) rather than 1089 medium ones (2 + 2 + 1)
-    ((0, 1, 4096, 4096, 4096), "mfma large whole pipelined split 1"),   # exactly one round of large tiles
+    ((0, 1, 4096, 4096, 4096), "mfma large whole pipelined staged 2 split 1"),   # exactly one round of large tiles
     ((0, 1, 3072, 4096, 4096), "mfma medium whole pipelined split 1"),  # 192 large tiles leave a quarter of the chip idle
-    ((0, 1, 2048, 2048, 2048), "mfma medium whole pipelined split 1"),
-    ((0, 1, 1024, 2048, 512), "mfma wide whole pipelined split 1"),   # 128 medium tiles on 256 units: 256 wide ones
+    ((0, 1, 2048, 2048, 2048), "mfma medium whole pipelined staged 2 split 1"),
+    ((0, 1, 1024, 2048, 512), "mfma wide whole pipelined staged 2 split 1"),   # 128 medium tiles on 256 units: 256 wide ones
     ((0, 1, 1, 4096, 4096), "skinny"),                               # configuration 5
     ((0, 1, 4, 4096, 4096), "skinny"),
     ((0, 1, 16, 4096, 4096), "skinny"),
@@ -241,24 +241,24 @@ GEMM_PLANS = [
     ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
     ((0, 1, 1000, 333, 777), "mfma small ragged pipelined split 2"),   # configuration 5, ragged: two rounds of the one-launch kernel would take longer
     ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
-    ((0, 1, 17, 11008, 4096), "mfma flat ragged pipelined split 2"),          # one workgroup per compute unit: 86 tiles x 2
+    ((0, 1, 17, 11008, 4096), "mfma flat ragged pipelined staged 2 split 2"),          # one workgroup per compute unit: 86 tiles x 2
     ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
-    ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
+    ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
     ((0, 1, 96, 4096, 4096), "mfma flat whole split 8"),             # 65..96 rows: three row tiles of 32, not two of 64
-    ((0, 1, 64, 64, 8192), "mfma small whole pipelined split 16"),             # one tile, a long reduction
+    ((0, 1, 64, 64, 8192), "mfma small whole pipelined staged 4 split 16"),             # one tile, a long reduction
     ((0, 1, 768, 768, 4096), "mfma medium ragged pipelined split 7"),   # 36 medium tiles x 7 parts of 592 steps: one workgroup per unit
-    ((0, 1, 1024, 1024, 8192), "mfma medium whole pipelined split 4"),   # 64 medium tiles x 4 parts of 2048 steps
-    ((0, 1, 1024, 1024, 1024), "mfma small whole pipelined split 1"),   # 256 small tiles, one per unit, on the pipelined schedule
+    ((0, 1, 1024, 1024, 8192), "mfma medium whole pipelined staged 2 split 4"),   # 64 medium tiles x 4 parts of 2048 steps
+    ((0, 1, 1024, 1024, 1024), "mfma small whole pipelined staged 4 split 1"),   # 256 small tiles, one per unit, on the pipelined schedule
     ((0, 1, 128, 128, 4096), "mfma small whole pipelined split 16"),   # too long for the one-launch kernel
-    ((0, 0, 512, 4096, 4096), "mfma wide whole pipelined split 1"),   # a [K, N] operand: the 64 x 128 tile, one per unit
-    ((1, 0, 512, 4096, 4096), "mfma wide whole pipelined split 1"),
-    ((0, 1, 512, 4096, 4096), "mfma wide whole pipelined split 1"),
-    ((0, 1, 256, 4096, 4096), "mfma small whole pipelined split 1"),   # 256 small tiles, one per unit, four tiles of K on their way each
-    ((0, 1, 1000, 1000, 1000), "mfma small ragged pipelined split 1"),
-    ((0, 0, 1000, 1000, 1000), "mfma small ragged pipelined split 1"),
+    ((0, 0, 512, 4096, 4096), "mfma wide whole pipelined staged 4 split 1"),   # a [K, N] operand: the 64 x 128 tile, one per unit
+    ((1, 0, 512, 4096, 4096), "mfma wide whole pipelined staged 4 split 1"),
+    ((0, 1, 512, 4096, 4096), "mfma wide whole pipelined staged 4 split 1"),
+    ((0, 1, 256, 4096, 4096), "mfma small whole pipelined staged 4 split 1"),   # 256 small tiles, one per unit, four tiles of K on their way each
+    ((0, 1, 1000, 1000, 1000), "mfma small ragged pipelined staged 4 split 1"),
+    ((0, 0, 1000, 1000, 1000), "mfma small ragged pipelined staged 4 split 1"),
     ((0, 1, 600, 600, 6000), "mfma medium ragged pipelined split 10"),  # 25 medium tiles x 10 parts: parts need not be a power of two
-    ((0, 0, 72, 4096, 11008), "mfma medium ragged pipelined split 8"),  # 65..96 rows that are no multiple of 32, [K, N] operand
-    ((0, 1, 72, 4096, 11008), "mfma flat ragged pipelined split 8"),
+    ((0, 0, 72, 4096, 11008), "mfma medium ragged pipelined staged 2 split 8"),  # 65..96 rows that are no multiple of 32, [K, N] operand
+    ((0, 1, 72, 4096, 11008), "mfma flat ragged pipelined staged 2 split 8"),
     ((0, 1, 0, 5, 5), "nothing"),
 ]
 

@@ -865,6 +865,55 @@ def test_split_k_with_a_large_output(m, n, k, bias_act):
     check(got, ref_all.astype(np.float32), what="split-K %dx%dx%d whole output" % (m, n, k))
 
 
+# The pipelined kernels keep one, two or four tiles on their way in registers; the loop over the tiles is
+# unrolled over those sets, with whole rounds and a remainder.  One case per (tile, variant, depth) and, across
+# the reduction lengths, every remainder of the tile count, with and without a masked last tile.
+STAGED = [
+    ((1024, 1024, 512), "small whole pipelined staged 4"), ((1024, 1024, 544), "small whole pipelined staged 4"),
+    ((1024, 1024, 576), "small whole pipelined staged 4"), ((1024, 1024, 608), "small whole pipelined staged 4"),
+    ((1000, 1000, 1013), "small ragged pipelined staged 4"), ((1000, 1000, 1050), "small ragged pipelined staged 4"),
+    ((999, 1001, 1090), "small ragged pipelined staged 4"), ((1001, 999, 1120), "small ragged pipelined staged 4"),
+    ((1024, 2048, 512), "wide whole pipelined staged 2"), ((1024, 2048, 544), "wide whole pipelined staged 2"),
+    ((512, 4096, 4096), "wide whole pipelined staged 4"), ((512, 4096, 4128), "wide whole pipelined staged 4"),
+    ((512, 4096, 4160), "wide whole pipelined staged 4"), ((512, 4096, 4192), "wide whole pipelined staged 4"),
+    ((1000, 2000, 1111), "wide ragged pipelined staged 2"), ((1000, 2000, 1150), "wide ragged pipelined staged 2"),
+    ((2048, 2048, 1024), "medium whole pipelined staged 2"), ((2048, 2048, 1056), "medium whole pipelined staged 2"),
+    ((2000, 2000, 1050), "medium ragged pipelined staged 2"), ((2000, 2000, 1100), "medium ragged pipelined staged 2"),
+    ((4096, 4096, 512), "large whole pipelined staged 2"), ((4096, 4096, 528), "large whole pipelined staged 2"),
+    ((4000, 4000, 530), "large ragged pipelined staged 2"), ((4000, 4000, 550), "large ragged pipelined staged 2"),
+    ((24, 8192, 4100), "flat ragged pipelined staged 2"), ((31, 16384, 2100), "flat ragged pipelined staged 2"),
+]
+
+
+@pytest.mark.parametrize("shape,variant", STAGED, ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else v.replace(" ", "_"))
+def test_staged_tiles_every_remainder(shape, variant):
+    m, n, k = shape
+    rng = np.random.default_rng(m * 7 + n * 3 + k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    sample = sorted(set([0, 1, m // 3, m - 2, m - 1] + list(range(5, m, max(1, m // 12)))))
+    for ta, tb in ((0, 1), (0, 0), (1, 0)):
+        assert variant in VMath.gemm_plan(ta, tb, m, n, k), VMath.gemm_plan(ta, tb, m, n, k)
+        a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+        b = rng.uniform(-0.05, 0.05, (n, k) if tb else (k, n)).astype(np.float32)
+        c = DB(m * n * 4)
+        VMath.fill_float(0, c, m * n, 77.0)
+        VMath.gemm_f32(0, ta, tb, m, n, k, dev(a), a.shape[1], dev(b), b.shape[1], c, n, dev(bias), kai.ACT["relu"], None, False)
+        got = c.to_numpy((m, n))
+        a64 = (a.T if ta else a).astype(np.float64)
+        b64 = (b.T if tb else b).astype(np.float64)
+        ref_all = np.maximum(a64 @ b64 + bias, 0.0).astype(np.float32)
+        if (ta, tb) == (0, 1):
+            ref_rows = ko.matmul_rows(b, a, sample)
+        elif (ta, tb) == (0, 0):
+            ref_rows = ko.matmul_backward_x(np.ascontiguousarray(a[sample]), b)
+        else:
+            ref_rows = ko.matmul_backward_w(np.ascontiguousarray(a[:, sample]), b, len(sample), n)
+        ref_rows = ko.activate(ko.add_bias(ref_rows, bias), "relu")
+        what = "%dx%dx%d form %d%d" % (m, n, k, ta, tb)
+        check(got[sample], ref_rows, what=what + " sampled rows")
+        check(got, ref_all, what=what + " whole output")
+
+
 def test_scratch_growth_does_not_wait_for_the_device():
     # Growth allocates the larger buffer and keeps the old one: no device-wide wait, no free.  Shown by
     # queueing ~0.1 s of products, then issuing a call that makes the scratch grow: it returns while the queue
