@@ -12,8 +12,8 @@
 // the first blocks_x workgroups compute gx (its reduction over yvec cut into parts so that a part is about as
 // long as the reduction of gw), the next compute gw, the last few sum the columns of ga (one thread per column,
 // rows ascending: the order of a sequential loop).  Workgroups are dealt out in id order, so the compute units
-// hold workgroups of both products side by side.  Both products run the tile loop of gemm_mfma.h (64 x 64 tile,
-// four waves, 32 reduction steps per tile, four tiles in flight) with the masked A operand; they share one LDS
+// hold workgroups of both products side by side.  Both products run the pipelined tile loop of gemm_mfma.h (64 rows
+// x 64 or 128 columns, four waves, 32 reduction steps per tile) with the masked A operand; they share one LDS
 // allocation.
 #include <algorithm>
 #include <string>
@@ -25,13 +25,17 @@ namespace kai {
 
 namespace {
 
-constexpr int kPairTile = 64, kPairBK = 32, kPairDepth = 4;
-using PairAx = TileShape<true, kPairTile, kPairBK>;    // gx: A = gy, reduction index contiguous
-using PairBx = TileShape<false, kPairTile, kPairBK>;   //     B = w, output index contiguous
-using PairAw = TileShape<false, kPairTile, kPairBK>;   // gw: A = gy^T, B = x, both output index contiguous
-using PairBw = TileShape<false, kPairTile, kPairBK>;
-constexpr int kPairLdsX = 2 * (PairAx::kFloats + PairBx::kFloats), kPairLdsW = 2 * (PairAw::kFloats + PairBw::kFloats);
-constexpr int kPairLds = kPairLdsX > kPairLdsW ? kPairLdsX : kPairLdsW;
+constexpr int kPairTile = 64, kPairBK = 32;
+// The tiles are 64 rows x BN columns of gx or gw (BN = 128 where xvec allows: a third less to load per flop).
+template <int BN>
+struct PairTiles {
+    using Ax = TileShape<true, kPairTile, kPairBK>;    // gx: A = gy, reduction index contiguous
+    using Bx = TileShape<false, BN, kPairBK>;          //     B = w, output index contiguous
+    using Aw = TileShape<false, kPairTile, kPairBK>;   // gw: A = gy^T, B = x, both output index contiguous
+    using Bw = TileShape<false, BN, kPairBK>;
+    static constexpr int kLdsX = 2 * (Ax::kFloats + Bx::kFloats), kLdsW = 2 * (Aw::kFloats + Bw::kFloats);
+    static constexpr int kLds = kLdsX > kLdsW ? kLdsX : kLdsW;
+};
 
 // The bias gradient of 64 columns: gb[c] (=|+=) sum over the rows of gy[m,c] * f'(pre[m,c]), rows ascending (the
 // order of the reference's sequential loop, so the sum is bit-identical to it).  All 256 threads fetch blocks of
@@ -80,29 +84,32 @@ __device__ __forceinline__ void masked_colsum_64(const GemmParams& pw, int col0,
 
 // blockIdx.x < blocks_b: 64 columns of the bias gradient (first, so that these light workgroups run beside the
 // others from the start); then blocks_x tiles of the parts of gx; then the tiles of gw.
-static_assert(kColsumRows * 64 <= kPairLds, "the column-sum block must fit the shared LDS allocation");
+template <int BN, int DEPTH>
 __global__ void __launch_bounds__(256, 2)
     dense_backward_pair_kernel(const GemmParams px, const GemmParams pw, const int blocks_b, const int blocks_x,
                                const int tiles_x) {
-    __shared__ __attribute__((aligned(16))) float lds[kPairLds];
+    using T = PairTiles<BN>;
+    static_assert(kColsumRows * 64 <= T::kLds, "the column-sum block must fit the shared LDS allocation");
+    constexpr int NBN = BN / 64;
+    __shared__ __attribute__((aligned(16))) float lds[T::kLds];
     const int bid = (int)blockIdx.x - blocks_b;
     if (bid < 0) {
         masked_colsum_64(pw, (int)blockIdx.x * 64, lds);
     } else if (bid < blocks_x) {
-        gemm_tile_body<2, 2, 1, 1, kPairBK, true, false, false, 0, kPairDepth, false, true>(
-            px, bid % tiles_x, bid / tiles_x, reinterpret_cast<float(*)[PairAx::kFloats]>(lds),
-            reinterpret_cast<float(*)[PairBx::kFloats]>(lds + 2 * PairAx::kFloats));
+        gemm_tile_body<2, 2, 1, NBN, kPairBK, true, false, false, 1, DEPTH, false, true>(
+            px, bid % tiles_x, bid / tiles_x, reinterpret_cast<float(*)[T::Ax::kFloats]>(lds),
+            reinterpret_cast<float(*)[T::Bx::kFloats]>(lds + 2 * T::Ax::kFloats));
     } else {
-        gemm_tile_body<2, 2, 1, 1, kPairBK, false, false, false, 0, kPairDepth, false, true>(
-            pw, bid - blocks_x, 0, reinterpret_cast<float(*)[PairAw::kFloats]>(lds),
-            reinterpret_cast<float(*)[PairBw::kFloats]>(lds + 2 * PairAw::kFloats));
+        gemm_tile_body<2, 2, 1, NBN, kPairBK, false, false, false, 1, DEPTH, false, true>(
+            pw, bid - blocks_x, 0, reinterpret_cast<float(*)[T::Aw::kFloats]>(lds),
+            reinterpret_cast<float(*)[T::Bw::kFloats]>(lds + 2 * T::Aw::kFloats));
     }
 }
 
-GemmParams pair_params(const GemmDesc& d, bool a_kc, bool b_kc) {
+GemmParams pair_params(const GemmDesc& d, bool a_kc, bool b_kc, int bn) {
     GemmParams p = make_params(d, a_kc, b_kc);
     p.tiles_m = (p.M + kPairTile - 1) / kPairTile;
-    p.tiles_n = (p.N + kPairTile - 1) / kPairTile;
+    p.tiles_n = (p.N + bn - 1) / bn;
     p.group_m = 4;
     p.edge_buf = 1;
     return p;
@@ -160,9 +167,15 @@ int launch_dense_backward_pair(float* pgx, float* pgw, float* pgb, const float* 
     dw.M = yvec; dw.N = xvec; dw.K = ndat;
     dw.a_rs = 1; dw.a_ks = yvec; dw.b_rs = 1; dw.b_ks = xvec; dw.c_rs = xvec; dw.c_cs = 1;
     dw.acc = acc;
-    GemmParams gx = pair_params(dx, true, false), gw = pair_params(dw, false, false);
-    if (!fits_without_edges(gx, true, false, kPairTile, kPairTile, kPairBK) || !fits_buffer_offsets(gx, true, false, kPairTile, kPairTile) ||
-        !fits_without_edges(gw, false, false, kPairTile, kPairTile, kPairBK) || !fits_buffer_offsets(gw, false, false, kPairTile, kPairTile))
+    // 128 columns per tile where that still gives every compute unit a workgroup (batch 256, 1024 -> 1024: 19.8 ->
+    // 18.5 us; 512^3 with its 64 wide tiles: 16.1 -> 21.4); more than one tile on its way in registers from eight
+    // tiles per workgroup on (batch 128, 1024 -> 1024 with four: 13.4 -> 13.7 us)
+    const int64_t wide_blocks = (ndat / kPairTile) * (xvec / 128) * split + (yvec / kPairTile) * (xvec / 128);
+    const int bn = xvec % 128 == 0 && wide_blocks >= compute_units() ? 128 : kPairTile;
+    const bool deep = yvec / split / kPairBK >= 8 && ndat / kPairBK >= 8;
+    GemmParams gx = pair_params(dx, true, false, bn), gw = pair_params(dw, false, false, bn);
+    if (!fits_without_edges(gx, true, false, kPairTile, bn, kPairBK) || !fits_buffer_offsets(gx, true, false, kPairTile, bn) ||
+        !fits_without_edges(gw, false, false, kPairTile, bn, kPairBK) || !fits_buffer_offsets(gw, false, false, kPairTile, bn))
         return fail(KAI_ERR_INVALID_ARGUMENT, "dense backward: shape does not fit the paired launch");
     gx.A2 = ppre; gx.a_mask = a_mask; gx.leaky = leaky;
     gw.A2 = ppre; gw.a_mask = a_mask; gw.leaky = leaky;
@@ -170,8 +183,11 @@ int launch_dense_backward_pair(float* pgx, float* pgw, float* pgb, const float* 
     const int tiles_x = gx.tiles_m * gx.tiles_n, tiles_w = gw.tiles_m * gw.tiles_n;
     const int blocks_x = tiles_x * split;
     const int blocks_b = pgb ? (int)(yvec / 64) : 0;
-    dense_backward_pair_kernel<<<dim3((unsigned)(blocks_b + blocks_x + tiles_w)), dim3(256), 0, stream>>>(
-        gx, gw, blocks_b, blocks_x, tiles_x);
+    const dim3 grid((unsigned)(blocks_b + blocks_x + tiles_w));
+    if (bn == 128 && deep) dense_backward_pair_kernel<128, 2><<<grid, dim3(256), 0, stream>>>(gx, gw, blocks_b, blocks_x, tiles_x);
+    else if (bn == 128) dense_backward_pair_kernel<128, 1><<<grid, dim3(256), 0, stream>>>(gx, gw, blocks_b, blocks_x, tiles_x);
+    else if (deep) dense_backward_pair_kernel<64, 4><<<grid, dim3(256), 0, stream>>>(gx, gw, blocks_b, blocks_x, tiles_x);
+    else dense_backward_pair_kernel<64, 1><<<grid, dim3(256), 0, stream>>>(gx, gw, blocks_b, blocks_x, tiles_x);
     KAI_TRY(check_launch("dense_backward_pair_kernel"));
     if (split > 1) {
         SplitReduceParams r{};

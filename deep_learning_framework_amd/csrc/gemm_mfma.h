@@ -566,7 +566,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 // over K, one thread per row reading the tile from LDS, k ascending across tiles: a fixed order
 // that is the order of a sequential loop.
 //
-// AMASK (PIPE 0, whole tiles only): the A tile is multiplied element by element with the derivative of
+// AMASK (whole tiles only): the A tile is multiplied element by element with the derivative of
 // relu / leaky relu at a second tensor A2 of the same layout on its way to LDS (GemmParams::a_mask): the
 // backward products of a dense layer read the output gradient and the pre-activation directly.
 //
@@ -587,7 +587,7 @@ __device__ __forceinline__ void gemm_tile_body(
     constexpr int NCHB = TB::kChunks / NT;
     static_assert(TA::kChunks % NT == 0 && TB::kChunks % NT == 0, "tile must divide over the threads");
     static_assert(BK % 8 == 0, "BK must hold whole groups of 8 k");
-    static_assert(!AMASK || (PIPE == 0 && !EDGE), "the masked A operand exists for whole tiles on the simple schedule");
+    static_assert(!AMASK || !EDGE, "the masked A operand exists for whole tiles only");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -860,8 +860,32 @@ __device__ __forceinline__ void gemm_tile_body(
                 load_global(kt);
             }
         };
+        // AMASK: the pre-activation tile kt into the registers beside staging set `set`; mask_chunk turns chunk i
+        // of that set into A * f'(A2) on its way to LDS
+        auto load_a2_chunk = [&](int kt, auto setc, int i) {
+            if constexpr (AMASK)
+                load_tile_chunk_buf<A_KC, BM, BK, NT>(rax2[decltype(setc)::value], rsrc_a2, kt * BK * (int)p.a_ks * 4,
+                                                      (int)a_ld * 4, (int)toff_a * 4, i);
+        };
+        auto mask_chunk = [&](auto setc, int i) {
+            if constexpr (AMASK) {
+                constexpr int set = decltype(setc)::value;
+                if (a_masked) {   // uniform
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        rax[set][i][j] = ((rax2[set][i][j] > 0) ? 1.0f : a_mask_slope) * rax[set][i][j];
+                }
+            }
+        };
+        constexpr std::integral_constant<int, 0> set0{};
         if (nkt > 0) {
             load_whole(0);
+            if constexpr (AMASK) {
+#pragma unroll
+                for (int i = 0; i < NCHA; i++) load_a2_chunk(0, set0, i);
+#pragma unroll
+                for (int i = 0; i < NCHA; i++) mask_chunk(set0, i);
+            }
             store_tile_lds<A_KC, BM, BK, NT>(lds_a[0], ra, tid);
             store_tile_lds<B_KC, BN, BK, NT>(lds_b[0], rb, tid);
         }
@@ -892,12 +916,20 @@ __device__ __forceinline__ void gemm_tile_body(
                             read_frag_piece<B_KC, NBN, BN, BK>(fb[fill], lds_b[rbuf], wn0, rkg, l32, half, sl - kReadsA);
                     }
                     if (store && sl < kWrites) {
-                        if (sl < NCHA) store_tile_chunk<A_KC, BM, BK, NT>(lds_a[wbuf], ra, tid, sl);
-                        else store_tile_chunk<B_KC, BN, BK, NT>(lds_b[wbuf], rb, tid, sl - NCHA);
+                        if (sl < NCHA) {
+                            if constexpr (AMASK) mask_chunk(setc, sl);
+                            store_tile_chunk<A_KC, BM, BK, NT>(lds_a[wbuf], ra, tid, sl);
+                        } else {
+                            store_tile_chunk<B_KC, BN, BK, NT>(lds_b[wbuf], rb, tid, sl - NCHA);
+                        }
                     }
                     if (gload && sl < kWrites) {
-                        if (sl < NCHA) load_tile_chunk_buf<A_KC, BM, BK, NT>(ra, rsrc_a, ga_off, (int)a_ld * 4, (int)toff_a * 4, sl);
-                        else load_tile_chunk_buf<B_KC, BN, BK, NT>(rb, rsrc_b, gb_off, (int)b_ld * 4, (int)toff_b * 4, sl - NCHA);
+                        if (sl < NCHA) {
+                            load_tile_chunk_buf<A_KC, BM, BK, NT>(ra, rsrc_a, ga_off, (int)a_ld * 4, (int)toff_a * 4, sl);
+                            if constexpr (AMASK) load_a2_chunk(gkt, setc, sl);
+                        } else {
+                            load_tile_chunk_buf<B_KC, BN, BK, NT>(rb, rsrc_b, gb_off, (int)b_ld * 4, (int)toff_b * 4, sl - NCHA);
+                        }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     // fewer MFMAs than slots (one block per wave and an operand whose fragments take four reads):
@@ -931,9 +963,14 @@ __device__ __forceinline__ void gemm_tile_body(
         // them into the free LDS buffer, one store per slot; the last group refills them with tile
         // kt+2, one global load per slot, so that the waves of a workgroup never queue all their
         // loads on the address unit at once and every load has most of a tile to land.
-        constexpr std::integral_constant<int, 0> set0{};
         if constexpr (DEPTH == 1) {
-            if (nkt > 1) load_whole(1);
+            if (nkt > 1) {
+                load_whole(1);
+                if constexpr (AMASK) {
+#pragma unroll
+                    for (int i = 0; i < NCHA; i++) load_a2_chunk(1, set0, i);
+                }
+            }
         } else if (nkt > 0) {
             // DEPTH > 1: tile t waits in staging set t % DEPTH, requested DEPTH tiles before its turn -- the
             // workgroups that have a compute unit to themselves and stream an operand from HBM need that much
@@ -945,6 +982,10 @@ __device__ __forceinline__ void gemm_tile_body(
 #pragma unroll
                 for (int i = 0; i < NCHA; i++)
                     load_tile_chunk_buf<A_KC, BM, BK, NT>(rax[d % DEPTH], rsrc_a, kt * BK * (int)p.a_ks * 4, (int)a_ld * 4, (int)toff_a * 4, i);
+                if constexpr (AMASK) {
+#pragma unroll
+                    for (int i = 0; i < NCHA; i++) load_a2_chunk(kt, std::integral_constant<int, d % DEPTH>{}, i);
+                }
 #pragma unroll
                 for (int i = 0; i < NCHB; i++)
                     load_tile_chunk_buf<B_KC, BN, BK, NT>(rbx[d % DEPTH], rsrc_b, kt * BK * (int)p.b_ks * 4, (int)b_ld * 4, (int)toff_b * 4, i);

@@ -136,6 +136,7 @@ def test_dense_backward_bias_gradient_fused_or_not(ndat, yvec, xvec, acc):
 @pytest.mark.parametrize("ndat,yvec,xvec,act,acc,one_launch", [
     (256, 1024, 1024, "relu", False, True),      # configuration 2: gx cut into 4 parts of 256 steps
     (256, 1024, 1024, "leaky", True, True),
+    (128, 1024, 1024, "relu", True, True),       # 128-column tiles, 8 parts of 4 tiles: one tile staged at a time
     (64, 512, 128, "relu", True, True),          # gx cut into 4 parts of 128
     (128, 256, 320, "none", False, True),        # two parts of 128
     (512, 512, 512, "leaky", False, True),       # no cut: a part would be shorter than gw's reduction
