@@ -544,7 +544,9 @@ def test_softmax_activation_rows():
                                                       (2, 700, 8, 24), (1, 1100, 4, 6), (3, 1200, 1, 40), (1, 608, 12, 8),
                                                       # several heads per batch entry, lengths and head sizes in whole
                                                       # 32s: the kernels that take four heads per workgroup
-                                                      (2, 64, 4, 32), (1, 96, 8, 64), (3, 32, 12, 32), (4, 128, 4, 96)])
+                                                      (2, 64, 4, 32), (1, 96, 8, 64), (3, 32, 12, 32), (4, 128, 4, 96),
+                                                      # whole 128-query tiles of four heads, one workgroup per compute unit
+                                                      (4, 512, 4, 64)])
 def test_attention_ops_small(nbat, ntimes, nhead, npiece):
     nvec = nhead * npiece
     rng = np.random.default_rng(nbat * 100 + ntimes * 10 + nhead)
