@@ -64,7 +64,10 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // SLICES: K is a multiple of 8 x 512, so every wave owns the same number of slices of 512 steps and the tile loop
 // of a slice is written out (16 tiles, every wait counted exactly by the compiler): 12.2 us at M = 4 against
 // 12.9 us for the rolled loop that other lengths use.
-template <bool WHOLE, bool SLICES>
+//
+// XL (with SLICES): 1 = at most 8 rows of X (one load per tile), 2 = more (two); 0 = decided per tile from M.  With
+// the number of X loads a compile-time constant and every tile inside K, the written-out slice has no branch left.
+template <bool WHOLE, bool SLICES, int XL = 0>
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
@@ -132,7 +135,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
             const int kc = min(kt, p.K - kSsTileK) * 4;
 #pragma unroll
             for (int j = 0; j < kSsLoadsPerTile; j++)
-                if (kSsRowsPerLoad * j < p.M)   // uniform
+                if (XL ? j < XL : kSsRowsPerLoad * j < p.M)   // uniform
                     dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, xoff[j], kc, 0));
             return;
         }
@@ -145,13 +148,13 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         }
     };
     auto consume = [&](const f32x4(&w)[kSsLoadsPerTile], const f32x4(&x)[kSsLoadsPerTile], int kt) {
-        if (kt < p.K) {   // uniform
+        if ((SLICES && XL) || kt < p.K) {   // uniform
 #pragma unroll
             for (int j = 0; j < kSsLoadsPerTile; j++) {
                 const int row = kSsRowsPerLoad * j + lrow;
                 *reinterpret_cast<f32x4*>(tw + row * kSsTileStride + lk) =
                     WHOLE ? w[j] : keep_if(w[j], n0 + row < p.N && kt + lk < p.K);
-                if (kSsRowsPerLoad * j < p.M)
+                if (XL ? j < XL : kSsRowsPerLoad * j < p.M)
                     *reinterpret_cast<f32x4*>(tx + row * kSsTileStride + lk) =
                         WHOLE ? x[j] : keep_if(x[j], row < p.M && kt + lk < p.K);
             }
@@ -267,7 +270,8 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
                        ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
     const bool slices = p.K % (kSsWaves * 512) == 0;
     const dim3 grid((unsigned)blocks), block(kSsThreads);
-    if (whole && slices) skinny_stream_kernel<true, true><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    if (whole && slices && p.M <= 8) skinny_stream_kernel<true, true, 1><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (whole && slices) skinny_stream_kernel<true, true, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     else if (whole) skinny_stream_kernel<true, false><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     else skinny_stream_kernel<false, false><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     return check_launch("skinny_stream_kernel");
