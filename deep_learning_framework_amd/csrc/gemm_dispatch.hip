@@ -43,27 +43,24 @@ struct GemmPlan {
     int wavesplit_edge = 0;   // 16 or 32: the product runs on the kernel that cuts K over the waves of a workgroup
 };
 
-// Expected duration in microseconds of the wave-split kernel with T x T blocks, from measurements over 60 shapes
-// (a fixed cost, then the larger of the stream of operand bytes through the compute units' address units and
-// one wave's chain of rounds along K; an operand that is not K-contiguous adds about an eighth), or a negative
-// value outside the measured range.
-double wavesplit_estimate(const GemmDesc& d, int T, bool rounds_counted = false) {
+// Expected duration in microseconds of the wave-split kernel with T x T blocks, or a negative value outside the
+// measured range; fitted to sweeps over 64..768 rows x 256..2048 columns x 64..2048 steps in the three operand
+// forms.  Up to one workgroup per compute unit the time is one workgroup's: a floor of 3.9 us, then 2.5 ns per step
+// with 16 x 16 blocks (3.2 ns with both operands K-contiguous, the slowest form there) and 6.4 ns with 32 x 32
+// blocks.  Beyond that, every further 256 workgroups add a round that overlaps the end of the one before.
+double wavesplit_estimate(const GemmDesc& d, int T) {
     const int64_t wgs = ((d.M + T - 1) / T) * ((d.N + T - 1) / T);
-    const double K = (double)d.K;
-    const double forms = 1.0 + 0.12 * ((d.a_ks != 1) + (d.b_ks != 1));
-    if (T == 16) {
-        if (d.K > 2048 || wgs > 1024) return -1.0;
-        return (3.8 + std::max(1.3e-5 * (double)wgs * K, 3.1e-3 * std::max(0.0, K - 256.0))) * forms;
-    }
-    if (d.K > 1024 || wgs > 512 || (d.K < 256 && wgs > 256)) return -1.0;
-    if (!rounds_counted) return (4.0 + std::max(2.7e-5 * (double)wgs * K, 6.45e-3 * K)) * forms;
-    // The workgroups of 16 waves run one per compute unit at a time: beyond that many a second round follows
-    // (512 x 1024 x 256: 11.6 us against 6.5 for 512 x 512 x 256).  This closer figure is the one compared with
-    // the tiled kernels' expected time.
     const int64_t cus = compute_units();
-    const double rounds = (double)((wgs + cus - 1) / cus);
-    const double one = std::max(2.7e-5 * (double)std::min(wgs, cus) * K, 6.45e-3 * K);
-    return (4.0 + rounds * one + 3.0 * (rounds - 1.0)) * forms;
+    const double K = (double)d.K;
+    if (wgs > 1024) return -1.0;
+    const double more_rounds = (double)((wgs + cus - 1) / cus - 1);
+    if (T == 16) {
+        if (d.K > 2048) return -1.0;
+        const double per_step = (d.a_ks == 1 && d.b_ks == 1) ? 3.2e-3 : 2.5e-3;
+        return std::max(3.9, 2.9 + per_step * K) + more_rounds * 3.2e-3 * K;
+    }
+    if (d.K > 1024) return -1.0;
+    return std::max(3.9, 2.7 + 6.4e-3 * K) + 1.0e-3 * (double)std::min(wgs, cus) + more_rounds * (0.2 + 8.0e-3 * K);
 }
 
 // Number of parts for a long reduction on the 64x64 tile.  A compute unit that holds one workgroup spends
@@ -174,7 +171,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         const double limit = plan.skinny ? (d.M <= 4 ? 0.0 : 7.0) : 12.5;
         if (best > 0 && best <= limit) {
             ws_edge = take16 ? 16 : 32;
-            ws_cost = take16 ? best : wavesplit_estimate(dn, 32, true);
+            ws_cost = best;
         }
     }
 
@@ -222,11 +219,9 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         }
     }
 
-    // (the model is trusted against the one-launch kernel for the pipelined kernels only; for the simple schedule
-    // with K parts it is too optimistic at these sizes: 256 x 1024 x 777 with a [K, N] operand 13.6 us for its
-    // choice against 10.4)
-    const bool tiles_pipelined = modelled && (plan.tile != kTileSmall || (plan.a_kc && plan.b_kc));
-    if (ws_edge && !(tiles_pipelined && tiles_cost < 0.95 * ws_cost)) {
+    // (over 840 shapes x forms the choice between the two estimates is within a tenth of the faster kernel in all
+    // but eleven cases, 1.45 x at worst)
+    if (ws_edge && !(modelled && tiles_cost < 0.95 * ws_cost)) {
         plan.wavesplit_edge = ws_edge;
         modelled = false;
         plan.split = 1;

@@ -39,7 +39,8 @@ struct WaveSplitParams {
     const float* leaky;
     int M, N, K;
     int64_t a_rs, a_ks, b_rs, b_ks, ldc;
-    int tiles_n;
+    int tiles_fast;       // blocks along the output dimension that consecutive workgroups walk
+    int m_fast;           // ... which is M (else N)
     int act, accflag, has_alpha;
 };
 
@@ -54,12 +55,14 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
     return r;
 }
 
-template <int T, bool A_KC, bool B_KC>
+// U: k-groups per wave and round: for a reduction of up to eight groups per wave (T = 32: K <= 1024, T = 16:
+// K <= 2048) exactly as many as it needs, in ONE round with every load of a wave in flight at once; else four, in
+// as many rounds as K needs.
+template <int T, bool A_KC, bool B_KC, int U = kWsFlight>
 __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const WaveSplitParams p) {
     static_assert(T == 32 || T == 16, "block edge");
     constexpr int KG = T == 32 ? 8 : 16;        // k per group
     constexpr int NR = T == 32 ? 16 : 4;        // accumulator registers per lane
-    constexpr int U = kWsFlight;
     constexpr int GS = T == 32 ? kWsWaves : 1;  // distance between a wave's groups of one round
     __shared__ float red[kWsWaves * NR * 64];
 
@@ -67,7 +70,12 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
     const int lane = tid & 63, wave = tid >> 6;
     const int r = T == 32 ? (lane & 31) : (lane & 15);   // row of the block this lane feeds, for both operands
     const int kq = T == 32 ? (lane >> 5) : (lane >> 4);  // which 4 k of the group
-    const int tm = blockIdx.x / p.tiles_n, tn = blockIdx.x % p.tiles_n;
+    // Consecutive workgroups go round the eight XCDs: they walk along the output dimension with more blocks, so that
+    // an XCD's workgroups share the whole of the smaller operand and an eighth of the larger one behind its L2 (with
+    // 4 column blocks and 64 row blocks numbered column-fastest, every XCD fetched half of A: 1024 x 64 x 2048 took
+    // 13.4 us against 8.7 for 64 x 1024 x 2048)
+    const int slow = blockIdx.x / p.tiles_fast, fast = blockIdx.x % p.tiles_fast;
+    const int tm = p.m_fast ? fast : slow, tn = p.m_fast ? slow : fast;
     const int m0 = tm * T, n0 = tn * T;
     // rows past the end are read from the last row and never stored
     const float* __restrict__ arow = p.A + (int64_t)min(m0 + r, p.M - 1) * p.a_rs;
@@ -131,12 +139,17 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
                 else
                     acc[u & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(am[j], bm[j], acc[u & 1], 0, 0, 0);
             }
+            // one round of eight: the products of a group start when its two loads have landed, not when all have
+            if (U != kWsFlight) __builtin_amdgcn_sched_barrier(0);
         }
     };
     int g0 = wave * (T == 32 ? 1 : U);
     if (g0 < ngroups) {   // uniform per wave
         load(g0);
-        for (int next = g0 + U * kWsWaves; next < ngroups; next += U * kWsWaves) {
+        // every load of the round is issued before the first product (left alone, the scheduler sinks the loads
+        // to their uses to save registers: two in flight instead of sixteen)
+        __builtin_amdgcn_sched_barrier(0);
+        for (int next = g0 + U * kWsWaves; U == kWsFlight && next < ngroups; next += U * kWsWaves) {
             f32x4 a_now[U], b_now[U];
 #pragma unroll
             for (int u = 0; u < U; u++) {
@@ -202,13 +215,13 @@ bool wavesplit_applies(const GemmDesc& d) {
            d.K <= (1 << 24) && d.act >= kActNone && d.act <= kActSwish;
 }
 
-template <int T>
+template <int T, int U>
 static void launch_wavesplit_forms(const WaveSplitParams& p, bool a_kc, bool b_kc, dim3 grid, hipStream_t stream) {
     const dim3 block(64 * kWsWaves);
-    if (a_kc && b_kc) gemm_wavesplit_kernel<T, true, true><<<grid, block, 0, stream>>>(p);
-    else if (a_kc) gemm_wavesplit_kernel<T, true, false><<<grid, block, 0, stream>>>(p);
-    else if (b_kc) gemm_wavesplit_kernel<T, false, true><<<grid, block, 0, stream>>>(p);
-    else gemm_wavesplit_kernel<T, false, false><<<grid, block, 0, stream>>>(p);
+    if (a_kc && b_kc) gemm_wavesplit_kernel<T, true, true, U><<<grid, block, 0, stream>>>(p);
+    else if (a_kc) gemm_wavesplit_kernel<T, true, false, U><<<grid, block, 0, stream>>>(p);
+    else if (b_kc) gemm_wavesplit_kernel<T, false, true, U><<<grid, block, 0, stream>>>(p);
+    else gemm_wavesplit_kernel<T, false, false, U><<<grid, block, 0, stream>>>(p);
 }
 
 int launch_gemm_wavesplit(const GemmDesc& d, int block_edge, hipStream_t stream) {
@@ -220,11 +233,35 @@ int launch_gemm_wavesplit(const GemmDesc& d, int block_edge, hipStream_t stream)
     const int64_t T = block_edge;
     const int64_t tiles_m = (d.M + T - 1) / T, tiles_n = (d.N + T - 1) / T;
     if (tiles_m * tiles_n > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
-    p.tiles_n = (int)tiles_n;
+    p.m_fast = tiles_m > tiles_n;
+    p.tiles_fast = (int)(p.m_fast ? tiles_m : tiles_n);
     const dim3 grid((unsigned)(tiles_m * tiles_n));
     const bool a_kc = d.a_ks == 1, b_kc = d.b_ks == 1;
-    if (block_edge == 32) launch_wavesplit_forms<32>(p, a_kc, b_kc, grid, stream);
-    else launch_wavesplit_forms<16>(p, a_kc, b_kc, grid, stream);
+    // Up to eight groups per wave (groups of 8 k for T = 32, of 16 k for T = 16, over 16 waves): ONE round of exactly
+    // as many groups as K needs, every load of a wave in flight at once (256 x 1024 x 1024: 11.0 -> 10.6 us, the
+    // [K, N] form 10.3 -> 9.7; 64 x 512 x 2048 on 16-blocks 8.4 -> 7.4).  Exactly: a group past the end of K is
+    // loaded and multiplied all the same, and the four waves of a SIMD share its matrix core (256 x 1024 x 640 with
+    // a round of eight: 10.6 us, of five: 7.6; K <= 384 on 32-blocks took 6 us whatever K was).  Longer
+    // reductions: rounds of four.
+    const int64_t kg = block_edge == 32 ? 8 : 16;
+    const int64_t per_wave = ((d.K + kg - 1) / kg + kWsWaves - 1) / kWsWaves;
+    auto forms = [&](auto tc, auto uc) {
+        launch_wavesplit_forms<decltype(tc)::value, decltype(uc)::value>(p, a_kc, b_kc, grid, stream);
+    };
+    auto rounds = [&](auto tc) {
+        switch (per_wave) {
+        case 1: forms(tc, std::integral_constant<int, 1>{}); break;
+        case 2: forms(tc, std::integral_constant<int, 2>{}); break;
+        case 3: forms(tc, std::integral_constant<int, 3>{}); break;
+        case 5: forms(tc, std::integral_constant<int, 5>{}); break;
+        case 6: forms(tc, std::integral_constant<int, 6>{}); break;
+        case 7: forms(tc, std::integral_constant<int, 7>{}); break;
+        case 8: forms(tc, std::integral_constant<int, 8>{}); break;
+        default: forms(tc, std::integral_constant<int, kWsFlight>{}); break;
+        }
+    };
+    if (block_edge == 32) rounds(std::integral_constant<int, 32>{});
+    else rounds(std::integral_constant<int, 16>{});
     return check_launch("gemm_wavesplit_kernel");
 }
 

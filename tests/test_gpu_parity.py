@@ -989,6 +989,8 @@ WAVE_SPLIT = [
     (16, 16, 2048), (50, 70, 4), (33, 17, 1), (512, 1024, 512), (192, 1000, 1000), (9, 200, 1030), (128, 512, 260),
     # rows that start at odd float addresses (128-bit loads at 4-byte alignment) and one to three k after the rounds
     (64, 512, 783), (256, 1024, 1023), (1000, 333, 777), (130, 70, 2),
+    # one round of eight groups per wave (16 x 16 blocks: 1792 < K <= 2048; 32 x 32 blocks: 640 <= K <= 1024)
+    (40, 100, 1901), (64, 512, 2000), (256, 512, 650),
 ]
 
 
