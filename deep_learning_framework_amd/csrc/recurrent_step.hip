@@ -21,7 +21,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kRsTile = 16;     // rows and units per workgroup
 constexpr int kRsSplits = 2;    // waves along the reduction, per gate
-constexpr int kRsFlight = 4;    // chunks of 16 reduction steps a wave keeps in flight
+// chunks of 16 reduction steps a wave keeps in flight: 4 or 8 (kRsFlight template parameter), the smaller one where it
+// covers a wave's share in one round (a chunk past the end is loaded and multiplied all the same)
 
 struct RecStepParams {
     float* r;              // [ndat, nrec] output of the step
@@ -39,7 +40,7 @@ struct RecStepParams {
 
 __device__ __forceinline__ float keep_bits(float x, int keep) { return __int_as_float(__float_as_int(x) & keep); }
 
-template <int NG>
+template <int NG, int kRsFlight>
 __global__ void __launch_bounds__(64 * NG * kRsSplits) recurrent_step_kernel(RecStepParams p) {
     __shared__ float part[kRsSplits][NG][kRsTile * kRsTile];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -87,6 +88,8 @@ __global__ void __launch_bounds__(64 * NG * kRsSplits) recurrent_step_kernel(Rec
                 av[j] = *reinterpret_cast<const f32x4*>(ap + kc);
                 bv[j] = *reinterpret_cast<const f32x4*>(bp + kc);
             }
+            // every load of the round before the first product (the scheduler would sink them to their uses)
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < kRsFlight; j++) {
 #pragma unroll
@@ -156,7 +159,9 @@ template <int NG>
 int launch_step(const RecStepParams& p, hipStream_t stream) {
     const int64_t blocks = ((p.ndat + kRsTile - 1) / kRsTile) * ((p.nrec + kRsTile - 1) / kRsTile);
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "recurrent step: too many tiles");
-    recurrent_step_kernel<NG><<<dim3((unsigned)blocks), dim3(64 * NG * kRsSplits), 0, stream>>>(p);
+    const int64_t chunks = (p.nrec + 15) / 16, per = (chunks + kRsSplits - 1) / kRsSplits;
+    if (per <= 4) recurrent_step_kernel<NG, 4><<<dim3((unsigned)blocks), dim3(64 * NG * kRsSplits), 0, stream>>>(p);
+    else recurrent_step_kernel<NG, 8><<<dim3((unsigned)blocks), dim3(64 * NG * kRsSplits), 0, stream>>>(p);
     return check_launch("recurrent_step_kernel");
 }
 
