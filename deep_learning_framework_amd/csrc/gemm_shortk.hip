@@ -243,9 +243,12 @@ using TileBh = TileShape<true, kShBN, kSkK>;   // [32][68]
 // loop, which lets the compiler count the loads and stores in flight exactly (behind a branch it waits for all).
 // PAIR: one LDS buffer for the A slices instead of two, so that two workgroups share a compute unit and one
 // computes while the other waits for its stores (a second barrier per step lets the buffer be overwritten).
-template <int NG, bool WHOLE, bool PAIR>
+// ONE: the workgroup has one query tile (four steps): no slice is requested or staged beyond the fourth, at
+// compile time (the unconditional form would request three surplus slices, 96 KB per workgroup, for the four it needs).
+template <int NG, bool WHOLE, bool PAIR, bool ONE = false>
 __global__ void __launch_bounds__(kSkThreads, PAIR ? 2 : 1) shortk_heads_kernel(const GemmParams p) {
     static_assert(!WHOLE || NG * 8 == kSkK, "whole panels hold all 64 reduction steps");
+    static_assert(!ONE || WHOLE, "the one-tile form exists for whole tiles");
     __shared__ __attribute__((aligned(16))) float lds_a[PAIR ? 1 : 2][TileA::kFloats];
     __shared__ __attribute__((aligned(16))) float lds_b[kShHeads][TileBh::kFloats];
 
@@ -320,6 +323,12 @@ __global__ void __launch_bounds__(kSkThreads, PAIR ? 2 : 1) shortk_heads_kernel(
 #pragma unroll
         for (int j = 0; j < kShHeads; j++) {
             if (!WHOLE && (p.N - n0 < kShBN || p.K < kSkK)) mask_panel<kShBN>(rb[j], p.N - n0, p.K, tid);
+            // whole tiles: the scale goes into the key panel once per workgroup instead of into every output (64
+            // multiplies per lane and tile, which would take their time from the MFMAs)
+            if (WHOLE) {
+#pragma unroll
+                for (int c = 0; c < NCHB; c++) rb[j][c] *= alpha;
+            }
             store_tile_lds<true, kShBN, kSkK, kSkThreads>(lds_b[j], rb[j], tid);
         }
         stage_a(0, 0, std::integral_constant<int, 0>{});
@@ -333,18 +342,21 @@ __global__ void __launch_bounds__(kSkThreads, PAIR ? 2 : 1) shortk_heads_kernel(
         const int m0 = (tm_first + it) * kSkBM;
         const bool rows_inside = WHOLE || m0 + wm0 < p.M;   // wave-uniform
         f32x16 acc[kShHeads];
+        if (!WHOLE) {
 #pragma unroll
-        for (int j = 0; j < kShHeads; j++)
+            for (int j = 0; j < kShHeads; j++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+                for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+        }
 
         static_for<0, kShHeads>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             const int s = it * kShHeads + j;
+            constexpr bool loads = !ONE || j + AHEAD < kShHeads, stages = !ONE || j + 1 < kShHeads;
             // whole tiles: every load and LDS store is unconditional (behind a branch the compiler waits for
             // everything in flight where the paths join): past the last step the last slice comes again and a
             // surplus copy goes to LDS that nobody reads any more
-            if (WHOLE || s + 1 < nstep)
+            if (loads && (WHOLE || s + 1 < nstep))
                 load_a(min(s + AHEAD, nstep - 1), std::integral_constant<int, WHOLE ? (j + AHEAD) % kShHeads : 0>{});
             const float* la = lds_a[PAIR ? 0 : s & 1];
             if (rows_inside) {
@@ -354,13 +366,17 @@ __global__ void __launch_bounds__(kSkThreads, PAIR ? 2 : 1) shortk_heads_kernel(
                     read_frag<true, 1, kSkBM, kSkK>(fa, la, wm0, kg, l32, half);
                     read_frag<true, 1, kShBN, kSkK>(fb, lds_b[j], 0, kg, l32, half);
 #pragma unroll
-                    for (int t = 0; t < 4; t++)
-                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(0, t), fb.get(0, t), acc[j], 0, 0, 0);
+                    for (int t = 0; t < 4; t++) {
+                        // whole tiles: the first product of an accumulator starts from a zero constant (no 64 moves)
+                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa.get(0, t), fb.get(0, t),
+                                                                     (WHOLE && kg == 0 && t == 0) ? zero : acc[j], 0, 0, 0);
+                    }
                 }
             }
             // the next slice moves to LDS before this tile's stores are issued
-            if (PAIR) __syncthreads();   // every wave has read this step's slice
-            if (WHOLE || s + 1 < nstep)
+            if (PAIR && stages) __syncthreads();   // every wave has read this step's slice
+            if (stages && (WHOLE || s + 1 < nstep))
                 stage_a(min(s + 1, nstep - 1), (s + 1) & 1, std::integral_constant<int, WHOLE ? (j + 1) % kShHeads : 0>{});
             if (j + 1 < kShHeads) __syncthreads();
         });
@@ -371,7 +387,7 @@ __global__ void __launch_bounds__(kSkThreads, PAIR ? 2 : 1) shortk_heads_kernel(
                 constexpr int r = decltype(rc)::value;
                 const int row = m0 + wm0 + 8 * (r >> 2) + 4 * half + (r & 3);
                 f32x4 o = {acc[0][r], acc[1][r], acc[2][r], acc[3][r]};
-                o *= alpha;
+                if (!WHOLE) o *= alpha;
                 if (WHOLE || (row < p.M && col < p.N))
                     *reinterpret_cast<f32x4*>(Cz + (int64_t)row * p.c_rs + (int64_t)col * p.c_cs) = o;
             });
@@ -448,7 +464,8 @@ int launch_gemm_shortk_heads(GemmParams p, int64_t nbatch, hipStream_t stream) {
     const int64_t blocks = runs * p.tiles_n * hgroups * outer;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
     const dim3 grid((unsigned)blocks, 1, 1);
-    if (whole && pair) shortk_heads_kernel<8, true, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+    if (whole && pair && run == 1) shortk_heads_kernel<8, true, true, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+    else if (whole && pair) shortk_heads_kernel<8, true, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     else if (whole) shortk_heads_kernel<8, true, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     else if (p.K <= 32) shortk_heads_kernel<4, false, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     else shortk_heads_kernel<8, false, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
