@@ -288,6 +288,13 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
     xc, wc = x.cpu().numpy(), w.cpu().numpy()
     row("cfg5 ragged 1000x777x333", gpu_us(lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0)),
         flops=2.0 * m * n * k, cpu=cpu_us(lambda: ko.matmul(wc, xc)))
+    # batches of a per-shard size against a wide weight matrix (kai_matmul, the matrix warm in the caches)
+    for m, n, k in ((64, 4096, 4096), (96, 4096, 4096), (144, 4096, 4096), (256, 2048, 2048)):
+        x = torch.randn((m, k), device=dev, generator=g)
+        w = torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05
+        y = torch.empty((m, n), device=dev)
+        row("batch of %d rows: Y = X.W^T, W %d x %d (%s)" % (m, n, k, kai.VMath.gemm_plan(0, 1, m, n, k)),
+            gpu_us(lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0)), flops=2.0 * m * n * k)
     # one LSTM layer forward as the engine's loop issues it (vtensor.cpp:2455-2492): 32 steps of 64 x 256 -> 4 x 256
     nt_, nd_, ni_, nr_ = 32, 64, 256, 256
     xs = torch.randn((nt_, nd_, ni_), device=dev, generator=g)

@@ -219,6 +219,59 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         }
     }
 
+    // 129..160 rows: five rows of 32 x 128 tiles compute 160 rows where three rows of 64-row tiles compute 192.
+    // A workgroup takes 0.44 us per 32 steps (0.47 alone on its compute unit), launch and parts as above: within
+    // 4 % of the measured times at 130..160 rows against 2048..8192 columns wherever the workgroups fill their
+    // rounds (see below), 10 % low at 8192 x 8192, where the five row blocks re-read the other operand from
+    // beyond L2.  Taken where that is 7 % below the other tiles' estimate: over 57 shapes in the three operand
+    // forms 1.05 x on average (144 x 4096 x 4096 53.4 -> 49.5 us, 144 x 3072 x 4096 44.8 -> 39, 144 x 6144 x 4096
+    // 85 -> 70, 144 x 8192 x 4096 96 -> 88, 160 x 4096 x 11008 130 -> 123; ties at 2560 x 2560 and 1024 x 4096).
+    // Reductions under 2048 steps lost (4096 x 1024: 19.3 -> 21) and 11008 columns measured between 9 % slower
+    // and 8 % faster: both stay with the other tiles.
+    if (modelled && d.M > 128 && d.M <= 160 && d.N >= 1024 && d.N <= 8192 && d.K >= 2048 && d.N * d.K <= (1ll << 26)) {
+        const GemmParams pp = make_params(dn, plan.a_kc, plan.b_kc);
+        if (fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, 32, 128)) {
+            const int64_t tiles = 5 * ((d.N + 127) / 128);
+            double flat_best = 0.0;
+            int64_t flat_split = 0, flat_len = 0;
+            for (int64_t sp = 1; sp <= kSplitMax; sp++) {
+                int64_t k_len = d.K;
+                if (sp > 1) {
+                    if (d.K < kSplitFromK || sp * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) break;
+                    k_len = d.K % (16 * sp) == 0 ? d.K / sp : ((d.K + sp - 1) / sp + 15) / 16 * 16;
+                    if (k_len < 256) break;
+                    if ((d.K + k_len - 1) / k_len != sp) continue;
+                }
+                const int64_t per_cu = (tiles * sp + cus - 1) / cus;
+                // measured against the other tiles: one workgroup per compute unit +15..22 %, two 0..+13 %, where
+                // they cover at least 85 % of the units (200 of 256: -3 %, 390 and 420 of 512: -7 %); whole rounds
+                // beyond (1280 workgroups: five per unit) +5..10 %, partly filled ones -16..+10 %
+                const int64_t wgs = tiles * sp;
+                if (wgs > 2 * cus ? wgs % cus != 0 : 100 * wgs < 85 * per_cu * cus) continue;
+                // three workgroups fit a compute unit (45 KB of LDS each); a last round of one per unit lands
+                // three to a unit on a third of the chip and costs a round of two (980 workgroups of 16 steps:
+                // 37.6 us in the loop where 4 x 16 x 0.44 = 28 were expected; 1280: 35, as expected)
+                const int64_t rounds = per_cu + (per_cu > 3 && per_cu % 3 == 1 ? 1 : 0);
+                double c = (double)rounds * ((double)k_len / 32.0) * (per_cu == 1 ? 0.47 : 0.44) *
+                           (plan.a_kc && plan.b_kc ? 1.0 : 1.02);
+                if (k_len % 32 != 0) c += 1.5 * (double)per_cu;
+                c += 3.5 + (sp > 1 ? 3.5 + 0.1 * (double)sp + (double)(2 * sp + 1) * (double)(d.M * d.N) * 4.0 / 6.0e6 : 0.0);
+                if (flat_split == 0 || c < 0.98 * flat_best) {
+                    flat_best = c;
+                    flat_split = sp;
+                    flat_len = k_len;
+                }
+            }
+            if (flat_split > 0 && flat_best < 0.93 * tiles_cost) {
+                tiles_cost = flat_best;
+                plan.tile = kTileFlat;
+                plan.split = flat_split;
+                plan.k_part = flat_split > 1 ? flat_len : 0;
+                plan.ragged_parts = flat_split > 1 && d.K % (16 * flat_split) != 0;
+            }
+        }
+    }
+
     // (over 840 shapes x forms the choice between the two estimates is within a tenth of the faster kernel in all
     // but eleven cases, 1.45 x at worst)
     if (ws_edge && !(modelled && tiles_cost < 0.95 * ws_cost)) {

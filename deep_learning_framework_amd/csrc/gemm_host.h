@@ -213,9 +213,12 @@ inline GemmVariant pick_gemm_variant(const GemmParams& p, bool a_kc, bool b_kc, 
         // at most 32 rows against many columns (a batch of 17..32 rows against a weight matrix): four waves side
         // by side, so that the matrix cores do not spend half their time on rows that do not exist.  With edges
         // the pipelined schedule is the faster one (80 x 4096 x 4096: 41.2 -> 36.6 us, 72 x 4096 x 11008:
-        // 88.6 -> 79.9, 17 and 24 rows 22.9 -> 22.4); whole tiles lose with it (32 x 11008 x 4096: 50 -> 65: the
-        // stream of the other operand wants the four tiles in flight that the simple schedule keeps)
-        if (whole(32, 128, 32)) return {tile, kKindWhole, 32, 4};
+        // 88.6 -> 79.9, 17 and 24 rows 22.9 -> 22.4), and so it is with whole tiles in several rows of tiles
+        // (96 x 4096 x 4096: 35.7 -> 33.1 us, 96 x 2048 x 2048 17.9 -> 15.9, 96 x 4096 x 11008 76.2 -> 72.6,
+        // 160 x 4096 x 4096 56.4 -> 52.0; the variant without range checks measured the same as the one with
+        // them, so there is only the latter); one row of whole tiles loses with it (32 x 11008 x 4096:
+        // 50 -> 65: the stream of the other operand wants the four tiles in flight that the simple schedule keeps)
+        if (whole(32, 128, 32) && p.M <= 32) return {tile, kKindWhole, 32, 4};
         if (fits_ragged_pipe(p, a_kc, b_kc, 32, 128))
             return {tile, kKindRaggedPipelined, 32, staging_depth(tile, p, 0, nbatch, 32)};
         return {tile, kKindGeneral, 32, 4};

@@ -244,7 +244,18 @@ GEMM_PLANS = [
     ((0, 1, 17, 11008, 4096), "mfma flat ragged pipelined staged 2 split 2"),          # one workgroup per compute unit: 86 tiles x 2
     ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
-    ((0, 1, 96, 4096, 4096), "mfma flat whole split 8"),             # 65..96 rows: three row tiles of 32, not two of 64
+    ((0, 1, 96, 4096, 4096), "mfma flat ragged pipelined split 8"),  # 65..96 rows: three row tiles of 32, not two of 64
+    ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # one row of whole 32 x 128 tiles: the simple schedule
+    # 129..160 rows: five row tiles of 32 where their workgroups fill the compute units' rounds
+    ((0, 1, 144, 4096, 4096), "mfma flat ragged pipelined staged 2 split 3"),     # 480 workgroups
+    ((0, 0, 160, 4096, 4096), "mfma flat ragged pipelined staged 2 split 3"),
+    ((1, 0, 144, 8192, 4096), "mfma flat ragged pipelined staged 2 split 4"),     # 1280: five whole rounds
+    ((0, 1, 144, 6144, 4096), "mfma flat ragged pipelined staged 2 split 1"),     # 240
+    ((0, 1, 144, 5120, 5120), "mfma small ragged pipelined staged 4 split 1"),    # no part count fills the rounds
+    ((0, 1, 144, 4096, 1024), "mfma small ragged pipelined staged 4 split 1"),    # short reduction
+    ((0, 1, 144, 11008, 4096), "mfma small ragged pipelined split 4"),            # more than 8192 columns
+    ((0, 1, 128, 4096, 4096), "mfma small whole pipelined staged 4 split 2"),     # 128 rows: two whole 64-row tiles
+    ((0, 1, 161, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),    # 161 rows: six row tiles of 32 = three of 64
     ((0, 1, 64, 64, 8192), "mfma small whole pipelined staged 4 split 16"),             # one tile, a long reduction
     ((0, 1, 768, 768, 4096), "mfma medium ragged pipelined split 7"),   # 36 medium tiles x 7 parts of 592 steps: one workgroup per unit
     ((0, 1, 1024, 1024, 8192), "mfma medium whole pipelined staged 2 split 4"),   # 64 medium tiles x 4 parts of 2048 steps

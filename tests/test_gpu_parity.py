@@ -885,6 +885,11 @@ STAGED = [
     ((4096, 4096, 512), "large whole pipelined staged 2"), ((4096, 4096, 528), "large whole pipelined staged 2"),
     ((4000, 4000, 530), "large ragged pipelined staged 2"), ((4000, 4000, 550), "large ragged pipelined staged 2"),
     ((24, 8192, 4100), "flat ragged pipelined staged 2"), ((31, 16384, 2100), "flat ragged pipelined staged 2"),
+    # several rows of 32 x 128 tiles: 129..160 rows with parts of unequal length, whole tiles in equal parts,
+    # steps after the last whole tile of 32
+    ((144, 4096, 4096), "flat ragged pipelined staged 2 split 3"), ((160, 2048, 2048), "flat ragged pipelined split 3"),
+    ((96, 2048, 2048), "flat ragged pipelined split 4"), ((130, 3072, 2100), "flat ragged pipelined staged 2 split 2"),
+    ((150, 1100, 2500), "flat ragged pipelined split 5"),
 ]
 
 
