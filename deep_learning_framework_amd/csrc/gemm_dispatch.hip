@@ -227,11 +227,13 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // forms 1.05 x on average (144 x 4096 x 4096 53.4 -> 49.5 us, 144 x 3072 x 4096 44.8 -> 39, 144 x 6144 x 4096
     // 85 -> 70, 144 x 8192 x 4096 96 -> 88, 160 x 4096 x 11008 130 -> 123; ties at 2560 x 2560 and 1024 x 4096).
     // Reductions under 2048 steps lost (4096 x 1024: 19.3 -> 21) and 11008 columns measured between 9 % slower
-    // and 8 % faster: both stay with the other tiles.
-    if (modelled && d.M > 128 && d.M <= 160 && d.N >= 1024 && d.N <= 8192 && d.K >= 2048 && d.N * d.K <= (1ll << 26)) {
+    // and 8 % faster: both stay with the other tiles.  193..224 rows likewise, seven rows of tiles against four
+    // (200 x 3072 x 4096 56 -> 50 us, 224 x 4608 x 4608 91 -> 77, 200 x 3072 x 3072 42 -> 39; 50 shapes x 3 forms
+    // 1.04-1.05 x on average, nothing slower than measurement noise).
+    if (modelled && ((d.M > 128 && d.M <= 160) || (d.M > 192 && d.M <= 224)) && d.N >= 1024 && d.N <= 8192 && d.K >= 2048 && d.N * d.K <= (1ll << 26)) {
         const GemmParams pp = make_params(dn, plan.a_kc, plan.b_kc);
         if (fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, 32, 128)) {
-            const int64_t tiles = 5 * ((d.N + 127) / 128);
+            const int64_t tiles = ((d.M + 31) / 32) * ((d.N + 127) / 128);
             double flat_best = 0.0;
             int64_t flat_split = 0, flat_len = 0;
             for (int64_t sp = 1; sp <= kSplitMax; sp++) {
@@ -245,9 +247,13 @@ GemmPlan plan_gemm(const GemmDesc& d) {
                 const int64_t per_cu = (tiles * sp + cus - 1) / cus;
                 // measured against the other tiles: one workgroup per compute unit +15..22 %, two 0..+13 %, where
                 // they cover at least 85 % of the units (200 of 256: -3 %, 390 and 420 of 512: -7 %); whole rounds
-                // beyond (1280 workgroups: five per unit) +5..10 %, partly filled ones -16..+10 %
+                // beyond (1280 workgroups: five per unit) +5..10 %, partly filled ones -16..+10 %, fourteen rounds
+                // of 16 parts -8 %
                 const int64_t wgs = tiles * sp;
-                if (wgs > 2 * cus ? wgs % cus != 0 : 100 * wgs < 85 * per_cu * cus) continue;
+                // (seven row tiles against four of 64 rows save an eighth, not a sixth: 448 workgroups of 512 lost
+                // 3..7 % there, 504 and 252 gained 6..20 %)
+                const int64_t min_fill = d.M <= 160 ? 85 : 95;
+                if (wgs > 2 * cus ? wgs % cus != 0 || wgs > 6 * cus : 100 * wgs < min_fill * per_cu * cus) continue;
                 // three workgroups fit a compute unit (45 KB of LDS each); a last round of one per unit lands
                 // three to a unit on a third of the chip and costs a round of two (980 workgroups of 16 steps:
                 // 37.6 us in the loop where 4 x 16 x 0.44 = 28 were expected; 1280: 35, as expected)

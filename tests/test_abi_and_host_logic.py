@@ -256,6 +256,11 @@ GEMM_PLANS = [
     ((0, 1, 144, 11008, 4096), "mfma small ragged pipelined split 4"),            # more than 8192 columns
     ((0, 1, 128, 4096, 4096), "mfma small whole pipelined staged 4 split 2"),     # 128 rows: two whole 64-row tiles
     ((0, 1, 161, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),    # 161 rows: six row tiles of 32 = three of 64
+    # 193..224 rows: seven row tiles of 32 against four of 64, where they fill at least 95 % of the compute units
+    ((0, 1, 200, 3072, 4096), "mfma flat ragged pipelined staged 2 split 3"),     # 504 workgroups
+    ((0, 0, 224, 4608, 4608), "mfma flat ragged pipelined staged 2 split 1"),     # 252
+    ((0, 1, 200, 8192, 4096), "mfma small ragged pipelined staged 4 split 1"),    # 448 of 512: stays
+    ((0, 0, 200, 4096, 8192), "mfma medium ragged pipelined staged 2 split 4"),   # 14 whole rounds of 16 parts: stays
     ((0, 1, 64, 64, 8192), "mfma small whole pipelined staged 4 split 16"),             # one tile, a long reduction
     ((0, 1, 768, 768, 4096), "mfma medium ragged pipelined split 7"),   # 36 medium tiles x 7 parts of 592 steps: one workgroup per unit
     ((0, 1, 1024, 1024, 8192), "mfma medium whole pipelined staged 2 split 4"),   # 64 medium tiles x 4 parts of 2048 steps

@@ -890,6 +890,7 @@ STAGED = [
     ((144, 4096, 4096), "flat ragged pipelined staged 2 split 3"), ((160, 2048, 2048), "flat ragged pipelined split 3"),
     ((96, 2048, 2048), "flat ragged pipelined split 4"), ((130, 3072, 2100), "flat ragged pipelined staged 2 split 2"),
     ((150, 1100, 2500), "flat ragged pipelined split 5"),
+    ((200, 3072, 4096), "flat ragged pipelined staged 2 split 3"), ((224, 4608, 2304), "flat ragged pipelined staged 2 split 1"),
 ]
 
 
