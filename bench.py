@@ -98,7 +98,7 @@ def cpu_baseline(a_rows, bt, bias, seconds_hint=10.0):
     }, y, rows
 
 
-def per_config_table(torch, kai, stream, dev, with_cpu):
+def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
     """The other BASELINE configurations (they are parity cases; reported here for completeness): GPU time
     per call from HIP events over back-to-back launches (after about 40 ms of the same call untimed; the median
     of three runs of `iters` launches), achieved rate, and the oracle's single-thread time."""
@@ -118,7 +118,7 @@ def per_config_table(torch, kai, stream, dev, with_cpu):
         # then on); an in-place op works on one spare copy of its input meanwhile
         spare = prep() if prep else None
         t0 = time.perf_counter()
-        while time.perf_counter() - t0 < 0.04:
+        while time.perf_counter() - t0 < warm_ms * 1e-3:
             for _ in range(20):
                 if prep:
                     fn(spare)
@@ -374,6 +374,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="skip the table of the other configurations")
+    ap.add_argument("--row-warmup-ms", type=float, default=40.0,
+                    help="untimed warm-up before each row of the table (a profiler run passes a small value to keep its trace short)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path is built and measured on a single MI355X "
@@ -513,7 +515,7 @@ def main():
     else:
         out["cpu_baseline"] = None
     if not args.headline_only:
-        out["per_config"] = per_config_table(torch, kai, stream, dev, not args.no_cpu_baseline)
+        out["per_config"] = per_config_table(torch, kai, stream, dev, not args.no_cpu_baseline, args.row_warmup_ms)
     print(json.dumps(out))
 
 
