@@ -98,18 +98,61 @@ gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__ X, const
                 acc[r] += w[r][j][0] * x[j][0] + w[r][j][1] * x[j][1] + w[r][j][2] * x[j][2] + w[r][j][3] * x[j][3];
     };
 
+    // The same chunk as 16 segments of 256 steps that start at segment seg0 of the row's nseg whole ones and wrap
+    // round (rows a multiple of 32 KiB apart, below)
+    auto wrapped_chunk = [&](int seg0, int nseg) {
+        f32x4 w[R][CH];
+        f32x4 x[CH];
+        int koff[CH];
+#pragma unroll
+        for (int j = 0; j < CH; j++) {
+            int sg = seg0 + j;
+            if (sg >= nseg) sg -= nseg;
+            koff[j] = 256 * sg + 4 * lane;
+        }
+#pragma unroll
+        for (int j = 0; j < CH; j++) {
+            w[0][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[0] + koff[j]));
+            x[j] = *reinterpret_cast<const f32x4*>(p.X + koff[j]);
+        }
+#pragma unroll
+        for (int r = 1; r < R; r++)
+#pragma unroll
+            for (int j = 0; j < CH; j++)
+                w[r][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(wrow[r] + koff[j]));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int j = 0; j < CH; j++)
+                acc[r] += w[r][j][0] * x[j][0] + w[r][j][1] * x[j][1] + w[r][j][2] * x[j][2] + w[r][j][3] * x[j][3];
+    };
+
     if constexpr (K4096) {
         full_chunk(0);
     } else {
-        // whole chunks, each wave starting at a chunk of its own and wrapping round: with rows a large power of
-        // two apart, waves that all walk their rows from k = 0 keep meeting in the same HBM channels
-        // (8192 x 8192: 50 -> 46 us, 4096 x 16384: 48 -> 44)
+        // whole chunks, each wave starting at a place of its own and wrapping round: with rows a large power of
+        // two apart, waves that all walk their rows from k = 0 keep meeting in the same HBM channels.  Rows a
+        // multiple of 32 KiB apart: the start moves in steps of 4 KiB (8192 x 8192: 50 us from k = 0, 44.5 with a
+        // chunk of 4096 steps as the unit, 41.3 with 4 KiB; 4096 x 8192: 24.1 -> 22.6, 4096 x 16384: 43.9 -> 41.4).
+        // Other lengths keep whole chunks as the unit (5120 x 5120: 20.4 us against 21.2 with the finer one).
         const int nfull = p.K / (256 * CH);
-        const int first = nfull > 1 ? (int)((blockIdx.x * (kSkinnyThreads / 64) + wave) % nfull) : 0;
-        for (int i = 0; i < nfull; i++) {
-            int c = first + i;
-            if (c >= nfull) c -= nfull;
-            full_chunk(c * 256 * CH);
+        const int wave_id = (int)(blockIdx.x * (kSkinnyThreads / 64) + wave);
+        if (nfull > 1 && p.ldw % 8192 == 0) {
+            const int nseg = nfull * CH;
+            int seg = (wave_id * 4) % nseg;
+            for (int i = 0; i < nfull; i++) {
+                wrapped_chunk(seg, nseg);
+                seg += CH;
+                if (seg >= nseg) seg -= nseg;
+            }
+        } else {
+            const int first = nfull > 1 ? wave_id % nfull : 0;
+            for (int i = 0; i < nfull; i++) {
+                int c = first + i;
+                if (c >= nfull) c -= nfull;
+                full_chunk(c * 256 * CH);
+            }
         }
         const int kc = nfull * 256 * CH;
         if (kc < p.K) {

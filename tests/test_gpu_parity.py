@@ -375,7 +375,10 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # batch 1 at K = 4096 (the straight-line kernel) with rows that do not fill the last wave
                                    (1, 4096, 1027), (1, 4096, 257),
                                    # 2..4 rows with X shared through LDS: K in (3072, 4096], N >= 1024
-                                   (3, 3080, 1030), (2, 4096, 1024), (4, 3588, 2050)])
+                                   (3, 3080, 1030), (2, 4096, 1024), (4, 3588, 2050),
+                                   # rows a multiple of 32 KiB apart: every wave starts at a place of its own in its
+                                   # rows / slices and wraps round
+                                   (16, 8192, 512), (12, 16384, 272), (1, 16384, 260), (2, 8192, 4112), (1, 24576, 130)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     rng = np.random.default_rng(m + k + n)
     w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
