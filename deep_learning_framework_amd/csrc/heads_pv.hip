@@ -118,28 +118,6 @@ __global__ void __launch_bounds__(kHpThreads) heads_pv_kernel(HeadsPvParams p) {
             *reinterpret_cast<f32x4*>(&lds_x[buf][0][0] + xlds[c]) = sx[c];
         }
     };
-    auto compute = [&](int buf) {
-        const float* pl = lds_p[buf][wave];
-        const float* xl = lds_x[buf][wave];
-#pragma unroll
-        for (int s = 0; s < kHpTile / 8; s++) {
-            // reduction steps 8s + 4 * half + e: operand element e of both operands
-            float a[4], bq[4];
-            if (!TRANS) {
-                const f32x4 av = *reinterpret_cast<const f32x4*>(pl + l32 * kHpPStride + 8 * s + 4 * half);
-#pragma unroll
-                for (int e = 0; e < 4; e++) a[e] = av[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; e++) a[e] = pl[(8 * s + 4 * half + e) * kHpPStride + l32];
-            }
-#pragma unroll
-            for (int e = 0; e < 4; e++) bq[e] = xl[(8 * s + 4 * half + e) * kHpXStride + l32];
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], bq[e], acc, 0, 0, 0);
-        }
-    };
-
     // prologue: tiles 0 .. depth-1 into the register slots, tile 0 on to LDS, its slot refilled
     static_for<0, kHpDepth>([&](auto dc) {
         constexpr int d = decltype(dc)::value;
@@ -149,14 +127,59 @@ __global__ void __launch_bounds__(kHpThreads) heads_pv_kernel(HeadsPvParams p) {
     load_into(kHpDepth, rp[0], rx[0]);
     __syncthreads();
     // At the top of tile kt: LDS[kt & 1] holds tile kt, slot (kt + j) % depth holds tile kt + j, j = 1 .. depth.
-    // The next tile goes to the free LDS buffer before the MFMAs of this one, its slot is refilled at once.
+    // The next tile goes to the free LDS buffer between the MFMAs of this one, its slot is refilled behind them.
+    // One tile: the MFMAs of tile kt (LDS[cur]) with everything else between them -- a wave issues its 16
+    // dependent MFMAs 64 cycles apart and has those gaps to spend: the operands of step s + 1 are read while
+    // step s multiplies, and piece s of the next tile goes from its register slot to the other LDS buffer behind
+    // the MFMAs of step s (written as one block before the MFMAs, the 12 LDS stores of a tile and their waits
+    // were a phase of their own: 1.2 us per tile against 0.43 us of MFMAs).
+    auto read_ops = [&](const float* pl, const float* xl, int s, float (&a)[4], float (&bq)[4]) {
+        if (!TRANS) {
+            const f32x4 av = *reinterpret_cast<const f32x4*>(pl + l32 * kHpPStride + 8 * s + 4 * half);
+#pragma unroll
+            for (int e = 0; e < 4; e++) a[e] = av[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) a[e] = pl[(8 * s + 4 * half + e) * kHpPStride + l32];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) bq[e] = xl[(8 * s + 4 * half + e) * kHpXStride + l32];
+    };
+    static_assert(kHpChunks == kHpTile / 8, "one piece of the next tile per group of four MFMAs");
     auto stage = [&](auto dc, int kt, bool guard) {
         constexpr int d = decltype(dc)::value;
         constexpr int nslot = (d + 1) % kHpDepth;
         const int cur = kt & 1;
-        if (!guard || kt + 1 < nkt) store_lds(cur ^ 1, rp[nslot], rx[nslot]);
+        const bool st = !guard || kt + 1 < nkt;   // the same for every thread
+        const float* pl = lds_p[cur][wave];
+        const float* xl = lds_x[cur][wave];
+        float a[2][4], bq[2][4];
+        read_ops(pl, xl, 0, a[0], bq[0]);
+        static_for<0, kHpChunks>([&](auto sc) {
+            constexpr int s = decltype(sc)::value;
+            constexpr int o = s & 1;
+            if constexpr (s + 1 < kHpChunks) read_ops(pl, xl, s + 1, a[o ^ 1], bq[o ^ 1]);
+            const f32x4 v = rp[nslot][s];
+            __builtin_amdgcn_sched_barrier(0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[o][0], bq[o][0], acc, 0, 0, 0);
+            if (st) {
+                lds_p[cur ^ 1][0][plds[s]] = v[0];
+                lds_p[cur ^ 1][1][plds[s]] = v[1];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[o][1], bq[o][1], acc, 0, 0, 0);
+            if (st) {
+                lds_p[cur ^ 1][2][plds[s]] = v[2];
+                lds_p[cur ^ 1][3][plds[s]] = v[3];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[o][2], bq[o][2], acc, 0, 0, 0);
+            if (st) *reinterpret_cast<f32x4*>(&lds_x[cur ^ 1][0][0] + xlds[s]) = rx[nslot][s];
+            __builtin_amdgcn_sched_barrier(0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[o][3], bq[o][3], acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        });
         load_into(kt + 1 + kHpDepth, rp[nslot], rx[nslot]);
-        compute(cur);
         __syncthreads();
     };
     int kt0 = 0;
