@@ -47,8 +47,10 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // amdgpu_waves_per_eu(1, 2): two waves per SIMD are all the grid ever gives a CU, so the register
 // allocator is told not to trade loads in flight for an occupancy it cannot use.
-template <int R, bool K4096>
-__global__ void __launch_bounds__(kSkinnyThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
+// THREADS: 256, or 128 / 64 where 256-thread workgroups would not cover the compute units (1024 x 4096: 128
+// workgroups 5.06 us, 256 of 128 threads 4.5)
+template <int R, bool K4096, int THREADS>
+__global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 2)))
 gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t N,
                  const int K, const int act_acc, float* __restrict__ Y, const float* __restrict__ bias,
                  float* __restrict__ Y2, const float* __restrict__ leaky_ptr) {
@@ -60,7 +62,7 @@ gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__ X, const
     constexpr int CH = 16;   // float4 per lane per chunk of 4096 k
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int64_t n0 = ((int64_t)blockIdx.x * (kSkinnyThreads / 64) + wave) * R;
+    const int64_t n0 = ((int64_t)blockIdx.x * (THREADS / 64) + wave) * R;
     // rows past the end are clamped to the last row (loaded, never stored): no early exit, so the
     // kernel arguments are fetched in one round trip and the first loads go out at once
     const float* __restrict__ wrow[R];
@@ -137,7 +139,7 @@ gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__ X, const
         // chunk of 4096 steps as the unit, 41.3 with 4 KiB; 4096 x 8192: 24.1 -> 22.6, 4096 x 16384: 43.9 -> 41.4).
         // Other lengths keep whole chunks as the unit (5120 x 5120: 20.4 us against 21.2 with the finer one).
         const int nfull = p.K / (256 * CH);
-        const int wave_id = (int)(blockIdx.x * (kSkinnyThreads / 64) + wave);
+        const int wave_id = (int)(blockIdx.x * (THREADS / 64) + wave);
         if (nfull > 1 && p.ldw % 8192 == 0) {
             const int nseg = nfull * CH;
             int seg = (wave_id * 4) % nseg;
@@ -187,18 +189,28 @@ gemv_rows_kernel(const float* __restrict__ W, const float* __restrict__ X, const
     }
 }
 
+template <int THREADS>
+static void launch_gemv_rows_threads(const SkinnyParams& p, int64_t blocks, int act_acc, hipStream_t stream) {
+    constexpr int R = 2;
+    if (p.K == 4096)
+        gemv_rows_kernel<R, true, THREADS><<<dim3((unsigned)blocks), dim3(THREADS), 0, stream>>>(
+            p.W, p.X, p.ldw, p.N, p.K, act_acc, p.Y, p.bias, p.Y2, p.leaky);
+    else
+        gemv_rows_kernel<R, false, THREADS><<<dim3((unsigned)blocks), dim3(THREADS), 0, stream>>>(
+            p.W, p.X, p.ldw, p.N, p.K, act_acc, p.Y, p.bias, p.Y2, p.leaky);
+}
+
 static int launch_gemv_rows(const SkinnyParams& p, hipStream_t stream) {
     constexpr int R = 2;
-    const int64_t rows_per_block = (kSkinnyThreads / 64) * R;
+    int threads = kSkinnyThreads;
+    while (threads > 64 && (p.N + (threads / 64) * R - 1) / ((threads / 64) * R) < compute_units()) threads /= 2;
+    const int64_t rows_per_block = (threads / 64) * R;
     const int64_t blocks = (p.N + rows_per_block - 1) / rows_per_block;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
     const int act_acc = (p.act & 0xff) | (p.accflag ? 0x100 : 0);
-    if (p.K == 4096)
-        gemv_rows_kernel<R, true><<<dim3((unsigned)blocks), dim3(kSkinnyThreads), 0, stream>>>(
-            p.W, p.X, p.ldw, p.N, p.K, act_acc, p.Y, p.bias, p.Y2, p.leaky);
-    else
-        gemv_rows_kernel<R, false><<<dim3((unsigned)blocks), dim3(kSkinnyThreads), 0, stream>>>(
-            p.W, p.X, p.ldw, p.N, p.K, act_acc, p.Y, p.bias, p.Y2, p.leaky);
+    if (threads == 256) launch_gemv_rows_threads<256>(p, blocks, act_acc, stream);
+    else if (threads == 128) launch_gemv_rows_threads<128>(p, blocks, act_acc, stream);
+    else launch_gemv_rows_threads<64>(p, blocks, act_acc, stream);
     return check_launch("gemv_rows_kernel");
 }
 
