@@ -210,8 +210,9 @@ inline GemmVariant pick_gemm_variant(const GemmParams& p, bool a_kc, bool b_kc, 
             return {tile, kKindRaggedPipelined, 32, staging_depth(tile, p, groups(128, 128), nbatch, 32)};
         return {tile, kKindGeneral, 16, 1};
     case kTileFlat:
-        // at most 32 rows against many columns (a batch of 17..32 rows against a weight matrix): four waves side
-        // by side, so that the matrix cores do not spend half their time on rows that do not exist.  With edges
+        // 17..32 rows against many columns (a batch against a weight matrix), or several rows of such tiles where
+        // 64-row tiles would pad more (65..96, 129..160, 193..224 rows): four waves side by side, so that the matrix
+        // cores do not spend half their time on rows that do not exist.  With edges
         // the pipelined schedule is the faster one (80 x 4096 x 4096: 41.2 -> 36.6 us, 72 x 4096 x 11008:
         // 88.6 -> 79.9, 17 and 24 rows 22.9 -> 22.4), and so it is with whole tiles in several rows of tiles
         // (96 x 4096 x 4096: 35.7 -> 33.1 us, 96 x 2048 x 2048 17.9 -> 15.9, 96 x 4096 x 11008 76.2 -> 72.6,

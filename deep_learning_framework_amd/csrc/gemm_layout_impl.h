@@ -6,7 +6,8 @@
 //   medium 128x128 tile, 4 waves of 64x64, 2 workgroups per CU -- fills the chip at mid sizes
 //   small   64x64  tile, 4 waves of 32x32                      -- small or very ragged products
 //   wide    64x128 tile, 4 waves of 32x64                      -- whole tiles, fewer workgroups than the small tile
-//   flat    32x128 tile, 4 waves of 32x32 side by side         -- at most 32 rows against many columns
+//   flat    32x128 tile, 4 waves of 32x32 side by side         -- 17..32 rows against many columns, and row counts that
+//                                                                 fill an odd number of 32-row tiles (65..96, 129..160, 193..224)
 // On the two bigger tiles, operands that allow 128-bit loads run the pipelined kernel: predicate-free
 // when the shape is a whole multiple of the tile, else with range-checked buffer resources and one
 // masked K-tile at the end.  The wide tile and the small tile run the pipelined kernel too, each with one to four
