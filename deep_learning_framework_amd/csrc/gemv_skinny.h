@@ -45,6 +45,7 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream);
 
 // skinny_stream.hip: aligned operands, K split over workgroups (uses the library's scratch memory)
 bool skinny_stream_applies(const SkinnyParams& p);
+bool skinny_stream32_applies(const SkinnyParams& p);   // 17..32 rows
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream);
 
 }  // namespace kai

@@ -560,7 +560,10 @@ static int launch_skinny_mfma(const SkinnyParams& p, bool vec, hipStream_t strea
 
 int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
     if (p.M <= 0 || p.N <= 0) return KAI_OK;
-    if (p.M > kSkinnyMaxRows) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
+    if (p.M > kSkinnyMaxRows) {
+        if (skinny_stream32_applies(p)) return launch_skinny_stream(p, stream);
+        return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
+    }
     const bool vec = p.K % 4 == 0 && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X);
     if (vec && p.K >= 256) {
         if (p.M == 1) return launch_gemv_rows(p, stream);

@@ -67,13 +67,20 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 //
 // XL (with SLICES): 1 = at most 8 rows of X (one load per tile), 2 = more (two); 0 = decided per tile from M.  With
 // the number of X loads a compile-time constant and every tile inside K, the written-out slice has no branch left.
-template <bool WHOLE, bool SLICES, int XL = 0>
+//
+// XB: blocks of 16 rows of X.  2 (17..32 rows; whole tiles and written-out slices only, XL = 3 or 4): a tile of W meets
+// two tiles of X and a wave keeps two accumulators -- W still streams once, where a tiled product of 17..32 rows
+// cuts K over workgroups and sums the parts in a second launch.
+template <bool WHOLE, bool SLICES, int XL = 0, int XB = 1>
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
     const SkinnyParams p = skinny_params(W, X, ldw, ldx, N, M, K, Y, t);
     __shared__ __attribute__((aligned(16))) float lds_w[kSsWaves][16 * kSsTileStride];
-    __shared__ __attribute__((aligned(16))) float lds_x[kSsWaves][16 * kSsTileStride];
+    static_assert(XB == 1 || (XB == 2 && WHOLE && SLICES && XL > kSsLoadsPerTile && XL <= 2 * kSsLoadsPerTile),
+                  "two blocks of X rows exist for whole tiles in written-out slices");
+    constexpr int kXLoads = kSsLoadsPerTile * XB;   // 128-bit loads per lane that cover a tile of X
+    __shared__ __attribute__((aligned(16))) float lds_x[kSsWaves][16 * XB * kSsTileStride];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -88,10 +95,12 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
 
     // rows of X that are never loaded stay zero in the tile
 #pragma unroll
-    for (int j = 0; j < kSsLoadsPerTile; j++)
+    for (int j = 0; j < kXLoads; j++)
         *reinterpret_cast<f32x4*>(tx + (kSsRowsPerLoad * j + lrow) * kSsTileStride + lk) = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[XB];
+#pragma unroll
+    for (int b = 0; b < XB; b++) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
     // One tile = 16 rows x kSsTileK k of W and of X, kSsLoadsPerTile 128-bit loads per lane each.  Addresses past
     // K are clamped into the row (every load is unconditional); what they return is zeroed on the way to LDS.
     // WHOLE: resources and per-lane offsets (bytes)
@@ -105,10 +114,11 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         uniform_ptr(p.W + n0 * p.ldw), 0, (int)(((int64_t)15 * p.ldw + p.K) * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
         uniform_ptr(p.X), 0, (int)(((int64_t)(p.M - 1) * p.ldx + p.K) * 4), 0x00020000);
-    int woff[kSsLoadsPerTile], xoff[kSsLoadsPerTile];
+    int woff[kSsLoadsPerTile], xoff[kXLoads];
 #pragma unroll
-    for (int j = 0; j < kSsLoadsPerTile; j++) {
-        woff[j] = (int)(((int64_t)(kSsRowsPerLoad * j + lrow) * p.ldw + lk) * 4);
+    for (int j = 0; j < kSsLoadsPerTile; j++) woff[j] = (int)(((int64_t)(kSsRowsPerLoad * j + lrow) * p.ldw + lk) * 4);
+#pragma unroll
+    for (int j = 0; j < kXLoads; j++) {
         // a row past M must land behind the end of the resource whatever ldx is: the last row's end is the limit
         const int m = kSsRowsPerLoad * j + lrow;
         xoff[j] = m < p.M ? (int)(((int64_t)m * p.ldx + lk) * 4) : 0x7FFFFFF0;
@@ -130,11 +140,11 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
             dst[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src));
         }
     };
-    auto load_x = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
+    auto load_x = [&](f32x4(&dst)[kXLoads], int kt) {
         if constexpr (WHOLE) {
             const int kc = min(kt, p.K - kSsTileK) * 4;
 #pragma unroll
-            for (int j = 0; j < kSsLoadsPerTile; j++)
+            for (int j = 0; j < kXLoads; j++)
                 if (XL ? j < XL : kSsRowsPerLoad * j < p.M)   // uniform
                     dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, xoff[j], kc, 0));
             return;
@@ -147,13 +157,17 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
             }
         }
     };
-    auto consume = [&](const f32x4(&w)[kSsLoadsPerTile], const f32x4(&x)[kSsLoadsPerTile], int kt) {
+    auto consume = [&](const f32x4(&w)[kSsLoadsPerTile], const f32x4(&x)[kXLoads], int kt) {
         if ((SLICES && XL) || kt < p.K) {   // uniform
 #pragma unroll
             for (int j = 0; j < kSsLoadsPerTile; j++) {
                 const int row = kSsRowsPerLoad * j + lrow;
                 *reinterpret_cast<f32x4*>(tw + row * kSsTileStride + lk) =
                     WHOLE ? w[j] : keep_if(w[j], n0 + row < p.N && kt + lk < p.K);
+            }
+#pragma unroll
+            for (int j = 0; j < kXLoads; j++) {
+                const int row = kSsRowsPerLoad * j + lrow;
                 if (XL ? j < XL : kSsRowsPerLoad * j < p.M)
                     *reinterpret_cast<f32x4*>(tx + row * kSsTileStride + lk) =
                         WHOLE ? x[j] : keep_if(x[j], row < p.M && kt + lk < p.K);
@@ -162,9 +176,12 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
 #pragma unroll
             for (int s = 0; s < kSsTileK / 16; s++) {
                 const f32x4 wv = *reinterpret_cast<const f32x4*>(tw + r * kSsTileStride + 16 * s + 4 * g);
-                const f32x4 xv = *reinterpret_cast<const f32x4*>(tx + r * kSsTileStride + 16 * s + 4 * g);
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[e], wv[e], acc, 0, 0, 0);
+                for (int b = 0; b < XB; b++) {
+                    const f32x4 xv = *reinterpret_cast<const f32x4*>(tx + (16 * b + r) * kSsTileStride + 16 * s + 4 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[e], wv[e], acc[b], 0, 0, 0);
+                }
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -179,7 +196,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         // lengths unchanged).  At 4096 steps the plain order is the faster one (12.1 against 12.4 us).
         const int stag = p.K >= 8192 ? 2 * wave : 0;
         for (int k0 = wave * kSlice; k0 < p.K; k0 += kSsWaves * kSlice) {
-            f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kSsLoadsPerTile];
+            f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kXLoads];
             ss_static_for<0, kSsRing>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
                 load_w(w[t], k0 + ((t + stag) & (kTiles - 1)) * kSsTileK);
@@ -209,7 +226,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         const int tiles_base = tiles_total / kSsWaves, tiles_rem = tiles_total % kSsWaves;
         const int t_count = tiles_base + (wave < tiles_rem ? 1 : 0);
         const int k_begin = (wave * tiles_base + min(wave, tiles_rem)) * kSsTileK;
-        f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kSsLoadsPerTile];
+        f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kXLoads];
         ss_static_for<0, kSsRing>([&](auto tc) {
             constexpr int t = decltype(tc)::value;
             load_w(w[t], k_begin + t * kSsTileK);
@@ -237,12 +254,15 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         });
     }
 
-    // acc[v] = D[m = 4 * g + v][n = n0 + r]; the tiles are free now: wave w parks its result in its W tile
+    // acc[b][v] = D[m = 16 * b + 4 * g + v][n = n0 + r]; the tiles are free now: wave w parks its result in its W tile
+    static_assert(256 * XB <= 16 * kSsTileStride, "a wave's results fit its W tile");
     __syncthreads();
 #pragma unroll
-    for (int v = 0; v < 4; v++) tw[(4 * g + v) * 16 + r] = acc[v];
+    for (int b = 0; b < XB; b++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) tw[(16 * b + 4 * g + v) * 16 + r] = acc[b][v];
     __syncthreads();
-    if (tid < 256) {
+    if (tid < 256 * XB) {
         const int m = tid >> 4, j = tid & 15;
         const int64_t n = n0 + j;
         if (m < p.M && n < p.N) {
@@ -261,6 +281,18 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
 
 }  // namespace
 
+// 17..32 rows: whole tiles, written-out slices, workgroups that cover the compute units, a matrix of at most 192 MB.
+// Measured against a row of 32 x 128 tiles with K in parts, us per call at 17 / 32 rows, the matrix streamed from
+// HBM (rotating buffers) | still in the last-level cache: 4096 x 4096 21.2 -> 15.0 / 21.3 -> 17.9 | 16.7 -> 14.4 /
+// 20.2 -> 17.2; 11008 x 4096 45.4 -> 38.3 / 49.7 -> 45.8 | 39.0 -> 36.1 / 47.3 -> 44.2; 4096 x 8192 37.4 -> 28.9 /
+// 38.7 -> 34.0 | 25.8 -> 27.9 / 29.6 -> 33.0; 8192 x 8192 (256 MB, left out) 64.8 -> 54.5 / 67.5 -> 64.9 |
+// 44.0 -> 52.2 / 51.3 -> 63.5.
+bool skinny_stream32_applies(const SkinnyParams& p) {
+    return p.M > kSkinnyMaxRows && p.M <= 2 * kSkinnyMaxRows && p.K % (kSsWaves * 512) == 0 && p.N % 16 == 0 &&
+           p.N >= 16 * (int64_t)compute_units() && p.N * (int64_t)p.K * 4 <= (192ll << 20) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
+           (15 * p.ldw + p.K) * 4 < (1ll << 31) && ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
+}
+
 bool skinny_stream_applies(const SkinnyParams& p) {
     return p.M >= 1 && p.M <= kSkinnyMaxRows && p.K >= 64 && p.K % 4 == 0 && p.ldw % 4 == 0 && p.ldx % 4 == 0 &&
            aligned16(p.W) && aligned16(p.X);
@@ -275,6 +307,12 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
                        ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
     const bool slices = p.K % (kSsWaves * 512) == 0;
     const dim3 grid((unsigned)blocks), block(kSsThreads);
+    if (p.M > kSkinnyMaxRows) {
+        if (!skinny_stream32_applies(p)) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
+        if (p.M <= 24) skinny_stream_kernel<true, true, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        else skinny_stream_kernel<true, true, 4, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        return check_launch("skinny_stream_kernel");
+    }
     if (whole && slices && p.M <= 8) skinny_stream_kernel<true, true, 1><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     else if (whole && slices) skinny_stream_kernel<true, true, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     else if (whole) skinny_stream_kernel<true, false><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);

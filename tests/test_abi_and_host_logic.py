@@ -240,12 +240,15 @@ GEMM_PLANS = [
     ((0, 1, 16, 1024, 1024), "wavesplit 16"),                        # 5..16 rows against a small weight matrix
     ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
     ((0, 1, 1000, 333, 777), "mfma small ragged pipelined split 2"),   # configuration 5, ragged: two rounds of the one-launch kernel would take longer
-    ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
-    ((0, 1, 17, 11008, 4096), "mfma flat ragged pipelined staged 2 split 2"),          # one workgroup per compute unit: 86 tiles x 2
-    ((0, 1, 32, 8192, 8192), "mfma flat whole split 4"),
+    ((0, 1, 32, 4096, 5120), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
+    ((0, 0, 17, 11008, 4096), "mfma flat ragged pipelined staged 2 split 2"),          # one workgroup per compute unit: 86 tiles x 2
+    ((0, 1, 17, 11008, 4096), "skinny"),
+    ((0, 0, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
     ((0, 1, 96, 4096, 4096), "mfma flat ragged pipelined split 8"),  # 65..96 rows: three row tiles of 32, not two of 64
-    ((0, 1, 32, 4096, 4096), "mfma flat whole split 8"),             # one row of whole 32 x 128 tiles: the simple schedule
+    ((0, 1, 32, 4096, 4096), "skinny"),                              # 17..32 rows, K a multiple of 4096: W streams once
+    ((0, 1, 32, 4096, 11008), "mfma flat whole split 8"),            # one row of whole 32 x 128 tiles: the simple schedule
+    ((0, 0, 32, 4096, 4096), "mfma flat whole split 8"),             # ... and a [K, N] weight matrix
     # 129..160 rows: five row tiles of 32 where their workgroups fill the compute units' rounds
     ((0, 1, 144, 4096, 4096), "mfma flat ragged pipelined staged 2 split 3"),     # 480 workgroups
     ((0, 0, 160, 4096, 4096), "mfma flat ragged pipelined staged 2 split 3"),
