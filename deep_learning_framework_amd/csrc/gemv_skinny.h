@@ -1,4 +1,5 @@
-// Skinny (at most 16 rows) products: parameters and launcher, see gemv_skinny.hip.
+// Skinny products (at most 16 rows; 17..32 on the streaming kernel where skinny_stream32_applies): parameters and
+// launcher, see gemv_skinny.hip.
 #pragma once
 
 #include "kai_common.h"

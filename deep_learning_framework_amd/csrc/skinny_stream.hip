@@ -1,6 +1,6 @@
-// Skinny products (at most 16 rows of X) whose operands allow aligned 128-bit loads:
+// Skinny products (at most 16 rows of X, in one variant 32) whose operands allow aligned 128-bit loads:
 //
-//   y[m,n] (=|+=) act( sum_k x[m,k] * w[n,k] + bias[n] ),   m < M <= 16
+//   y[m,n] (=|+=) act( sum_k x[m,k] * w[n,k] + bias[n] ),   m < M <= 16 (32)
 //
 // A workgroup of eight waves owns 16 rows of W and all of K; wave w owns a contiguous eighth of the tiles of
 // 32 reduction steps.  Everything up to the final sum is private to a wave, so there is no
