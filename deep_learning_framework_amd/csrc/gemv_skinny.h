@@ -47,6 +47,8 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream);
 // skinny_stream.hip: aligned operands, K split over workgroups (uses the library's scratch memory)
 bool skinny_stream_applies(const SkinnyParams& p);
 bool skinny_stream32_applies(const SkinnyParams& p);   // 17..32 rows
+bool skinny_stream8_applies(const SkinnyParams& p);    // workgroups of 8 rows of W
+int launch_skinny_stream8(const SkinnyParams& p, hipStream_t stream);
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream);
 
 }  // namespace kai

@@ -567,6 +567,7 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
     const bool vec = p.K % 4 == 0 && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X);
     if (vec && p.K >= 256) {
         if (p.M == 1) return launch_gemv_rows(p, stream);
+        if (skinny_stream8_applies(p)) return launch_skinny_stream8(p, stream);
         // 3 and 4 rows: the streaming kernel once its workgroups (16 rows of W each) cover the chip (measured at
         // 4096 x 4096: 12.6 against 16.0 us, 11008 x 4096: 30 against 40; at 2048 x 8192, 128 workgroups:
         // 19.8 against 15.3); 2 rows: the streaming kernel where its slices are written out (K a multiple of 4096:

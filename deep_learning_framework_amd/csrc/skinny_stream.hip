@@ -71,7 +71,10 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // XB: blocks of 16 rows of X.  2 (17..32 rows; whole tiles and written-out slices only, XL = 3 or 4): a tile of W meets
 // two tiles of X and a wave keeps two accumulators -- W still streams once, where a tiled product of 17..32 rows
 // cuts K over workgroups and sums the parts in a second launch.
-template <bool WHOLE, bool SLICES, int XL = 0, int XB = 1>
+//
+// WR: rows of W per workgroup, 16, or 8 (whole tiles only) where workgroups of 16 rows would not cover the compute
+// units: the second half of the W tile then stays zero and only eight columns of the result are stored.
+template <bool WHOLE, bool SLICES, int XL = 0, int XB = 1, int WR = 16>
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
@@ -79,6 +82,8 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     __shared__ __attribute__((aligned(16))) float lds_w[kSsWaves][16 * kSsTileStride];
     static_assert(XB == 1 || (XB == 2 && WHOLE && SLICES && XL > kSsLoadsPerTile && XL <= 2 * kSsLoadsPerTile),
                   "two blocks of X rows exist for whole tiles in written-out slices");
+    static_assert(WR == 16 || (WR == 8 && WHOLE && XB == 1 && kSsRowsPerLoad == 8), "eight rows of W: one load per tile");
+    constexpr int kWLoads = WR / kSsRowsPerLoad;    // 128-bit loads per lane that cover the workgroup's rows of a W tile
     constexpr int kXLoads = kSsLoadsPerTile * XB;   // 128-bit loads per lane that cover a tile of X
     __shared__ __attribute__((aligned(16))) float lds_x[kSsWaves][16 * XB * kSsTileStride];
 
@@ -87,13 +92,16 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15;    // row of W inside the block's 16 / row of X
     const int g = lane >> 4;    // k group of the MFMA operand
-    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int64_t n0 = (int64_t)blockIdx.x * WR;
     const int lrow = lane / kSsLanesPerRow;          // a load covers kSsRowsPerLoad rows x kSsTileK k
     const int lk = (lane % kSsLanesPerRow) * 4;
     float* tw = lds_w[wave];
     float* tx = lds_x[wave];
 
-    // rows of X that are never loaded stay zero in the tile
+    // rows of W beyond the workgroup's WR and rows of X that are never loaded stay zero in the tiles
+#pragma unroll
+    for (int j = kWLoads; j < kSsLoadsPerTile; j++)
+        *reinterpret_cast<f32x4*>(tw + (kSsRowsPerLoad * j + lrow) * kSsTileStride + lk) = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < kXLoads; j++)
         *reinterpret_cast<f32x4*>(tx + (kSsRowsPerLoad * j + lrow) * kSsTileStride + lk) = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -111,7 +119,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
     };
     const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
-        uniform_ptr(p.W + n0 * p.ldw), 0, (int)(((int64_t)15 * p.ldw + p.K) * 4), 0x00020000);
+        uniform_ptr(p.W + n0 * p.ldw), 0, (int)(((int64_t)(WR - 1) * p.ldw + p.K) * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
         uniform_ptr(p.X), 0, (int)(((int64_t)(p.M - 1) * p.ldx + p.K) * 4), 0x00020000);
     int woff[kSsLoadsPerTile], xoff[kXLoads];
@@ -129,7 +137,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
             // counting on the range check for the scalar part of the address; it is never consumed
             const int kc = min(kt, p.K - kSsTileK) * 4;
 #pragma unroll
-            for (int j = 0; j < kSsLoadsPerTile; j++)   // aux 2: non-temporal, as the general variant's loads
+            for (int j = 0; j < kWLoads; j++)   // aux 2: non-temporal, as the general variant's loads
                 dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff[j], kc, 2));
             return;
         }
@@ -160,7 +168,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     auto consume = [&](const f32x4(&w)[kSsLoadsPerTile], const f32x4(&x)[kXLoads], int kt) {
         if ((SLICES && XL) || kt < p.K) {   // uniform
 #pragma unroll
-            for (int j = 0; j < kSsLoadsPerTile; j++) {
+            for (int j = 0; j < kWLoads; j++) {
                 const int row = kSsRowsPerLoad * j + lrow;
                 *reinterpret_cast<f32x4*>(tw + row * kSsTileStride + lk) =
                     WHOLE ? w[j] : keep_if(w[j], n0 + row < p.N && kt + lk < p.K);
@@ -265,7 +273,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     if (tid < 256 * XB) {
         const int m = tid >> 4, j = tid & 15;
         const int64_t n = n0 + j;
-        if (m < p.M && n < p.N) {
+        if (m < p.M && n < p.N && j < WR) {
             float v = 0.f;
 #pragma unroll
             for (int i = 0; i < kSsWaves; i++) v += lds_w[i][tid];
@@ -296,6 +304,28 @@ bool skinny_stream32_applies(const SkinnyParams& p) {
 bool skinny_stream_applies(const SkinnyParams& p) {
     return p.M >= 1 && p.M <= kSkinnyMaxRows && p.K >= 64 && p.K % 4 == 0 && p.ldw % 4 == 0 && p.ldx % 4 == 0 &&
            aligned16(p.W) && aligned16(p.X);
+}
+
+// Eight rows of W per workgroup: whole tiles in written-out slices, N / 8 workgroups that cover at least half of the
+// compute units and at most all of them (one round).  Measured against 16-row workgroups (5..16 rows) and the
+// slice kernels (2..4 rows), us per call with W from HBM: 2048 x 4096 M = 4 / 8 / 16 11.8 / 9.9 / 11.9 -> 8.0 / 8.2 /
+// 9.9, 1024 x 4096 11.2 / 9.2 / 11.3 -> 7.5 / 7.6 / 9.2, 2048 x 8192 M = 8 / 16 18.3 / 21.9 -> 14.7 / 17.6.  With more
+// than 4096 steps the slice kernels keep 2..4 rows (1024 x 8192 M = 2: 8.5 against 12.7); N = 2560 and 3072 (a
+// second, partly filled round) lost 15..40 % at 8 and 16 rows, and so did the rolled loop for other K at most row counts.
+bool skinny_stream8_applies(const SkinnyParams& p) {
+    const int64_t cus = compute_units();
+    return skinny_stream_applies(p) && p.M >= 2 && (p.K == 4096 || p.M >= 5) && p.N % 8 == 0 && p.K % (kSsWaves * 512) == 0 &&
+           p.N <= 8 * cus && p.N >= 4 * cus && (7 * p.ldw + p.K) * 4 < (1ll << 31) &&
+           ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
+}
+
+int launch_skinny_stream8(const SkinnyParams& p, hipStream_t stream) {
+    if (!skinny_stream8_applies(p)) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: shape not served with 8-row workgroups");
+    const SkinnyTail t = skinny_tail(p);
+    const dim3 grid((unsigned)(p.N / 8)), block(kSsThreads);
+    if (p.M <= 8) skinny_stream_kernel<true, true, 1, 1, 8><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else skinny_stream_kernel<true, true, 2, 1, 8><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    return check_launch("skinny_stream_kernel");
 }
 
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {

@@ -380,7 +380,9 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # rows / slices and wraps round
                                    (16, 8192, 512), (12, 16384, 272), (1, 16384, 260), (2, 8192, 4112), (1, 24576, 130),
                                    # 17..32 rows on the streaming kernel: two blocks of 16 rows of X per tile of W
-                                   (17, 4096, 4096), (24, 8192, 4112), (25, 4096, 4096), (32, 4096, 4096)])
+                                   (17, 4096, 4096), (24, 8192, 4112), (25, 4096, 4096), (32, 4096, 4096),
+                                   # workgroups of 8 rows of W where those of 16 would not cover the compute units
+                                   (8, 4096, 2048), (16, 8192, 1024), (3, 4096, 1544), (2, 4096, 2048), (9, 12288, 1032)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     rng = np.random.default_rng(m + k + n)
     w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
