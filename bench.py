@@ -98,7 +98,7 @@ def cpu_baseline(a_rows, bt, bias, seconds_hint=10.0):
     }, y, rows
 
 
-def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
+def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None):
     """The other BASELINE configurations (they are parity cases; reported here for completeness): GPU time
     per call from HIP events over back-to-back launches (after about 40 ms of the same call untimed; the median
     of three runs of `iters` launches), achieved rate, and the oracle's single-thread time."""
@@ -159,7 +159,12 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
 
     rows = []
 
-    def row(name, us, flops=None, nbytes=None, cpu=None):
+    def row(name, fn, iters=50, prep=None, flops=None, nbytes=None, cpu=None):
+        """One row: `fn` timed on the GPU (see gpu_us), `cpu` (a callable) the oracle's time for the same work."""
+        if only and not any(o in name for o in only):
+            return
+        us = gpu_us(fn, iters, prep)
+        cpu = cpu_us(cpu) if cpu is not None else None
         r = {"case": name, "gpu_us": round(us, 2)}
         if flops:
             r["tflops"] = round(flops / us * 1e-6, 2)
@@ -181,24 +186,28 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
     o8 = torch.empty((n8, n8), device=dev)
     f8 = 2.0 * n8 ** 3
     row("8192^3 NT  Y = relu(X.W^T + b)  (kai_dense_forward)",
-        gpu_us(lambda: L.kai_dense_forward(0, P(o8), None, P(w8), P(b8), P(x8), I(n8), I(n8), I(n8), relu, None), iters=10),
+        lambda: L.kai_dense_forward(0, P(o8), None, P(w8), P(b8), P(x8), I(n8), I(n8), I(n8), relu, None), iters=10,
         flops=f8)
     row("8192^3 NT  Y = X.W^T  (kai_matmul)",
-        gpu_us(lambda: L.kai_matmul(0, P(o8), P(w8), P(x8), I(n8), I(n8), I(n8), 0), iters=10), flops=f8)
+        lambda: L.kai_matmul(0, P(o8), P(w8), P(x8), I(n8), I(n8), I(n8), 0), iters=10, flops=f8)
     row("8192^3 NN  dX = dY.W  (kai_matmul_backward_x)",
-        gpu_us(lambda: L.kai_matmul_backward_x(0, P(o8), P(x8), P(w8), I(n8), I(n8), I(n8), 0), iters=10), flops=f8)
+        lambda: L.kai_matmul_backward_x(0, P(o8), P(x8), P(w8), I(n8), I(n8), I(n8), 0), iters=10, flops=f8)
     row("8192^3 TN  dW = dY^T.X  (kai_matmul_backward_w)",
-        gpu_us(lambda: L.kai_matmul_backward_w(0, P(o8), P(x8), P(w8), I(n8), I(n8), I(n8), 0), iters=10), flops=f8)
+        lambda: L.kai_matmul_backward_w(0, P(o8), P(x8), P(w8), I(n8), I(n8), I(n8), 0), iters=10, flops=f8)
+    # the same launch with a transcendental activation: applied to the accumulators in registers, one store
+    row("8192^3 NT  Y = gelu(X.W^T + b)  (kai_dense_forward)",
+        lambda: L.kai_dense_forward(0, P(o8), None, P(w8), P(b8), P(x8), I(n8), I(n8), I(n8), kai.ACT["gelu"], None), iters=10,
+        flops=f8)
     del x8, w8, b8, o8
     # cfg1: dense forward 64 x 784 -> 512, fused
     x = torch.randn((64, 784), device=dev, generator=g)
     w = (torch.rand((512, 784), device=dev, generator=g) * 2 - 1) / 28.0
     b = torch.zeros(512, device=dev)
     y = torch.empty((64, 512), device=dev)
-    us = gpu_us(lambda: L.kai_dense_forward(0, P(y), None, P(w), P(b), P(x), I(512), I(64), I(784), relu, None))
+    us = lambda: L.kai_dense_forward(0, P(y), None, P(w), P(b), P(x), I(512), I(64), I(784), relu, None)
     xc, wc, bc = x.cpu().numpy(), w.cpu().numpy(), b.cpu().numpy()
     row("cfg1 dense fwd 64x784->512 +bias+relu (1 launch)", us, flops=2.0 * 64 * 784 * 512,
-        cpu=cpu_us(lambda: ko.activate(ko.add_bias(ko.matmul(wc, xc), bc), "relu")))
+        cpu=lambda: ko.activate(ko.add_bias(ko.matmul(wc, xc), bc), "relu"))
     # cfg2: batch 256, 1024 -> 1024
     x = torch.randn((256, 1024), device=dev, generator=g)
     w = (torch.rand((1024, 1024), device=dev, generator=g) * 2 - 1) / 32.0
@@ -207,19 +216,24 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
     y, gx, gw, gb = (torch.empty_like(x), torch.empty_like(x), torch.empty_like(w), torch.empty_like(b))
     f = 2.0 * 256 * 1024 * 1024
     xc, wc, bc, gyc = x.cpu().numpy(), w.cpu().numpy(), b.cpu().numpy(), gy.cpu().numpy()
-    row("cfg2 Y = X.W^T + b (fused)", gpu_us(lambda: L.kai_dense_forward(0, P(y), None, P(w), P(b), P(x), I(1024), I(256), I(1024), 0, None)),
-        flops=f, cpu=cpu_us(lambda: ko.add_bias(ko.matmul(wc, xc), bc)))
-    row("cfg2 dX = dY.W", gpu_us(lambda: L.kai_matmul_backward_x(0, P(gx), P(gy), P(w), I(1024), I(256), I(1024), 0)),
-        flops=f, cpu=cpu_us(lambda: ko.matmul_backward_x(gyc, wc)))
-    row("cfg2 dW = dY^T.X", gpu_us(lambda: L.kai_matmul_backward_w(0, P(gw), P(gy), P(x), I(1024), I(256), I(1024), 0)),
-        flops=f, cpu=cpu_us(lambda: ko.matmul_backward_w(gyc, xc, 1024, 1024)))
-    row("cfg2 db = colsum(dY)", gpu_us(lambda: L.kai_add_bias_backward_b(0, P(gb), P(gy), I(256), I(1024), 0)),
-        nbytes=4.0 * 256 * 1024, cpu=cpu_us(lambda: ko.add_bias_backward_b(gyc, 1024)))
+    row("cfg2 Y = X.W^T + b (fused)", lambda: L.kai_dense_forward(0, P(y), None, P(w), P(b), P(x), I(1024), I(256), I(1024), 0, None),
+        flops=f, cpu=lambda: ko.add_bias(ko.matmul(wc, xc), bc))
+    alpha = torch.tensor([0.1], device=dev)
+    for name in ("relu", "leaky", "sigmoid", "tanh", "gelu", "selu", "mish", "swish"):
+        row("cfg2 Y = %s(X.W^T + b) (fused)" % name,
+            lambda: L.kai_dense_forward(0, P(y), None, P(w), P(b), P(x), I(1024), I(256), I(1024), kai.ACT[name], P(alpha)),
+            flops=f)
+    row("cfg2 dX = dY.W", lambda: L.kai_matmul_backward_x(0, P(gx), P(gy), P(w), I(1024), I(256), I(1024), 0),
+        flops=f, cpu=lambda: ko.matmul_backward_x(gyc, wc))
+    row("cfg2 dW = dY^T.X", lambda: L.kai_matmul_backward_w(0, P(gw), P(gy), P(x), I(1024), I(256), I(1024), 0),
+        flops=f, cpu=lambda: ko.matmul_backward_w(gyc, xc, 1024, 1024))
+    row("cfg2 db = colsum(dY)", lambda: L.kai_add_bias_backward_b(0, P(gb), P(gy), I(256), I(1024), 0),
+        nbytes=4.0 * 256 * 1024, cpu=lambda: ko.add_bias_backward_b(gyc, 1024))
     pre = torch.randn((256, 1024), device=dev, generator=g)
     work = torch.empty_like(pre)
     row("cfg2 dense backward with ReLU: dX, dW, db from dY and the pre-activation (kai_dense_backward)",
-        gpu_us(lambda: L.kai_dense_backward(0, P(gx), P(gw), P(gb), P(work), P(gy), P(w), P(x), P(pre), I(1024), I(256),
-                                            I(1024), relu, None, 0)),
+        lambda: L.kai_dense_backward(0, P(gx), P(gw), P(gb), P(work), P(gy), P(w), P(x), P(pre), I(1024), I(256),
+                                            I(1024), relu, None, 0),
         flops=2 * f)
     # cfg4: attention, both mappings of 32 batch x heads, seq 512, head dim 64
     for nbat, nhead, nvec in ((32, 1, 64), (4, 8, 512)):
@@ -233,26 +247,26 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
         fl = 2.0 * 32 * T * T * D
         qc, kc, vc = q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy()
         row(tag + "S = Q.K^T/8 (mult_on_heads)",
-            gpu_us(lambda: L.kai_mult_on_heads(0, P(s0), P(k), P(q), I(nbat), I(T), I(nvec), I(nhead), I(D), P(coef))),
-            flops=fl, cpu=cpu_us(lambda: ko.mult_on_heads(kc, qc, nhead, 0.125)))
+            lambda: L.kai_mult_on_heads(0, P(s0), P(k), P(q), I(nbat), I(T), I(nvec), I(nhead), I(D), P(coef)),
+            flops=fl, cpu=lambda: ko.mult_on_heads(kc, qc, nhead, 0.125))
         row(tag + "softmax_direct_on_axis (in place)",
-            gpu_us(lambda b: L.kai_softmax_direct_on_axis(0, P(b), I(nbat * T), I(T), I(nhead)), iters=20,
-                   prep=lambda: s0.clone()),
-            nbytes=8.0 * 32 * T * T, cpu=cpu_us(lambda: ko.softmax_direct_on_axis(s0.cpu().numpy(), nbat * T, T, nhead)))
+            lambda b: L.kai_softmax_direct_on_axis(0, P(b), I(nbat * T), I(T), I(nhead)), iters=20,
+                   prep=lambda: s0.clone(),
+            nbytes=8.0 * 32 * T * T, cpu=lambda: ko.softmax_direct_on_axis(s0.cpu().numpy(), nbat * T, T, nhead))
         pbuf.copy_(s0)
         L.kai_softmax_direct_on_axis(0, P(pbuf), I(nbat * T), I(T), I(nhead))
         row(tag + "O = P.V (mix_values)",
-            gpu_us(lambda: L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))),
-            flops=fl, cpu=cpu_us(lambda: ko.mix_values(pbuf.cpu().numpy(), vc, nhead)))
+            lambda: L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D)),
+            flops=fl, cpu=lambda: ko.mix_values(pbuf.cpu().numpy(), vc, nhead))
         def three_calls():
             L.kai_mult_on_heads(0, P(pbuf), P(k), P(q), I(nbat), I(T), I(nvec), I(nhead), I(D), P(coef))
             L.kai_softmax_direct_on_axis(0, P(pbuf), I(nbat * T), I(T), I(nhead))
             L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))
 
-        row(tag + "the three calls back to back", gpu_us(three_calls), flops=2 * fl)
+        row(tag + "the three calls back to back", three_calls, flops=2 * fl)
         row(tag + "all three fused, forward only (kai_attention_forward)",
-            gpu_us(lambda: L.kai_attention_forward(0, P(o), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
-                                                   P(coef), 0)),
+            lambda: L.kai_attention_forward(0, P(o), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
+                                                   P(coef), 0),
             flops=2 * fl)
         # the backward calls of the same block (vtensor.cpp:3142-3166 of the reference)
         go = torch.randn((nbat, T, nvec), device=dev, generator=g)
@@ -261,20 +275,20 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
         gq = torch.empty_like(q)
         goc = go.cpu().numpy() if with_cpu else None
         row(tag + "gP = gO.V^T (mix_values_backward_prop)",
-            gpu_us(lambda: L.kai_mix_values_backward_prop(0, P(gp), P(go), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))),
-            flops=fl, cpu=cpu_us(lambda: ko.mix_values_backward_prop(goc, vc, nhead)))
+            lambda: L.kai_mix_values_backward_prop(0, P(gp), P(go), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D)),
+            flops=fl, cpu=lambda: ko.mix_values_backward_prop(goc, vc, nhead))
         row(tag + "gV = P^T.gO (mix_values_backward_value)",
-            gpu_us(lambda: L.kai_mix_values_backward_value(0, P(gv), P(go), P(pbuf), I(nbat), I(T), I(nvec), I(nhead), I(D))),
-            flops=fl, cpu=cpu_us(lambda: ko.mix_values_backward_value(goc, pbuf.cpu().numpy(), nhead)))
+            lambda: L.kai_mix_values_backward_value(0, P(gv), P(go), P(pbuf), I(nbat), I(T), I(nvec), I(nhead), I(D)),
+            flops=fl, cpu=lambda: ko.mix_values_backward_value(goc, pbuf.cpu().numpy(), nhead))
         gp0 = gp.clone()
         row(tag + "softmax_direct_on_axis_backward (in place)",
-            gpu_us(lambda b: L.kai_softmax_direct_on_axis_backward(0, P(b), P(pbuf), I(nbat), I(T), I(nhead), P(coef)),
-                   iters=20, prep=lambda: gp0.clone()),
+            lambda b: L.kai_softmax_direct_on_axis_backward(0, P(b), P(pbuf), I(nbat), I(T), I(nhead), P(coef)),
+                   iters=20, prep=lambda: gp0.clone(),
             nbytes=12.0 * 32 * T * T,
-            cpu=cpu_us(lambda: ko.softmax_direct_on_axis_backward(gp0.cpu().numpy(), pbuf.cpu().numpy(), 0.125)))
+            cpu=lambda: ko.softmax_direct_on_axis_backward(gp0.cpu().numpy(), pbuf.cpu().numpy(), 0.125))
         row(tag + "gQ = gS.K (mult_on_heads_backward)",
-            gpu_us(lambda: L.kai_mult_on_heads_backward(0, P(gq), P(gp), P(k), I(nbat), I(T), I(nvec), I(nhead), I(D))),
-            flops=fl, cpu=cpu_us(lambda: ko.mult_on_heads_backward(gp.cpu().numpy(), kc, nhead)))
+            lambda: L.kai_mult_on_heads_backward(0, P(gq), P(gp), P(k), I(nbat), I(T), I(nvec), I(nhead), I(D)),
+            flops=fl, cpu=lambda: ko.mult_on_heads_backward(gp.cpu().numpy(), kc, nhead))
     # cfg5: skinny (cold: six rotating weight buffers) and ragged
     K = N = 4096
     ws = [torch.rand((N, K), device=dev, generator=g) * 0.1 - 0.05 for _ in range(6)]
@@ -289,23 +303,23 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
 
         wc = ws[0].cpu().numpy() if with_cpu else None
         xc = x.cpu().numpy()
-        row("cfg5 M=%d x 4096 x 4096 (cold)" % m, gpu_us(call, iters=120), flops=2.0 * m * N * K,
-            nbytes=4.0 * (K * N + m * K + m * N), cpu=cpu_us(lambda: ko.matmul(wc, xc)))
+        row("cfg5 M=%d x 4096 x 4096 (cold)" % m, call, iters=120, flops=2.0 * m * N * K,
+            nbytes=4.0 * (K * N + m * K + m * N), cpu=lambda: ko.matmul(wc, xc))
     del ws
     m, k, n = 1000, 777, 333
     x = torch.randn((m, k), device=dev, generator=g)
     w = torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05
     y = torch.empty((m, n), device=dev)
     xc, wc = x.cpu().numpy(), w.cpu().numpy()
-    row("cfg5 ragged 1000x777x333", gpu_us(lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0)),
-        flops=2.0 * m * n * k, cpu=cpu_us(lambda: ko.matmul(wc, xc)))
+    row("cfg5 ragged 1000x777x333", lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0),
+        flops=2.0 * m * n * k, cpu=lambda: ko.matmul(wc, xc))
     # batches of a per-shard size against a wide weight matrix (kai_matmul, the matrix warm in the caches)
     for m, n, k in ((32, 4096, 4096), (64, 4096, 4096), (96, 4096, 4096), (144, 4096, 4096), (256, 2048, 2048)):
         x = torch.randn((m, k), device=dev, generator=g)
         w = torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05
         y = torch.empty((m, n), device=dev)
         row("batch of %d rows: Y = X.W^T, W %d x %d (%s)" % (m, n, k, kai.VMath.gemm_plan(0, 1, m, n, k)),
-            gpu_us(lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0)), flops=2.0 * m * n * k)
+            lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0), flops=2.0 * m * n * k)
     # one LSTM layer forward as the engine's loop issues it (vtensor.cpp:2455-2492): 32 steps of 64 x 256 -> 4 x 256
     nt_, nd_, ni_, nr_ = 32, 64, 256, 256
     xs = torch.randn((nt_, nd_, ni_), device=dev, generator=g)
@@ -332,11 +346,11 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
             L.kai_lstm_process(0, P(rec[t]), P(sta[t]), P(sta[t - 1]) if t > 0 else None, P(aff[t]), I(nd_), I(nr_), I(ni_))
 
     lstm_flops = 2.0 * nt_ * nd_ * 4 * nr_ * (ni_ + nr_)
-    row("lstm layer forward, 32 steps x (64 x 256 -> 4 x 256), per-step calls", gpu_us(lambda: lstm_layer(False), iters=10),
+    row("lstm layer forward, 32 steps x (64 x 256 -> 4 x 256), per-step calls", lambda: lstm_layer(False), iters=10,
         flops=lstm_flops)
-    row("lstm layer forward, same, input products of all steps in one call", gpu_us(lambda: lstm_layer(True), iters=10),
+    row("lstm layer forward, same, input products of all steps in one call", lambda: lstm_layer(True), iters=10,
         flops=lstm_flops)
-    row("lstm layer forward, same, one kai_lstm_step per step", gpu_us(lambda: lstm_layer(True, True), iters=10),
+    row("lstm layer forward, same, one kai_lstm_step per step", lambda: lstm_layer(True, True), iters=10,
         flops=lstm_flops)
     # the same calls recorded once into a HIP graph and replayed (the counterpart of the engine's call replay)
     side = torch.cuda.Stream()
@@ -346,7 +360,7 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
         with torch.cuda.graph(graph, stream=side):
             lstm_layer(True, fused)
         kai.set_stream(stream.cuda_stream)
-        row("lstm layer forward, %s, replayed from a HIP graph" % name, gpu_us(graph.replay, iters=10), flops=lstm_flops)
+        row("lstm layer forward, %s, replayed from a HIP graph" % name, graph.replay, iters=10, flops=lstm_flops)
         del graph
     # transposes next to the path: the head split [4,512,8,64] -> [4,8,512,64] of configuration 4 and a plain 4096^2
     shape, axes = (4, 512, 8, 64), (0, 2, 1, 3)
@@ -357,13 +371,13 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0):
                         dtype=torch.int32, device=dev)
     xc = x.cpu().numpy()
     row("transpose [4,512,8,64] -> [4,8,512,64]",
-        gpu_us(lambda: L.kai_transpose(0, P(y), P(x), P(info), I(4), I(x.numel()))),
-        nbytes=8.0 * x.numel(), cpu=cpu_us(lambda: ko.transpose(xc, axes)))
+        lambda: L.kai_transpose(0, P(y), P(x), P(info), I(4), I(x.numel())),
+        nbytes=8.0 * x.numel(), cpu=lambda: ko.transpose(xc, axes))
     x = torch.randn((4096, 4096), device=dev, generator=g)
     y = torch.empty_like(x)
     xc = x.cpu().numpy()
-    row("transpose_bin 4096 x 4096", gpu_us(lambda: L.kai_transpose_bin(0, P(y), P(x), I(4096), I(4096))),
-        nbytes=8.0 * x.numel(), cpu=cpu_us(lambda: ko.transpose_bin(xc, 4096, 4096)))
+    row("transpose_bin 4096 x 4096", lambda: L.kai_transpose_bin(0, P(y), P(x), I(4096), I(4096)),
+        nbytes=8.0 * x.numel(), cpu=lambda: ko.transpose_bin(xc, 4096, 4096))
     return rows
 
 
@@ -374,6 +388,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="skip the table of the other configurations")
+    ap.add_argument("--only", action="append", default=None, metavar="TEXT",
+                    help="measure only the rows of the table whose name contains TEXT (may be given several times)")
     ap.add_argument("--row-warmup-ms", type=float, default=40.0,
                     help="untimed warm-up before each row of the table (a profiler run passes a small value to keep its trace short)")
     args = ap.parse_args()
@@ -515,7 +531,7 @@ def main():
     else:
         out["cpu_baseline"] = None
     if not args.headline_only:
-        out["per_config"] = per_config_table(torch, kai, stream, dev, not args.no_cpu_baseline, args.row_warmup_ms)
+        out["per_config"] = per_config_table(torch, kai, stream, dev, not args.no_cpu_baseline, args.row_warmup_ms, args.only)
     print(json.dumps(out))
 
 

@@ -91,7 +91,7 @@ int64_t small_tile_split(int64_t tiles, int64_t K, int64_t cus) {
 // best measured one on average, 8 % at worst).  A workgroup takes a fixed time per 32 reduction steps whatever
 // shares its compute unit -- small 0.48 us with both operands K-contiguous, else 0.57 / 0.54 / 0.52 with one / two /
 // three workgroups per unit and 0.49 with more (the simple schedule), wide 0.95, medium 1.8 (two resident at
-// most); edge tiles cost a twentieth more -- so the kernel takes
+// most); edge tiles cost a twentieth more (not on the small tile with two K-contiguous operands) -- so the kernel takes
 // rounds x steps x that, plus 3.5 us of launch, first loads and epilogue; the parts cost a second launch
 // (3.5 us + 0.1 per part) and their traffic (each part written and read once, at about 6 TB/s).
 double tiled_cost(int tile, bool both_kc, bool whole, int64_t M, int64_t N, int64_t k_len, int64_t parts, int64_t cus) {
@@ -110,7 +110,10 @@ double tiled_cost(int tile, bool both_kc, bool whole, int64_t M, int64_t N, int6
         pipelined = false;   // the simple schedule
         t = (double)per_cu * steps * 0.49;
     } else {
-        double c = both_kc ? 0.48 : (per_cu == 1 ? 0.57 : per_cu == 2 ? 0.54 : 0.52) * (whole ? 1.0 : 1.05);
+        // (the surcharge for edge tiles applies to the forms with an operand that is not K-contiguous only: the
+        // sweeps this was fitted to were run with exactly this expression, and with both operands K-contiguous the
+        // edge variant's range-checked loads measured like the whole-tile ones)
+        const double c = both_kc ? 0.48 : (per_cu == 1 ? 0.57 : per_cu == 2 ? 0.54 : 0.52) * (whole ? 1.0 : 1.05);
         t = (double)per_cu * steps * c;
     }
     // the pipelined kernels run the steps after the last whole tile of 32 as a tile of their own, loaded, masked
@@ -150,6 +153,9 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // large tile wins: it moves half as much through LDS per flop (8000^3: 7.1 against 7.5 ms).
     const int64_t short_side = d.M < d.N ? d.M : d.N;
     const int64_t cus = compute_units();
+    // bytes of partial sums this product may use: the library scratch grows up to kSplitScratchMax, a caller's
+    // fixed buffer (the allocation-free entry point) may be smaller, and the part count is then chosen to fit it
+    const int64_t scratch_cap = d.scratch ? std::min(kSplitScratchMax, d.scratch_bytes) : kSplitScratchMax;
     const int64_t t256 = tiles_of(d.M, d.N, d.nbatch, 256), t128 = tiles_of(d.M, d.N, d.nbatch, 128);
     if (short_side > 128 && t256 >= (3 * cus) / 4 && 4 * ((t256 + cus - 1) / cus) <= (t128 + cus - 1) / cus)
         plan.tile = kTileLarge;
@@ -206,7 +212,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
                     int64_t k_len = d.K;
                     bool equal = true;
                     if (sp > 1) {
-                        if (d.K < kSplitFromK || sp * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) break;
+                        if (d.K < kSplitFromK || sp * d.M * d.N * (int64_t)sizeof(float) > scratch_cap) break;
                         equal = d.K % (16 * sp) == 0;
                         k_len = equal ? d.K / sp : ((d.K + sp - 1) / sp + 15) / 16 * 16;
                         // parts of at least 256 steps, 512 for the larger tiles (their first tile takes longer to arrive)
@@ -249,7 +255,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
             for (int64_t sp = 1; sp <= kSplitMax; sp++) {
                 int64_t k_len = d.K;
                 if (sp > 1) {
-                    if (d.K < kSplitFromK || sp * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) break;
+                    if (d.K < kSplitFromK || sp * d.M * d.N * (int64_t)sizeof(float) > scratch_cap) break;
                     k_len = d.K % (16 * sp) == 0 ? d.K / sp : ((d.K + sp - 1) / sp + 15) / 16 * 16;
                     if (k_len < 256) break;
                     if ((d.K + k_len - 1) / k_len != sp) continue;
@@ -313,7 +319,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         const bool one_flat_row = plan.tile == kTileFlat && d.M <= 32;
         if ((plan.tile == kTileSmall || plan.tile == kTileFlat) && d.K >= 1024 && !one_flat_row)
             split = small_tile_split(tiles, d.K, cus);
-        while (split > 1 && split * d.M * d.N * (int64_t)sizeof(float) > kSplitScratchMax) split /= 2;
+        while (split > 1 && split * d.M * d.N * (int64_t)sizeof(float) > scratch_cap) split /= 2;
         if (split > d.K / kSplitMinK) split = d.K / kSplitMinK;
         if (split > kSplitMax) split = kSplitMax;
         // equal parts of whole 16-step tiles if some part count allows it; else parts of whole tiles with a

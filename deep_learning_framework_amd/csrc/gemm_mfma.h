@@ -364,9 +364,9 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 }
 
 // Epilogue of one output tile.  In registers: alpha, += C (acc), bias, optional store of the
-// pre-activation, then none / relu / leaky relu.  The transcendental activations are applied in a
-// second, rolled pass in which each thread re-reads the values it has just stored: that keeps the
-// unrolled part small enough for the accumulators to stay in registers for the whole kernel.
+// pre-activation, the activation, one store.  none / relu / leaky relu are written out per element; the
+// transcendental codes run in a rolled loop over the 16 rows of a block (see there), so that the kernel
+// holds one copy of their code per block and the accumulators stay in registers for the whole kernel.
 template <int NBM, int NBN, bool A_KC, bool B_KC>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[NBM][NBN], int m0, int n0,
                                               int64_t c_off, int wm0, int wn0, int l32, int half, float alpha,
@@ -445,19 +445,43 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                 for (int r = 0; r < 16; r++)
                     if (row_ok(r) && col_ok) *reinterpret_cast<vecw*>(C2 + rowoff(r) + col) = o[r];
             }
-            if (act != kActNone) {
+            if (slow_act) {
+                // The values go back into the accumulator vectors (compile-time indices) and a ROLLED loop picks
+                // row r out of them with a run-time index (a register-indexed move, the index is wave-uniform):
+                // one copy of the transcendental code per 32-row block instead of one per element, every value
+                // transformed in registers and stored once.
+                static_for<0, 16>([&](auto rc) {
+                    constexpr int r = decltype(rc)::value;
+                    static_for<0, NBN>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        acc[i][j][r] = o[r][j];
+                    });
+                });
+#pragma nounroll
+                for (int r = 0; r < 16; r++) {
+                    vecw x;
+                    static_for<0, VW>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        x[j] = apply_act(acc[i][j % NBN][r], act, leaky);
+                    });
+                    const int d = (A_KC ? 1 : NBM) * (8 * (r >> 2) + (r & 3));
+                    if (row0 + d < p.M && col_ok) *reinterpret_cast<vecw*>(C + base0 + (int64_t)d * p.c_rs + col) = x;
+                }
+            } else {
+                if (act != kActNone) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+#pragma unroll
+                        for (int j = 0; j < VW; j++) {
+                            float v = o[r][j];
+                            activate_cheap(v);
+                            o[r][j] = v;
+                        }
+                }
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-#pragma unroll
-                    for (int j = 0; j < VW; j++) {
-                        float v = o[r][j];
-                        activate_cheap(v);
-                        o[r][j] = v;
-                    }
+                    if (row_ok(r) && col_ok) *reinterpret_cast<vecw*>(C + rowoff(r) + col) = o[r];
             }
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                if (row_ok(r) && col_ok) *reinterpret_cast<vecw*>(C + rowoff(r) + col) = o[r];
         } else {
             float v[NBN][16];
             int cols[NBN];
@@ -507,38 +531,41 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                     for (int r = 0; r < 16; r++)
                         if (row_ok(r) && cols[j] < p.N) C2[rowoff(r) + coloff[j]] = v[j][r];
             }
-            if (act != kActNone) {
+            if (slow_act) {
+                // as above: back into the accumulator vectors, then one rolled loop over the 16 rows of the block
+                static_for<0, NBN>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    static_for<0, 16>([&](auto rc) {
+                        constexpr int r = decltype(rc)::value;
+                        acc[i][j][r] = v[j][r];
+                    });
+                });
+#pragma nounroll
+                for (int r = 0; r < 16; r++) {
+                    const int d = (A_KC ? 1 : NBM) * (8 * (r >> 2) + (r & 3));
+                    const bool ok = row0 + d < p.M;
+                    const int64_t ro = base0 + (int64_t)d * p.c_rs;
+                    static_for<0, NBN>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        const float x = apply_act(acc[i][j][r], act, leaky);
+                        if (ok && cols[j] < p.N) C[ro + coloff[j]] = x;
+                    });
+                }
+            } else {
+                if (act != kActNone) {
+#pragma unroll
+                    for (int j = 0; j < NBN; j++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) activate_cheap(v[j][r]);
+                }
 #pragma unroll
                 for (int j = 0; j < NBN; j++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) activate_cheap(v[j][r]);
+                    for (int r = 0; r < 16; r++)
+                        if (row_ok(r) && cols[j] < p.N) C[rowoff(r) + coloff[j]] = v[j][r];
             }
-#pragma unroll
-            for (int j = 0; j < NBN; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    if (row_ok(r) && cols[j] < p.N) C[rowoff(r) + coloff[j]] = v[j][r];
         }
     });
-
-    if (slow_act) {
-#pragma nounroll
-        for (int i = 0; i < NBM; i++) {
-#pragma nounroll
-            for (int r = 0; r < 16; r++) {
-                const int row = row_of(i, r);
-                if (row >= p.M) continue;
-#pragma nounroll
-                for (int j = 0; j < NBN; j++) {
-                    const int col = col_of(j);
-                    if (col < p.N) {
-                        const int64_t idx = (int64_t)row * p.c_rs + (int64_t)col * p.c_cs;
-                        C[idx] = apply_act(C[idx], act, leaky);
-                    }
-                }
-            }
-        }
-    }
 }
 
 // EDGE = false: the host has checked that M, N, K are multiples of the tile, that both operands

@@ -33,6 +33,14 @@ int noalloc_scratch(float** out) {
         return kai::fail(KAI_ERR_INVALID_ARGUMENT, "kai_matmul_noalloc: device index out of range");
     std::lock_guard<std::mutex> lock(g_noalloc_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
+        // The look-up may load the code object onto this device, which allocates: it must not happen while the
+        // calling thread's stream is being captured.  kai_matmul_noalloc_scratch_bytes() or any earlier call on
+        // the device does it ahead of time.
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(kai::current_stream(), &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+            return kai::fail(KAI_ERR_GPU, "kai_matmul_noalloc: first use on this device while its stream is being captured; "
+                                          "call kai_matmul_noalloc_scratch_bytes() on the device before the capture");
+        (void)hipGetLastError();
         float* ptr = nullptr;
         KAI_TRY(kai::check_hip(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)),
                                "hipGetSymbolAddress(scratch)"));
@@ -67,4 +75,10 @@ extern "C" int kai_matmul_noalloc(int device, float* py, const float* pw, const 
     return launch_gemm(d, current_stream());
 }
 
-extern "C" int64_t kai_matmul_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
+// Also the set-up call: it looks up the array's address on the current device, so that a later kai_matmul_noalloc
+// there has nothing left to do but launch (a failure of the look-up is reported by that later call).
+extern "C" int64_t kai_matmul_noalloc_scratch_bytes(void) {
+    float* ptr = nullptr;
+    (void)noalloc_scratch(&ptr);
+    return kNoAllocScratchBytes;
+}

@@ -142,8 +142,15 @@ int launch_skinny_rows(const GemmDesc& d, hipStream_t stream) {
     int64_t splits = compute_units() / slices;
     if (splits < 1) splits = 1;
     if (splits > 16) splits = 16;
-    const int64_t k_part = ((d.K + splits - 1) / splits + unit - 1) / unit * unit;
-    splits = (d.K + k_part - 1) / k_part;
+    const int64_t k_first = ((d.K + splits - 1) / splits + unit - 1) / unit * unit;
+    splits = (d.K + k_first - 1) / k_first;
+    // a caller's fixed buffer: fewer, longer parts until their sums fit it
+    int64_t k_len = k_first;
+    while (d.scratch && splits > 1 && splits * d.M * d.N * (int64_t)sizeof(float) > d.scratch_bytes) {
+        k_len += unit;
+        splits = (d.K + k_len - 1) / k_len;
+    }
+    const int64_t k_part = k_len;
     float* part = d.scratch;
     const int64_t part_bytes = splits * d.M * d.N * (int64_t)sizeof(float);
     if (part == nullptr) KAI_TRY(workspace(part_bytes, &part));

@@ -295,9 +295,12 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
 // 20.2 -> 17.2; 11008 x 4096 45.4 -> 38.3 / 49.7 -> 45.8 | 39.0 -> 36.1 / 47.3 -> 44.2; 4096 x 8192 37.4 -> 28.9 /
 // 38.7 -> 34.0 | 25.8 -> 27.9 / 29.6 -> 33.0; 8192 x 8192 (256 MB, left out) 64.8 -> 54.5 / 67.5 -> 64.9 |
 // 44.0 -> 52.2 / 51.3 -> 63.5.
+// Rows longer than 4096 steps are taken only up to 96 MB: a weight matrix that a serving loop multiplies again and
+// again stays in the last-level cache, and there 4096 x 8192 lost 8..11 % (the warm figures above).
 bool skinny_stream32_applies(const SkinnyParams& p) {
     return p.M > kSkinnyMaxRows && p.M <= 2 * kSkinnyMaxRows && p.K % (kSsWaves * 512) == 0 && p.N % 16 == 0 &&
-           p.N >= 16 * (int64_t)compute_units() && p.N * (int64_t)p.K * 4 <= (192ll << 20) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
+           p.N >= 16 * (int64_t)compute_units() && p.N * (int64_t)p.K * 4 <= (192ll << 20) &&
+           (p.K <= 4096 || p.N * (int64_t)p.K * 4 <= (96ll << 20)) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
            (15 * p.ldw + p.K) * 4 < (1ll << 31) && ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
 }
 

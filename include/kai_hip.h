@@ -136,13 +136,19 @@ int kai_matmul_backward_w(int device, float* pgw, const float* pgy, const float*
                           int64_t xvec, int acc);
 
 /* kai_matmul for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same kernels and
- * the same result as kai_matmul; it calls no hipMalloc / hipFree and never touches the library's heap scratch.
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and the same kernels as
+ * kai_matmul; it calls no hipMalloc / hipFree and never touches the library's heap scratch.
  * A product whose reduction is cut into parts keeps the partial sums in a fixed 32 MiB array inside the
- * library's code object (each GPU the library runs on holds its copy until the process ends); a product whose
- * partial sums would need more (kai_matmul_noalloc_scratch_bytes) is refused with KAI_ERR_INVALID_ARGUMENT and
+ * library's code object (each GPU the library runs on holds its copy until the process ends); the number of parts
+ * is chosen so that their sums fit the array, so a product that kai_matmul would cut finer runs here with fewer
+ * parts (equal to kai_matmul up to the order of the partial sums, bit for bit wherever the part count is the
+ * same).  Should a product ever need more than the array holds it is refused with KAI_ERR_INVALID_ARGUMENT and
  * a message that names both sizes.  All calls on one GPU share that array: calls that overlap on one GPU race
- * and must be serialised by the caller.  The first call on a device looks up the array's address. */
+ * and must be serialised by the caller.
+ * The first use on a device looks up the array's address, which may load the code object there: that must happen
+ * BEFORE a stream capture begins.  kai_matmul_noalloc_scratch_bytes() does the look-up for the current device
+ * (call it once per device at set-up) and returns the array's size; a first kai_matmul_noalloc made while the
+ * thread's stream is being captured fails with KAI_ERR_GPU instead of allocating. */
 int kai_matmul_noalloc(int device, float* py, const float* pw, const float* px, int64_t yvec, int64_t ndat,
                        int64_t xvec, int acc);
 int64_t kai_matmul_noalloc_scratch_bytes(void);
