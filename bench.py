@@ -289,6 +289,27 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
         row(tag + "gQ = gS.K (mult_on_heads_backward)",
             lambda: L.kai_mult_on_heads_backward(0, P(gq), P(gp), P(k), I(nbat), I(T), I(nvec), I(nhead), I(D)),
             flops=fl, cpu=lambda: ko.mult_on_heads_backward(gp.cpu().numpy(), kc, nhead))
+        # the same backward middle (vtensor.cpp:3145-3154) as the reference's five calls back to back, and as one call
+        mo = torch.empty_like(o)
+        L.kai_mix_values(0, P(mo), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))
+        gk = torch.empty_like(q)
+
+        def five_calls():
+            L.kai_mix_values_backward_prop(0, P(gp), P(go), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))
+            L.kai_mix_values_backward_value(0, P(gv), P(go), P(pbuf), I(nbat), I(T), I(nvec), I(nhead), I(D))
+            L.kai_softmax_direct_on_axis_backward(0, P(gp), P(pbuf), I(nbat), I(T), I(nhead), P(coef))
+            L.kai_mult_on_heads_backward(0, P(gk), P(gp), P(q), I(nbat), I(T), I(nvec), I(nhead), I(D))
+            L.kai_mult_on_heads_backward(0, P(gq), P(gp), P(k), I(nbat), I(T), I(nvec), I(nhead), I(D))
+
+        row(tag + "backward: the five calls back to back", five_calls, flops=4 * fl)
+        row(tag + "backward: gQ, gK, gV in one call, two launches (kai_attention_backward)",
+            lambda: L.kai_attention_backward(0, P(gq), P(gk), P(gv), P(go), P(pbuf), P(mo), P(q), P(k), P(v), I(nbat), I(T),
+                                             I(nvec), I(nhead), I(D), P(coef), 0),
+            flops=4 * fl)
+        row(tag + "backward: the same without the mixed output (row sums in a first pass)",
+            lambda: L.kai_attention_backward(0, P(gq), P(gk), P(gv), P(go), P(pbuf), None, P(q), P(k), P(v), I(nbat), I(T),
+                                             I(nvec), I(nhead), I(D), P(coef), 0),
+            flops=5 * fl)
     # cfg5: skinny (cold: six rotating weight buffers) and ragged
     K = N = 4096
     ws = [torch.rand((N, K), device=dev, generator=g) * 0.1 - 0.05 for _ in range(6)]

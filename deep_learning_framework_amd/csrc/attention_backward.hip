@@ -1,0 +1,397 @@
+// The backward middle of the attention block in one kernel per output kind:
+//   gP = gM.V^T                     VMath::mix_values_backward_prop        (vmath.cu:7029-7077 of the reference)
+//   gS = coef * P * (gP - sum P*gP) VMath::softmax_direct_on_axis_backward (vmath.cu:6920-6973)
+//   gS[k > q] = 0 when masked       VMath::set_mh_attention_mask, backward (vmath.cu:6833-6860)
+//   gK[t] = sum_k gS[t,k] * Q[k]    VMath::mult_on_heads_backward          (vmath.cu:6783-6829)
+//   gQ[t] = sum_k gS[t,k] * K[k]    VMath::mult_on_heads_backward, second call
+// as VTensor::multihead_attention_backprop issues them (vtensor.cpp:3145-3154).  The reference indexes gp by the
+// OUTPUT row t for the key gradient and the query gradient alike (vmath.cu:6790-6797), so gP -> gS -> gK, gQ are all
+// local to a row t: a workgroup that owns 64 rows of one (batch entry, head) forms the row's gP tile by tile, turns
+// it into gS in registers and multiplies it into both outputs.  Neither gP nor gS is ever stored.  The value
+// gradient gV = P^T.gM is a reduction over rows and keeps its own launch (mix_values_backward_value).
+//
+// The sum over k of P*gP that the softmax derivative needs equals sum_d gM[t,d] * M[t,d] with M = P.V, the mixed
+// output of the forward pass, which the engine keeps for the output projection's weight gradient (vtensor.cpp:3050):
+// given M the row constant costs one dot product of length D; without it a first pass over the keys forms it from
+// P and gP as the reference writes it.
+//
+// Layout of the computation: as in attention_fused.hip, transposed with the rows t along the lanes.
+// v_mfma_f32_16x16x4_f32, lane = (l % 16, l / 16):  gP^T[key, t] = V[key, :] . gM[t, :] puts the gradient of
+// (t, key 4g + v) into register v of lane (t, g), where the matching P values are loaded to (128-bit loads with one
+// head, strided 32-bit loads otherwise), and the registers that hold gS^T are, as they are, the B operand of
+// gQ^T += K^T.gS^T and gK^T += Q^T.gS^T.  Eight waves = 4 groups of 16 rows x 2 halves of every key tile; the halves
+// meet in LDS at the end, in a fixed order.
+#include <float.h>
+
+#include "elementwise.h"
+
+namespace kai {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kAbQGroups = 4;          // waves along the rows t, 16 rows each
+constexpr int kAbKGroups = 2;          // waves along the keys of a tile
+constexpr int kAbWaves = kAbQGroups * kAbKGroups;
+constexpr int kAbThreads = 64 * kAbWaves;
+constexpr int kAbRows = 16 * kAbQGroups;   // rows t per workgroup
+
+struct AttnBwdParams {
+    const float* gM;     // gradient of the mixed output, [nbat, ntimes, nvec]
+    const float* M;      // the mixed output, or null
+    const float* P;      // probabilities, [nbat, ntimes, ntimes, nhead]
+    const float* Q;
+    const float* K;
+    const float* V;
+    float* gQ;
+    float* gK;
+    const float* coef;   // device scalar, null reads as 0
+    int64_t nvec;            // row stride of Q, K, V, gM, M, gQ, gK
+    int64_t batch_stride;    // ntimes * nvec
+    int64_t p_batch_stride;  // ntimes * ntimes * nhead
+    int ntimes, nhead, npiece;
+    int masked;
+};
+
+// DB = head size / 16; KB = blocks of 16 keys per wave and tile (a tile holds 32 * KB keys); PVEC: one head and
+// rows of P that allow 128-bit loads.
+template <int DB, int KB, bool PVEC>
+__global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(const AttnBwdParams p) {
+    constexpr int D = 16 * DB;
+    constexpr int kKeys = 16 * KB * kAbKGroups;
+    constexpr int kStride = D + 4;           // tiles [keys][D] lie in LDS as in memory
+    constexpr int kTile = kKeys * kStride;
+    constexpr int kChunksPerKey = D / 4;
+    constexpr int kTileChunks = kKeys * kChunksPerKey;
+    constexpr int NCH = (kTileChunks + kAbThreads - 1) / kAbThreads;   // 128-bit chunks per thread, operand and tile
+    constexpr bool kPartial = kTileChunks % kAbThreads != 0;
+    constexpr int NP = PVEC ? KB : 4 * KB;   // loads of P per lane and tile
+    // [buffer][operand V, K, Q][tile]
+    __shared__ __attribute__((aligned(16))) float lds[2][3][kTile];
+    static_assert(8 * DB * 64 * kAbQGroups + 64 * kAbQGroups <= 6 * kTile, "the merge buffer must fit the tiles");
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int qg = wave % kAbQGroups;
+    const int kgp = wave / kAbQGroups;
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+    const int T = p.ntimes;
+    const int H = p.nhead;
+    const int b = blockIdx.y / H, h = blockIdx.y % H;
+    const int t0 = blockIdx.x * kAbRows;
+    const int64_t base = (int64_t)b * p.batch_stride + (int64_t)h * p.npiece;
+    const float coef = p.coef ? *p.coef : 0.f;
+
+    // this lane's row and its fragments of gM, scaled by coef once: gS = P * (coef*gP - coef*sum)
+    const int t = t0 + 16 * qg + r16;
+    const int tc = min(t, T - 1);            // rows past the end are clamped, never stored
+    f32x4 gf[DB];
+#pragma unroll
+    for (int s = 0; s < DB; s++)
+        gf[s] = coef * *reinterpret_cast<const f32x4*>(p.gM + base + (int64_t)tc * p.nvec + 16 * s + 4 * g);
+
+    auto uniform_ptr = [](const float* q) -> float* {
+        const uint64_t a = reinterpret_cast<uint64_t>(q);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
+    };
+    // Buffer resources: the rows of V, K, Q of this (batch entry, head) up to the last key, and this batch
+    // entry's block of P from this head's first element on.  Keys past the end read as zeros.
+    const int extent = (int)(((int64_t)(T - 1) * p.nvec + D) * 4);   // bytes; the host keeps these below 2 GiB
+    const int extent_p = (int)((((int64_t)T * T - 1) * H + 1) * 4);
+    const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.V + base), 0, extent, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.K + base), 0, extent, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.Q + base), 0, extent, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_p =
+        __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.P + (int64_t)b * p.p_batch_stride + h), 0, extent_p, 0x00020000);
+    const int tile_bytes = kKeys * (int)p.nvec * 4;
+    const int p_tile_bytes = kKeys * H * 4;
+    int choff[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * kAbThreads;
+        choff[i] = ((c / kChunksPerKey) * (int)p.nvec + (c % kChunksPerKey) * 4) * 4;
+    }
+    // P[t, key, h] with key = tile * kKeys + 16 * KB * kgp + 16 * kb + 4 * g + v
+    int poff[NP];
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        const int key = 16 * KB * kgp + 4 * g + (PVEC ? 16 * i : 16 * (i / 4) + (i % 4));
+        poff[i] = (int)((((int64_t)tc * T + key) * H) * 4);
+    }
+
+    f32x4 rv[NCH], rk[NCH], rq[NCH];
+    auto load_v = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * kAbThreads;
+            if (!kPartial || c < kTileChunks)
+                rv[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_v, choff[i], kt * tile_bytes, 0));
+        }
+    };
+    auto load_kq = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * kAbThreads;
+            if (!kPartial || c < kTileChunks) {
+                rk[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, choff[i], kt * tile_bytes, 0));
+                rq[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, choff[i], kt * tile_bytes, 0));
+            }
+        }
+    };
+    auto store_v = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * kAbThreads;
+            if (!kPartial || c < kTileChunks)
+                *reinterpret_cast<f32x4*>(&lds[buf][0][(c / kChunksPerKey) * kStride + (c % kChunksPerKey) * 4]) = rv[i];
+        }
+    };
+    auto store_kq = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * kAbThreads;
+            if (!kPartial || c < kTileChunks) {
+                *reinterpret_cast<f32x4*>(&lds[buf][1][(c / kChunksPerKey) * kStride + (c % kChunksPerKey) * 4]) = rk[i];
+                *reinterpret_cast<f32x4*>(&lds[buf][2][(c / kChunksPerKey) * kStride + (c % kChunksPerKey) * 4]) = rq[i];
+            }
+        }
+    };
+    // this wave's P values of one tile: pr[kb][v] = P[t, key0 + 16*kb + 4*g + v, h]
+    auto load_p = [&](f32x4 (&pr)[KB], int kt) {
+        if (PVEC) {
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+                pr[kb] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, poff[kb], kt * p_tile_bytes, 0));
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    pr[kb][v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_p, poff[4 * kb + v], kt * p_tile_bytes, 0));
+        }
+    };
+    // gP^T of this wave's keys: KB blocks of 16 keys x 16 rows, scaled by coef through gf
+    auto grad_p = [&](f32x4 (&gp)[KB], const float* lv) {
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) gp[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < DB; s++) {
+            f32x4 vf[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+                vf[kb] = *reinterpret_cast<const f32x4*>(lv + (16 * kb + r16) * kStride + 16 * s + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int kb = 0; kb < KB; kb++)
+                    gp[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[kb][e], gf[s][e], gp[kb], 0, 0, 0);
+        }
+    };
+
+    const int nkt_all = (T + kKeys - 1) / kKeys;
+    const int t_last = min(t0 + kAbRows, T) - 1;
+    // key tiles that hold a key at or below the diagonal of some row of this workgroup
+    const int nkt = p.masked ? min(t_last / kKeys + 1, nkt_all) : nkt_all;
+
+    // ---- the row constant coef * sum_k P[t,k] * gP[t,k] ---------------------------------------------------------
+    float delta = 0.f;
+    if (p.M != nullptr) {
+        const float* mrow = p.M + base + (int64_t)tc * p.nvec;
+#pragma unroll
+        for (int s = 0; s < DB; s++) {
+            const f32x4 mv = *reinterpret_cast<const f32x4*>(mrow + 16 * s + 4 * g);
+            delta += gf[s][0] * mv[0] + gf[s][1] * mv[1] + gf[s][2] * mv[2] + gf[s][3] * mv[3];
+        }
+        delta += __shfl_xor(delta, 16);
+        delta += __shfl_xor(delta, 32);
+    } else {
+        // a pass of its own over ALL keys (the reference's sum does not look at the mask): V tiles only
+        f32x4 pr[KB];
+        load_v(0);
+        store_v(0);
+        __syncthreads();
+        for (int kt = 0; kt < nkt_all; kt++) {
+            const int buf = kt & 1;
+            load_v(min(kt + 1, nkt_all - 1));
+            load_p(pr, kt);
+            const int key0 = kt * kKeys + 16 * KB * kgp;
+            if (key0 < T) {
+                f32x4 gp[KB];
+                grad_p(gp, &lds[buf][0][16 * KB * kgp * kStride]);
+#pragma unroll
+                for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const int key = key0 + 16 * kb + 4 * g + v;
+                        delta += key < T ? pr[kb][v] * gp[kb][v] : 0.f;
+                    }
+            }
+            if (kt + 1 < nkt_all) store_v(buf ^ 1);
+            __syncthreads();
+        }
+        delta += __shfl_xor(delta, 16);
+        delta += __shfl_xor(delta, 32);
+        // the two key halves add their parts
+        float* ex = &lds[0][0][0];
+        if (kgp == 1) ex[qg * 64 + lane] = delta;
+        __syncthreads();
+        if (kgp == 0) {
+            delta += ex[qg * 64 + lane];
+            ex[qg * 64 + lane] = delta;
+        }
+        __syncthreads();
+        delta = ex[qg * 64 + lane];
+        __syncthreads();
+    }
+
+    // ---- gS tile by tile, multiplied into both outputs ----------------------------------------------------------
+    f32x4 acc_q[DB], acc_k[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+        acc_q[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+        acc_k[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    f32x4 p_next[KB];
+    load_v(0);
+    load_kq(0);
+    load_p(p_next, 0);
+    store_v(0);
+    store_kq(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < nkt; kt++) {
+        const int buf = kt & 1;
+        const int nxt = min(kt + 1, nkt - 1);      // the surplus loads of the last tile are never used
+        f32x4 pr[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) pr[kb] = p_next[kb];
+        load_v(nxt);
+        load_kq(nxt);
+        load_p(p_next, nxt);
+        const int key0 = kt * kKeys + 16 * KB * kgp;    // first key of this wave's part of the tile
+        // a part past the end, or entirely above the diagonal of the workgroup's last row, adds nothing
+        if (key0 < T && !(p.masked && key0 > t_last)) {
+            const float* lv = &lds[buf][0][16 * KB * kgp * kStride];
+            const float* lk = &lds[buf][1][16 * KB * kgp * kStride];
+            const float* lq = &lds[buf][2][16 * KB * kgp * kStride];
+            f32x4 gs[KB];
+            grad_p(gs, lv);
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) gs[kb] = pr[kb] * (gs[kb] - delta);
+            // keys past the end or above the diagonal of some row of this wave (wave-uniform test)
+            const bool edge_tile = key0 + 16 * KB > T || (p.masked && key0 + 16 * KB - 1 > t0 + 16 * qg);
+            if (edge_tile) {
+#pragma unroll
+                for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const int key = key0 + 16 * kb + 4 * g + v;
+                        if (key >= T || (p.masked && key > t)) gs[kb][v] = 0.f;
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // gQ^T[d, t] += sum_key K[key, d] * gS[t, key];  gK^T[d, t] += sum_key Q[key, d] * gS[t, key]
+            // (32-bit reads down a column of the tile: consecutive lanes, consecutive d)
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int row = (16 * kb + 4 * g + e) * kStride + r16;
+#pragma unroll
+                    for (int db = 0; db < DB; db++) {
+                        acc_q[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(lk[row + 16 * db], gs[kb][e], acc_q[db], 0, 0, 0);
+                        acc_k[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(lq[row + 16 * db], gs[kb][e], acc_k[db], 0, 0, 0);
+                    }
+                }
+        }
+        if (kt + 1 < nkt) {
+            store_v(buf ^ 1);
+            store_kq(buf ^ 1);
+        }
+        __syncthreads();
+    }
+
+    // the second key half hands its sums over through LDS; the first adds them and stores
+    float* mg = &lds[0][0][0] + (qg * 64 + lane);
+    constexpr int kMergeStride = 64 * kAbQGroups;
+    if (kgp == 1) {
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                mg[(4 * db + v) * kMergeStride] = acc_q[db][v];
+                mg[(4 * DB + 4 * db + v) * kMergeStride] = acc_k[db][v];
+            }
+    }
+    __syncthreads();
+    if (kgp == 1) return;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            acc_q[db][v] += mg[(4 * db + v) * kMergeStride];
+            acc_k[db][v] += mg[(4 * DB + 4 * db + v) * kMergeStride];
+        }
+    // acc[db][v] = gradient of (row t, d = 16*db + 4*g + v)
+    if (t < T) {
+        float* oq = p.gQ + base + (int64_t)t * p.nvec;
+        float* ok = p.gK + base + (int64_t)t * p.nvec;
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+            *reinterpret_cast<f32x4*>(oq + 16 * db + 4 * g) = acc_q[db];
+            *reinterpret_cast<f32x4*>(ok + 16 * db + 4 * g) = acc_k[db];
+        }
+    }
+}
+
+}  // namespace
+
+bool attention_backward_applies(const float* gq, const float* gk, const float* gm, const float* m, const float* pp,
+                                const float* q, const float* k, const float* v, int64_t ntimes, int64_t nvec,
+                                int64_t nhead, int64_t npiece) {
+    // the gradients and the mixed output are [nbat, ntimes, nhead, npiece] like the output of mix_values, the
+    // projections [nbat, ntimes, nvec]: the same thing only when the heads fill the vector
+    return nhead * npiece == nvec && npiece % 16 == 0 && npiece >= 16 && npiece <= 128 && nvec % 4 == 0 && ntimes >= 1 &&
+           ntimes <= kMaxDim && ntimes * nvec * 4 < (1ll << 31) && ntimes * ntimes * nhead * 4 < (1ll << 31) &&
+           nhead >= 1 && aligned16(gq) && aligned16(gk) && aligned16(gm) && (m == nullptr || aligned16(m)) &&
+           aligned16(q) && aligned16(k) && aligned16(v) && (reinterpret_cast<uintptr_t>(pp) & 3u) == 0;
+}
+
+template <int DB, int KB>
+static void launch_rows(const AttnBwdParams& p, bool pvec, dim3 grid, hipStream_t stream) {
+    if (pvec) attention_backward_rows_kernel<DB, KB, true><<<grid, dim3(kAbThreads), 0, stream>>>(p);
+    else attention_backward_rows_kernel<DB, KB, false><<<grid, dim3(kAbThreads), 0, stream>>>(p);
+}
+
+int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const float* m, const float* pp,
+                                   const float* q, const float* k, const float* v, int64_t nbat, int64_t ntimes,
+                                   int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
+                                   hipStream_t stream) {
+    AttnBwdParams p{};
+    p.gM = gm; p.M = m; p.P = pp; p.Q = q; p.K = k; p.V = v; p.gQ = gq; p.gK = gk; p.coef = hcoef;
+    p.nvec = nvec; p.batch_stride = ntimes * nvec; p.p_batch_stride = ntimes * ntimes * nhead;
+    p.ntimes = (int)ntimes; p.nhead = (int)nhead; p.npiece = (int)npiece;
+    p.masked = masked;
+    const int64_t ttiles = (ntimes + kAbRows - 1) / kAbRows;
+    if (ttiles > kMaxDim || nbat * nhead > 65535) return fail(KAI_ERR_INVALID_ARGUMENT, "attention backward: grid too large");
+    const dim3 grid((unsigned)ttiles, (unsigned)(nbat * nhead));
+    const bool pvec = nhead == 1 && ntimes % 4 == 0 && aligned16(pp);
+    switch (npiece / 16) {
+    case 1: launch_rows<1, 2>(p, pvec, grid, stream); break;
+    case 2: launch_rows<2, 2>(p, pvec, grid, stream); break;
+    case 3: launch_rows<3, 2>(p, pvec, grid, stream); break;
+    case 4: launch_rows<4, 2>(p, pvec, grid, stream); break;
+    case 5: launch_rows<5, 2>(p, pvec, grid, stream); break;
+    case 6: launch_rows<6, 2>(p, pvec, grid, stream); break;
+    case 7: launch_rows<7, 1>(p, pvec, grid, stream); break;
+    default: launch_rows<8, 1>(p, pvec, grid, stream); break;
+    }
+    return check_launch("attention_backward_rows_kernel");
+}
+
+}  // namespace kai

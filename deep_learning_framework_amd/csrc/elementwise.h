@@ -92,4 +92,13 @@ int launch_attention_fused(float* o, const float* q, const float* k, const float
                            int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
                            hipStream_t stream);
 
+// attention_backward.hip: gQ and gK of the attention block from gM, P (and M) without storing gP or gS
+bool attention_backward_applies(const float* gq, const float* gk, const float* gm, const float* m, const float* pp,
+                                const float* q, const float* k, const float* v, int64_t ntimes, int64_t nvec,
+                                int64_t nhead, int64_t npiece);
+int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const float* m, const float* pp,
+                                   const float* q, const float* k, const float* v, int64_t nbat, int64_t ntimes,
+                                   int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
+                                   hipStream_t stream);
+
 }  // namespace kai

@@ -838,4 +838,30 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
     return kai_mix_values(device, py, pp, pV, nbat, ntimes, nvec, nhead, npiece);
 }
 
+int kai_attention_backward(int device, float* pgQ, float* pgK, float* pgV, const float* pgm, const float* pp,
+                           const float* pm, const float* pQ, const float* pK, const float* pV, int64_t nbat,
+                           int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
+                           int masked) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(pgQ); KAI_REQUIRE_PTR(pgK); KAI_REQUIRE_PTR(pgV); KAI_REQUIRE_PTR(pgm); KAI_REQUIRE_PTR(pp);
+    KAI_REQUIRE_PTR(pQ); KAI_REQUIRE_PTR(pK); KAI_REQUIRE_PTR(pV);
+    // the value gradient is a reduction over the rows: its own launch either way
+    KAI_TRY(kai_mix_values_backward_value(device, pgV, pgm, pp, nbat, ntimes, nvec, nhead, npiece));
+    if (attention_backward_applies(pgQ, pgK, pgm, pm, pp, pQ, pK, pV, ntimes, nvec, nhead, npiece))
+        return launch_attention_backward_rows(pgQ, pgK, pgm, pm, pp, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece,
+                                              hCoef, masked != 0, current_stream());
+    // any other shape: the reference's calls one by one, the gradient of the probabilities in the library's scratch
+    const int64_t pbytes = nbat * ntimes * ntimes * nhead * (int64_t)sizeof(float);
+    float* pgp = nullptr;
+    KAI_TRY(workspace(pbytes, &pgp));
+    ScratchHold held(pbytes);
+    KAI_TRY(kai_mix_values_backward_prop(device, pgp, pgm, pV, nbat, ntimes, nvec, nhead, npiece));
+    KAI_TRY(kai_softmax_direct_on_axis_backward(device, pgp, pp, nbat, ntimes, nhead, hCoef));
+    if (masked) KAI_TRY(kai_set_mh_attention_mask(device, pgp, nbat, ntimes, nhead, 0));
+    KAI_TRY(kai_mult_on_heads_backward(device, pgK, pgp, pQ, nbat, ntimes, nvec, nhead, npiece));
+    return kai_mult_on_heads_backward(device, pgQ, pgp, pK, nbat, ntimes, nvec, nhead, npiece);
+}
+
 }  // extern "C"

@@ -330,6 +330,25 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
                           int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
                           int masked);
 
+/* The backward middle of the same block in two launches: the calls of VTensor::multihead_attention_backprop between
+ * the output projection and the input projections (vtensor.cpp:3145-3154),
+ *   mix_values_backward_prop, mix_values_backward_value, softmax_direct_on_axis_backward,
+ *   [set_mh_attention_mask(backward) when masked != 0], mult_on_heads_backward (key gradient from pQ),
+ *   mult_on_heads_backward (query gradient from pK),
+ * without the [nbat, ntimes, ntimes, nhead] gradient of the probabilities reaching memory.  The reference indexes
+ * that gradient by the output row for the key and the query gradient alike (vmath.cu:6790-6797); this entry point
+ * follows it as written.  pgm: gradient of the mixed output; pp: the probabilities the forward pass kept; pm: the
+ * mixed output of the forward pass (the engine keeps it, vtensor.cpp:3050), or null -- with it the softmax
+ * derivative's row sum is one dot product (sum_k P*gP = sum_d gM*M), without it a first pass over the keys forms
+ * it.  Outputs: pgQ, pgK, pgV, each [nbat, ntimes, nvec].  Head sizes that are multiples of 16 up to 128 with
+ * nhead * npiece == nvec and 16-byte aligned operands run fused (the value gradient in its own launch); any other
+ * shape runs the six calls with the gradient of the probabilities in the library's scratch memory.  Results equal
+ * the separate calls up to the order of the sums. */
+int kai_attention_backward(int device, float* pgQ, float* pgK, float* pgV, const float* pgm, const float* pp,
+                           const float* pm, const float* pQ, const float* pK, const float* pV, int64_t nbat,
+                           int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
+                           int masked);
+
 #ifdef __cplusplus
 }
 #endif

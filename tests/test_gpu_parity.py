@@ -727,6 +727,72 @@ def test_cfg4_attention_backward(nbat, nhead, nvec):
         check(g.to_numpy(q.shape), ko.mult_on_heads_backward(ref_gs, src, nhead), what="cfg4 mult_on_heads_backward " + name)
 
 
+# the backward middle of the block in one call (kai_attention_backward) against the oracle's chain of the six calls
+# it replaces: both cfg4 mappings, the small geometries of test_attention_ops_small (most of them fall back to the
+# separate kernels: head sizes that are no multiple of 16), head sizes 16 .. 128, ragged lengths, masked and not,
+# with the mixed output given (row sums as one dot product) and without it (a first pass over the keys)
+ATTENTION_BACKWARD_SHAPES = [(32, 512, 1, 64), (4, 512, 8, 64),
+                             (2, 5, 1, 3), (3, 17, 4, 8), (1, 64, 2, 64), (2, 33, 3, 5), (1, 130, 1, 64), (1, 7, 200, 2),
+                             (2, 100, 4, 16), (1, 130, 8, 64), (1, 70, 4, 6), (1, 96, 12, 24), (2, 700, 8, 24),
+                             (1, 1100, 4, 6), (3, 1200, 1, 40), (1, 608, 12, 8), (2, 64, 4, 32), (1, 96, 8, 64),
+                             (3, 32, 12, 32), (4, 128, 4, 96), (4, 512, 4, 64),
+                             (2, 384, 12, 64), (1, 500, 16, 96), (2, 1024, 8, 128), (3, 200, 6, 32), (1, 77, 2, 16),
+                             (2, 129, 3, 48), (1, 257, 2, 80), (1, 100, 1, 112), (1, 1, 1, 16), (2, 66, 1, 128)]
+
+
+@pytest.mark.parametrize("nbat,ntimes,nhead,npiece", ATTENTION_BACKWARD_SHAPES)
+def test_attention_backward_one_call(nbat, ntimes, nhead, npiece):
+    nvec = nhead * npiece
+    rng = np.random.default_rng(nbat * 1000 + ntimes * 10 + nhead + npiece)
+    q, k, v, gm = (rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32) for _ in range(4))
+    coef = 1.0 / np.sqrt(npiece)
+    hcoef = kai.hyper(coef)
+    dq, dk, dv, dgm = dev(q), dev(k), dev(v), dev(gm)
+    big = nbat * ntimes * ntimes * nhead >= (1 << 22)
+    for masked in ((False,) if big and ntimes != 512 else (False, True)):
+        s = ko.mult_on_heads(k, q, nhead, coef)
+        if masked:
+            s = ko.set_mh_attention_mask(s, True)
+        p = ko.softmax_direct_on_axis(s, nbat * ntimes, ntimes, nhead)
+        m = ko.mix_values(p, v, nhead)
+        ref_gv = ko.mix_values_backward_value(gm, p, nhead)
+        gs = ko.softmax_direct_on_axis_backward(ko.mix_values_backward_prop(gm, v, nhead), p, coef)
+        if masked:
+            gs = ko.set_mh_attention_mask(gs, False)
+        ref_gk = ko.mult_on_heads_backward(gs, q, nhead)     # the key gradient is formed with Q, by the output row
+        ref_gq = ko.mult_on_heads_backward(gs, k, nhead)
+        dp, dm = dev(p), dev(m)
+        for with_m in (True, False):
+            gq, gk, gv = (dev(np.full(q.shape, np.nan, np.float32)) for _ in range(3))
+            VMath.attention_backward(0, gq, gk, gv, dgm, dp, dm if with_m else None, dq, dk, dv, nbat, ntimes, nvec,
+                                     nhead, npiece, hcoef, masked)
+            what = " (%d x %d x %d heads of %d, masked %s, mixed output %s)" % (nbat, ntimes, nhead, npiece, masked, with_m)
+            check(gq.to_numpy(q.shape), ref_gq, what="query gradient" + what)
+            check(gk.to_numpy(q.shape), ref_gk, what="key gradient" + what)
+            check(gv.to_numpy(q.shape), ref_gv, what="value gradient" + what)
+
+
+def test_attention_backward_one_call_when_the_heads_do_not_fill_the_vector():
+    # nhead * npiece < nvec: the gradients of the mixed output are compact, those of the projections are not; the
+    # separate kernels take it (columns of the outputs beyond the heads are not written, as with the reference)
+    nbat, ntimes, nvec, nhead, npiece = 2, 70, 80, 2, 32
+    rng = np.random.default_rng(5)
+    q, k, v = (rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32) for _ in range(3))
+    gm = rng.standard_normal((nbat, ntimes, nhead * npiece)).astype(np.float32)
+    coef = 1.0 / np.sqrt(npiece)
+    used = slice(0, nhead * npiece)
+    qc, kc, vc = (np.ascontiguousarray(t[:, :, used]) for t in (q, k, v))
+    p = ko.softmax_direct_on_axis(ko.mult_on_heads(kc, qc, nhead, coef), nbat * ntimes, ntimes, nhead)
+    gs = ko.softmax_direct_on_axis_backward(ko.mix_values_backward_prop(gm, vc, nhead), p, coef)
+    gq, gk, gv = (dev(np.zeros(q.shape, np.float32)) for _ in range(3))
+    VMath.attention_backward(0, gq, gk, gv, dev(gm), dev(p), None, dev(q), dev(k), dev(v), nbat, ntimes, nvec, nhead,
+                             npiece, kai.hyper(coef), False)
+    check(gq.to_numpy(q.shape)[:, :, used], ko.mult_on_heads_backward(gs, kc, nhead), what="query gradient")
+    check(gk.to_numpy(q.shape)[:, :, used], ko.mult_on_heads_backward(gs, qc, nhead), what="key gradient")
+    check(gv.to_numpy(q.shape)[:, :, used], ko.mix_values_backward_value(gm, p, nhead), what="value gradient")
+    assert (gq.to_numpy(q.shape)[:, :, nhead * npiece:] == 0).all()
+
+
 # one case per kernel variant: rows in registers (1 head; 2..128 heads, short and long axis), rows through
 # LDS (long axis, odd lengths), one thread per head (more than 128 heads)
 SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8), (3, 20, 128), (2, 9, 129),
