@@ -268,6 +268,10 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
             lambda: L.kai_attention_forward(0, P(o), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
                                                    P(coef), 0),
             flops=2 * fl)
+        row(tag + "all three in one launch, probabilities stored (kai_attention_forward_train)",
+            lambda: L.kai_attention_forward_train(0, P(o), P(pbuf), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
+                                                  P(coef), 0),
+            flops=2 * fl)
         # the backward calls of the same block (vtensor.cpp:3142-3166 of the reference)
         go = torch.randn((nbat, T, nvec), device=dev, generator=g)
         gp = torch.empty_like(s0)

@@ -31,6 +31,20 @@ namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// Workgroup id -> (batch entry, head, row tile).  Hardware deals consecutive workgroup ids round-robin over the 8
+// XCDs, so ids congruent mod 8 share an L2.  They are renumbered so that each XCD gets a contiguous run of the
+// order (batch entry, row tile, head): the workgroups that read the same K, V and Q rows (all row tiles of a batch
+// entry and head) and, with several heads, the same lines of the head-interleaved probabilities (all heads of a
+// batch entry and row tile) then sit behind one L2 instead of fetching them into all eight.
+__device__ __forceinline__ void attention_block_of(int bid, int total, int ntiles, int nhead, int& b, int& h, int& tile) {
+    int id = bid;
+    if ((total & 7) == 0) id = (bid & 7) * (total >> 3) + (bid >> 3);
+    h = id % nhead;
+    const int r = id / nhead;
+    tile = r % ntiles;
+    b = r / ntiles;
+}
+
 constexpr int kAbQGroups = 4;          // waves along the rows t, 16 rows each
 constexpr int kAbKGroups = 2;          // waves along the keys of a tile
 constexpr int kAbWaves = kAbQGroups * kAbKGroups;
@@ -80,8 +94,9 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     const int g = lane >> 4;
     const int T = p.ntimes;
     const int H = p.nhead;
-    const int b = blockIdx.y / H, h = blockIdx.y % H;
-    const int t0 = blockIdx.x * kAbRows;
+    int b, h, ttile;
+    attention_block_of(blockIdx.x, gridDim.x, (T + kAbRows - 1) / kAbRows, H, b, h, ttile);
+    const int t0 = ttile * kAbRows;
     const int64_t base = (int64_t)b * p.batch_stride + (int64_t)h * p.npiece;
     const float coef = p.coef ? *p.coef : 0.f;
 
@@ -175,21 +190,43 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
                     pr[kb][v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_p, poff[4 * kb + v], kt * p_tile_bytes, 0));
         }
     };
-    // gP^T of this wave's keys: KB blocks of 16 keys x 16 rows, scaled by coef through gf
-    auto grad_p = [&](f32x4 (&gp)[KB], const float* lv) {
+    // gP^T of this wave's keys: KB blocks of 16 keys x 16 rows, scaled by coef through gf.  All fragments of V are
+    // requested before the first product (vf), and every block is summed in NCHAIN independent chains over the head
+    // dimension, so that no product waits for the one issued just before it.
+    constexpr int NCHAIN = (KB == 2 ? 2 : 4) < DB ? (KB == 2 ? 2 : 4) : DB;
+    // (head sizes from 96 on: the fragments of V are read chain group by chain group instead, for want of registers)
+    constexpr int NVF = DB <= 5 ? DB : NCHAIN;
+    auto read_v = [&](f32x4 (&vf)[NVF][KB], const float* lv, int s0) {
 #pragma unroll
-        for (int kb = 0; kb < KB; kb++) gp[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < DB; s++) {
-            f32x4 vf[KB];
+        for (int s = 0; s < NVF; s++)
 #pragma unroll
             for (int kb = 0; kb < KB; kb++)
-                vf[kb] = *reinterpret_cast<const f32x4*>(lv + (16 * kb + r16) * kStride + 16 * s + 4 * g);
+                vf[s][kb] = *reinterpret_cast<const f32x4*>(lv + (16 * kb + r16) * kStride + 16 * (s0 + s) + 4 * g);
+    };
+    auto grad_p = [&](f32x4 (&gp)[KB], f32x4 (&vf)[NVF][KB], const float* lv) {
+        f32x4 part[KB][NCHAIN];
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int c = 0; c < NCHAIN; c++) part[kb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s0 = 0; s0 < DB; s0 += NCHAIN) {
+            if (NVF < DB && s0 > 0) read_v(vf, lv, s0);
 #pragma unroll
             for (int e = 0; e < 4; e++)
 #pragma unroll
-                for (int kb = 0; kb < KB; kb++)
-                    gp[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[kb][e], gf[s][e], gp[kb], 0, 0, 0);
+                for (int c = 0; c < NCHAIN; c++)
+#pragma unroll
+                    for (int kb = 0; kb < KB; kb++)
+                        if (s0 + c < DB)
+                            part[kb][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[NVF < DB ? c : s0 + c][kb][e], gf[s0 + c][e],
+                                                                              part[kb][c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+            gp[kb] = part[kb][0];
+#pragma unroll
+            for (int c = 1; c < NCHAIN; c++) gp[kb] += part[kb][c];
         }
     };
 
@@ -221,8 +258,10 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
             load_p(pr, kt);
             const int key0 = kt * kKeys + 16 * KB * kgp;
             if (key0 < T) {
-                f32x4 gp[KB];
-                grad_p(gp, &lds[buf][0][16 * KB * kgp * kStride]);
+                f32x4 gp[KB], vf[NVF][KB];
+                const float* lv = &lds[buf][0][16 * KB * kgp * kStride];
+                read_v(vf, lv, 0);
+                grad_p(gp, vf, lv);
 #pragma unroll
                 for (int kb = 0; kb < KB; kb++)
 #pragma unroll
@@ -279,8 +318,33 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
             const float* lv = &lds[buf][0][16 * KB * kgp * kStride];
             const float* lk = &lds[buf][1][16 * KB * kgp * kStride];
             const float* lq = &lds[buf][2][16 * KB * kgp * kStride];
+            // Every LDS read of the tile is requested ahead of the products that hide its latency: the fragments of V
+            // and the first block's columns of K and Q before the gP products, the second block's columns before
+            // the first block's products.  (Left to itself the compiler reads each column just before its product
+            // and the matrix cores wait for LDS again and again.)
+            // kq[kb][e][0][db] = K[key 16*kb + 4*g + e, d 16*db + r16], kq[kb][e][1][db] the same of Q: 32-bit reads
+            // down a column of the tile (consecutive lanes, consecutive d)
+            f32x4 vf[NVF][KB];
+            float kq[KB][4][2][DB];
+            auto read_kq = [&](int kb) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int row = (16 * kb + 4 * g + e) * kStride + r16;
+#pragma unroll
+                    for (int db = 0; db < DB; db++) {
+                        kq[kb][e][0][db] = lk[row + 16 * db];
+                        kq[kb][e][1][db] = lq[row + 16 * db];
+                    }
+                }
+            };
+            read_v(vf, lv, 0);
+            read_kq(0);
+            __builtin_amdgcn_sched_barrier(0);
             f32x4 gs[KB];
-            grad_p(gs, lv);
+            grad_p(gs, vf, lv);
+            __builtin_amdgcn_sched_barrier(0);
+            if (KB > 1) read_kq(KB - 1);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kb = 0; kb < KB; kb++) gs[kb] = pr[kb] * (gs[kb] - delta);
             // keys past the end or above the diagonal of some row of this wave (wave-uniform test)
@@ -296,18 +360,15 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
                 __builtin_amdgcn_sched_barrier(0);
             }
             // gQ^T[d, t] += sum_key K[key, d] * gS[t, key];  gK^T[d, t] += sum_key Q[key, d] * gS[t, key]
-            // (32-bit reads down a column of the tile: consecutive lanes, consecutive d)
 #pragma unroll
             for (int kb = 0; kb < KB; kb++)
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int row = (16 * kb + 4 * g + e) * kStride + r16;
+                for (int e = 0; e < 4; e++)
 #pragma unroll
                     for (int db = 0; db < DB; db++) {
-                        acc_q[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(lk[row + 16 * db], gs[kb][e], acc_q[db], 0, 0, 0);
-                        acc_k[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(lq[row + 16 * db], gs[kb][e], acc_k[db], 0, 0, 0);
+                        acc_q[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[kb][e][0][db], gs[kb][e], acc_q[db], 0, 0, 0);
+                        acc_k[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[kb][e][1][db], gs[kb][e], acc_k[db], 0, 0, 0);
                     }
-                }
         }
         if (kt + 1 < nkt) {
             store_v(buf ^ 1);
@@ -378,8 +439,8 @@ int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const 
     p.ntimes = (int)ntimes; p.nhead = (int)nhead; p.npiece = (int)npiece;
     p.masked = masked;
     const int64_t ttiles = (ntimes + kAbRows - 1) / kAbRows;
-    if (ttiles > kMaxDim || nbat * nhead > 65535) return fail(KAI_ERR_INVALID_ARGUMENT, "attention backward: grid too large");
-    const dim3 grid((unsigned)ttiles, (unsigned)(nbat * nhead));
+    if (ttiles * nbat * nhead > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention backward: grid too large");
+    const dim3 grid((unsigned)(ttiles * nbat * nhead));
     const bool pvec = nhead == 1 && ntimes % 4 == 0 && aligned16(pp);
     switch (npiece / 16) {
     case 1: launch_rows<1, 2>(p, pvec, grid, stream); break;
@@ -387,7 +448,7 @@ int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const 
     case 3: launch_rows<3, 2>(p, pvec, grid, stream); break;
     case 4: launch_rows<4, 2>(p, pvec, grid, stream); break;
     case 5: launch_rows<5, 2>(p, pvec, grid, stream); break;
-    case 6: launch_rows<6, 2>(p, pvec, grid, stream); break;
+    case 6: launch_rows<6, 1>(p, pvec, grid, stream); break;
     case 7: launch_rows<7, 1>(p, pvec, grid, stream); break;
     default: launch_rows<8, 1>(p, pvec, grid, stream); break;
     }

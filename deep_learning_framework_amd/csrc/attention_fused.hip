@@ -15,6 +15,8 @@
 // operands.  K and V tiles lie in LDS as in memory.
 #include <float.h>
 
+#include <type_traits>
+
 #include "elementwise.h"
 
 namespace kai {
@@ -22,6 +24,29 @@ namespace kai {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// loop with compile-time indices (register arrays must never be indexed by a run-time value)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
+// Workgroup id -> (batch entry, head, row tile).  Hardware deals consecutive workgroup ids round-robin over the 8
+// XCDs, so ids congruent mod 8 share an L2.  They are renumbered so that each XCD gets a contiguous run of the
+// order (batch entry, row tile, head): the workgroups that read the same K and V rows (all row tiles of a batch
+// entry and head) and, with several heads, the same lines of the head-interleaved probabilities (all heads of a
+// batch entry and row tile) then sit behind one L2 instead of fetching them into all eight.
+__device__ __forceinline__ void attention_block_of(int bid, int total, int ntiles, int nhead, int& b, int& h, int& tile) {
+    int id = bid;
+    if ((total & 7) == 0) id = (bid & 7) * (total >> 3) + (bid >> 3);
+    h = id % nhead;
+    const int r = id / nhead;
+    tile = r % ntiles;
+    b = r / ntiles;
+}
 
 constexpr int kFaQGroups = 4;          // waves along the queries, 16 rows each
 constexpr int kFaKGroups = 2;          // waves along the keys: each takes 32 of a tile's 64 keys
@@ -66,8 +91,9 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
     const int r16 = lane & 15;
     const int g = lane >> 4;
     const int T = p.ntimes;
-    const int b = blockIdx.y / p.nhead, h = blockIdx.y % p.nhead;
-    const int q0 = blockIdx.x * kFaQ;
+    int b, h, qtile;
+    attention_block_of(blockIdx.x, gridDim.x, (T + kFaQ - 1) / kFaQ, p.nhead, b, h, qtile);
+    const int q0 = qtile * kFaQ;
     const int64_t base = (int64_t)b * p.batch_stride + (int64_t)h * p.npiece;
     const float* __restrict__ Qb = p.Q + base;
     const float* __restrict__ Kb = p.K + base;
@@ -252,6 +278,247 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
     }
 }
 
+
+// ---- the same block for TRAINING: the probabilities are also stored, as the backward pass needs them -------------
+//
+// With the probabilities to be written normalised, the running renormalisation of the kernel above does not apply:
+// a query's maximum and sum must be known before its first probability is stored.  Here a wave keeps ALL of its
+// scores in registers (8 per tile of 64 keys: lengths up to 64 * NT) -- first every key tile of K passes through
+// LDS and leaves its scores, then maximum, exponentials and sum are formed in registers (the two key halves exchange
+// theirs through LDS), then every tile of V passes through the same LDS buffers while the finished probabilities
+// are stored and multiplied into the output.  Each product is computed once; P is written once and never read.
+struct ProbsParams {
+    FusedParams f;
+    float* P;                 // [nbat, ntimes, ntimes, nhead]
+    int64_t p_batch_stride;   // ntimes * ntimes * nhead
+};
+
+template <int DB, int NT, bool PVEC>
+__global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const ProbsParams pp) {
+    const FusedParams& p = pp.f;
+    constexpr int D = 16 * DB;
+    constexpr int kStride = D + 4;
+    constexpr int kChunksPerKey = D / 4;
+    constexpr int kTileChunks = kFaKeys * kChunksPerKey;
+    constexpr int NCH = (kTileChunks + kFaThreads - 1) / kFaThreads;
+    constexpr bool kPartial = kTileChunks % kFaThreads != 0;
+    __shared__ __attribute__((aligned(16))) float lds_t[2][kFaKeys * kStride];   // K tiles, then V tiles
+    __shared__ float lds_x[2][64 * kFaQGroups];                                   // exchange of maxima and sums
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int qg = wave % kFaQGroups;
+    const int kgp = wave / kFaQGroups;
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+    const int T = p.ntimes;
+    const int H = p.nhead;
+    int b, h, qtile;
+    attention_block_of(blockIdx.x, gridDim.x, (T + kFaQ - 1) / kFaQ, H, b, h, qtile);
+    const int q0 = qtile * kFaQ;
+    const int64_t base = (int64_t)b * p.batch_stride + (int64_t)h * p.npiece;
+    const float* __restrict__ Qb = p.Q + base;
+    const float coef = p.coef ? *p.coef : 0.f;
+    const float c2 = coef * 1.44269504088896340736f;
+
+    const int q = q0 + 16 * qg + r16;
+    const int qc = min(q, T - 1);
+    f32x4 qf[DB];
+#pragma unroll
+    for (int s = 0; s < DB; s++) qf[s] = c2 * *reinterpret_cast<const f32x4*>(Qb + (int64_t)qc * p.nvec + 16 * s + 4 * g);
+
+    const int nkt_all = (T + kFaKeys - 1) / kFaKeys;
+    const int q_last = min(q0 + kFaQ, T) - 1;
+    // key tiles that hold an unmasked key for some query of this workgroup; the others hold zeros only
+    const int nkt = p.masked ? min(q_last / kFaKeys + 1, nkt_all) : nkt_all;
+
+    auto uniform_ptr = [](const float* ptr) -> float* {
+        const uint64_t a = reinterpret_cast<uint64_t>(ptr);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
+    };
+    const int extent = (int)(((int64_t)(T - 1) * p.nvec + D) * 4);
+    const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.K + base), 0, extent, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.V + base), 0, extent, 0x00020000);
+    const int tile_bytes = kFaKeys * (int)p.nvec * 4;
+    int choff[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+        const int c = tid + i * kFaThreads;
+        choff[i] = ((c / kChunksPerKey) * (int)p.nvec + (c % kChunksPerKey) * 4) * 4;
+    }
+    f32x4 rt[NCH];
+    auto load_tile = [&](const __amdgpu_buffer_rsrc_t& rsrc, int kt) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * kFaThreads;
+            if (!kPartial || c < kTileChunks)
+                rt[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, choff[i], kt * tile_bytes, 0));
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int c = tid + i * kFaThreads;
+            if (!kPartial || c < kTileChunks)
+                *reinterpret_cast<f32x4*>(&lds_t[buf][(c / kChunksPerKey) * kStride + (c % kChunksPerKey) * 4]) = rt[i];
+        }
+    };
+
+    // ---- scores of every key tile into registers: sc[kt][kb][v] = (query q, key 64*kt + 32*kgp + 16*kb + 4*g + v) -----
+    f32x4 sc[NT][2];
+    load_tile(rsrc_k, 0);
+    store_tile(0);
+    __syncthreads();
+    static_for<0, NT>([&](auto ktc) {
+        constexpr int kt = decltype(ktc)::value;
+        if (kt < nkt) {
+            constexpr int buf = kt & 1;
+            if (kt + 1 < nkt) load_tile(rsrc_k, kt + 1);
+            const int key0 = kt * kFaKeys + 32 * kgp;
+            const float* lk = lds_t[buf] + 32 * kgp * kStride;
+            sc[kt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+            sc[kt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < DB; s++) {
+                f32x4 kf[2];
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+                    kf[kb] = *reinterpret_cast<const f32x4*>(lk + (16 * kb + r16) * kStride + 16 * s + 4 * g);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+#pragma unroll
+                    for (int kb = 0; kb < 2; kb++)
+                        sc[kt][kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[kb][e], qf[s][e], sc[kt][kb], 0, 0, 0);
+            }
+            const bool edge_tile = key0 + 32 > T || (p.masked && key0 + 31 > q0 + 16 * qg);   // wave-uniform
+            if (edge_tile) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const int key = key0 + 16 * kb + 4 * g + v;
+                        if (key >= T || (p.masked && key > q)) sc[kt][kb][v] = -INFINITY;
+                    }
+            }
+            if (kt + 1 < nkt) store_tile(buf ^ 1);
+            __syncthreads();
+        } else {
+            sc[kt][0] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            sc[kt][1] = sc[kt][0];
+        }
+    });
+    // the first tile of V is on its way while the softmax runs
+    load_tile(rsrc_v, 0);
+
+    // ---- maximum, exponentials, sum: in registers; the two key halves exchange through LDS ---------------------------
+    float m = -INFINITY;
+    static_for<0, NT>([&](auto ktc) {
+        constexpr int kt = decltype(ktc)::value;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+            m = fmaxf(m, fmaxf(fmaxf(sc[kt][kb][0], sc[kt][kb][1]), fmaxf(sc[kt][kb][2], sc[kt][kb][3])));
+    });
+    m = fmaxf(m, __shfl_xor(m, 16));
+    m = fmaxf(m, __shfl_xor(m, 32));
+    lds_x[kgp][qg * 64 + lane] = m;
+    __syncthreads();
+    m = fmaxf(m, lds_x[kgp ^ 1][qg * 64 + lane]);   // key 0 is never masked: the maximum is finite
+    float l = 0.f;
+    static_for<0, NT>([&](auto ktc) {
+        constexpr int kt = decltype(ktc)::value;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                sc[kt][kb][v] = __builtin_amdgcn_exp2f(sc[kt][kb][v] - m);
+                l += sc[kt][kb][v];
+            }
+    });
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    __syncthreads();                                  // every wave has read the maxima
+    lds_x[kgp][qg * 64 + lane] = l;
+    store_tile(0);                                    // V tile 0 (the K tiles are done with)
+    __syncthreads();
+    l += lds_x[kgp ^ 1][qg * 64 + lane];
+    const float rl = 1.0f / l;
+
+    // ---- probabilities stored, and multiplied into the output tile by tile -------------------------------------------
+    f32x4 acc_o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++) acc_o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float* Pq = pp.P + (int64_t)b * pp.p_batch_stride + ((int64_t)qc * T) * H + h;   // P[b, q, 0, h]
+    static_for<0, NT>([&](auto ktc) {
+        constexpr int kt = decltype(ktc)::value;
+        if (kt < nkt_all) {
+            constexpr int buf = kt & 1;
+            const int key0 = kt * kFaKeys + 32 * kgp;
+            f32x4 pr[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) pr[kb] = sc[kt][kb] * rl;
+            if (kt < nkt) {
+                if (kt + 1 < nkt) load_tile(rsrc_v, kt + 1);
+                if (key0 < T && !(p.masked && key0 > q_last)) {
+                    const float* lv = lds_t[buf] + 32 * kgp * kStride;
+#pragma unroll
+                    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float* vp = lv + (16 * kb + 4 * g + e) * kStride + r16;
+#pragma unroll
+                            for (int db = 0; db < DB; db++)
+                                acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(vp[16 * db], pr[kb][e], acc_o[db], 0, 0, 0);
+                        }
+                }
+            }
+            // the probabilities of this tile: masked keys hold exp(-inf) = 0 exactly, also in the tiles above the diagonal
+            if (q < T) {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+                    const int key = key0 + 16 * kb + 4 * g;
+                    if (PVEC) {
+                        if (key < T) *reinterpret_cast<f32x4*>(Pq + key) = pr[kb];
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; v++)
+                            if (key + v < T) Pq[(int64_t)(key + v) * H] = pr[kb][v];
+                    }
+                }
+            }
+            if (kt < nkt) {
+                if (kt + 1 < nkt) store_tile(buf ^ 1);
+                __syncthreads();
+            }
+        }
+    });
+
+    // merge the two key halves of the output
+    float* mg = &lds_t[0][0] + (qg * 64 + lane);
+    constexpr int kMergeStride = 64 * kFaQGroups;
+    static_assert(4 * DB * 64 * kFaQGroups <= 2 * kFaKeys * kStride, "merge buffer must fit the tiles");
+    if (kgp == 1) {
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) mg[(4 * db + v) * kMergeStride] = acc_o[db][v];
+    }
+    __syncthreads();
+    if (kgp == 1) return;
+    if (q < T) {
+        float* out = p.O + base + (int64_t)q * p.nvec;
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+            f32x4 o = acc_o[db];
+#pragma unroll
+            for (int v = 0; v < 4; v++) o[v] += mg[(4 * db + v) * kMergeStride];
+            *reinterpret_cast<f32x4*>(out + 16 * db + 4 * g) = o;
+        }
+    }
+}
+
 }  // namespace
 
 bool attention_fused_applies(const float* q, const float* k, const float* v, const float* o, int64_t ntimes,
@@ -273,12 +540,52 @@ int launch_attention_fused(float* o, const float* q, const float* k, const float
     p.ntimes = (int)ntimes; p.nhead = (int)nhead; p.npiece = (int)npiece;
     p.masked = masked;
     const int64_t qtiles = (ntimes + kFaQ - 1) / kFaQ;
-    if (qtiles > kMaxDim || nbat * nhead > 65535) return fail(KAI_ERR_INVALID_ARGUMENT, "attention: grid too large");
-    const dim3 grid((unsigned)qtiles, (unsigned)(nbat * nhead));
+    if (qtiles * nbat * nhead > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention: grid too large");
+    const dim3 grid((unsigned)(qtiles * nbat * nhead));
     if (npiece == 16) attention_fused_kernel<1><<<grid, dim3(kFaThreads), 0, stream>>>(p);
     else if (npiece == 32) attention_fused_kernel<2><<<grid, dim3(kFaThreads), 0, stream>>>(p);
     else attention_fused_kernel<4><<<grid, dim3(kFaThreads), 0, stream>>>(p);
     return check_launch("attention_fused_kernel");
+}
+
+bool attention_probs_applies(const float* q, const float* k, const float* v, const float* o, const float* pp,
+                             int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece) {
+    return attention_fused_applies(q, k, v, o, ntimes, nvec, nhead, npiece) && ntimes <= 1024 &&
+           (reinterpret_cast<uintptr_t>(pp) & 3u) == 0;
+}
+
+template <int DB>
+static void launch_probs(const ProbsParams& p, bool pvec, int64_t ntimes, dim3 grid, hipStream_t stream) {
+    const dim3 block(kFaThreads);
+    if (ntimes <= 256) {
+        if (pvec) attention_probs_kernel<DB, 4, true><<<grid, block, 0, stream>>>(p);
+        else attention_probs_kernel<DB, 4, false><<<grid, block, 0, stream>>>(p);
+    } else if (ntimes <= 512) {
+        if (pvec) attention_probs_kernel<DB, 8, true><<<grid, block, 0, stream>>>(p);
+        else attention_probs_kernel<DB, 8, false><<<grid, block, 0, stream>>>(p);
+    } else {
+        if (pvec) attention_probs_kernel<DB, 16, true><<<grid, block, 0, stream>>>(p);
+        else attention_probs_kernel<DB, 16, false><<<grid, block, 0, stream>>>(p);
+    }
+}
+
+int launch_attention_probs(float* o, float* pp, const float* q, const float* k, const float* v, int64_t nbat,
+                           int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
+                           hipStream_t stream) {
+    ProbsParams p{};
+    p.f.Q = q; p.f.K = k; p.f.V = v; p.f.O = o; p.f.coef = hcoef;
+    p.f.nvec = nvec; p.f.batch_stride = ntimes * nvec;
+    p.f.ntimes = (int)ntimes; p.f.nhead = (int)nhead; p.f.npiece = (int)npiece;
+    p.f.masked = masked;
+    p.P = pp; p.p_batch_stride = ntimes * ntimes * nhead;
+    const int64_t qtiles = (ntimes + kFaQ - 1) / kFaQ;
+    if (qtiles * nbat * nhead > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention: grid too large");
+    const dim3 grid((unsigned)(qtiles * nbat * nhead));
+    const bool pvec = nhead == 1 && ntimes % 4 == 0 && aligned16(pp);
+    if (npiece == 16) launch_probs<1>(p, pvec, ntimes, grid, stream);
+    else if (npiece == 32) launch_probs<2>(p, pvec, ntimes, grid, stream);
+    else launch_probs<4>(p, pvec, ntimes, grid, stream);
+    return check_launch("attention_probs_kernel");
 }
 
 }  // namespace kai

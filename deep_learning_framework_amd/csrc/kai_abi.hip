@@ -838,6 +838,23 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
     return kai_mix_values(device, py, pp, pV, nbat, ntimes, nvec, nhead, npiece);
 }
 
+int kai_attention_forward_train(int device, float* py, float* pp, const float* pQ, const float* pK, const float* pV,
+                                int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece,
+                                const float* hCoef, int masked) {
+    KAI_REQUIRE_DEVICE(device);
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    if (nbat == 0 || ntimes == 0 || nhead == 0) return KAI_OK;
+    KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pp); KAI_REQUIRE_PTR(pQ); KAI_REQUIRE_PTR(pK); KAI_REQUIRE_PTR(pV);
+    if (npiece > 0 && attention_probs_applies(pQ, pK, pV, py, pp, ntimes, nvec, nhead, npiece))
+        return launch_attention_probs(py, pp, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked != 0,
+                                      current_stream());
+    // any other shape: the reference's calls one by one
+    KAI_TRY(kai_mult_on_heads(device, pp, pK, pQ, nbat, ntimes, nvec, nhead, npiece, hCoef));
+    if (masked) KAI_TRY(kai_set_mh_attention_mask(device, pp, nbat, ntimes, nhead, 1));
+    KAI_TRY(kai_softmax_direct_on_axis(device, pp, nbat * ntimes, ntimes, nhead));
+    return kai_mix_values(device, py, pp, pV, nbat, ntimes, nvec, nhead, npiece);
+}
+
 int kai_attention_backward(int device, float* pgQ, float* pgK, float* pgV, const float* pgm, const float* pp,
                            const float* pm, const float* pQ, const float* pK, const float* pV, int64_t nbat,
                            int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,

@@ -66,6 +66,7 @@ SIGNATURES = {
     "kai_gemm_plan": [_INT, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _INT, _INT, _INT, ctypes.c_char_p, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
     "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
+    "kai_attention_forward_train": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
     "kai_attention_backward": [_INT, _F, _F, _F, _F, _F, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
     "kai_cosinesim": [_INT, _F, _F, _F, _I64, _I64, _I64],
     "kai_copy": [_INT, _F, _F, _I64],
@@ -421,6 +422,11 @@ class VMath:
     def attention_forward(device, py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked):
         _ck(load().kai_attention_forward(device, _addr(py), _addr(pQ), _addr(pK), _addr(pV), nbat, ntimes, nvec,
                                          nhead, npiece, _addr(hCoef), int(bool(masked))))
+
+    @staticmethod
+    def attention_forward_train(device, py, pp, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked):
+        _ck(load().kai_attention_forward_train(device, _addr(py), _addr(pp), _addr(pQ), _addr(pK), _addr(pV), nbat,
+                                               ntimes, nvec, nhead, npiece, _addr(hCoef), int(bool(masked))))
 
     @staticmethod
     def attention_backward(device, pgQ, pgK, pgV, pgm, pp, pm, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef,

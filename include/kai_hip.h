@@ -330,6 +330,15 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
                           int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
                           int masked);
 
+/* The same block for training: pp[nbat, ntimes, ntimes, nhead] also receives the probabilities, as the separate
+ * calls leave them (masked keys exactly 0), for the backward pass (VTensor::mh_attention keeps them,
+ * vtensor.cpp:3005, 3048).  One launch for head sizes 16, 32 and 64 with nhead * npiece == nvec, 16-byte aligned
+ * operands and ntimes <= 1024 (a wave keeps the scores of its queries in registers between the maximum and the
+ * stores); any other shape runs the four separate kernels.  Equal to the separate calls up to rounding. */
+int kai_attention_forward_train(int device, float* py, float* pp, const float* pQ, const float* pK, const float* pV,
+                                int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece,
+                                const float* hCoef, int masked);
+
 /* The backward middle of the same block in two launches: the calls of VTensor::multihead_attention_backprop between
  * the output projection and the input projections (vtensor.cpp:3145-3154),
  *   mix_values_backward_prop, mix_values_backward_value, softmax_direct_on_axis_backward,

@@ -826,6 +826,39 @@ def test_attention_forward_fused(nbat, ntimes, nhead, npiece, masked):
     check(o.to_numpy((nbat, ntimes, nvec)), ref, what="fused attention")
 
 
+# the training form of the block in one call (kai_attention_forward_train): mixed output AND probabilities against
+# the oracle's four steps; both cfg4 mappings, the three register depths (lengths up to 256 / 512 / 1024), ragged
+# lengths, masked and not (masked keys must be exactly 0), and shapes that fall back to the separate kernels
+@pytest.mark.parametrize("nbat,ntimes,nhead,npiece", [(32, 512, 1, 64), (4, 512, 8, 64), (2, 130, 4, 32), (3, 77, 2, 16),
+                                                      (1, 1000, 2, 64), (2, 64, 3, 64), (2, 100, 2, 24), (1, 50, 3, 7),
+                                                      (1, 1, 1, 16), (2, 300, 1, 32), (1, 1024, 1, 16), (1, 1030, 2, 32),
+                                                      (2, 257, 1, 64), (1, 640, 4, 64), (3, 33, 5, 16)])
+def test_attention_forward_train(nbat, ntimes, nhead, npiece):
+    nvec = nhead * npiece
+    rng = np.random.default_rng(nbat * 1000 + ntimes * 10 + nhead + npiece)
+    q, k, v = (rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32) for _ in range(3))
+    coef = 1.0 / np.sqrt(npiece)
+    dq, dk, dv = dev(q), dev(k), dev(v)
+    pshape = (nbat, ntimes, ntimes, nhead)
+    for masked in (False, True):
+        s = ko.mult_on_heads(k, q, nhead, coef)
+        if masked:
+            s = ko.set_mh_attention_mask(s, True)
+        pr = ko.softmax_direct_on_axis(s, nbat * ntimes, ntimes, nhead).reshape(pshape)
+        ref = ko.mix_values(pr, v, nhead)
+        o = dev(np.full((nbat, ntimes, nvec), np.nan, np.float32))
+        pp = dev(np.full(pshape, np.nan, np.float32))
+        VMath.attention_forward_train(0, o, pp, dq, dk, dv, nbat, ntimes, nvec, nhead, npiece, kai.hyper(coef), masked)
+        what = " (%d x %d x %d heads of %d, masked %s)" % (nbat, ntimes, nhead, npiece, masked)
+        got_p = pp.to_numpy(pshape)
+        check(got_p, pr, what="probabilities" + what)
+        check(o.to_numpy((nbat, ntimes, nvec)), ref, what="mixed output" + what)
+        np.testing.assert_allclose(got_p.sum(axis=2), 1.0, rtol=0, atol=2e-6)
+        if masked:
+            upper = np.triu(np.ones((ntimes, ntimes), bool), 1)
+            assert (got_p[:, upper] == 0).all()       # keys after the query: exactly 0
+
+
 def test_attention_forward_when_the_heads_do_not_fill_the_vector():
     # nhead * npiece < nvec: the engine never does this, the interface allows it.  The output is the compact
     # [nbat, ntimes, nhead, npiece] of mix_values whatever the head size (the one-launch kernel steps aside).
