@@ -23,6 +23,8 @@
 // meet in LDS at the end, in a fixed order.
 #include <float.h>
 
+#include <type_traits>
+
 #include "elementwise.h"
 
 namespace kai {
@@ -30,6 +32,15 @@ namespace kai {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// loop with compile-time indices (register arrays must never be indexed by a run-time value)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
 
 // Workgroup id -> (batch entry, head, row tile).  Hardware deals consecutive workgroup ids round-robin over the 8
 // XCDs, so ids congruent mod 8 share an L2.  They are renumbered so that each XCD gets a contiguous run of the
@@ -289,12 +300,36 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     }
 
     // ---- gS tile by tile, multiplied into both outputs ----------------------------------------------------------
+    //
+    // The products of a tile are dealt with in NG groups of 2 * KB * 4 (gP, one 16-wide slice s of the head dimension)
+    // or 2 * DB (gQ and gK, one key column e of one block kb) matrix instructions.  The schedule is written out,
+    // with fences between the groups so that the compiler keeps it:
+    //   * the LDS reads of group i + 1 are issued BEFORE the products of group i (operands double buffered), so no
+    //     product waits for LDS, and the eight waves do not all hit LDS in one burst at the start of a tile;
+    //   * the global loads of the next tile are dealt out one per group over the first groups (issued together
+    //     they fill the address unit's queue and every wave waits at its next load), its LDS stores two per group
+    //     over the last groups;
+    //   * the barrier sits before the LAST group, whose operands are in registers by then and whose products cover
+    //     the first reads of the next tile.
+    // Measured on the first version of this loop (all reads, then all products; cfg4, one head, 36.8 us): without the
+    // LDS reads and the tile traffic it took 26.1 us, the time of its matrix instructions plus launch and first
+    // loads; the reads added 5.5 us and the tile traffic 5.2 us on top instead of running under them.
     f32x4 acc_q[DB], acc_k[DB];
 #pragma unroll
     for (int db = 0; db < DB; db++) {
         acc_q[db] = f32x4{0.f, 0.f, 0.f, 0.f};
         acc_k[db] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    constexpr int NA = DB;            // groups of gP products: one per slice s
+    constexpr int NC = 4 * KB;        // groups of gQ / gK products: one per (kb, e)
+    constexpr int NG = NA + NC;
+    constexpr int NLOAD = 3 * NCH;    // global loads of a tile per thread (V, K, Q chunks), then the loads of P
+    constexpr int kLoadsPerGroup = (NLOAD + 1 + (NG - 3) - 1) / (NG - 3);     // all issued by group NG - 3
+    constexpr int kStoresPerGroup = 2;
+    constexpr int kStoreGroups = (NLOAD + kStoresPerGroup - 1) / kStoresPerGroup;
+    constexpr int kFirstStoreGroup = NG - 1 - kStoreGroups;                   // the last store is in group NG - 2
+    static_assert(kFirstStoreGroup >= 1, "too many chunks for this schedule");
+
     f32x4 p_next[KB];
     load_v(0);
     load_kq(0);
@@ -303,78 +338,126 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     store_kq(0);
     __syncthreads();
 
+    // operand registers of the groups, double buffered by group parity
+    f32x4 vf[2][KB];
+    float kf[2][DB], qf2[2][DB];
+    // the LDS reads of group i of the tile in buffer `buf`
+    auto stage = [&](auto ic, int buf) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int par = i & 1;
+        const float* lv = &lds[buf][0][16 * KB * kgp * kStride];
+        if constexpr (i < NA) {
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++)
+                vf[par][kb] = *reinterpret_cast<const f32x4*>(lv + (16 * kb + r16) * kStride + 16 * i + 4 * g);
+        } else {
+            constexpr int kb = (i - NA) / 4, e = (i - NA) % 4;
+            const float* lk = &lds[buf][1][16 * KB * kgp * kStride] + (16 * kb + 4 * g + e) * kStride + r16;
+            const float* lq = &lds[buf][2][16 * KB * kgp * kStride] + (16 * kb + 4 * g + e) * kStride + r16;
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                kf[par][db] = lk[16 * db];
+                qf2[par][db] = lq[16 * db];
+            }
+        }
+    };
+    // one chunk of the next tile's global loads / of its LDS stores, by number: V chunks, K chunks, Q chunks
+    auto load_one = [&](auto jc, int kt) {
+        constexpr int j = decltype(jc)::value;
+        constexpr int i = j % NCH;
+        const int c = tid + i * kAbThreads;
+        if (!kPartial || c < kTileChunks) {
+            if constexpr (j / NCH == 0) rv[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_v, choff[i], kt * tile_bytes, 0));
+            else if constexpr (j / NCH == 1) rk[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, choff[i], kt * tile_bytes, 0));
+            else rq[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_q, choff[i], kt * tile_bytes, 0));
+        }
+    };
+    auto store_one = [&](auto jc, int buf) {
+        constexpr int j = decltype(jc)::value;
+        constexpr int i = j % NCH;
+        const int c = tid + i * kAbThreads;
+        if (!kPartial || c < kTileChunks) {
+            float* dst = &lds[buf][j / NCH][(c / kChunksPerKey) * kStride + (c % kChunksPerKey) * 4];
+            *reinterpret_cast<f32x4*>(dst) = j / NCH == 0 ? rv[i] : j / NCH == 1 ? rk[i] : rq[i];
+        }
+    };
+
+    stage(std::integral_constant<int, 0>{}, 0);
     for (int kt = 0; kt < nkt; kt++) {
         const int buf = kt & 1;
-        const int nxt = min(kt + 1, nkt - 1);      // the surplus loads of the last tile are never used
+        const int nxt = min(kt + 1, nkt - 1);      // the surplus loads and stores of the last tile are never used
+        const int key0 = kt * kKeys + 16 * KB * kgp;    // first key of this wave's part of the tile
         f32x4 pr[KB];
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) pr[kb] = p_next[kb];
-        load_v(nxt);
-        load_kq(nxt);
-        load_p(p_next, nxt);
-        const int key0 = kt * kKeys + 16 * KB * kgp;    // first key of this wave's part of the tile
-        // a part past the end, or entirely above the diagonal of the workgroup's last row, adds nothing
-        if (key0 < T && !(p.masked && key0 > t_last)) {
-            const float* lv = &lds[buf][0][16 * KB * kgp * kStride];
-            const float* lk = &lds[buf][1][16 * KB * kgp * kStride];
-            const float* lq = &lds[buf][2][16 * KB * kgp * kStride];
-            // Every LDS read of the tile is requested ahead of the products that hide its latency: the fragments of V
-            // and the first block's columns of K and Q before the gP products, the second block's columns before
-            // the first block's products.  (Left to itself the compiler reads each column just before its product
-            // and the matrix cores wait for LDS again and again.)
-            // kq[kb][e][0][db] = K[key 16*kb + 4*g + e, d 16*db + r16], kq[kb][e][1][db] the same of Q: 32-bit reads
-            // down a column of the tile (consecutive lanes, consecutive d)
-            f32x4 vf[NVF][KB];
-            float kq[KB][4][2][DB];
-            auto read_kq = [&](int kb) {
+        f32x4 part[KB][NCHAIN];
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int row = (16 * kb + 4 * g + e) * kStride + r16;
+        for (int kb = 0; kb < KB; kb++)
 #pragma unroll
-                    for (int db = 0; db < DB; db++) {
-                        kq[kb][e][0][db] = lk[row + 16 * db];
-                        kq[kb][e][1][db] = lq[row + 16 * db];
-                    }
-                }
-            };
-            read_v(vf, lv, 0);
-            read_kq(0);
-            __builtin_amdgcn_sched_barrier(0);
-            f32x4 gs[KB];
-            grad_p(gs, vf, lv);
-            __builtin_amdgcn_sched_barrier(0);
-            if (KB > 1) read_kq(KB - 1);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kb = 0; kb < KB; kb++) gs[kb] = pr[kb] * (gs[kb] - delta);
-            // keys past the end or above the diagonal of some row of this wave (wave-uniform test)
-            const bool edge_tile = key0 + 16 * KB > T || (p.masked && key0 + 16 * KB - 1 > t0 + 16 * qg);
-            if (edge_tile) {
-#pragma unroll
-                for (int kb = 0; kb < KB; kb++)
-#pragma unroll
-                    for (int v = 0; v < 4; v++) {
-                        const int key = key0 + 16 * kb + 4 * g + v;
-                        if (key >= T || (p.masked && key > t)) gs[kb][v] = 0.f;
-                    }
-                __builtin_amdgcn_sched_barrier(0);
+            for (int c = 0; c < NCHAIN; c++) part[kb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 gs[KB];
+        static_for<0, NG>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            constexpr int par = i & 1;
+            // -- the next group's operands
+            if constexpr (i + 1 < NG) {
+                stage(std::integral_constant<int, i + 1>{}, buf);
+            } else {
+                __syncthreads();     // the next tile is in LDS, and every wave has read this one
+                if (kt + 1 < nkt) stage(std::integral_constant<int, 0>{}, buf ^ 1);
             }
-            // gQ^T[d, t] += sum_key K[key, d] * gS[t, key];  gK^T[d, t] += sum_key Q[key, d] * gS[t, key]
-#pragma unroll
-            for (int kb = 0; kb < KB; kb++)
+            // -- this group's share of the next tile's traffic
+            static_for<0, kLoadsPerGroup>([&](auto lc) {
+                constexpr int j = i * kLoadsPerGroup + decltype(lc)::value;
+                if constexpr (j < NLOAD) load_one(std::integral_constant<int, j>{}, nxt);
+                else if constexpr (j == NLOAD) load_p(p_next, nxt);
+            });
+            if constexpr (i >= kFirstStoreGroup && i < NG - 1) {
+                static_for<0, kStoresPerGroup>([&](auto sc) {
+                    constexpr int j = (i - kFirstStoreGroup) * kStoresPerGroup + decltype(sc)::value;
+                    if constexpr (j < NLOAD) store_one(std::integral_constant<int, j>{}, buf ^ 1);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // -- this group's products
+            if constexpr (i < NA) {
+                constexpr int c = i % NCHAIN;
 #pragma unroll
                 for (int e = 0; e < 4; e++)
 #pragma unroll
-                    for (int db = 0; db < DB; db++) {
-                        acc_q[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[kb][e][0][db], gs[kb][e], acc_q[db], 0, 0, 0);
-                        acc_k[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(kq[kb][e][1][db], gs[kb][e], acc_k[db], 0, 0, 0);
+                    for (int kb = 0; kb < KB; kb++)
+                        part[kb][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[par][kb][e], gf[i][e], part[kb][c], 0, 0, 0);
+                if constexpr (i == NA - 1) {
+                    // gS = P * (coef * gP - coef * row sum); keys past the end or above the diagonal give nothing
+#pragma unroll
+                    for (int kb = 0; kb < KB; kb++) {
+                        gs[kb] = part[kb][0];
+#pragma unroll
+                        for (int cc = 1; cc < NCHAIN; cc++) gs[kb] += part[kb][cc];
+                        gs[kb] = pr[kb] * (gs[kb] - delta);
                     }
-        }
-        if (kt + 1 < nkt) {
-            store_v(buf ^ 1);
-            store_kq(buf ^ 1);
-        }
-        __syncthreads();
+                    const bool edge_tile = key0 + 16 * KB > T || (p.masked && key0 + 16 * KB - 1 > t0 + 16 * qg);   // wave-uniform
+                    if (edge_tile) {
+#pragma unroll
+                        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+                            for (int v = 0; v < 4; v++) {
+                                const int key = key0 + 16 * kb + 4 * g + v;
+                                if (key >= T || (p.masked && key > t)) gs[kb][v] = 0.f;
+                            }
+                    }
+                }
+            } else {
+                // gQ^T[d, t] += K[key, d] * gS[t, key];  gK^T[d, t] += Q[key, d] * gS[t, key]  for key = 16*kb + 4*g + e
+                constexpr int kb = (i - NA) / 4, e = (i - NA) % 4;
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    acc_q[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[par][db], gs[kb][e], acc_q[db], 0, 0, 0);
+                    acc_k[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(qf2[par][db], gs[kb][e], acc_k[db], 0, 0, 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
     }
 
     // the second key half hands its sums over through LDS; the first adds them and stores

@@ -293,32 +293,48 @@ struct ProbsParams {
     int64_t p_batch_stride;   // ntimes * ntimes * nhead
 };
 
-template <int DB, int NT, bool PVEC>
+// HG = heads per workgroup.  1: the eight waves are 4 groups of 16 queries x 2 halves of every key tile, all of one
+// head; a lane stores the probabilities of 4 consecutive keys of its query (one 128-bit store with one head in
+// all, PVEC, else four 32-bit stores nhead floats apart).  4 (head counts that are multiples of 4): the waves are
+// 4 HEADS x 2 key halves of the same 16 queries, the K / V tiles hold the rows of the four heads side by side as
+// they lie in memory, and the probabilities of a tile meet in LDS so that a lane stores the four heads of one
+// (query, key) as one 128-bit word: written head by head, 4 bytes every 4 * nhead, the stores of the probabilities
+// alone took longer than everything else together (cfg4 with 8 heads: 58 us against 29 with one head).
+template <int DB, int NT, int HG, bool PVEC>
 __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const ProbsParams pp) {
     const FusedParams& p = pp.f;
     constexpr int D = 16 * DB;
-    constexpr int kStride = D + 4;
-    constexpr int kChunksPerKey = D / 4;
+    constexpr int kRows = HG == 1 ? kFaQ : 16;        // queries per workgroup
+    constexpr int kStride = HG * D + 4;               // tile [64 keys][HG heads x D]
+    constexpr int kChunksPerKey = HG * D / 4;
     constexpr int kTileChunks = kFaKeys * kChunksPerKey;
     constexpr int NCH = (kTileChunks + kFaThreads - 1) / kFaThreads;
     constexpr bool kPartial = kTileChunks % kFaThreads != 0;
+    constexpr int kPStride = kFaKeys + 4;             // exchange buffer [4 heads][16 queries][64 keys]: a plane per head
+    constexpr int kPPlane = 16 * kPStride;
     __shared__ __attribute__((aligned(16))) float lds_t[2][kFaKeys * kStride];   // K tiles, then V tiles
     __shared__ float lds_x[2][64 * kFaQGroups];                                   // exchange of maxima and sums
+    __shared__ __attribute__((aligned(16))) float lds_p[HG == 4 ? 4 * kPPlane : 4];
+    static_assert(HG == 1 || HG == 4, "one head or four heads per workgroup");
+    static_assert(!(HG == 4 && PVEC), "PVEC is the one-head store");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int qg = wave % kFaQGroups;
+    const int w4 = wave % kFaQGroups;
     const int kgp = wave / kFaQGroups;
+    const int qg = HG == 1 ? w4 : 0;      // which 16 queries of the workgroup
+    const int hd = HG == 1 ? 0 : w4;      // which head of the workgroup
     const int r16 = lane & 15;
     const int g = lane >> 4;
     const int T = p.ntimes;
     const int H = p.nhead;
-    int b, h, qtile;
-    attention_block_of(blockIdx.x, gridDim.x, (T + kFaQ - 1) / kFaQ, H, b, h, qtile);
-    const int q0 = qtile * kFaQ;
-    const int64_t base = (int64_t)b * p.batch_stride + (int64_t)h * p.npiece;
-    const float* __restrict__ Qb = p.Q + base;
+    int b, hgrp, qtile;
+    attention_block_of(blockIdx.x, gridDim.x, (T + kRows - 1) / kRows, H / HG, b, hgrp, qtile);
+    const int h0 = hgrp * HG;             // first head of the workgroup
+    const int q0 = qtile * kRows;
+    const int64_t base = (int64_t)b * p.batch_stride + (int64_t)h0 * p.npiece;   // the workgroup's heads, side by side
+    const float* __restrict__ Qb = p.Q + base + hd * D;
     const float coef = p.coef ? *p.coef : 0.f;
     const float c2 = coef * 1.44269504088896340736f;
 
@@ -329,7 +345,7 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
     for (int s = 0; s < DB; s++) qf[s] = c2 * *reinterpret_cast<const f32x4*>(Qb + (int64_t)qc * p.nvec + 16 * s + 4 * g);
 
     const int nkt_all = (T + kFaKeys - 1) / kFaKeys;
-    const int q_last = min(q0 + kFaQ, T) - 1;
+    const int q_last = min(q0 + kRows, T) - 1;
     // key tiles that hold an unmasked key for some query of this workgroup; the others hold zeros only
     const int nkt = p.masked ? min(q_last / kFaKeys + 1, nkt_all) : nkt_all;
 
@@ -339,7 +355,7 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
         return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
     };
-    const int extent = (int)(((int64_t)(T - 1) * p.nvec + D) * 4);
+    const int extent = (int)(((int64_t)(T - 1) * p.nvec + HG * D) * 4);
     const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.K + base), 0, extent, 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(p.V + base), 0, extent, 0x00020000);
     const int tile_bytes = kFaKeys * (int)p.nvec * 4;
@@ -376,9 +392,9 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
         constexpr int kt = decltype(ktc)::value;
         if (kt < nkt) {
             constexpr int buf = kt & 1;
-            if (kt + 1 < nkt) load_tile(rsrc_k, kt + 1);
+            load_tile(rsrc_k, min(kt + 1, nkt - 1));   // unconditional: a load behind a branch is waited for at once; the surplus one is never stored
             const int key0 = kt * kFaKeys + 32 * kgp;
-            const float* lk = lds_t[buf] + 32 * kgp * kStride;
+            const float* lk = lds_t[buf] + 32 * kgp * kStride + hd * D;
             sc[kt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
             sc[kt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -423,9 +439,9 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
     });
     m = fmaxf(m, __shfl_xor(m, 16));
     m = fmaxf(m, __shfl_xor(m, 32));
-    lds_x[kgp][qg * 64 + lane] = m;
+    lds_x[kgp][w4 * 64 + lane] = m;
     __syncthreads();
-    m = fmaxf(m, lds_x[kgp ^ 1][qg * 64 + lane]);   // key 0 is never masked: the maximum is finite
+    m = fmaxf(m, lds_x[kgp ^ 1][w4 * 64 + lane]);   // key 0 is never masked: the maximum is finite
     float l = 0.f;
     static_for<0, NT>([&](auto ktc) {
         constexpr int kt = decltype(ktc)::value;
@@ -440,17 +456,17 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
     __syncthreads();                                  // every wave has read the maxima
-    lds_x[kgp][qg * 64 + lane] = l;
+    lds_x[kgp][w4 * 64 + lane] = l;
     store_tile(0);                                    // V tile 0 (the K tiles are done with)
     __syncthreads();
-    l += lds_x[kgp ^ 1][qg * 64 + lane];
+    l += lds_x[kgp ^ 1][w4 * 64 + lane];
     const float rl = 1.0f / l;
 
     // ---- probabilities stored, and multiplied into the output tile by tile -------------------------------------------
     f32x4 acc_o[DB];
 #pragma unroll
     for (int db = 0; db < DB; db++) acc_o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
-    float* Pq = pp.P + (int64_t)b * pp.p_batch_stride + ((int64_t)qc * T) * H + h;   // P[b, q, 0, h]
+    float* Pq = pp.P + (int64_t)b * pp.p_batch_stride + ((int64_t)qc * T) * H + h0 + hd;   // P[b, q, 0, h]
     static_for<0, NT>([&](auto ktc) {
         constexpr int kt = decltype(ktc)::value;
         if (kt < nkt_all) {
@@ -459,10 +475,18 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
             f32x4 pr[2];
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) pr[kb] = sc[kt][kb] * rl;
+            if (HG == 4) {
+                // this wave's head of (query r16, keys 32*kgp + 16*kb + 4*g + 0..3) into its plane of the exchange
+                // buffer: one 128-bit write per key block (written as the fourth part of 4-float groups, the 64 lanes
+                // of a write would share 8 banks)
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+                    *reinterpret_cast<f32x4*>(&lds_p[hd * kPPlane + r16 * kPStride + 32 * kgp + 16 * kb + 4 * g]) = pr[kb];
+            }
             if (kt < nkt) {
-                if (kt + 1 < nkt) load_tile(rsrc_v, kt + 1);
+                load_tile(rsrc_v, min(kt + 1, nkt - 1));
                 if (key0 < T && !(p.masked && key0 > q_last)) {
-                    const float* lv = lds_t[buf] + 32 * kgp * kStride;
+                    const float* lv = lds_t[buf] + 32 * kgp * kStride + hd * D;
 #pragma unroll
                     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -475,7 +499,19 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
                 }
             }
             // the probabilities of this tile: masked keys hold exp(-inf) = 0 exactly, also in the tiles above the diagonal
-            if (q < T) {
+            if (HG == 4) {
+                __syncthreads();   // the four heads of every (query, key) of the tile are in the exchange buffer
+#pragma unroll
+                for (int i = 0; i < 16 * kFaKeys / kFaThreads; i++) {
+                    const int idx = tid + i * kFaThreads;
+                    const int qq = idx / kFaKeys, kk = idx % kFaKeys;
+                    const int key = kt * kFaKeys + kk;
+                    const float* src = &lds_p[qq * kPStride + kk];
+                    const f32x4 w = {src[0], src[kPPlane], src[2 * kPPlane], src[3 * kPPlane]};
+                    if (q0 + qq < T && key < T)
+                        *reinterpret_cast<f32x4*>(pp.P + (int64_t)b * pp.p_batch_stride + (((int64_t)(q0 + qq) * T + key) * H + h0)) = w;
+                }
+            } else if (q < T) {
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) {
                     const int key = key0 + 16 * kb + 4 * g;
@@ -491,12 +527,14 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
             if (kt < nkt) {
                 if (kt + 1 < nkt) store_tile(buf ^ 1);
                 __syncthreads();
+            } else if (HG == 4) {
+                __syncthreads();   // the exchange buffer is free again
             }
         }
     });
 
     // merge the two key halves of the output
-    float* mg = &lds_t[0][0] + (qg * 64 + lane);
+    float* mg = &lds_t[0][0] + (w4 * 64 + lane);
     constexpr int kMergeStride = 64 * kFaQGroups;
     static_assert(4 * DB * 64 * kFaQGroups <= 2 * kFaKeys * kStride, "merge buffer must fit the tiles");
     if (kgp == 1) {
@@ -508,7 +546,7 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
     __syncthreads();
     if (kgp == 1) return;
     if (q < T) {
-        float* out = p.O + base + (int64_t)q * p.nvec;
+        float* out = p.O + base + hd * D + (int64_t)q * p.nvec;
 #pragma unroll
         for (int db = 0; db < DB; db++) {
             f32x4 o = acc_o[db];
@@ -554,20 +592,24 @@ bool attention_probs_applies(const float* q, const float* k, const float* v, con
            (reinterpret_cast<uintptr_t>(pp) & 3u) == 0;
 }
 
-template <int DB>
+template <int DB, int HG>
 static void launch_probs(const ProbsParams& p, bool pvec, int64_t ntimes, dim3 grid, hipStream_t stream) {
     const dim3 block(kFaThreads);
+    constexpr bool kVecOk = HG == 1;
     if (ntimes <= 256) {
-        if (pvec) attention_probs_kernel<DB, 4, true><<<grid, block, 0, stream>>>(p);
-        else attention_probs_kernel<DB, 4, false><<<grid, block, 0, stream>>>(p);
+        if (kVecOk && pvec) attention_probs_kernel<DB, 4, HG, kVecOk><<<grid, block, 0, stream>>>(p);
+        else attention_probs_kernel<DB, 4, HG, false><<<grid, block, 0, stream>>>(p);
     } else if (ntimes <= 512) {
-        if (pvec) attention_probs_kernel<DB, 8, true><<<grid, block, 0, stream>>>(p);
-        else attention_probs_kernel<DB, 8, false><<<grid, block, 0, stream>>>(p);
+        if (kVecOk && pvec) attention_probs_kernel<DB, 8, HG, kVecOk><<<grid, block, 0, stream>>>(p);
+        else attention_probs_kernel<DB, 8, HG, false><<<grid, block, 0, stream>>>(p);
     } else {
-        if (pvec) attention_probs_kernel<DB, 16, true><<<grid, block, 0, stream>>>(p);
-        else attention_probs_kernel<DB, 16, false><<<grid, block, 0, stream>>>(p);
+        if (kVecOk && pvec) attention_probs_kernel<DB, 16, HG, kVecOk><<<grid, block, 0, stream>>>(p);
+        else attention_probs_kernel<DB, 16, HG, false><<<grid, block, 0, stream>>>(p);
     }
 }
+
+// four heads per workgroup: head counts in whole fours and rows of the probabilities that allow 128-bit stores
+static bool probs_four_heads(const float* pp, int64_t nhead) { return nhead % 4 == 0 && aligned16(pp); }
 
 int launch_attention_probs(float* o, float* pp, const float* q, const float* k, const float* v, int64_t nbat,
                            int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
@@ -578,13 +620,21 @@ int launch_attention_probs(float* o, float* pp, const float* q, const float* k, 
     p.f.ntimes = (int)ntimes; p.f.nhead = (int)nhead; p.f.npiece = (int)npiece;
     p.f.masked = masked;
     p.P = pp; p.p_batch_stride = ntimes * ntimes * nhead;
-    const int64_t qtiles = (ntimes + kFaQ - 1) / kFaQ;
-    if (qtiles * nbat * nhead > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention: grid too large");
-    const dim3 grid((unsigned)(qtiles * nbat * nhead));
+    const bool four = probs_four_heads(pp, nhead);
+    const int64_t qtiles = four ? (ntimes + 15) / 16 : (ntimes + kFaQ - 1) / kFaQ;
+    const int64_t wgs = qtiles * nbat * (four ? nhead / 4 : nhead);
+    if (wgs > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention: grid too large");
+    const dim3 grid((unsigned)wgs);
     const bool pvec = nhead == 1 && ntimes % 4 == 0 && aligned16(pp);
-    if (npiece == 16) launch_probs<1>(p, pvec, ntimes, grid, stream);
-    else if (npiece == 32) launch_probs<2>(p, pvec, ntimes, grid, stream);
-    else launch_probs<4>(p, pvec, ntimes, grid, stream);
+    if (four) {
+        if (npiece == 16) launch_probs<1, 4>(p, false, ntimes, grid, stream);
+        else if (npiece == 32) launch_probs<2, 4>(p, false, ntimes, grid, stream);
+        else launch_probs<4, 4>(p, false, ntimes, grid, stream);
+    } else {
+        if (npiece == 16) launch_probs<1, 1>(p, pvec, ntimes, grid, stream);
+        else if (npiece == 32) launch_probs<2, 1>(p, pvec, ntimes, grid, stream);
+        else launch_probs<4, 1>(p, pvec, ntimes, grid, stream);
+    }
     return check_launch("attention_probs_kernel");
 }
 
