@@ -314,6 +314,34 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
             lambda: L.kai_attention_backward(0, P(gq), P(gk), P(gv), P(go), P(pbuf), None, P(q), P(k), P(v), I(nbat), I(T),
                                              I(nvec), I(nhead), I(D), P(coef), 0),
             flops=5 * fl)
+    # a BERT-base sized block: 2 x 384 tokens, 12 heads of 64 (the head count is no power of two)
+    nbat, T, nhead, D = 2, 384, 12, 64
+    nvec = nhead * D
+    q, k, v, go = (torch.randn((nbat, T, nvec), device=dev, generator=g) for _ in range(4))
+    pbuf = torch.empty((nbat, T, T, nhead), device=dev)
+    o, gq, gk, gv = (torch.empty_like(q) for _ in range(4))
+    coef = torch.tensor([0.125], device=dev)
+    fl = 2.0 * nbat * nhead * T * T * D
+    tag = "attention 2 x 384 x 12 heads of 64: "
+
+    def three_calls_12():
+        L.kai_mult_on_heads(0, P(pbuf), P(k), P(q), I(nbat), I(T), I(nvec), I(nhead), I(D), P(coef))
+        L.kai_softmax_direct_on_axis(0, P(pbuf), I(nbat * T), I(T), I(nhead))
+        L.kai_mix_values(0, P(o), P(pbuf), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D))
+
+    row(tag + "the three forward calls back to back", three_calls_12, flops=2 * fl)
+    row(tag + "forward only, one launch (kai_attention_forward, %s)" % kai.VMath.attention_plan("forward", nbat, T, nvec, nhead, D),
+        lambda: L.kai_attention_forward(0, P(o), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D), P(coef), 0),
+        flops=2 * fl)
+    row(tag + "forward with the probabilities stored (kai_attention_forward_train, %s)" % kai.VMath.attention_plan("forward_train", nbat, T, nvec, nhead, D),
+        lambda: L.kai_attention_forward_train(0, P(o), P(pbuf), P(q), P(k), P(v), I(nbat), I(T), I(nvec), I(nhead), I(D),
+                                              P(coef), 0),
+        flops=2 * fl)
+    row(tag + "backward (kai_attention_backward, %s)" % kai.VMath.attention_plan("backward", nbat, T, nvec, nhead, D),
+        lambda: L.kai_attention_backward(0, P(gq), P(gk), P(gv), P(go), P(pbuf), P(o), P(q), P(k), P(v), I(nbat), I(T),
+                                         I(nvec), I(nhead), I(D), P(coef), 0),
+        flops=4 * fl)
+    del q, k, v, go, pbuf, o, gq, gk, gv
     # cfg5: skinny (cold: six rotating weight buffers) and ragged
     K = N = 4096
     ws = [torch.rand((N, K), device=dev, generator=g) * 0.1 - 0.05 for _ in range(6)]
@@ -406,6 +434,100 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
     return rows
 
 
+def plan_audit(torch, kai, stream, dev, out_path):
+    """Times the dispatcher's choice against every alternative it could have made (forced through
+    kai_gemm_force_plan) on shapes that sit on both sides of the thresholds coded in csrc/gemm_dispatch.hip, in the
+    three operand forms of the dense layer, and writes a table: chosen plan, its time, the fastest alternative, the
+    ratio.  A ratio above 1.08 marks a shape where the fitted rules have gone stale."""
+    import ctypes
+    L = kai.load()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    I = ctypes.c_int64
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    shapes = []
+    for nk in ((4096, 4096), (3584, 4096), (5120, 4096), (6656, 4096), (11008, 4096)):
+        for m in (128, 129, 160, 161, 192, 193, 224, 225):
+            shapes.append((m,) + nk)
+    for nk in ((2048, 2047), (2048, 2048), (4096, 2048)):
+        for m in (64, 144, 256):
+            shapes.append((m,) + nk)
+    shapes += [(64, 512, 784), (256, 1024, 1024), (1000, 333, 777), (512, 2048, 2048), (1024, 1024, 1024),
+               (32, 4096, 4096), (33, 4096, 4096), (96, 4096, 11008), (200, 6656, 4096), (144, 5120, 4096)]
+    tiles = ("medium", "wide", "small", "flat")
+    splits = (1, 2, 3, 4, 6, 8, 12, 16)
+    forms = (("NT", 0, 1), ("NN", 0, 0), ("TN", 1, 0))
+
+    def time_us(call, iters=20):
+        for _ in range(5):
+            call()
+        torch.cuda.synchronize()
+        reps = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(iters):
+                call()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            reps.append(e0.elapsed_time(e1) * 1e3 / iters)
+        return sorted(reps)[1]
+
+    rows = []
+    for m, n, k in shapes:
+        for form, ta, tb in forms:
+            a = torch.randn((k, m) if ta else (m, k), device=dev, generator=g)
+            b = torch.randn((n, k) if tb else (k, n), device=dev, generator=g) * 0.05
+            c = torch.empty((m, n), device=dev)
+            lda, ldb = (m if ta else k), (k if tb else n)
+
+            def call():
+                rc = L.kai_gemm_f32(0, ta, tb, I(m), I(n), I(k), P(a), I(lda), P(b), I(ldb), P(c), I(n), None, 0, None, 0)
+                if rc != 0:
+                    raise RuntimeError(L.kai_last_error().decode())
+
+            kai.VMath.gemm_force_plan(None)
+            chosen = kai.VMath.gemm_plan(ta, tb, m, n, k)
+            t_chosen = time_us(call)
+            call()
+            torch.cuda.synchronize()
+            want = c.clone()
+            seen = {chosen: t_chosen}
+            cands = ["%s split %d" % (t, sp) for t in tiles for sp in splits] + ["wavesplit 16", "wavesplit 32"]
+            for cand in cands:
+                kai.VMath.gemm_force_plan(cand)
+                text = kai.VMath.gemm_plan(ta, tb, m, n, k)
+                if text in seen:
+                    continue
+                seen[text] = time_us(call)
+                # a forced plan is a different order of the same sums: it must still be the same product
+                call()
+                torch.cuda.synchronize()
+                err = float(torch.linalg.norm((c - want).double()) / torch.linalg.norm(want.double()))
+                if not err <= 1e-5:
+                    raise RuntimeError("forced plan %r gives another result for %s %dx%dx%d: %.2e" % (text, form, m, n, k, err))
+            kai.VMath.gemm_force_plan(None)
+            # the audit times every candidate twice as often as the chosen plan was timed: time the chosen one again
+            seen[chosen] = min(seen[chosen], time_us(call))
+            best = min(seen, key=seen.get)
+            rows.append({"form": form, "M": m, "N": n, "K": k, "chosen": chosen, "chosen_us": round(seen[chosen], 2),
+                         "best": best, "best_us": round(seen[best], 2), "ratio": round(seen[chosen] / seen[best], 3),
+                         "candidates": len(seen)})
+    rows.sort(key=lambda r: -r["ratio"])
+    worst = rows[0]["ratio"]
+    geo = float(np.exp(np.mean([np.log(r["ratio"]) for r in rows])))
+    lines = ["| form | M x N x K | chosen plan | us | fastest alternative | us | chosen / fastest |", "|---|---|---|---|---|---|---|"]
+    for r in rows:
+        if r["ratio"] > 1.03 or r is rows[0]:
+            lines.append("| %s | %d x %d x %d | %s | %.2f | %s | %.2f | %.3f |" % (
+                r["form"], r["M"], r["N"], r["K"], r["chosen"], r["chosen_us"], r["best"], r["best_us"], r["ratio"]))
+    summary = {"cases": len(rows), "worst_ratio": worst, "geomean_ratio": round(geo, 4),
+               "over_1_08": sum(r["ratio"] > 1.08 for r in rows), "over_1_03": sum(r["ratio"] > 1.03 for r in rows)}
+    with open(out_path, "w") as f:
+        f.write(json.dumps(summary) + "\n\n" + "\n".join(lines) + "\n\n" + "\n".join(json.dumps(r) for r in rows) + "\n")
+    print(json.dumps({"plan_audit": summary, "written_to": out_path}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -413,6 +535,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="skip the table of the other configurations")
+    ap.add_argument("--plan-audit", metavar="FILE", default=None,
+                    help="instead of the benchmark: time the dispatcher's choice against every forced alternative on "
+                         "shapes around its thresholds and write the table to FILE")
     ap.add_argument("--only", action="append", default=None, metavar="TEXT",
                     help="measure only the rows of the table whose name contains TEXT (may be given several times)")
     ap.add_argument("--row-warmup-ms", type=float, default=40.0,
@@ -436,6 +561,10 @@ def main():
     stream = torch.cuda.current_stream()
     kai.set_stream(stream.cuda_stream)
     dev = torch.device("cuda:0")
+
+    if args.plan_audit:
+        plan_audit(torch, kai, stream, dev, args.plan_audit)
+        return
 
     n = 8192
     g = torch.Generator(device=dev)

@@ -564,7 +564,7 @@ bool attention_fused_applies(const float* q, const float* k, const float* v, con
     // the kernel writes its output with the row stride of the inputs; the output of the separate calls is
     // [nbat, ntimes, nhead, npiece], which is the same thing only when the heads fill the vector
     return nhead * npiece == nvec &&
-           (npiece == 16 || npiece == 32 || npiece == 64) && nvec % 4 == 0 && ntimes >= 1 && ntimes <= kMaxDim &&
+           npiece % 16 == 0 && npiece >= 16 && npiece <= 128 && nvec % 4 == 0 && ntimes >= 1 && ntimes <= kMaxDim &&
            ntimes * nvec * 4 < (1ll << 31) &&
            nhead >= 1 && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o);
 }
@@ -580,9 +580,16 @@ int launch_attention_fused(float* o, const float* q, const float* k, const float
     const int64_t qtiles = (ntimes + kFaQ - 1) / kFaQ;
     if (qtiles * nbat * nhead > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention: grid too large");
     const dim3 grid((unsigned)(qtiles * nbat * nhead));
-    if (npiece == 16) attention_fused_kernel<1><<<grid, dim3(kFaThreads), 0, stream>>>(p);
-    else if (npiece == 32) attention_fused_kernel<2><<<grid, dim3(kFaThreads), 0, stream>>>(p);
-    else attention_fused_kernel<4><<<grid, dim3(kFaThreads), 0, stream>>>(p);
+    switch (npiece / 16) {
+    case 1: attention_fused_kernel<1><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    case 2: attention_fused_kernel<2><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    case 3: attention_fused_kernel<3><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    case 4: attention_fused_kernel<4><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    case 5: attention_fused_kernel<5><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    case 6: attention_fused_kernel<6><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    case 7: attention_fused_kernel<7><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    default: attention_fused_kernel<8><<<grid, dim3(kFaThreads), 0, stream>>>(p); break;
+    }
     return check_launch("attention_fused_kernel");
 }
 
@@ -602,14 +609,22 @@ static void launch_probs(const ProbsParams& p, bool pvec, int64_t ntimes, dim3 g
     } else if (ntimes <= 512) {
         if (kVecOk && pvec) attention_probs_kernel<DB, 8, HG, kVecOk><<<grid, block, 0, stream>>>(p);
         else attention_probs_kernel<DB, 8, HG, false><<<grid, block, 0, stream>>>(p);
-    } else {
+    } else if constexpr (!(HG == 4 && DB == 4)) {
         if (kVecOk && pvec) attention_probs_kernel<DB, 16, HG, kVecOk><<<grid, block, 0, stream>>>(p);
         else attention_probs_kernel<DB, 16, HG, false><<<grid, block, 0, stream>>>(p);
     }
 }
 
 // four heads per workgroup: head counts in whole fours and rows of the probabilities that allow 128-bit stores
-static bool probs_four_heads(const float* pp, int64_t nhead) { return nhead % 4 == 0 && aligned16(pp); }
+// (head sizes up to 64: the tiles of four heads side by side must fit LDS twice)
+// (and not head size 64 beyond 512 keys: 128 score registers next to the staging registers of the wide tiles do not fit)
+static bool probs_four_heads(const float* pp, int64_t nhead, int64_t npiece, int64_t ntimes) {
+    return nhead % 4 == 0 && npiece <= 64 && !(npiece == 64 && ntimes > 512) && aligned16(pp);
+}
+
+bool attention_probs_four_heads(const float* pp, int64_t ntimes, int64_t nhead, int64_t npiece) {
+    return probs_four_heads(pp, nhead, npiece, ntimes);
+}
 
 int launch_attention_probs(float* o, float* pp, const float* q, const float* k, const float* v, int64_t nbat,
                            int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
@@ -620,20 +635,30 @@ int launch_attention_probs(float* o, float* pp, const float* q, const float* k, 
     p.f.ntimes = (int)ntimes; p.f.nhead = (int)nhead; p.f.npiece = (int)npiece;
     p.f.masked = masked;
     p.P = pp; p.p_batch_stride = ntimes * ntimes * nhead;
-    const bool four = probs_four_heads(pp, nhead);
+    const bool four = probs_four_heads(pp, nhead, npiece, ntimes);
     const int64_t qtiles = four ? (ntimes + 15) / 16 : (ntimes + kFaQ - 1) / kFaQ;
     const int64_t wgs = qtiles * nbat * (four ? nhead / 4 : nhead);
     if (wgs > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention: grid too large");
     const dim3 grid((unsigned)wgs);
     const bool pvec = nhead == 1 && ntimes % 4 == 0 && aligned16(pp);
     if (four) {
-        if (npiece == 16) launch_probs<1, 4>(p, false, ntimes, grid, stream);
-        else if (npiece == 32) launch_probs<2, 4>(p, false, ntimes, grid, stream);
-        else launch_probs<4, 4>(p, false, ntimes, grid, stream);
+        switch (npiece / 16) {
+        case 1: launch_probs<1, 4>(p, false, ntimes, grid, stream); break;
+        case 2: launch_probs<2, 4>(p, false, ntimes, grid, stream); break;
+        case 3: launch_probs<3, 4>(p, false, ntimes, grid, stream); break;
+        default: launch_probs<4, 4>(p, false, ntimes, grid, stream); break;
+        }
     } else {
-        if (npiece == 16) launch_probs<1, 1>(p, pvec, ntimes, grid, stream);
-        else if (npiece == 32) launch_probs<2, 1>(p, pvec, ntimes, grid, stream);
-        else launch_probs<4, 1>(p, pvec, ntimes, grid, stream);
+        switch (npiece / 16) {
+        case 1: launch_probs<1, 1>(p, pvec, ntimes, grid, stream); break;
+        case 2: launch_probs<2, 1>(p, pvec, ntimes, grid, stream); break;
+        case 3: launch_probs<3, 1>(p, pvec, ntimes, grid, stream); break;
+        case 4: launch_probs<4, 1>(p, pvec, ntimes, grid, stream); break;
+        case 5: launch_probs<5, 1>(p, pvec, ntimes, grid, stream); break;
+        case 6: launch_probs<6, 1>(p, pvec, ntimes, grid, stream); break;
+        case 7: launch_probs<7, 1>(p, pvec, ntimes, grid, stream); break;
+        default: launch_probs<8, 1>(p, pvec, ntimes, grid, stream); break;
+        }
     }
     return check_launch("attention_probs_kernel");
 }

@@ -95,6 +95,7 @@ int launch_attention_fused(float* o, const float* q, const float* k, const float
 // the same block with the probabilities stored as well (training): lengths up to 1024
 bool attention_probs_applies(const float* q, const float* k, const float* v, const float* o, const float* pp,
                              int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece);
+bool attention_probs_four_heads(const float* pp, int64_t ntimes, int64_t nhead, int64_t npiece);
 int launch_attention_probs(float* o, float* pp, const float* q, const float* k, const float* v, int64_t nbat,
                            int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
                            hipStream_t stream);

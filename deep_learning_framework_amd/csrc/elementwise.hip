@@ -282,11 +282,51 @@ int launch_transpose_bin(float* y, const float* x, int64_t nrow, int64_t ncol, h
     return check_launch("transpose_bin_kernel");
 }
 
+// The index arithmetic of one element (or one group of four): output position -> source position through the
+// table, with 32-bit integers where the tensor allows it (a 64-bit division costs several times a 32-bit one, and
+// there is one per axis and element).
+template <typename I, bool BACKWARD, bool VEC>
+__device__ __forceinline__ void transpose_axes_body(float* __restrict__ out, const float* __restrict__ in,
+                                                    const int64_t* yblk64, const int64_t* xblk64, int axis_size, int64_t n) {
+    I yblk[kTrMaxAxes], xblk[kTrMaxAxes];
+#pragma unroll
+    for (int m = 0; m < kTrMaxAxes; m++) {
+        yblk[m] = m < axis_size ? (I)yblk64[m] : (I)1;
+        xblk[m] = m < axis_size ? (I)xblk64[m] : (I)0;
+    }
+    const I count = (I)(VEC ? n / 4 : n);
+    const I stride = (I)gridDim.x * kEwThreads;
+    for (I i = (I)blockIdx.x * kEwThreads + threadIdx.x; i < count; i += stride) {
+        I xpos = 0, ypos = VEC ? i * 4 : i;
+#pragma unroll
+        for (int m = 0; m < kTrMaxAxes; m++) {      // written out: the table stays in registers
+            if (m < axis_size) {
+                const I c = ypos / yblk[m];
+                ypos -= c * yblk[m];
+                xpos += c * xblk[m];
+            }
+        }
+        if (VEC) {
+            // four consecutive elements of the innermost axis, which is the innermost axis on both sides
+            const I o = i * 4;
+            if (BACKWARD) *reinterpret_cast<f32x4*>(out + xpos) = *reinterpret_cast<const f32x4*>(in + o);
+            else *reinterpret_cast<f32x4*>(out + o) = *reinterpret_cast<const f32x4*>(in + xpos);
+        } else {
+            if (BACKWARD) out[xpos] = in[i];
+            else out[i] = in[xpos];
+        }
+    }
+}
+
+// The table lives in device memory (the engine builds it there), so the kernel itself looks whether the innermost
+// output axis is the innermost source axis (the head split / merge [B, T, H, D] <-> [B, H, T, D] of the attention
+// layers and every permutation of outer axes): then whole 128-bit words move, the innermost 4 * k floats being
+// contiguous on both sides.  `aligned16` is the host's check of the two base pointers.
 template <bool BACKWARD>
 __global__ void __launch_bounds__(kEwThreads) transpose_axes_kernel(float* __restrict__ out,
                                                                     const float* __restrict__ in,
                                                                     const int* __restrict__ pn, int axis_size,
-                                                                    int64_t n) {
+                                                                    int64_t n, int aligned16) {
     // the table is tiny and the same for every thread
     __shared__ int64_t yblk[kTrMaxAxes], xblk[kTrMaxAxes];
     if (threadIdx.x < axis_size) {
@@ -294,16 +334,18 @@ __global__ void __launch_bounds__(kEwThreads) transpose_axes_kernel(float* __res
         xblk[threadIdx.x] = pn[pn[threadIdx.x * 3] * 3 + 2];
     }
     __syncthreads();
-    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
-    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n; i += stride) {
-        int64_t xpos = 0, ypos = i;
-        for (int m = 0; m < axis_size; m++) {
-            const int64_t c = ypos / yblk[m];
-            ypos -= c * yblk[m];
-            xpos += c * xblk[m];
-        }
-        if (BACKWARD) out[xpos] = in[i];
-        else out[i] = in[xpos];
+    const int last = axis_size - 1;
+    // length of the innermost output axis = output elements per step of the axis before it
+    const int64_t inner = last > 0 ? yblk[last - 1] : n;
+    bool vec = aligned16 && yblk[last] == 1 && xblk[last] == 1 && inner % 4 == 0 && n % 4 == 0;
+    for (int m = 0; m < last; m++) vec = vec && xblk[m] % 4 == 0 && yblk[m] % 4 == 0;
+    const bool small = n < (1ll << 31);
+    if (vec) {
+        if (small) transpose_axes_body<int32_t, BACKWARD, true>(out, in, yblk, xblk, axis_size, n);
+        else transpose_axes_body<int64_t, BACKWARD, true>(out, in, yblk, xblk, axis_size, n);
+    } else {
+        if (small) transpose_axes_body<int32_t, BACKWARD, false>(out, in, yblk, xblk, axis_size, n);
+        else transpose_axes_body<int64_t, BACKWARD, false>(out, in, yblk, xblk, axis_size, n);
     }
 }
 
@@ -311,8 +353,11 @@ int launch_transpose(float* y, const float* x, const int* pn, int64_t axis_size,
                      hipStream_t stream) {
     if (n <= 0) return KAI_OK;
     if (axis_size < 1 || axis_size > kTrMaxAxes) return fail(KAI_ERR_INVALID_ARGUMENT, "transpose: 1 to 8 axes");
-    if (backward) transpose_axes_kernel<true><<<blocks_for(n), kEwThreads, 0, stream>>>(y, x, pn, (int)axis_size, n);
-    else transpose_axes_kernel<false><<<blocks_for(n), kEwThreads, 0, stream>>>(y, x, pn, (int)axis_size, n);
+    const int al = aligned16(y) && aligned16(x);
+    // a thread moves up to four elements: a quarter of the workgroups cover the tensor when it does (grid-stride)
+    const dim3 grid = blocks_for(al ? (n + 3) / 4 : n);
+    if (backward) transpose_axes_kernel<true><<<grid, kEwThreads, 0, stream>>>(y, x, pn, (int)axis_size, n, al);
+    else transpose_axes_kernel<false><<<grid, kEwThreads, 0, stream>>>(y, x, pn, (int)axis_size, n, al);
     return check_launch("transpose_axes_kernel");
 }
 

@@ -4,6 +4,7 @@
 // pair that matches how the operands lie in memory, with the tile that needs the fewest rounds
 // over the compute units.
 #include <algorithm>
+#include <cstdlib>
 #include <string>
 
 #include "elementwise.h"
@@ -32,6 +33,17 @@ static int launch_layout(const GemmParams& p, bool a_kc, bool b_kc, int64_t nbat
 
 namespace {
 
+// A maintainer's override of the choice below (kai_gemm_force_plan): the tile and / or the number of parts of the
+// reduction, or the one-launch kernel for small products.  Process-wide, meant for audits of the fitted rules
+// (bench.py --plan-audit times the chosen plan against every alternative), never set in production.
+struct ForcedPlan {
+    bool active = false;
+    int tile = -1;          // kTile* or -1: keep the chosen tile
+    int64_t split = 0;      // >= 1: this many parts; 0: keep the chosen number
+    int wavesplit = 0;      // 16 or 32: the wave-split kernel with blocks of that edge
+};
+ForcedPlan g_forced;
+
 struct GemmPlan {
     bool skinny = false;
     bool a_kc = false, b_kc = false;
@@ -41,6 +53,7 @@ struct GemmPlan {
     bool ragged_parts = false;   // the last part is shorter than k_part
     GemmDesc dn;   // the product with batch strides normalised
     int wavesplit_edge = 0;   // 16 or 32: the product runs on the kernel that cuts K over the waves of a workgroup
+    bool forced = false;      // set by an override: the tiled kernel (or the wave-split kernel) whatever else applies
 };
 
 // Expected duration in microseconds of the wave-split kernel with T x T blocks, or a negative value outside the
@@ -242,11 +255,12 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // beyond L2.  Taken where that is 7 % below the other tiles' estimate: over 57 shapes in the three operand
     // forms 1.05 x on average (144 x 4096 x 4096 53.4 -> 49.5 us, 144 x 3072 x 4096 44.8 -> 39, 144 x 6144 x 4096
     // 85 -> 70, 144 x 8192 x 4096 96 -> 88, 160 x 4096 x 11008 130 -> 123; ties at 2560 x 2560 and 1024 x 4096).
-    // Reductions under 2048 steps lost (4096 x 1024: 19.3 -> 21) and 11008 columns measured between 9 % slower
+    // Reductions of 1024 steps lost (4096 x 1024: 19.3 -> 21; 2047 steps measure like 2048: 144 x 2048 x 2047 23.3 -> 20.9
+    // in the audit of these rules, bench.py --plan-audit, so the bound sits a little below 2048) and 11008 columns measured between 9 % slower
     // and 8 % faster: both stay with the other tiles.  193..224 rows likewise, seven rows of tiles against four
     // (200 x 3072 x 4096 56 -> 50 us, 224 x 4608 x 4608 91 -> 77, 200 x 3072 x 3072 42 -> 39; 50 shapes x 3 forms
     // 1.04-1.05 x on average, nothing slower than measurement noise).
-    if (modelled && ((d.M > 128 && d.M <= 160) || (d.M > 192 && d.M <= 224)) && d.N >= 1024 && d.N <= 8192 && d.K >= 2048 && d.N * d.K <= (1ll << 26)) {
+    if (modelled && ((d.M > 128 && d.M <= 160) || (d.M > 192 && d.M <= 224)) && d.N >= 1024 && d.N <= 8192 && d.K >= 2000 && d.N * d.K <= (1ll << 26)) {
         const GemmParams pp = make_params(dn, plan.a_kc, plan.b_kc);
         if (fits_ragged_pipe(pp, plan.a_kc, plan.b_kc, 32, 128)) {
             const int64_t tiles = ((d.M + 31) / 32) * ((d.N + 127) / 128);
@@ -338,6 +352,37 @@ GemmPlan plan_gemm(const GemmDesc& d) {
             if (plan.split < 2) plan.split = 1;
         }
     }
+    if (g_forced.active && d.nbatch == 1 && d.rowsum == nullptr) {
+        if (g_forced.wavesplit) {
+            if (wavesplit_applies(dn) && wavesplit_estimate(dn, g_forced.wavesplit) > 0) {
+                plan.forced = true;
+                plan.skinny = false;
+                plan.wavesplit_edge = g_forced.wavesplit;
+                plan.split = 1; plan.k_part = 0; plan.ragged_parts = false;
+            }
+        } else {
+            plan.forced = true;
+            plan.skinny = false;
+            plan.wavesplit_edge = 0;
+            if (g_forced.tile >= 0) plan.tile = g_forced.tile;
+            if (g_forced.split >= 1) {
+                // the parts as the model above cuts them: equal where 16-step tiles allow it, else whole tiles with a
+                // shorter last part; a part count that the length does not give, or whose sums exceed the scratch,
+                // leaves one part
+                const int64_t sp = g_forced.split;
+                plan.split = 1; plan.k_part = 0; plan.ragged_parts = false;
+                if (sp >= 2 && sp <= kSplitMax && d.K >= 32 * sp && sp * d.M * d.N * (int64_t)sizeof(float) <= scratch_cap) {
+                    const bool equal = d.K % (16 * sp) == 0;
+                    const int64_t k_len = equal ? d.K / sp : ((d.K + sp - 1) / sp + 15) / 16 * 16;
+                    if ((d.K + k_len - 1) / k_len == sp) {
+                        plan.split = sp;
+                        plan.k_part = k_len;
+                        plan.ragged_parts = !equal;
+                    }
+                }
+            }
+        }
+    }
     return plan;
 }
 
@@ -346,6 +391,36 @@ bool valid_dims(const GemmDesc& d) {
 }
 
 }  // namespace
+
+// "auto" (or empty) clears the override; otherwise words: a tile name (large, medium, small, flat, wide), and / or
+// "split N" (1 .. 16), or "wavesplit 16" / "wavesplit 32".
+int set_forced_gemm_plan(const char* text) {
+    ForcedPlan f;
+    std::string t = text ? text : "";
+    size_t pos = 0;
+    auto next = [&]() -> std::string {
+        while (pos < t.size() && t[pos] == ' ') pos++;
+        const size_t b = pos;
+        while (pos < t.size() && t[pos] != ' ') pos++;
+        return t.substr(b, pos - b);
+    };
+    static const char* const tiles[] = {"large", "medium", "small", "flat", "wide"};
+    for (std::string w = next(); !w.empty(); w = next()) {
+        if (w == "auto") continue;
+        bool known = false;
+        for (int i = 0; i < 5; i++)
+            if (w == tiles[i]) { f.tile = i; f.active = known = true; }
+        if (w == "split" || w == "wavesplit") {
+            const std::string n = next();
+            const long v = n.empty() ? -1 : strtol(n.c_str(), nullptr, 10);
+            if (w == "split" && v >= 1 && v <= kSplitMax) { f.split = v; f.active = known = true; }
+            if (w == "wavesplit" && (v == 16 || v == 32)) { f.wavesplit = (int)v; f.active = known = true; }
+        }
+        if (!known) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm plan override: cannot read \"" + w + "\"");
+    }
+    g_forced = f;
+    return KAI_OK;
+}
 
 bool gemm_fuses_rowsum(const GemmDesc& d) {
     if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
@@ -361,11 +436,13 @@ std::string describe_gemm(const GemmDesc& d) {
     if (d.M == 0 || d.N == 0 || d.nbatch == 0) return "nothing";
     const GemmPlan plan = plan_gemm(d);
     if (plan.wavesplit_edge) return "wavesplit " + std::to_string(plan.wavesplit_edge);
-    if (skinny_rows_applies(plan.dn)) return "skinny rows";
-    if (plan.skinny) return "skinny";
-    if (shortk_nt_applies(plan.dn)) return "shortk_nt";
-    if (shortk_heads_applies(plan.dn)) return "shortk_heads";
-    if (heads_pv_applies(d)) return "heads_pv";
+    if (!plan.forced) {
+        if (skinny_rows_applies(plan.dn)) return "skinny rows";
+        if (plan.skinny) return "skinny";
+        if (shortk_nt_applies(plan.dn)) return "shortk_nt";
+        if (shortk_heads_applies(plan.dn)) return "shortk_heads";
+        if (heads_pv_applies(d)) return "heads_pv";
+    }
     const bool a_kc = plan.a_kc, b_kc = plan.b_kc;
     GemmDesc dt = plan.dn;
     if (plan.split >= 2) {
@@ -399,7 +476,7 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
         return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: this product cannot carry the fused row sum");
 
     if (plan.wavesplit_edge) return launch_gemm_wavesplit(plan.dn, plan.wavesplit_edge, stream);
-    if (skinny_rows_applies(plan.dn)) return launch_skinny_rows(plan.dn, stream);
+    if (!plan.forced && skinny_rows_applies(plan.dn)) return launch_skinny_rows(plan.dn, stream);
     if (plan.skinny) {
         SkinnyParams s{};
         s.W = d.B; s.X = d.A; s.Y = d.C; s.Y2 = d.C2; s.bias = d.bias; s.leaky = d.leaky;
@@ -410,10 +487,12 @@ int launch_gemm(const GemmDesc& d, hipStream_t stream) {
     }
 
     const bool a_kc = plan.a_kc, b_kc = plan.b_kc;
-    if (shortk_nt_applies(plan.dn)) return launch_gemm_shortk_nt(make_params(plan.dn, true, true), d.nbatch, stream);
-    if (shortk_heads_applies(plan.dn))
-        return launch_gemm_shortk_heads(make_params(plan.dn, true, true), d.nbatch, stream);
-    if (heads_pv_applies(d)) return launch_heads_pv(d, stream);
+    if (!plan.forced) {
+        if (shortk_nt_applies(plan.dn)) return launch_gemm_shortk_nt(make_params(plan.dn, true, true), d.nbatch, stream);
+        if (shortk_heads_applies(plan.dn))
+            return launch_gemm_shortk_heads(make_params(plan.dn, true, true), d.nbatch, stream);
+        if (heads_pv_applies(d)) return launch_heads_pv(d, stream);
+    }
     if (plan.split >= 2) {
         const int64_t split = plan.split;
         float* part = d.scratch;

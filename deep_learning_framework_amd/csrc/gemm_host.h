@@ -117,6 +117,8 @@ int launch_gemm_config(GemmParams p, int64_t nbatch, int group_m, hipStream_t st
 
 // picks kernel family, tile and variant; defined in gemm_dispatch.hip
 int launch_gemm(const GemmDesc& d, hipStream_t stream);
+// a maintainer's override of that choice (kai_gemm_force_plan); "auto" clears it
+int set_forced_gemm_plan(const char* text);
 // the decision of launch_gemm as text (host arithmetic only)
 std::string describe_gemm(const GemmDesc& d);
 // true when launch_gemm would compute GemmDesc::rowsum inside the product's own launch (d.rowsum is

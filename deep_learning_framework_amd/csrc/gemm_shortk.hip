@@ -71,16 +71,16 @@ __device__ __forceinline__ void mask_panel(f32x4 (&reg)[ROWS * kSkK / 4 / kSkThr
 }
 
 // NG: groups of 8 reduction steps that are computed (K <= 8 * NG; the panels are zero beyond K).
-// FULL = false: the epilogue only scales and stores (no accumulation into C, bias, second output
-// or activation), so nothing in the loop waits on a load issued after a store.
+// The epilogue only scales and stores (no accumulation into C, bias, second output or activation: products that
+// ask for those run the tiled kernels), so nothing in the loop waits on a load issued after a store.
 // Grid: one dimension over (batch, column panel, run), where a run is p.group_m consecutive row
 // tiles.  Hardware deals consecutive workgroup ids round-robin over the 8 XCDs; ids are renumbered
 // so that each XCD walks a contiguous range, which keeps the workgroups of one batch entry (they
 // share its A and B) behind one L2.
 // WHOLE: row and column counts in whole tiles, K = 64, 128-bit loads and stores: no clamp, mask or branch is left.
-template <int NG, bool FULL, bool WHOLE>
+template <int NG, bool WHOLE>
 __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams p) {
-    static_assert(!WHOLE || (NG * 8 == kSkK && !FULL), "whole panels: all 64 reduction steps, plain epilogue");
+    static_assert(!WHOLE || NG * 8 == kSkK, "whole panels: all 64 reduction steps");
     __shared__ __attribute__((aligned(16))) float lds_a[2][TileA::kFloats];
     __shared__ __attribute__((aligned(16))) float lds_b[TileB::kFloats];
 
@@ -147,7 +147,7 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
 #pragma unroll
             // plain epilogue: the scale goes into the panel once per workgroup instead of into every output (64
             // multiplies per lane and tile, which would take their time from the MFMAs)
-            for (int j = 0; j < 4; j++) lds_b[(k + j) * TileB::kStride + n] = FULL ? rb[i][j] : rb[i][j] * alpha;
+            for (int j = 0; j < 4; j++) lds_b[(k + j) * TileB::kStride + n] = rb[i][j] * alpha;
         }
         stage_a(tm_first, 0);
     }
@@ -191,9 +191,7 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
         if (WHOLE || more) stage_a(min(tm + 1, tm_first + ntile - 1), (it + 1) & 1);
 
         if (rows_inside) {
-            if (FULL) {
-                gemm_epilogue<1, 4, true, false>(p, acc, m0, n0, c_off, wm0, 0, l32, half, alpha, leaky);
-            } else {
+            {
                 float* C = p.C + c_off;
                 const int col = n0 + 4 * l32;
                 static_for<0, 16>([&](auto rc) {
@@ -404,7 +402,10 @@ constexpr int64_t kSkMinOutputs = 1ll << 22;
 
 bool shortk_nt_applies(const GemmDesc& d) {
     return d.a_ks == 1 && d.b_ks == 1 && d.c_cs == 1 && d.K >= 1 && d.K <= kSkK && d.rowsum == nullptr &&
-           d.k_part == 0 && d.M >= 64 && d.N >= 64 && d.M * d.N * d.nbatch >= kSkMinOutputs;
+           d.k_part == 0 && d.M >= 64 && d.N >= 64 && d.M * d.N * d.nbatch >= kSkMinOutputs &&
+           // plain epilogue only (scale and store): with accumulate / bias / second output / activation the kernel
+           // needed more registers than a wave has and spilled; no call of the engine's path asks for them here
+           !d.acc && d.bias == nullptr && d.C2 == nullptr && d.act == 0;
 }
 
 int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream) {
@@ -422,16 +423,15 @@ int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream) {
     const int64_t blocks = runs * p.tiles_n * nbatch;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: grid too large");
     const dim3 grid((unsigned)blocks, 1, 1);
-    const bool full = p.accflag || p.bias || p.C2 || p.act != kActNone;
-    const bool whole = !full && p.M % kSkBM == 0 && p.N % kSkBN == 0 && p.K == kSkK && p.a_vec && p.b_vec && p.c_vec;
+    if (p.accflag || p.bias || p.C2 || p.act != kActNone)
+        return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: the short-reduction kernel has no accumulate / bias / activation epilogue");
+    const bool whole = p.M % kSkBM == 0 && p.N % kSkBN == 0 && p.K == kSkK && p.a_vec && p.b_vec && p.c_vec;
     if (whole) {
-        shortk_nt_kernel<8, false, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+        shortk_nt_kernel<8, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     } else if (p.K <= 32) {
-        if (full) shortk_nt_kernel<4, true, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
-        else shortk_nt_kernel<4, false, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+        shortk_nt_kernel<4, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     } else {
-        if (full) shortk_nt_kernel<8, true, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
-        else shortk_nt_kernel<8, false, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
+        shortk_nt_kernel<8, false><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     }
     return check_launch("shortk_nt_kernel");
 }

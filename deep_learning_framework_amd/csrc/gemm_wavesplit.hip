@@ -149,15 +149,26 @@ __global__ void __launch_bounds__(64 * kWsWaves) gemm_wavesplit_kernel(const Wav
         // every load of the round is issued before the first product (left alone, the scheduler sinks the loads
         // to their uses to save registers: two in flight instead of sixteen)
         __builtin_amdgcn_sched_barrier(0);
+        // (32 x 32 blocks with two operands that are not K-contiguous: eight element loads per group with a 64-bit
+        // address each; a second set of operands in flight did not fit the 128 registers of a wave and spilled, so
+        // this form loads a round after it has multiplied the one before -- four waves per SIMD cover the wait)
+        constexpr bool kOverlap = !(T == 32 && !A_KC && !B_KC);
         for (int next = g0 + U * kWsWaves; U == kWsFlight && next < ngroups; next += U * kWsWaves) {
-            f32x4 a_now[U], b_now[U];
+            if constexpr (kOverlap) {
+                f32x4 a_now[U], b_now[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                a_now[u] = a[u];
-                b_now[u] = b[u];
+                for (int u = 0; u < U; u++) {
+                    a_now[u] = a[u];
+                    b_now[u] = b[u];
+                }
+                load(next);
+                multiply(a_now, b_now, g0);
+            } else {
+                multiply(a, b, g0);
+                __builtin_amdgcn_sched_barrier(0);
+                load(next);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            load(next);
-            multiply(a_now, b_now, g0);
             g0 = next;
         }
         multiply(a, b, g0);

@@ -355,34 +355,35 @@ __global__ void __launch_bounds__(64 * kSliceMaxWaves * kSliceLdsGroups) skinny_
         }
     }
     {
-        f32x4 xv[MT];
+        // two rows of X at a time: with four in flight next to the sixteen chunks of W a wave of this 16-wave
+        // workgroup ran out of its 128 registers
+        constexpr int XB = MT < 2 ? MT : 2;
         const int k = min(4 * tid, p.K - 4);
 #pragma unroll
-        for (int m = 0; m < MT; m++) xv[m] = *reinterpret_cast<const f32x4*>(p.X + (int64_t)min(m, p.M - 1) * p.ldx + k);
+        for (int m0 = 0; m0 < MT; m0 += XB) {
+            f32x4 xv[XB];
 #pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const int keep = (m < p.M && 4 * tid < p.K) ? -1 : 0;   // rows beyond M and steps beyond K read as zero
-            f32x4 z;
+            for (int m = 0; m < XB; m++)
+                xv[m] = *reinterpret_cast<const f32x4*>(p.X + (int64_t)min(m0 + m, p.M - 1) * p.ldx + k);
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float v = xv[m][e];
-                z[e] = __int_as_float(__float_as_int(v) & keep);
+            for (int m = 0; m < XB; m++) {
+                const int keep = (m0 + m < p.M && 4 * tid < p.K) ? -1 : 0;   // rows beyond M and steps beyond K read as zero
+                f32x4 z;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float v = xv[m][e];
+                    z[e] = __int_as_float(__float_as_int(v) & keep);
+                }
+                *reinterpret_cast<f32x4*>(&xs[(m0 + m) * kSliceLdsK + 4 * tid]) = z;
             }
-            *reinterpret_cast<f32x4*>(&xs[m * kSliceLdsK + 4 * tid]) = z;
         }
     }
     __syncthreads();
 
-    float acc[MT][RB];
-#pragma unroll
-    for (int m = 0; m < MT; m++)
-#pragma unroll
-        for (int r = 0; r < RB; r++) acc[m][r] = 0.f;
+    // W beyond K meets the zeros of X, but may hold anything: inf * 0 must not reach the sum
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        const int kk = ks + 4 * lane + 256 * j;           // < 4096: inside xs (zeros beyond K)
-        const int keep_k = (kk < p.K) ? -1 : 0;
-        // W beyond K meets the zeros of X, but may hold anything: inf * 0 must not reach the sum
+        const int keep_k = (ks + 4 * lane + 256 * j < p.K) ? -1 : 0;
 #pragma unroll
         for (int r = 0; r < RB; r++)
 #pragma unroll
@@ -390,22 +391,29 @@ __global__ void __launch_bounds__(64 * kSliceMaxWaves * kSliceLdsGroups) skinny_
                 const float v = w[r][j][e];
                 w[r][j][e] = __int_as_float(__float_as_int(v) & keep_k);
             }
+    }
+    // one row of X at a time, fenced: with the rows interleaved the sixteen chunks of W, the chunks of X of several
+    // rows and sixteen sums did not fit the 128 registers a wave of this 16-wave workgroup has
 #pragma unroll
-        for (int m = 0; m < MT; m++) {
+    for (int m = 0; m < MT; m++) {
+        float acc[RB];
+#pragma unroll
+        for (int r = 0; r < RB; r++) acc[r] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int kk = ks + 4 * lane + 256 * j;           // < 4096: inside xs (zeros beyond K)
             const f32x4 x = *reinterpret_cast<const f32x4*>(&xs[m * kSliceLdsK + kk]);
 #pragma unroll
             for (int r = 0; r < RB; r++)
-                acc[m][r] += w[r][j][0] * x[0] + w[r][j][1] * x[1] + w[r][j][2] * x[2] + w[r][j][3] * x[3];
+                acc[r] += w[r][j][0] * x[0] + w[r][j][1] * x[1] + w[r][j][2] * x[2] + w[r][j][3] * x[3];
         }
-    }
-
-#pragma unroll
-    for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int r = 0; r < RB; r++) {
-            const float v = wave_sum(acc[m][r]);
+            const float v = wave_sum(acc[r]);
             if (lane == 0) part[rg][m * RB + r][sl] = v;
         }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     __syncthreads();
     if (tid < kSliceLdsGroups * MT * RB) {
         const int g = tid / (MT * RB), t = tid % (MT * RB);
@@ -508,15 +516,18 @@ __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const Skinny
 
     // chunks of kMmUnroll steps: all loads of W and of X of a chunk are issued back to back (32 KiB in
     // flight per wave), then its MFMAs; the second wave of the SIMD computes meanwhile
-    for (int base = s_begin; base < s_end; base += kMmUnroll) {
-        f32x4v w[kMmUnroll], x[kMmUnroll];
+    // (element-wise loads, 128 of them per chunk of 16 steps with an address each, do not fit the registers:
+    // chunks of 8 steps there)
+    constexpr int UN = VEC ? kMmUnroll : kMmUnroll / 2;
+    for (int base = s_begin; base < s_end; base += UN) {
+        f32x4v w[UN], x[UN];
 #pragma unroll
-        for (int u = 0; u < kMmUnroll; u++) w[u] = load4(wp, (base + u) * 16 + 4 * g);
+        for (int u = 0; u < UN; u++) w[u] = load4(wp, (base + u) * 16 + 4 * g);
 #pragma unroll
-        for (int u = 0; u < kMmUnroll; u++) x[u] = load4(xp, (base + u) * 16 + 4 * g);
+        for (int u = 0; u < UN; u++) x[u] = load4(xp, (base + u) * 16 + 4 * g);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < kMmUnroll; u++) {
+        for (int u = 0; u < UN; u++) {
             const int k = (base + u) * 16 + 4 * g;
             const bool in = base + u < s_end;   // steps past the end of the slice add nothing
             const f32x4v wv = masked(w[u], k, wvalid && in);

@@ -6,6 +6,7 @@
 // mh_attention (:2978-3052) and multihead_attention_backprop (:3054-3227).
 #include <cstring>
 #include <cstdlib>
+#include <cstdio>
 #include <mutex>
 #include <vector>
 
@@ -836,6 +837,26 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
     if (masked) KAI_TRY(kai_set_mh_attention_mask(device, pp, nbat, ntimes, nhead, 1));
     KAI_TRY(kai_softmax_direct_on_axis(device, pp, nbat * ntimes, ntimes, nhead));
     return kai_mix_values(device, py, pp, pV, nbat, ntimes, nvec, nhead, npiece);
+}
+
+int kai_gemm_force_plan(const char* text) { return set_forced_gemm_plan(text); }
+
+int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, char* out,
+                       int buflen) {
+    KAI_REQUIRE(out != nullptr && buflen > 0, KAI_ERR_INVALID_POINTER, "null output buffer");
+    KAI_REQUIRE(which >= 0 && which <= 2, KAI_ERR_INVALID_ARGUMENT, "which must be 0 (forward), 1 (forward, training) or 2 (backward)");
+    KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
+    // 16-byte aligned operands are assumed: a pointer value that satisfies every alignment test
+    const float* a = reinterpret_cast<const float*>(uintptr_t(256));
+    std::string text = "separate";
+    if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) text = "nothing";
+    else if (which == 0 && attention_fused_applies(a, a, a, a, ntimes, nvec, nhead, npiece)) text = "fused";
+    else if (which == 1 && attention_probs_applies(a, a, a, a, a, ntimes, nvec, nhead, npiece))
+        text = attention_probs_four_heads(a, ntimes, nhead, npiece) ? "fused, four heads per workgroup" : "fused";
+    else if (which == 2 && attention_backward_applies(a, a, a, a, a, a, a, a, ntimes, nvec, nhead, npiece))
+        text = "fused rows + value gradient";
+    snprintf(out, (size_t)buflen, "%s", text.c_str());
+    return KAI_OK;
 }
 
 int kai_attention_forward_train(int device, float* py, float* pp, const float* pQ, const float* pK, const float* pV,

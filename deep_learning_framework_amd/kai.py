@@ -66,6 +66,8 @@ SIGNATURES = {
     "kai_gemm_plan": [_INT, _INT, _I64, _I64, _I64, _I64, _I64, _I64, _INT, _INT, _INT, ctypes.c_char_p, _INT],
     "kai_dense_forward": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _INT, _F],
     "kai_attention_forward": [_INT, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
+    "kai_gemm_force_plan": [ctypes.c_char_p],
+    "kai_attention_plan": [_INT, _I64, _I64, _I64, _I64, _I64, ctypes.c_char_p, _INT],
     "kai_attention_forward_train": [_INT, _F, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
     "kai_attention_backward": [_INT, _F, _F, _F, _F, _F, _F, _F, _F, _F, _I64, _I64, _I64, _I64, _I64, _F, _INT],
     "kai_cosinesim": [_INT, _F, _F, _F, _I64, _I64, _I64],
@@ -422,6 +424,21 @@ class VMath:
     def attention_forward(device, py, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked):
         _ck(load().kai_attention_forward(device, _addr(py), _addr(pQ), _addr(pK), _addr(pV), nbat, ntimes, nvec,
                                          nhead, npiece, _addr(hCoef), int(bool(masked))))
+
+    @staticmethod
+    def gemm_force_plan(text):
+        """Override the dispatcher's choice for later single products ("small split 4", "wavesplit 32", ...); "auto" or
+        None clears it.  For audits of the dispatch rules only."""
+        _ck(load().kai_gemm_force_plan((text or "auto").encode()))
+
+    @staticmethod
+    def attention_plan(which, nbat, ntimes, nvec, nhead, npiece):
+        """How an attention entry point would run this geometry (host arithmetic only): which = "forward",
+        "forward_train" or "backward"."""
+        buf = ctypes.create_string_buffer(128)
+        _ck(load().kai_attention_plan({"forward": 0, "forward_train": 1, "backward": 2}[which], nbat, ntimes, nvec, nhead,
+                                      npiece, buf, 128))
+        return buf.value.decode()
 
     @staticmethod
     def attention_forward_train(device, py, pp, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked):

@@ -139,7 +139,10 @@ class Tensor:
         return xgrad
 
     # ---- mh_attention: vtensor.cpp:2978-3052 ----------------------------------------------------------
-    def mh_attention(self, key, query, value, Kw, Kb, Qw, Qb, Vw, Vb, Ow, Ob, head_cnt, mask=False, coef=None):
+    def mh_attention(self, key, query, value, Kw, Kb, Qw, Qb, Vw, Vb, Ow, Ob, head_cnt, mask=False, coef=None,
+                     fused=False):
+        """``fused=False`` issues the reference's calls one by one; ``fused=True`` replaces the middle of the block
+        (mult_on_heads, mask, softmax_direct_on_axis, mix_values) by one kai_attention_forward_train."""
         x = self
         if len(x.shape) != 3 or x.shape[2] % head_cnt != 0:
             raise KaiError(VERR_BAD_SHAPE_TENSOR, "mh_attention")
@@ -168,11 +171,15 @@ class Tensor:
         VMath.add_bias(dev, K.ptr, K.ptr, Kb.ptr, n, nvec)
         VMath.add_bias(dev, Q.ptr, Q.ptr, Qb.ptr, n, nvec)
         VMath.add_bias(dev, V.ptr, V.ptr, Vb.ptr, n, nvec)
-        VMath.mult_on_heads(dev, probs.ptr, K.ptr, Q.ptr, nbat, ntimes, nvec, nhead, npiece, hcoef)
-        if mask:
-            VMath.set_mh_attention_mask(dev, probs.ptr, nbat, ntimes, nhead, True)
-        VMath.softmax_direct_on_axis(dev, probs.ptr, nbat * ntimes, ntimes, nhead)
-        VMath.mix_values(dev, mixed.ptr, probs.ptr, V.ptr, nbat, ntimes, nvec, nhead, npiece)
+        if fused:
+            VMath.attention_forward_train(dev, mixed.ptr, probs.ptr, Q.ptr, K.ptr, V.ptr, nbat, ntimes, nvec, nhead,
+                                          npiece, hcoef, mask)
+        else:
+            VMath.mult_on_heads(dev, probs.ptr, K.ptr, Q.ptr, nbat, ntimes, nvec, nhead, npiece, hcoef)
+            if mask:
+                VMath.set_mh_attention_mask(dev, probs.ptr, nbat, ntimes, nhead, True)
+            VMath.softmax_direct_on_axis(dev, probs.ptr, nbat * ntimes, ntimes, nhead)
+            VMath.mix_values(dev, mixed.ptr, probs.ptr, V.ptr, nbat, ntimes, nvec, nhead, npiece)
         VMath.matmul(dev, y.ptr, Ow.ptr, mixed.ptr, nvec, n, nvec, False)
         VMath.add_bias(dev, y.ptr, y.ptr, Ob.ptr, n, nvec)
         y.saved = {"op": "mh_attention", "x": x, "key": key, "query": query, "value": value, "Kw": Kw, "Qw": Qw, "Vw": Vw,
@@ -181,8 +188,9 @@ class Tensor:
         return y
 
     # vtensor.cpp:3054-3195 (the math calls; gradient registration is the engine's business)
-    def mh_attention_backprop(self, ygrad):
-        """Returns the 16 gradients by name.  ``g["x"]`` is the gradient of the tensor the operator was called on:
+    def mh_attention_backprop(self, ygrad, fused=False):
+        """Returns the 16 gradients by name (15 with ``fused=True``: one kai_attention_backward replaces the five or
+        six calls between the projections, and the gradient of the probabilities is never formed).  ``g["x"]`` is the gradient of the tensor the operator was called on:
         zero, plus the gradient of each of key / query / value that IS that tensor (self-attention,
         vtensor.cpp:3168-3195).  The reference's set_zero there passes an element count where bytes are meant
         and clears a quarter of the buffer; the whole buffer is cleared here."""
@@ -201,15 +209,21 @@ class Tensor:
         VMath.add_bias_backward_b(dev, g["Ob"].ptr, gy, n, nvec, False)
         VMath.matmul_backward_w(dev, g["Ow"].ptr, gy, s["mixed"].ptr, nvec, n, nvec, False)
         VMath.matmul_backward_x(dev, g["mixed"].ptr, gy, s["Ow"].ptr, nvec, n, nvec, False)
-        VMath.mix_values_backward_prop(dev, g["probs"].ptr, g["mixed"].ptr, s["V"].ptr, nbat, ntimes, nvec, nhead,
-                                       npiece)
-        VMath.mix_values_backward_value(dev, g["V"].ptr, g["mixed"].ptr, s["probs"].ptr, nbat, ntimes, nvec, nhead,
-                                        npiece)
-        VMath.softmax_direct_on_axis_backward(dev, g["probs"].ptr, s["probs"].ptr, nbat, ntimes, nhead, s["coef"])
-        if s["mask"]:
-            VMath.set_mh_attention_mask(dev, g["probs"].ptr, nbat, ntimes, nhead, False)
-        VMath.mult_on_heads_backward(dev, g["K"].ptr, g["probs"].ptr, s["Q"].ptr, nbat, ntimes, nvec, nhead, npiece)
-        VMath.mult_on_heads_backward(dev, g["Q"].ptr, g["probs"].ptr, s["K"].ptr, nbat, ntimes, nvec, nhead, npiece)
+        if fused:
+            del g["probs"]
+            VMath.attention_backward(dev, g["Q"].ptr, g["K"].ptr, g["V"].ptr, g["mixed"].ptr, s["probs"].ptr,
+                                     s["mixed"].ptr, s["Q"].ptr, s["K"].ptr, s["V"].ptr, nbat, ntimes, nvec, nhead,
+                                     npiece, s["coef"], s["mask"])
+        else:
+            VMath.mix_values_backward_prop(dev, g["probs"].ptr, g["mixed"].ptr, s["V"].ptr, nbat, ntimes, nvec, nhead,
+                                           npiece)
+            VMath.mix_values_backward_value(dev, g["V"].ptr, g["mixed"].ptr, s["probs"].ptr, nbat, ntimes, nvec, nhead,
+                                            npiece)
+            VMath.softmax_direct_on_axis_backward(dev, g["probs"].ptr, s["probs"].ptr, nbat, ntimes, nhead, s["coef"])
+            if s["mask"]:
+                VMath.set_mh_attention_mask(dev, g["probs"].ptr, nbat, ntimes, nhead, False)
+            VMath.mult_on_heads_backward(dev, g["K"].ptr, g["probs"].ptr, s["Q"].ptr, nbat, ntimes, nvec, nhead, npiece)
+            VMath.mult_on_heads_backward(dev, g["Q"].ptr, g["probs"].ptr, s["K"].ptr, nbat, ntimes, nvec, nhead, npiece)
         VMath.add_bias_backward_b(dev, g["Kb"].ptr, g["K"].ptr, n, nvec, False)
         VMath.add_bias_backward_b(dev, g["Qb"].ptr, g["Q"].ptr, n, nvec, False)
         VMath.add_bias_backward_b(dev, g["Vb"].ptr, g["V"].ptr, n, nvec, False)

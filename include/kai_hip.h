@@ -219,6 +219,15 @@ int kai_gemm_f32(int device, int transA, int transB, int64_t M, int64_t N, int64
 int kai_gemm_plan(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                   int has_bias, int actFunc, int acc, char* out, int buflen);
 
+/* No counterpart in the reference.  A maintainer's override of the dispatcher's choice for every later single
+ * (unbatched) product of the process, for audits of the fitted dispatch rules (bench.py --plan-audit times the
+ * chosen plan of a shape against every alternative): words in `text`, a tile name ("large", "medium", "small", "flat",
+ * "wide") and / or "split N" (N = 1 .. 16 parts of the reduction), or "wavesplit 16" / "wavesplit 32" (the one-launch
+ * kernel for small products, where it applies); "auto", "" or null clears the override.  A part count that the
+ * product cannot take runs as one part.  kai_gemm_plan reports what would run.  Process-wide and not synchronised
+ * with calls in flight on other threads: not for production use. */
+int kai_gemm_force_plan(const char* text);
+
 /* The engine's `dense` layer formula activate(add(matmul(x,w),b)) (api/vconst.cpp:11) in one launch:
  * py = act(x . w^T + b).  ppre, if not null, receives the pre-activation x . w^T + b that
  * VTensor::activate_backprop needs (vtensor.cpp:5697-5718).  pb may be null (no bias). */
@@ -322,17 +331,25 @@ int kai_eval_adam_delta(int device, float* pa, const float* pg, float* ps, float
  * mix_values(softmax_direct_on_axis(mask(mult_on_heads(K, Q, coef))), V), i.e. the middle of
  * VTensor::mh_attention (vtensor.cpp:3036-3043), without materialising the
  * [nbat, ntimes, ntimes, nhead] tensor (training needs that tensor and keeps the separate calls).
- * masked != 0 applies the causal mask of set_mh_attention_mask.  Head sizes 16, 32 and 64 with
- * 16-byte aligned operands run fused; any other shape runs the four separate kernels with the
+ * masked != 0 applies the causal mask of set_mh_attention_mask.  Head sizes that are multiples of 16 up to 128 with
+ * nhead * npiece == nvec and 16-byte aligned operands run fused; any other shape runs the four separate kernels with the
  * probabilities in the library's scratch memory.  The softmax is renormalised tile by tile, so the
  * result equals the separate calls up to rounding. */
 int kai_attention_forward(int device, float* py, const float* pQ, const float* pK, const float* pV, int64_t nbat,
                           int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hCoef,
                           int masked);
 
+/* No counterpart in the reference.  Writes into `out` how the attention entry points would run this geometry with
+ * 16-byte aligned operands, as text: which = 0 kai_attention_forward ("fused" or "separate"), 1
+ * kai_attention_forward_train ("fused", "fused, four heads per workgroup" or "separate"), 2 kai_attention_backward
+ * ("fused rows + value gradient" or "separate").  Host arithmetic only, nothing is launched and no GPU is needed.
+ * For maintainers and tests. */
+int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, char* out,
+                       int buflen);
+
 /* The same block for training: pp[nbat, ntimes, ntimes, nhead] also receives the probabilities, as the separate
  * calls leave them (masked keys exactly 0), for the backward pass (VTensor::mh_attention keeps them,
- * vtensor.cpp:3005, 3048).  One launch for head sizes 16, 32 and 64 with nhead * npiece == nvec, 16-byte aligned
+ * vtensor.cpp:3005, 3048).  One launch for head sizes that are multiples of 16 up to 128 with nhead * npiece == nvec, 16-byte aligned
  * operands and ntimes <= 1024 (a wave keeps the scores of its queries in registers between the maximum and the
  * stores); any other shape runs the four separate kernels.  Equal to the separate calls up to rounding. */
 int kai_attention_forward_train(int device, float* py, float* pp, const float* pQ, const float* pK, const float* pV,

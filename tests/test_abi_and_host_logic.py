@@ -302,3 +302,53 @@ def test_gemm_plan_checks_its_arguments():
     assert L.kai_gemm_plan(0, 1, 4, 4, 4, 4, 4, 4, 0, 9, 0, buf, 64) != 0        # softmax is no element-wise code
     assert L.kai_gemm_plan(0, 1, 4, 4, 4, 4, 4, 4, 0, 0, 0, None, 64) != 0       # null output
     assert L.kai_gemm_plan(0, 1, 4, 4, 4, 4, 4, 4, 0, 0, 0, buf, 4) == 0 and len(buf.value) == 3   # truncated, terminated
+
+
+def test_attention_plans():
+    """Which geometries the one-launch attention kernels take (host arithmetic, no GPU)."""
+    plan = kai.VMath.attention_plan
+    # both mappings of configuration 4
+    assert plan("forward", 32, 512, 64, 1, 64) == "fused"
+    assert plan("forward", 4, 512, 512, 8, 64) == "fused"
+    assert plan("forward_train", 32, 512, 64, 1, 64) == "fused"
+    assert plan("forward_train", 4, 512, 512, 8, 64) == "fused, four heads per workgroup"
+    assert plan("backward", 32, 512, 64, 1, 64) == "fused rows + value gradient"
+    assert plan("backward", 4, 512, 512, 8, 64) == "fused rows + value gradient"
+    # head sizes 96 and 128, twelve heads of 64, lengths that are no multiple of 32, six heads
+    for nbat, ntimes, nhead, npiece in ((2, 384, 12, 64), (1, 500, 16, 96), (2, 1024, 8, 128), (3, 200, 6, 32)):
+        nvec = nhead * npiece
+        assert plan("forward", nbat, ntimes, nvec, nhead, npiece) == "fused"
+        assert plan("forward_train", nbat, ntimes, nvec, nhead, npiece).startswith("fused")
+        assert plan("backward", nbat, ntimes, nvec, nhead, npiece) == "fused rows + value gradient"
+    # what the one-launch kernels leave to the separate ones: head sizes that are no multiple of 16 or beyond 128,
+    # heads that do not fill the vector, the training forward beyond 1024 keys
+    assert plan("forward", 2, 100, 48, 2, 24) == "separate"
+    assert plan("forward", 1, 64, 256, 1, 256) == "separate"
+    assert plan("forward", 2, 70, 80, 2, 32) == "separate"
+    assert plan("forward_train", 1, 1100, 64, 1, 64) == "separate"
+    assert plan("forward", 1, 1100, 64, 1, 64) == "fused"
+    assert plan("backward", 1, 64, 24, 1, 24) == "separate"
+    assert plan("backward", 0, 64, 64, 1, 64) == "nothing"
+
+
+def test_gemm_plan_override_for_audits():
+    """kai_gemm_force_plan: a maintainer's override of tile and part count, visible through kai_gemm_plan."""
+    V = kai.VMath
+    auto = V.gemm_plan(0, 1, 144, 4096, 4096)
+    try:
+        V.gemm_force_plan("small split 4")
+        assert V.gemm_plan(0, 1, 144, 4096, 4096) == "mfma small ragged pipelined staged 4 split 4"
+        V.gemm_force_plan("wavesplit 32")
+        assert V.gemm_plan(0, 1, 64, 512, 784) == "wavesplit 32"
+        assert V.gemm_plan(0, 1, 144, 4096, 4096) == auto          # outside that kernel's range: the choice stands
+        V.gemm_force_plan("medium")
+        assert V.gemm_plan(0, 1, 4, 4096, 4096).startswith("mfma medium")   # also where the skinny kernels would run
+        V.gemm_force_plan("flat split 16")
+        assert V.gemm_plan(0, 1, 144, 4096, 4096).endswith("split 16")
+        assert V.gemm_plan(0, 1, 144, 4096, 300).endswith("split 1")        # 16 parts of 300 steps: not offered
+        with pytest.raises(kai.KaiError) as e:
+            V.gemm_force_plan("bogus")
+        assert e.value.code == 510
+    finally:
+        V.gemm_force_plan(None)
+    assert V.gemm_plan(0, 1, 144, 4096, 4096) == auto
