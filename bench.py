@@ -199,6 +199,17 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
         lambda: L.kai_dense_forward(0, P(o8), None, P(w8), P(b8), P(x8), I(n8), I(n8), I(n8), kai.ACT["gelu"], None), iters=10,
         flops=f8)
     del x8, w8, b8, o8
+    # a product whose operands and output (1.5 GiB) exceed the 256 MB last-level cache: the HBM-side traffic of the
+    # 256 x 256 tiling is priced against HBM here (the summary under profiles/ holds the counters)
+    mb, nb, kb_ = 16384, 16384, 4096
+    xb = torch.rand((mb, kb_), device=dev, generator=g) * 2 - 1
+    wb = torch.rand((nb, kb_), device=dev, generator=g) * 2 - 1
+    bb = torch.randn(nb, device=dev, generator=g)
+    ob = torch.empty((mb, nb), device=dev)
+    row("16384 x 16384 x 4096 NT  Y = relu(X.W^T + b), operands and output beyond the last-level cache (kai_dense_forward)",
+        lambda: L.kai_dense_forward(0, P(ob), None, P(wb), P(bb), P(xb), I(nb), I(mb), I(kb_), relu, None), iters=5,
+        flops=2.0 * mb * nb * kb_)
+    del xb, wb, bb, ob
     # cfg1: dense forward 64 x 784 -> 512, fused
     x = torch.randn((64, 784), device=dev, generator=g)
     w = (torch.rand((512, 784), device=dev, generator=g) * 2 - 1) / 28.0

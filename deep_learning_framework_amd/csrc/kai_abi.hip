@@ -36,14 +36,29 @@ int check_launch(const char* kernel_name) { return check_hip(hipGetLastError(), 
 namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_ws_mutex;
-// Per device: the current scratch buffer and the smaller ones it replaced.  A replaced buffer is kept until
-// kai_shutdown: kernels already enqueued (on any stream) and HIP graphs that recorded its address stay valid,
-// and growing needs neither a wait for the device nor a hipFree (which waits, too).  Growth at least doubles
-// the size, so the retired buffers together are smaller than the current one.
-struct DeviceScratch {
+// Per device: one scratch buffer per STREAM that calls of the library have been enqueued on (the stream a thread
+// set with kai_set_stream; the null stream counts as one), so that calls on different streams of a device never
+// share partial sums, and the smaller buffers that grown ones replaced.  A replaced buffer is only retired: kernels
+// already enqueued that use it stay valid, and growing needs neither a wait for the device nor a hipFree (which
+// waits for the device, too).  Retired buffers are released at the library's own synchronisation points, when the
+// device is idle anyway (kai_device_synchronize, kai_shutdown) -- except those that were handed out while a stream
+// capture was active: a recorded graph keeps the address and may be replayed at any later time, so they stay until
+// kai_shutdown.  Growth at least doubles the size, so the retired buffers of a stream together are smaller than
+// its current one.
+struct StreamScratch {
+    hipStream_t stream = nullptr;
     void* ptr = nullptr;
     int64_t bytes = 0;
-    std::vector<void*> retired;
+    bool in_graph = false;     // handed out during a capture
+};
+struct RetiredScratch {
+    void* ptr;
+    int64_t bytes;
+    bool in_graph;
+};
+struct DeviceScratch {
+    std::vector<StreamScratch> streams;
+    std::vector<RetiredScratch> retired;
     int64_t retired_bytes = 0;
     int64_t growths = 0;
 };
@@ -52,11 +67,21 @@ int g_cu_count[kMaxDevices] = {};
 // bytes at the front of the scratch that an enclosing call of this thread holds (ScratchHold)
 thread_local int64_t tl_ws_held = 0;
 constexpr int64_t kScratchMin = 4ll << 20;
+constexpr size_t kMaxScratchStreams = 64;
 
-int grow_scratch(DeviceScratch& s, int64_t need) {
-    // an allocation is not allowed while the stream records a graph: the caller sizes the scratch first
+bool stream_is_capturing(hipStream_t st) {
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(current_stream(), &capturing) == hipSuccess && capturing != hipStreamCaptureStatusNone)
+    const hipError_t st_rc = hipStreamIsCapturing(st, &capturing);
+    if (st_rc != hipSuccess) {
+        (void)hipGetLastError();   // e.g. the query of the null stream while another stream records: not this call's error
+        return false;
+    }
+    return capturing != hipStreamCaptureStatusNone;
+}
+
+int grow_scratch(DeviceScratch& d, StreamScratch& s, int64_t need, bool capturing) {
+    // an allocation is not allowed while the stream records a graph: the caller sizes the scratch first
+    if (capturing)
         return fail(KAI_ERR_GPU, "the library scratch would have to grow to " + std::to_string(need) +
                                      " bytes while the stream is being captured: run the call once before the "
                                      "capture or call kai_reserve_scratch");
@@ -66,13 +91,24 @@ int grow_scratch(DeviceScratch& s, int64_t need) {
     void* fresh = nullptr;
     KAI_TRY(check_hip(hipMalloc(&fresh, (size_t)want), "hipMalloc(scratch)"));
     if (s.ptr) {
-        s.retired.push_back(s.ptr);
-        s.retired_bytes += s.bytes;
+        d.retired.push_back(RetiredScratch{s.ptr, s.bytes, s.in_graph});
+        d.retired_bytes += s.bytes;
     }
     s.ptr = fresh;
     s.bytes = want;
-    s.growths++;
+    s.in_graph = false;
+    d.growths++;
     return KAI_OK;
+}
+
+// the device is idle: every retired buffer that no recorded graph may still name goes back
+void release_retired(DeviceScratch& d) {
+    std::vector<RetiredScratch> kept;
+    for (const RetiredScratch& r : d.retired) {
+        if (r.in_graph || hipFree(r.ptr) != hipSuccess) kept.push_back(r);
+        else d.retired_bytes -= r.bytes;
+    }
+    d.retired.swap(kept);
 }
 }  // namespace
 
@@ -81,11 +117,25 @@ int workspace(int64_t bytes, float** out) {
     KAI_TRY(check_hip(hipGetDevice(&dev), "hipGetDevice"));
     if (dev < 0 || dev >= kMaxDevices) return fail(KAI_ERR_INVALID_ARGUMENT, "workspace: device index out of range");
     if (bytes < 0) return fail(KAI_ERR_INVALID_ARGUMENT, "workspace: negative size");
+    const hipStream_t st = current_stream();
+    const bool capturing = stream_is_capturing(st);
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    DeviceScratch& s = g_ws[dev];
+    DeviceScratch& d = g_ws[dev];
+    StreamScratch* s = nullptr;
+    for (StreamScratch& e : d.streams)
+        if (e.stream == st) s = &e;
+    if (s == nullptr) {
+        if (d.streams.size() >= kMaxScratchStreams)
+            return fail(KAI_ERR_INVALID_ARGUMENT, "workspace: more than 64 streams of one device have asked for scratch memory; "
+                                                  "kai_shutdown releases the buffers of streams that are gone");
+        d.streams.push_back(StreamScratch{});
+        s = &d.streams.back();
+        s->stream = st;
+    }
     const int64_t need = tl_ws_held + bytes;
-    if (s.bytes < need) KAI_TRY(grow_scratch(s, need));
-    *out = reinterpret_cast<float*>(static_cast<char*>(s.ptr) + tl_ws_held);
+    if (s->bytes < need) KAI_TRY(grow_scratch(d, *s, need, capturing));
+    if (capturing) s->in_graph = true;
+    *out = reinterpret_cast<float*>(static_cast<char*>(s->ptr) + tl_ws_held);
     return KAI_OK;
 }
 
@@ -110,17 +160,26 @@ static int release_workspaces() {
     int rc = KAI_OK;
     for (int d = 0; d < kMaxDevices; d++) {
         DeviceScratch& s = g_ws[d];
-        if (!s.ptr && s.retired.empty()) continue;
+        if (s.streams.empty() && s.retired.empty()) continue;
         if (hipSetDevice(d) == hipSuccess) {
             (void)hipDeviceSynchronize();
-            if (s.ptr && hipFree(s.ptr) != hipSuccess) rc = KAI_ERR_GPU;
-            for (void* p : s.retired)
-                if (hipFree(p) != hipSuccess) rc = KAI_ERR_GPU;
+            for (const StreamScratch& e : s.streams)
+                if (e.ptr && hipFree(e.ptr) != hipSuccess) rc = KAI_ERR_GPU;
+            for (const RetiredScratch& r : s.retired)
+                if (hipFree(r.ptr) != hipSuccess) rc = KAI_ERR_GPU;
         }
         s = DeviceScratch();
     }
     (void)hipSetDevice(old);
     return rc;
+}
+
+// after a successful wait for the current device
+static void release_retired_of_current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    release_retired(g_ws[dev]);
 }
 
 static bool act_is_elementwise(int act) { return act >= KAI_ACT_NONE && act <= KAI_ACT_SWISH; }
@@ -146,7 +205,11 @@ int kai_device_count(int* count) {
 
 int kai_set_device(int device) { return check_hip(hipSetDevice(device), "hipSetDevice"); }
 
-int kai_device_synchronize(void) { return check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
+int kai_device_synchronize(void) {
+    KAI_TRY(check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize"));
+    release_retired_of_current_device();   // the device is idle: scratch buffers that grown ones replaced go back
+    return KAI_OK;
+}
 
 int kai_set_stream(void* hip_stream) {
     tl_stream = reinterpret_cast<hipStream_t>(hip_stream);
@@ -170,7 +233,11 @@ int kai_scratch_info(int64_t* bytes, int64_t* growths, int64_t* retired_bytes) {
     KAI_TRY(check_hip(hipGetDevice(&dev), "hipGetDevice"));
     KAI_REQUIRE(dev >= 0 && dev < kMaxDevices, KAI_ERR_INVALID_ARGUMENT, "device index out of range");
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (bytes) *bytes = g_ws[dev].bytes;
+    if (bytes) {
+        *bytes = 0;
+        for (const StreamScratch& e : g_ws[dev].streams)
+            if (e.stream == current_stream()) *bytes = e.bytes;
+    }
     if (growths) *growths = g_ws[dev].growths;
     if (retired_bytes) *retired_bytes = g_ws[dev].retired_bytes;
     return KAI_OK;

@@ -24,12 +24,14 @@ int check_hip(hipError_t st, const char* what);
 int check_launch(const char* kernel_name);
 
 // Library-owned scratch memory on the CURRENT device (partial sums of a reduction cut into parts, row norms,
-// the probabilities of an attention call that runs as separate kernels).  Allocated on first use and released
-// by kai_shutdown.  When a call needs more than there is, a larger buffer is allocated and the old one is
-// kept until kai_shutdown, so growth never waits for the device and pointers handed out earlier (to
-// kernels in flight, to recorded graphs) stay valid.  While a stream capture is active, growth is refused
-// with an error.  Every call returns the front of the same buffer: calls that use it must be ordered on one
-// stream per device (the engine runs one thread and the null stream per device).
+// the probabilities of an attention call that runs as separate kernels), one buffer per stream that calls are
+// enqueued on (the calling thread's stream, kai_set_stream): calls on different streams of a device never share
+// it.  Allocated on first use and released by kai_shutdown.  When a call needs more than there is, a larger
+// buffer is allocated and the old one is retired -- kept, so that growth never waits for the device and
+// pointers handed out earlier (to kernels in flight, to recorded graphs) stay valid -- until the device is
+// idle at one of the library's own synchronisation points (kai_device_synchronize, kai_shutdown); buffers
+// handed out during a stream capture stay until kai_shutdown.  While a stream capture is active, growth is
+// refused with an error.  Every call on a stream returns the front of that stream's buffer.
 int workspace(int64_t bytes, float** out);
 // While an object of this type lives, workspace() calls of the same thread return memory BEHIND the first
 // `bytes` bytes of the scratch: for a call that keeps data in the scratch across inner calls which may ask

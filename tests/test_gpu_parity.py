@@ -240,6 +240,24 @@ def test_cfg3_size_backward_products_sampled_and_adjoint():
     assert abs(s_y - s_x) <= 1e-5 * scale and abs(s_y - s_w) <= 1e-5 * scale, (s_y, s_x, s_w, scale)
 
 
+def test_product_beyond_the_last_level_cache_row_sample():
+    # 16384 x 16384 x 4096: operands and output (1.5 GiB) exceed the 256 MB last-level cache, so every tile's
+    # operands come from HBM; sampled rows against the oracle, bias + ReLU fused
+    m, n, k = 16384, 16384, 4096
+    rng = np.random.default_rng(16)
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    w = rng.uniform(-1, 1, (n, k)).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    dx, dw, db = dev(x), dev(w), dev(b)
+    y = DB(m * n * 4)
+    VMath.dense_forward(0, y, None, dw, db, dx, n, m, k, kai.ACT["relu"], None)
+    got = y.to_numpy((m, n))
+    rows = np.unique(np.concatenate([[0, m - 1, 255, 256], rng.integers(0, m, 12)]))
+    ref = ko.activate(ko.add_bias(ko.matmul_rows(w, x, rows), b), "relu")
+    check(got[rows], ref, what="16384 x 16384 x 4096 sampled rows")
+    assert (got >= 0).all()
+
+
 # ---- configuration 4: attention batched matmul ---------------------------------------------------------------
 
 @pytest.mark.parametrize("nbat,nhead,nvec", [(32, 1, 64), (4, 8, 512)])
@@ -967,6 +985,69 @@ def test_split_k_scratch_survives_shutdown_and_growth():
     split_k(1024, 1024, 8192)
     attention_with_scratch()
     assert kai.scratch_info()[1] == n_growths and kai.scratch_info()[0] >= 48 << 20
+
+
+def test_split_k_products_on_two_streams_at_once_and_retired_scratch_returns():
+    # Each stream that calls are enqueued on has a scratch buffer of its own: products cut along K that run on two
+    # streams of the device at the same time do not share partial sums.  Buffers that grown ones replaced go back
+    # when the device is idle at kai_device_synchronize, without kai_shutdown.
+    import ctypes
+    kai.load()
+    hip = ctypes.CDLL("libamdhip64.so.7")        # the runtime the library itself is linked to, already loaded
+    hip.hipStreamCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+    hip.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+
+    def new_stream():
+        h = ctypes.c_void_p()
+        assert hip.hipStreamCreateWithFlags(ctypes.byref(h), 1) == 0      # hipStreamNonBlocking
+        return h.value
+
+    rng = np.random.default_rng(123)
+    kai.synchronize()
+    kai.shutdown()
+    s1, s2 = new_stream(), new_stream()
+    shapes = {s1: (256, 512, 16384), s2: (192, 384, 12288)}
+    data, outs = {}, {}
+    for st, (m, n, k) in shapes.items():
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+        data[st] = (x, w, dev(x), dev(w))
+        outs[st] = [DB(m * n * 4) for _ in range(6)]
+        assert int(VMath.gemm_plan(0, 1, m, n, k).rsplit(" ", 1)[1]) >= 8       # many parts: a long second launch each
+    kai.synchronize()
+    try:
+        for i in range(6):                      # alternating: the two streams' kernels overlap on the device
+            for st, (m, n, k) in shapes.items():
+                kai.set_stream(st)
+                x, w, dx, dw = data[st]
+                VMath.matmul(0, outs[st][i], dw, dx, n, m, k, False)
+        sizes = {}
+        for st in shapes:
+            kai.set_stream(st)
+            sizes[st] = kai.scratch_info()[0]
+        assert all(v >= 4 << 20 for v in sizes.values())     # a buffer per stream
+        # a larger product on the first stream: its buffer grows, the old one is retired, nothing waits
+        kai.set_stream(s1)
+        big = DB(1024 * 1024 * 4)
+        xb = rng.standard_normal((1024, 8192)).astype(np.float32)
+        wb = rng.uniform(-0.05, 0.05, (1024, 8192)).astype(np.float32)
+        VMath.matmul(0, big, dev(wb), dev(xb), 1024, 1024, 8192, False)
+        assert kai.scratch_info()[2] == sizes[s1]            # retired, not freed
+    finally:
+        kai.set_stream(None)
+    kai.synchronize()                                        # the device is idle: the retired buffer goes back
+    assert kai.scratch_info()[2] == 0
+    for st, (m, n, k) in shapes.items():
+        x, w, _, _ = data[st]
+        rows = list(range(0, m, 16))
+        ref = ko.matmul_rows(w, x, rows)
+        for i in range(6):
+            check(outs[st][i].to_numpy((m, n))[rows], ref, what="split-K on its own stream, call %d, %dx%dx%d" % (i, m, n, k))
+    rows = list(range(0, 1024, 64))
+    check(big.to_numpy((1024, 1024))[rows], ko.matmul_rows(wb, xb, rows), what="split-K after the growth")
+    kai.shutdown()
+    for st in (s1, s2):
+        assert hip.hipStreamDestroy(st) == 0
 
 
 # products cut along K whose outputs are larger than one capped element-wise grid covers (4096 workgroups x 256
