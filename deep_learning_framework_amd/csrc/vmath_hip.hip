@@ -138,6 +138,14 @@ void VMath::attention_forward(int device, float* py, float* pQ, float* pK, float
 void VMath::dense_forward(int device, float* py, float* ppre, float* pw, float* pb, float* px, int64 yvec, int64 ndat, int64 xvec, int actFunc, HYPER h) {
     raise_on(kai_dense_forward(device, py, ppre, pw, pb, px, yvec, ndat, xvec, actFunc, h));
 }
+void VMath::attention_forward_train(int device, float* py, float* pp, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked) {
+    raise_on(kai_attention_forward_train(device, py, pp, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked ? 1 : 0));
+}
+
+void VMath::attention_backward(int device, float* pgQ, float* pgK, float* pgV, float* pgm, float* pp, float* pm, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked) {
+    raise_on(kai_attention_backward(device, pgQ, pgK, pgV, pgm, pp, pm, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked ? 1 : 0));
+}
+
 void VMath::dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pga_work, float* pgy, float* pw, float* px, float* ppre, int64 yvec, int64 ndat, int64 xvec, int actFunc, HYPER h, bool acc) {
     raise_on(kai_dense_backward(device, pgx, pgw, pgb, pga_work, pgy, pw, px, ppre, yvec, ndat, xvec, actFunc, h, acc));
 }

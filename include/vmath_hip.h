@@ -100,6 +100,8 @@ public:
     static void apply_decay(int device, float* pd, float* pp, float* pg, int64 nrow, HYPER hL1Decay, HYPER hL2Decay);
     static void eval_adam_delta(int device, float* pa, float* pg, float* ps, float* pt, float* pn, int64 nrow, HYPER hRo1, HYPER hRo2, HYPER hEpsilon);
     static void attention_forward(int device, float* py, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked);
+    static void attention_forward_train(int device, float* py, float* pp, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked);
+    static void attention_backward(int device, float* pgQ, float* pgK, float* pgV, float* pgm, float* pp, float* pm, float* pQ, float* pK, float* pV, int64 nbat, int64 ntimes, int64 nvec, int64 nhead, int64 npiece, HYPER hCoef, bool masked);
     static void dense_forward(int device, float* py, float* ppre, float* pw, float* pb, float* px, int64 yvec, int64 ndat, int64 xvec, int actFunc, HYPER hLeakyAlpha);
     static void dense_backward(int device, float* pgx, float* pgw, float* pgb, float* pga_work, float* pgy, float* pw, float* px, float* ppre, int64 yvec, int64 ndat, int64 xvec, int actFunc, HYPER hLeakyAlpha, bool acc);
 };
