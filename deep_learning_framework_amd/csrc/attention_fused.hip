@@ -365,50 +365,86 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
         const int c = tid + i * kFaThreads;
         choff[i] = ((c / kChunksPerKey) * (int)p.nvec + (c % kChunksPerKey) * 4) * 4;
     }
-    f32x4 rt[NCH];
-    auto load_tile = [&](const __amdgpu_buffer_rsrc_t& rsrc, int kt) {
-#pragma unroll
-        for (int i = 0; i < NCH; i++) {
-            const int c = tid + i * kFaThreads;
-            if (!kPartial || c < kTileChunks)
-                rt[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, choff[i], kt * tile_bytes, 0));
-        }
+    // Staging registers of the tiles on their way, two sets: while tile kt is at work, tile kt + 1 (requested a tile
+    // earlier) moves to LDS and tile kt + 2 is requested.  The loads are dealt out over the groups of products of a
+    // tile instead of being issued together (issued together they fill the address unit's queue and every wave
+    // waits at its next load), the LDS stores sit in the group before the last, the barrier before the last group,
+    // whose operands are in registers by then and whose products cover the first LDS reads of the next tile; the
+    // LDS reads of a group are issued before the products of the group before it.  Fences keep the order.
+    f32x4 rt[2][NCH];
+    auto load_one = [&](auto setc, auto jc, const __amdgpu_buffer_rsrc_t& rsrc, int kt) {
+        constexpr int set = decltype(setc)::value, j = decltype(jc)::value;
+        const int c = tid + j * kFaThreads;
+        if (!kPartial || c < kTileChunks)
+            rt[set][j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, choff[j], kt * tile_bytes, 0));
     };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < NCH; i++) {
-            const int c = tid + i * kFaThreads;
-            if (!kPartial || c < kTileChunks)
-                *reinterpret_cast<f32x4*>(&lds_t[buf][(c / kChunksPerKey) * kStride + (c % kChunksPerKey) * 4]) = rt[i];
-        }
+    auto store_one = [&](auto setc, auto jc, int buf) {
+        constexpr int set = decltype(setc)::value, j = decltype(jc)::value;
+        const int c = tid + j * kFaThreads;
+        if (!kPartial || c < kTileChunks)
+            *reinterpret_cast<f32x4*>(&lds_t[buf][(c / kChunksPerKey) * kStride + (c % kChunksPerKey) * 4]) = rt[set][j];
     };
+    auto load_all = [&](auto setc, const __amdgpu_buffer_rsrc_t& rsrc, int kt) {
+        static_for<0, NCH>([&](auto jc) { load_one(setc, jc, rsrc, kt); });
+    };
+    auto store_all = [&](auto setc, int buf) {
+        static_for<0, NCH>([&](auto jc) { store_one(setc, jc, buf); });
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
 
     // ---- scores of every key tile into registers: sc[kt][kb][v] = (query q, key 64*kt + 32*kgp + 16*kb + 4*g + v) -----
+    // groups of 8 products: one 16-wide slice s of the head dimension, both key blocks
     f32x4 sc[NT][2];
-    load_tile(rsrc_k, 0);
-    store_tile(0);
+    f32x4 kf[2][2];      // operands of a group, double buffered by group parity
+    auto stage_k = [&](auto parc, int s, int buf) {
+        constexpr int par = decltype(parc)::value;
+        const float* lk = lds_t[buf] + 32 * kgp * kStride + hd * D;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+            kf[par][kb] = *reinterpret_cast<const f32x4*>(lk + (16 * kb + r16) * kStride + 16 * s + 4 * g);
+    };
+    constexpr int kLoadGroups1 = DB > 1 ? DB - 1 : 1;                      // groups that carry the loads of tile kt + 2
+    constexpr int kLPG1 = (NCH + kLoadGroups1 - 1) / kLoadGroups1;
+    constexpr int kStoreGroup1 = DB > 1 ? DB - 2 : 0;                       // the group that moves tile kt + 1 to LDS
+    load_all(I0{}, rsrc_k, 0);
+    load_all(I1{}, rsrc_k, min(1, nkt - 1));
+    store_all(I0{}, 0);
     __syncthreads();
+    stage_k(I0{}, 0, 0);
     static_for<0, NT>([&](auto ktc) {
         constexpr int kt = decltype(ktc)::value;
         if (kt < nkt) {
             constexpr int buf = kt & 1;
-            load_tile(rsrc_k, min(kt + 1, nkt - 1));   // unconditional: a load behind a branch is waited for at once; the surplus one is never stored
+            using SetNow = std::integral_constant<int, kt & 1>;          // held tile kt, free now: receives tile kt + 2
+            using SetNext = std::integral_constant<int, (kt + 1) & 1>;   // holds tile kt + 1
             const int key0 = kt * kFaKeys + 32 * kgp;
-            const float* lk = lds_t[buf] + 32 * kgp * kStride + hd * D;
+            const int kt2 = min(kt + 2, nkt - 1);                         // past the end: a surplus load, never stored
             sc[kt][0] = f32x4{0.f, 0.f, 0.f, 0.f};
             sc[kt][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < DB; s++) {
-                f32x4 kf[2];
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++)
-                    kf[kb] = *reinterpret_cast<const f32x4*>(lk + (16 * kb + r16) * kStride + 16 * s + 4 * g);
+            static_for<0, DB>([&](auto sc_) {
+                constexpr int s = decltype(sc_)::value;
+                constexpr int par = (kt * DB + s) & 1;
+                using ParNext = std::integral_constant<int, par ^ 1>;
+                if constexpr (s == kStoreGroup1) store_all(SetNext{}, buf ^ 1);
+                if constexpr (s + 1 < DB) {
+                    stage_k(ParNext{}, s + 1, buf);
+                } else {
+                    __syncthreads();     // tile kt + 1 is in LDS, and every wave has read tile kt
+                    if (kt + 1 < nkt) stage_k(ParNext{}, 0, buf ^ 1);
+                }
+                static_for<0, kLPG1>([&](auto lc) {
+                    constexpr int j = s * kLPG1 + decltype(lc)::value;
+                    if constexpr (j < NCH && (s < kLoadGroups1)) load_one(SetNow{}, std::integral_constant<int, j>{}, rsrc_k, kt2);
+                });
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int e = 0; e < 4; e++)
 #pragma unroll
                     for (int kb = 0; kb < 2; kb++)
-                        sc[kt][kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[kb][e], qf[s][e], sc[kt][kb], 0, 0, 0);
-            }
+                        sc[kt][kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[par][kb][e], qf[s][e], sc[kt][kb], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            });
             const bool edge_tile = key0 + 32 > T || (p.masked && key0 + 31 > q0 + 16 * qg);   // wave-uniform
             if (edge_tile) {
 #pragma unroll
@@ -419,15 +455,14 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
                         if (key >= T || (p.masked && key > q)) sc[kt][kb][v] = -INFINITY;
                     }
             }
-            if (kt + 1 < nkt) store_tile(buf ^ 1);
-            __syncthreads();
         } else {
             sc[kt][0] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
             sc[kt][1] = sc[kt][0];
         }
     });
-    // the first tile of V is on its way while the softmax runs
-    load_tile(rsrc_v, 0);
+    // the first two tiles of V are on their way while the softmax runs
+    load_all(I0{}, rsrc_v, 0);
+    load_all(I1{}, rsrc_v, min(1, nkt - 1));
 
     // ---- maximum, exponentials, sum: in registers; the two key halves exchange through LDS ---------------------------
     float m = -INFINITY;
@@ -457,78 +492,122 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
     l += __shfl_xor(l, 32);
     __syncthreads();                                  // every wave has read the maxima
     lds_x[kgp][w4 * 64 + lane] = l;
-    store_tile(0);                                    // V tile 0 (the K tiles are done with)
+    store_all(I0{}, 0);                               // V tile 0 (the K tiles are done with)
     __syncthreads();
     l += lds_x[kgp ^ 1][w4 * 64 + lane];
     const float rl = 1.0f / l;
 
     // ---- probabilities stored, and multiplied into the output tile by tile -------------------------------------------
+    // groups of 2 * DB products: two key columns e of one key block kb
     f32x4 acc_o[DB];
 #pragma unroll
     for (int db = 0; db < DB; db++) acc_o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float vfl[2][2][DB];
+    auto stage_v = [&](auto parc, int gi, int buf) {
+        constexpr int par = decltype(parc)::value;
+        const float* lv = lds_t[buf] + 32 * kgp * kStride + hd * D;
+        const int kb = gi >> 1, e0 = 2 * (gi & 1);
+#pragma unroll
+        for (int ee = 0; ee < 2; ee++) {
+            const float* vp = lv + (16 * kb + 4 * g + e0 + ee) * kStride + r16;
+#pragma unroll
+            for (int db = 0; db < DB; db++) vfl[par][ee][db] = vp[16 * db];
+        }
+    };
+    constexpr int kLPG2 = (NCH + 1) / 2;     // the loads of tile kt + 2 over groups 0 and 1, the stores of tile kt + 1 in group 2
     float* Pq = pp.P + (int64_t)b * pp.p_batch_stride + ((int64_t)qc * T) * H + h0 + hd;   // P[b, q, 0, h]
+    // the probabilities of a tile: masked keys hold exp(-inf) = 0 exactly, also in the tiles above the diagonal
+    auto store_p_direct = [&](const f32x4 (&pr)[2], int key0) {
+        if (q < T) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const int key = key0 + 16 * kb + 4 * g;
+                if (PVEC) {
+                    if (key < T) *reinterpret_cast<f32x4*>(Pq + key) = pr[kb];
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (key + v < T) Pq[(int64_t)(key + v) * H] = pr[kb][v];
+                }
+            }
+        }
+    };
+    // four heads per workgroup: this wave's head of (query r16, keys 32*kgp + 16*kb + 4*g + 0..3) into its plane of the
+    // exchange buffer, one 128-bit write per key block (written as the fourth part of 4-float groups, the 64 lanes
+    // of a write would share 8 banks); after a barrier a lane stores the four heads of a (query, key) as one word
+    auto exchange_write = [&](const f32x4 (&pr)[2]) {
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+            *reinterpret_cast<f32x4*>(&lds_p[hd * kPPlane + r16 * kPStride + 32 * kgp + 16 * kb + 4 * g]) = pr[kb];
+    };
+    auto exchange_store = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < 16 * kFaKeys / kFaThreads; i++) {
+            const int idx = tid + i * kFaThreads;
+            const int qq = idx / kFaKeys, kk = idx % kFaKeys;
+            const int key = kt * kFaKeys + kk;
+            const float* src = &lds_p[qq * kPStride + kk];
+            const f32x4 w = {src[0], src[kPPlane], src[2 * kPPlane], src[3 * kPPlane]};
+            if (q0 + qq < T && key < T)
+                *reinterpret_cast<f32x4*>(pp.P + (int64_t)b * pp.p_batch_stride + (((int64_t)(q0 + qq) * T + key) * H + h0)) = w;
+        }
+    };
+    stage_v(I0{}, 0, 0);
     static_for<0, NT>([&](auto ktc) {
         constexpr int kt = decltype(ktc)::value;
         if (kt < nkt_all) {
             constexpr int buf = kt & 1;
+            using SetNow = std::integral_constant<int, kt & 1>;
+            using SetNext = std::integral_constant<int, (kt + 1) & 1>;
             const int key0 = kt * kFaKeys + 32 * kgp;
             f32x4 pr[2];
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) pr[kb] = sc[kt][kb] * rl;
-            if (HG == 4) {
-                // this wave's head of (query r16, keys 32*kgp + 16*kb + 4*g + 0..3) into its plane of the exchange
-                // buffer: one 128-bit write per key block (written as the fourth part of 4-float groups, the 64 lanes
-                // of a write would share 8 banks)
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++)
-                    *reinterpret_cast<f32x4*>(&lds_p[hd * kPPlane + r16 * kPStride + 32 * kgp + 16 * kb + 4 * g]) = pr[kb];
-            }
             if (kt < nkt) {
-                load_tile(rsrc_v, min(kt + 1, nkt - 1));
-                if (key0 < T && !(p.masked && key0 > q_last)) {
-                    const float* lv = lds_t[buf] + 32 * kgp * kStride + hd * D;
-#pragma unroll
-                    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const float* vp = lv + (16 * kb + 4 * g + e) * kStride + r16;
-#pragma unroll
-                            for (int db = 0; db < DB; db++)
-                                acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(vp[16 * db], pr[kb][e], acc_o[db], 0, 0, 0);
-                        }
-                }
-            }
-            // the probabilities of this tile: masked keys hold exp(-inf) = 0 exactly, also in the tiles above the diagonal
-            if (HG == 4) {
-                __syncthreads();   // the four heads of every (query, key) of the tile are in the exchange buffer
-#pragma unroll
-                for (int i = 0; i < 16 * kFaKeys / kFaThreads; i++) {
-                    const int idx = tid + i * kFaThreads;
-                    const int qq = idx / kFaKeys, kk = idx % kFaKeys;
-                    const int key = kt * kFaKeys + kk;
-                    const float* src = &lds_p[qq * kPStride + kk];
-                    const f32x4 w = {src[0], src[kPPlane], src[2 * kPPlane], src[3 * kPPlane]};
-                    if (q0 + qq < T && key < T)
-                        *reinterpret_cast<f32x4*>(pp.P + (int64_t)b * pp.p_batch_stride + (((int64_t)(q0 + qq) * T + key) * H + h0)) = w;
-                }
-            } else if (q < T) {
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++) {
-                    const int key = key0 + 16 * kb + 4 * g;
-                    if (PVEC) {
-                        if (key < T) *reinterpret_cast<f32x4*>(Pq + key) = pr[kb];
-                    } else {
-#pragma unroll
-                        for (int v = 0; v < 4; v++)
-                            if (key + v < T) Pq[(int64_t)(key + v) * H] = pr[kb][v];
+                const int kt2 = min(kt + 2, nkt - 1);
+                static_for<0, 4>([&](auto gc) {
+                    constexpr int gi = decltype(gc)::value;
+                    constexpr int par = gi & 1;
+                    using ParNext = std::integral_constant<int, par ^ 1>;
+                    if constexpr (gi == 0) {
+                        if (HG == 4) exchange_write(pr);
+                        else store_p_direct(pr, key0);
                     }
-                }
-            }
-            if (kt < nkt) {
-                if (kt + 1 < nkt) store_tile(buf ^ 1);
-                __syncthreads();
+                    if constexpr (gi == 2) {
+                        store_all(SetNext{}, buf ^ 1);
+                        if (HG == 4) {
+                            __syncthreads();   // the four heads of every (query, key) of the tile are in the exchange buffer
+                            exchange_store(kt);
+                        }
+                    }
+                    if constexpr (gi < 3) {
+                        stage_v(ParNext{}, gi + 1, buf);
+                    } else {
+                        __syncthreads();       // tile kt + 1 is in LDS, every wave has read tile kt (and the exchange buffer)
+                        if (kt + 1 < nkt) stage_v(ParNext{}, 0, buf ^ 1);
+                    }
+                    if constexpr (gi < 2) {
+                        static_for<0, kLPG2>([&](auto lc) {
+                            constexpr int j = gi * kLPG2 + decltype(lc)::value;
+                            if constexpr (j < NCH) load_one(SetNow{}, std::integral_constant<int, j>{}, rsrc_v, kt2);
+                        });
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    constexpr int kb = gi >> 1, e0 = 2 * (gi & 1);
+#pragma unroll
+                    for (int ee = 0; ee < 2; ee++)
+#pragma unroll
+                        for (int db = 0; db < DB; db++)
+                            acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(vfl[par][ee][db], pr[kb][e0 + ee], acc_o[db], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             } else if (HG == 4) {
+                exchange_write(pr);
+                __syncthreads();
+                exchange_store(kt);
                 __syncthreads();   // the exchange buffer is free again
+            } else {
+                store_p_direct(pr, key0);
             }
         }
     });
@@ -610,7 +689,9 @@ static void launch_probs(const ProbsParams& p, bool pvec, int64_t ntimes, dim3 g
         if (kVecOk && pvec) attention_probs_kernel<DB, 8, HG, kVecOk><<<grid, block, 0, stream>>>(p);
         else attention_probs_kernel<DB, 8, HG, false><<<grid, block, 0, stream>>>(p);
     } else if constexpr (!(HG == 4 && DB == 4)) {
-        if (kVecOk && pvec) attention_probs_kernel<DB, 16, HG, kVecOk><<<grid, block, 0, stream>>>(p);
+        // (head sizes above 96 with more than 512 keys: the variant with 128-bit stores of P does not fit its
+        // registers; one head per batch entry stores its probabilities element by element there)
+        if (kVecOk && pvec && DB <= 6) attention_probs_kernel<DB, 16, HG, (kVecOk && DB <= 6)><<<grid, block, 0, stream>>>(p);
         else attention_probs_kernel<DB, 16, HG, false><<<grid, block, 0, stream>>>(p);
     }
 }

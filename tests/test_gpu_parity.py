@@ -867,7 +867,8 @@ def test_attention_forward_fused(nbat, ntimes, nhead, npiece, masked):
                                                       (1, 1, 1, 16), (2, 300, 1, 32), (1, 1024, 1, 16), (1, 1030, 2, 32),
                                                       (2, 257, 1, 64), (1, 640, 4, 64), (3, 33, 5, 16),
                                                       (2, 384, 12, 64), (1, 500, 16, 96), (1, 1024, 8, 128),
-                                                      (3, 200, 6, 32), (1, 300, 4, 48), (1, 100, 1, 128)])
+                                                      (3, 200, 6, 32), (1, 300, 4, 48), (1, 100, 1, 128), (1, 512, 2, 128),
+                                                      (1, 700, 2, 96), (1, 600, 1, 128)])
 def test_attention_forward_train(nbat, ntimes, nhead, npiece):
     nvec = nhead * npiece
     plan = VMath.attention_plan("forward_train", nbat, ntimes, nvec, nhead, npiece)
