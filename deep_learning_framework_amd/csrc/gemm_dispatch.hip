@@ -41,6 +41,7 @@ struct ForcedPlan {
     int tile = -1;          // kTile* or -1: keep the chosen tile
     int64_t split = 0;      // >= 1: this many parts; 0: keep the chosen number
     int wavesplit = 0;      // 16 or 32: the wave-split kernel with blocks of that edge
+    int stream_rows = 0;    // 16, 32 or 48: rows of W per workgroup of the skinny streaming kernel (does not force a tile)
 };
 ForcedPlan g_forced;
 
@@ -393,7 +394,8 @@ bool valid_dims(const GemmDesc& d) {
 }  // namespace
 
 // "auto" (or empty) clears the override; otherwise words: a tile name (large, medium, small, flat, wide), and / or
-// "split N" (1 .. 16), or "wavesplit 16" / "wavesplit 32".
+// "split N" (1 .. 16), or "wavesplit 16" / "wavesplit 32"; "stream 16" / "stream 32" / "stream 48" only sets the rows
+// of W per workgroup of the skinny streaming kernel for the products that kernel takes anyway.
 int set_forced_gemm_plan(const char* text) {
     ForcedPlan f;
     std::string t = text ? text : "";
@@ -410,15 +412,17 @@ int set_forced_gemm_plan(const char* text) {
         bool known = false;
         for (int i = 0; i < 5; i++)
             if (w == tiles[i]) { f.tile = i; f.active = known = true; }
-        if (w == "split" || w == "wavesplit") {
+        if (w == "split" || w == "wavesplit" || w == "stream") {
             const std::string n = next();
             const long v = n.empty() ? -1 : strtol(n.c_str(), nullptr, 10);
             if (w == "split" && v >= 1 && v <= kSplitMax) { f.split = v; f.active = known = true; }
             if (w == "wavesplit" && (v == 16 || v == 32)) { f.wavesplit = (int)v; f.active = known = true; }
+            if (w == "stream" && (v == 16 || v == 32 || v == 48)) { f.stream_rows = (int)v; known = true; }
         }
         if (!known) return fail(KAI_ERR_INVALID_ARGUMENT, "gemm plan override: cannot read \"" + w + "\"");
     }
     g_forced = f;
+    set_skinny_stream_rows_override(f.stream_rows);
     return KAI_OK;
 }
 
@@ -438,7 +442,13 @@ std::string describe_gemm(const GemmDesc& d) {
     if (plan.wavesplit_edge) return "wavesplit " + std::to_string(plan.wavesplit_edge);
     if (!plan.forced) {
         if (skinny_rows_applies(plan.dn)) return "skinny rows";
-        if (plan.skinny) return "skinny";
+        if (plan.skinny) {
+            // the streaming kernel with workgroups of 32 or 48 rows of W says so
+            SkinnyParams sp{};
+            sp.W = d.B; sp.X = d.A; sp.ldw = d.b_rs; sp.ldx = d.a_rs; sp.N = d.N; sp.M = (int)d.M; sp.K = (int)d.K;
+            const int wide = skinny_stream_wide_rows(sp);
+            return wide ? "skinny stream " + std::to_string(wide) : "skinny";
+        }
         if (shortk_nt_applies(plan.dn)) return "shortk_nt";
         if (shortk_heads_applies(plan.dn)) return "shortk_heads";
         if (heads_pv_applies(d)) return "heads_pv";

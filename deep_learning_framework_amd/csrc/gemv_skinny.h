@@ -50,5 +50,7 @@ bool skinny_stream32_applies(const SkinnyParams& p);   // 17..32 rows
 bool skinny_stream8_applies(const SkinnyParams& p);    // workgroups of 8 rows of W
 int launch_skinny_stream8(const SkinnyParams& p, hipStream_t stream);
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream);
+int skinny_stream_wide_rows(const SkinnyParams& p);    // 32 or 48 rows of W per workgroup, 0 = workgroups of 16 rows
+void set_skinny_stream_rows_override(int rows);        // audits: 16, 32 or 48 rows of W per workgroup, 0 = the rule
 
 }  // namespace kai

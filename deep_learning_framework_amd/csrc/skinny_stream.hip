@@ -79,17 +79,27 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // cuts K over workgroups and sums the parts in a second launch.
 //
 // WR: rows of W per workgroup, 16, or 8 (whole tiles only) where workgroups of 16 rows would not cover the compute
-// units: the second half of the W tile then stays zero and only eight columns of the result are stored.
+// units: the second half of the W tile then stays zero and only eight columns of the result are stored.  32 and 48
+// (whole tiles, written-out slices) where N / WR workgroups still cover the compute units: every workgroup loads
+// all of X whatever it owns of W, and through the same load paths, so at 16 rows of W the tiles of X are as many
+// bytes as those of W (twice as many with two blocks of X rows) and the compute unit's load path, not HBM, sets
+// the time; with two or three blocks of W rows a tile of X meets two or three tiles of W.  The last workgroup may
+// own fewer blocks (N a multiple of 16): the rows behind N lie behind the end of its resource and read as zero.
 template <bool WHOLE, bool SLICES, int XL = 0, int XB = 1, int WR = 16>
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
     const SkinnyParams p = skinny_params(W, X, ldw, ldx, N, M, K, Y, t);
-    __shared__ __attribute__((aligned(16))) float lds_w[kSsWaves][16 * kSsTileStride];
+    constexpr int WB = WR <= 16 ? 1 : WR / 16;      // blocks of 16 rows of W
+    constexpr int kWTileRows = 16 * WB;
+    __shared__ __attribute__((aligned(16))) float lds_w[kSsWaves][kWTileRows * kSsTileStride];
     static_assert(XB == 1 || (XB == 2 && WHOLE && SLICES && XL > kSsLoadsPerTile && XL <= 2 * kSsLoadsPerTile),
                   "two blocks of X rows exist for whole tiles in written-out slices");
-    static_assert(WR == 16 || (WR == 8 && WHOLE && XB == 1 && kSsRowsPerLoad == 8), "eight rows of W: one load per tile");
+    static_assert(WR == 16 || (WR == 8 && WHOLE && XB == 1 && kSsRowsPerLoad == 8) ||
+                      ((WR == 32 || WR == 48) && WHOLE && SLICES && XL > 0),
+                  "eight rows of W: one load per tile; 32 and 48: whole tiles in written-out slices");
     constexpr int kWLoads = WR / kSsRowsPerLoad;    // 128-bit loads per lane that cover the workgroup's rows of a W tile
+    constexpr int kWRegs = kWLoads > kSsLoadsPerTile ? kWLoads : kSsLoadsPerTile;
     constexpr int kXLoads = kSsLoadsPerTile * XB;   // 128-bit loads per lane that cover a tile of X
     __shared__ __attribute__((aligned(16))) float lds_x[kSsWaves][16 * XB * kSsTileStride];
 
@@ -112,9 +122,11 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     for (int j = 0; j < kXLoads; j++)
         *reinterpret_cast<f32x4*>(tx + (kSsRowsPerLoad * j + lrow) * kSsTileStride + lk) = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    f32x4 acc[XB];
+    f32x4 acc[WB][XB];
 #pragma unroll
-    for (int b = 0; b < XB; b++) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int a = 0; a < WB; a++)
+#pragma unroll
+        for (int b = 0; b < XB; b++) acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
     // One tile = 16 rows x kSsTileK k of W and of X, kSsLoadsPerTile 128-bit loads per lane each.  Addresses past
     // K are clamped into the row (every load is unconditional); what they return is zeroed on the way to LDS.
     // WHOLE: resources and per-lane offsets (bytes)
@@ -124,20 +136,25 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
         return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
     };
+    const int w_rows = WR > 16 ? (int)min((int64_t)WR, p.N - n0) : WR;   // rows of W this workgroup has (uniform)
     const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
-        uniform_ptr(p.W + n0 * p.ldw), 0, (int)(((int64_t)(WR - 1) * p.ldw + p.K) * 4), 0x00020000);
+        uniform_ptr(p.W + n0 * p.ldw), 0, (int)(((int64_t)(w_rows - 1) * p.ldw + p.K) * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
         uniform_ptr(p.X), 0, (int)(((int64_t)(p.M - 1) * p.ldx + p.K) * 4), 0x00020000);
-    int woff[kSsLoadsPerTile], xoff[kXLoads];
+    int woff[kWRegs], xoff[kXLoads];
 #pragma unroll
-    for (int j = 0; j < kSsLoadsPerTile; j++) woff[j] = (int)(((int64_t)(kSsRowsPerLoad * j + lrow) * p.ldw + lk) * 4);
+    for (int j = 0; j < kWRegs; j++) {
+        // a row past the workgroup's last must land behind the end of the resource whatever ldw is
+        const int row = kSsRowsPerLoad * j + lrow;
+        woff[j] = WR > 16 && row >= w_rows ? 0x7FFFFFF0 : (int)(((int64_t)row * p.ldw + lk) * 4);
+    }
 #pragma unroll
     for (int j = 0; j < kXLoads; j++) {
         // a row past M must land behind the end of the resource whatever ldx is: the last row's end is the limit
         const int m = kSsRowsPerLoad * j + lrow;
         xoff[j] = m < p.M ? (int)(((int64_t)m * p.ldx + lk) * 4) : 0x7FFFFFF0;
     }
-    auto load_w = [&](f32x4(&dst)[kSsLoadsPerTile], int kt) {
+    auto load_w = [&](f32x4(&dst)[kWRegs], int kt) {
         if constexpr (WHOLE) {
             // a tile past the end of K (a wave's last slice may be short) re-reads the last whole tile instead of
             // counting on the range check for the scalar part of the address; it is never consumed
@@ -171,7 +188,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
             }
         }
     };
-    auto consume = [&](const f32x4(&w)[kSsLoadsPerTile], const f32x4(&x)[kXLoads], int kt) {
+    auto consume = [&](const f32x4(&w)[kWRegs], const f32x4(&x)[kXLoads], int kt) {
         if ((SLICES && XL) || kt < p.K) {   // uniform
 #pragma unroll
             for (int j = 0; j < kWLoads; j++) {
@@ -189,12 +206,31 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
             __builtin_amdgcn_wave_barrier();   // LDS serves a wave's accesses in order; the compiler must too
 #pragma unroll
             for (int s = 0; s < kSsTileK / 16; s++) {
-                const f32x4 wv = *reinterpret_cast<const f32x4*>(tw + r * kSsTileStride + 16 * s + 4 * g);
+                if constexpr (WB == 1) {
+                    const f32x4 wv = *reinterpret_cast<const f32x4*>(tw + r * kSsTileStride + 16 * s + 4 * g);
 #pragma unroll
-                for (int b = 0; b < XB; b++) {
-                    const f32x4 xv = *reinterpret_cast<const f32x4*>(tx + (16 * b + r) * kSsTileStride + 16 * s + 4 * g);
+                    for (int b = 0; b < XB; b++) {
+                        const f32x4 xv = *reinterpret_cast<const f32x4*>(tx + (16 * b + r) * kSsTileStride + 16 * s + 4 * g);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[e], wv[e], acc[b], 0, 0, 0);
+                        for (int e = 0; e < 4; e++)
+                            acc[0][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[e], wv[e], acc[0][b], 0, 0, 0);
+                    }
+                } else {
+                    // all operands of the 16 steps first, then the products with the accumulators taking turns
+                    f32x4 wv[WB], xv[XB];
+#pragma unroll
+                    for (int a = 0; a < WB; a++)
+                        wv[a] = *reinterpret_cast<const f32x4*>(tw + (16 * a + r) * kSsTileStride + 16 * s + 4 * g);
+#pragma unroll
+                    for (int b = 0; b < XB; b++)
+                        xv[b] = *reinterpret_cast<const f32x4*>(tx + (16 * b + r) * kSsTileStride + 16 * s + 4 * g);
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+#pragma unroll
+                        for (int a = 0; a < WB; a++)
+#pragma unroll
+                            for (int b = 0; b < XB; b++)
+                                acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[b][e], wv[a][e], acc[a][b], 0, 0, 0);
                 }
             }
             __builtin_amdgcn_wave_barrier();
@@ -210,7 +246,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         // lengths unchanged).  At 4096 steps the plain order is the faster one (12.1 against 12.4 us).
         const int stag = p.K >= 8192 ? 2 * wave : 0;
         for (int k0 = wave * kSlice; k0 < p.K; k0 += kSsWaves * kSlice) {
-            f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kXLoads];
+            f32x4 w[kSsRing][kWRegs], x[kSsRing][kXLoads];
             ss_static_for<0, kSsRing>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
                 load_w(w[t], k0 + ((t + stag) & (kTiles - 1)) * kSsTileK);
@@ -240,7 +276,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         const int tiles_base = tiles_total / kSsWaves, tiles_rem = tiles_total % kSsWaves;
         const int t_count = tiles_base + (wave < tiles_rem ? 1 : 0);
         const int k_begin = (wave * tiles_base + min(wave, tiles_rem)) * kSsTileK;
-        f32x4 w[kSsRing][kSsLoadsPerTile], x[kSsRing][kXLoads];
+        f32x4 w[kSsRing][kWRegs], x[kSsRing][kXLoads];
         ss_static_for<0, kSsRing>([&](auto tc) {
             constexpr int t = decltype(tc)::value;
             load_w(w[t], k_begin + t * kSsTileK);
@@ -268,21 +304,27 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         });
     }
 
-    // acc[b][v] = D[m = 16 * b + 4 * g + v][n = n0 + r]; the tiles are free now: wave w parks its result in its W tile
-    static_assert(256 * XB <= 16 * kSsTileStride, "a wave's results fit its W tile");
+    // acc[a][b][v] = D[m = 16 * b + 4 * g + v][n = n0 + 16 * a + r]; the tiles are free now: wave w parks its
+    // results in its W tile, a 16 x 16 block per (a, b)
+    static_assert(256 * XB * WB <= kWTileRows * kSsTileStride, "a wave's results fit its W tile");
     __syncthreads();
 #pragma unroll
-    for (int b = 0; b < XB; b++)
+    for (int a = 0; a < WB; a++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) tw[(16 * b + 4 * g + v) * 16 + r] = acc[b][v];
+        for (int b = 0; b < XB; b++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) tw[((a * XB + b) * 16 + 4 * g + v) * 16 + r] = acc[a][b][v];
     __syncthreads();
-    if (tid < 256 * XB) {
-        const int m = tid >> 4, j = tid & 15;
-        const int64_t n = n0 + j;
-        if (m < p.M && n < p.N && j < WR) {
+#pragma unroll
+    for (int i0 = 0; i0 < 256 * XB * WB; i0 += kSsThreads) {
+        const int e = i0 + tid;
+        const int blk = e >> 8, a = blk / XB, b = blk % XB;
+        const int m = 16 * b + ((e >> 4) & 15), j = e & 15;
+        const int64_t n = n0 + 16 * a + j;
+        if (e < 256 * XB * WB && m < p.M && n < p.N && j < WR) {
             float v = 0.f;
 #pragma unroll
-            for (int i = 0; i < kSsWaves; i++) v += lds_w[i][tid];
+            for (int i = 0; i < kSsWaves; i++) v += lds_w[i][e];
             const float leaky = p.leaky ? *p.leaky : 0.f;
             const int64_t idx = (int64_t)m * p.ldy + n;
             if (p.accflag) v += p.Y[idx];
@@ -337,10 +379,56 @@ int launch_skinny_stream8(const SkinnyParams& p, hipStream_t stream) {
     return check_launch("skinny_stream_kernel");
 }
 
+namespace {
+int g_stream_rows_override = 0;
+
+template <int WR>
+int launch_wide(const SkinnyParams& p, const SkinnyTail& t, hipStream_t stream) {
+    const dim3 grid((unsigned)((p.N + WR - 1) / WR)), block(kSsThreads);
+    if (p.M <= 8) skinny_stream_kernel<true, true, 1, 1, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (p.M <= 16) skinny_stream_kernel<true, true, 2, 1, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (p.M <= 24) skinny_stream_kernel<true, true, 3, 2, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else skinny_stream_kernel<true, true, 4, 2, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    return check_launch("skinny_stream_kernel");
+}
+}  // namespace
+
+void set_skinny_stream_rows_override(int rows) { g_stream_rows_override = rows; }
+
+// Rows of W per workgroup where workgroups of 32 or 48 rows take the product, 0 where those of 16 rows keep it.
+// Fewer, larger workgroups load fewer bytes of X but leave a compute unit with one workgroup's eight waves, which
+// pull less through its load path than the sixteen of two resident 16-row workgroups; so they pay only from 9 rows
+// of X on, and only where their number fills the compute units.  Measured, us per call with W from HBM, 16-row
+// workgroups -> these (K = 4096): 11008 columns (230 workgroups of 48) 8 / 16 / 24 / 32 rows 29.6 / 33.9 / 40.8 / 45.4 ->
+// 29.5 / 29.9 / 34.8 / 36.4; 12288 (256 of 48) 31.0 / 34.7 / 41.9 / 47.2 -> 32.9 / 32.9 / 38.5 / 39.3; 32000 (667 of 48)
+// 16 rows 90.2 -> 84.8; 8192 (256 of 32) 16 / 24 / 32 rows 23.9 / 28.5 / 32.0 -> 28.2 / 28.9 / 29.8; 7168 (224 of 32)
+// 23.8 / 27.7 / 30.7 -> 25.1 / 26.5 / 27.8; 6144 (192 of 32) 22.9 / 26.5 / 29.9 -> 22.5 / 24.8 / 26.1; 16384 (342 of 48,
+// 512 of 32) 16 rows 45.6 -> 51.4 / 51.8.  Hence: 48 rows from 9 rows of X on where the workgroups fill their rounds
+// over the compute units to 85 %; 32 rows from 17 rows of X on where the workgroups are one round, at least three
+// quarters full.
+int skinny_stream_wide_rows(const SkinnyParams& p) {
+    if (g_stream_rows_override == 16) return 0;
+    const bool base = p.M > kSkinnyMaxRows ? skinny_stream32_applies(p) : (p.M >= 2 && skinny_stream_applies(p));
+    if (!base || p.K % (kSsWaves * 512) != 0 || p.N % 16 != 0 || (47 * p.ldw + p.K) * 4 >= (1ll << 31) ||
+        ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 >= 0x7FFFFFF0ll)
+        return 0;
+    if (g_stream_rows_override == 32 || g_stream_rows_override == 48) return g_stream_rows_override;
+    if (p.M <= 8) return 0;
+    const int64_t cus = compute_units();
+    const int64_t groups48 = (p.N + 47) / 48, rounds48 = (groups48 + cus - 1) / cus;
+    if (groups48 * 100 >= 85 * rounds48 * cus && (rounds48 == 1 || p.M <= kSkinnyMaxRows)) return 48;
+    const int64_t groups32 = (p.N + 31) / 32;
+    if (p.M > kSkinnyMaxRows && groups32 <= cus && groups32 * 4 >= 3 * cus) return 32;
+    return 0;
+}
+
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     const int64_t blocks = (p.N + 15) / 16;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
     const SkinnyTail t = skinny_tail(p);
+    const int wide = skinny_stream_wide_rows(p);
+    if (wide == 48) return launch_wide<48>(p, t, stream);
+    if (wide == 32) return launch_wide<32>(p, t, stream);
     // whole tiles, and byte offsets inside a workgroup's 16 rows of W and inside X that fit 31 bits
     const bool whole = p.N % 16 == 0 && p.K % kSsTileK == 0 && (15 * p.ldw + p.K) * 4 < (1ll << 31) &&
                        ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;

@@ -223,7 +223,9 @@ int kai_gemm_plan(int transA, int transB, int64_t M, int64_t N, int64_t K, int64
  * (unbatched) product of the process, for audits of the fitted dispatch rules (bench.py --plan-audit times the
  * chosen plan of a shape against every alternative): words in `text`, a tile name ("large", "medium", "small", "flat",
  * "wide") and / or "split N" (N = 1 .. 16 parts of the reduction), or "wavesplit 16" / "wavesplit 32" (the one-launch
- * kernel for small products, where it applies); "auto", "" or null clears the override.  A part count that the
+ * kernel for small products, where it applies); "stream 16" / "stream 32" / "stream 48" sets only the rows of W
+ * that a workgroup of the skinny streaming kernel owns, for the products that kernel takes anyway, and forces no
+ * tile; "auto", "" or null clears the override.  A part count that the
  * product cannot take runs as one part.  kai_gemm_plan reports what would run.  Process-wide and not synchronised
  * with calls in flight on other threads: not for production use. */
 int kai_gemm_force_plan(const char* text);

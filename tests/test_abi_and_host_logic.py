@@ -242,7 +242,12 @@ GEMM_PLANS = [
     ((0, 1, 1000, 333, 777), "mfma small ragged pipelined split 2"),   # configuration 5, ragged: two rounds of the one-launch kernel would take longer
     ((0, 1, 32, 4096, 5120), "mfma flat whole split 8"),             # 17..32 rows: the 32 x 128 tile
     ((0, 0, 17, 11008, 4096), "mfma flat ragged pipelined staged 2 split 2"),          # one workgroup per compute unit: 86 tiles x 2
-    ((0, 1, 17, 11008, 4096), "skinny"),
+    ((0, 1, 17, 11008, 4096), "skinny stream 48"),                   # 230 workgroups of 48 rows of W fill the compute units
+    ((0, 1, 16, 11008, 4096), "skinny stream 48"),                   # from 9 rows of X on
+    ((0, 1, 8, 11008, 4096), "skinny"),
+    ((0, 1, 32, 8192, 4096), "skinny stream 32"),                    # 256 workgroups of 32 rows, 17..32 rows of X only
+    ((0, 1, 16, 8192, 4096), "skinny"),
+    ((0, 1, 16, 16384, 4096), "skinny"),                             # 342 workgroups of 48: the second round a third full
     ((0, 0, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
     ((0, 1, 96, 4096, 4096), "mfma flat ragged pipelined split 8"),  # 65..96 rows: three row tiles of 32, not two of 64

@@ -400,8 +400,14 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # 17..32 rows on the streaming kernel: two blocks of 16 rows of X per tile of W
                                    (17, 4096, 4096), (24, 8192, 4112), (25, 4096, 4096), (32, 4096, 4096),
                                    # workgroups of 8 rows of W where those of 16 would not cover the compute units
-                                   (8, 4096, 2048), (16, 8192, 1024), (3, 4096, 1544), (2, 4096, 2048), (9, 12288, 1032)])
+                                   (8, 4096, 2048), (16, 8192, 1024), (3, 4096, 1544), (2, 4096, 2048), (9, 12288, 1032),
+                                   # workgroups of 48 and 32 rows of W where they fill the compute units (the last one
+                                   # of 11008 and of 7184 owns 16 rows)
+                                   (32, 4096, 11008), (16, 4096, 11008), (9, 4096, 12288), (24, 4096, 7184), (17, 4096, 6144)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
+    if n >= 6144:
+        want = "skinny stream %d" % (48 if n >= 11008 else 32)
+        assert VMath.gemm_plan(0, 1, m, n, k) == want
     rng = np.random.default_rng(m + k + n)
     w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
     x = rng.standard_normal((m, k)).astype(np.float32)
@@ -416,6 +422,35 @@ def test_skinny_shapes_bias_act_acc(m, k, n):
     ya = dev(y0)
     VMath.matmul(0, ya, dw, dx, n, m, k, True)
     check(ya.to_numpy((m, n)), ko.matmul(w, x, acc_into=y0), what="skinny acc")
+
+
+@pytest.mark.parametrize("rows", [32, 48])
+def test_skinny_stream_with_wide_workgroups_forced(rows):
+    # every variant of the streaming kernel with 32 / 48 rows of W per workgroup (one or two loads of X per tile, one
+    # or two blocks of X rows), on a matrix whose last workgroup owns fewer blocks, with padded rows, bias,
+    # activation and acc; the override is the audit hook, the dispatcher's own rule is asserted elsewhere
+    rng = np.random.default_rng(rows)
+    n, k, padw, padx = 4112, 4096, 4, 8
+    w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+    wp = np.full((n, k + padw), np.nan, np.float32); wp[:, :k] = w
+    bias = rng.standard_normal(n).astype(np.float32)
+    dwp, dbias = dev(wp), dev(bias)
+    try:
+        VMath.gemm_force_plan("stream %d" % rows)
+        for m in (2, 8, 9, 16, 17, 24, 25, 32):
+            assert VMath.gemm_plan(0, 1, m, n, k, k + padx, k + padw, n) == "skinny stream %d" % rows
+            x = rng.standard_normal((m, k)).astype(np.float32)
+            xp = np.full((m, k + padx), np.nan, np.float32); xp[:, :k] = x
+            y0 = rng.standard_normal((m, n)).astype(np.float32)
+            acc, act = bool(m % 2), ("tanh" if m % 3 == 0 else "relu")
+            y = dev(y0)
+            VMath.gemm_f32(0, 0, 1, m, n, k, dev(xp), k + padx, dwp, k + padw, y, n, dbias, kai.ACT[act], None, acc)
+            ref = ko.activate(ko.add_bias(ko.matmul(w, x, acc_into=y0 if acc else None), bias), act)
+            got = y.to_numpy((m, n))
+            assert np.isfinite(got).all(), m
+            check(got, ref, what="%d rows of X, workgroups of %d rows of W" % (m, rows))
+    finally:
+        VMath.gemm_force_plan("auto")
 
 
 @pytest.mark.parametrize("m,k,n", [(1, 4096, 4096), (4, 2500, 4100), (5, 2100, 1500), (9, 9000, 1024), (16, 3000, 1028),
@@ -1161,12 +1196,15 @@ def test_scratch_growth_does_not_wait_for_the_device():
     t_queued = time.perf_counter()
     VMath.matmul_backward_x(0, y, dgy, dw, k, m, nn, False)
     t_call = time.perf_counter()
+    grown = kai.scratch_info()                         # host bookkeeping only: does not wait either
     kai.synchronize()
     t_done = time.perf_counter()
     after = kai.scratch_info()
-    print("queueing %.1f ms, growing call %.2f ms, drain %.1f ms, scratch %s -> %s"
-          % ((t_queued - t0) * 1e3, (t_call - t_queued) * 1e3, (t_done - t_call) * 1e3, before, after))
-    assert after[1] == before[1] + 1 and after[0] >= 8 << 20 and after[2] == before[0]
+    print("queueing %.1f ms, growing call %.2f ms, drain %.1f ms, scratch %s -> %s -> %s"
+          % ((t_queued - t0) * 1e3, (t_call - t_queued) * 1e3, (t_done - t_call) * 1e3, before, grown, after))
+    # the old buffer is only retired while the queue may still use it, and goes back once the device is idle
+    assert grown[1] == before[1] + 1 and grown[0] >= 8 << 20 and grown[2] == before[0]
+    assert after[:2] == grown[:2] and after[2] == 0
     rows = list(range(0, m, 32))
     check(y.to_numpy((m, nn))[rows], ko.matmul_backward_x(gy[rows], w), what="product after growth")
     if (t_done - t_call) > 0.02:                       # the queue was still busy when the call returned
