@@ -94,15 +94,6 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     constexpr int NP = PVEC ? KB : 4 * KB;   // loads of P per lane and tile
     // [buffer][operand V, K, Q][tile]
     __shared__ __attribute__((aligned(16))) float lds[2][3][kTile];
-    // Without 128-bit loads of P (several heads: the values of a head lie 4 * nhead bytes apart) a load in the
-    // layout the products need would touch 64 cache lines, a row of P per lane.  The workgroup's 64 rows x kKeys
-    // values of a tile are loaded with the keys along the lanes instead (16 lines per load with 8 heads) and pass
-    // through LDS: [buffer][row][key], rows kPStride floats apart (8 modulo 32: the 128-bit reads are conflict-free).
-    constexpr bool PCOOP = !PVEC;
-    constexpr int kPStride = kKeys + 8;
-    constexpr int NPC = kAbRows * kKeys / kAbThreads;      // 32-bit loads of P per thread and tile
-    constexpr int kPRowsPerLoad = kAbThreads / kKeys;
-    __shared__ __attribute__((aligned(16))) float lds_p[PCOOP ? 2 * kAbRows * kPStride : 4];
     static_assert(8 * DB * 64 * kAbQGroups + 64 * kAbQGroups <= 6 * kTile, "the merge buffer must fit the tiles");
 
     const int tid = threadIdx.x;
@@ -158,25 +149,6 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
         const int key = 16 * KB * kgp + 4 * g + (PVEC ? 16 * i : 16 * (i / 4) + (i % 4));
         poff[i] = (int)((((int64_t)tc * T + key) * H) * 4);
     }
-
-    // the cooperative loads of P: value j of this thread is P[t0 + tid / kKeys + j * kPRowsPerLoad, key tid % kKeys]
-    int pcoff[PCOOP ? NPC : 1];
-    float pc[PCOOP ? NPC : 1];
-    if constexpr (PCOOP) {
-#pragma unroll
-        for (int j = 0; j < NPC; j++) {
-            const int row = min(t0 + tid / kKeys + j * kPRowsPerLoad, T - 1);   // rows past the end are clamped, never stored
-            pcoff[j] = (int)((((int64_t)row * T + tid % kKeys) * H) * 4);
-        }
-    }
-    auto load_pc = [&](auto jc, int kt) {
-        constexpr int j = decltype(jc)::value;
-        pc[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_p, pcoff[j], kt * p_tile_bytes, 0));
-    };
-    auto store_pc = [&](auto jc, int buf) {
-        constexpr int j = decltype(jc)::value;
-        lds_p[buf * (kAbRows * kPStride) + (tid / kKeys + j * kPRowsPerLoad) * kPStride + tid % kKeys] = pc[j];
-    };
 
     f32x4 rv[NCH], rk[NCH], rq[NCH];
     auto load_v = [&](int kt) {
@@ -357,23 +329,11 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     constexpr int kStoreGroups = (NLOAD + kStoresPerGroup - 1) / kStoresPerGroup;
     constexpr int kFirstStoreGroup = NG - 1 - kStoreGroups;                   // the last store is in group NG - 2
     static_assert(kFirstStoreGroup >= 1, "too many chunks for this schedule");
-    constexpr int kPcPerGroup = 2;
-    static_assert(!PCOOP || (NPC + kPcPerGroup - 1) / kPcPerGroup <= NG - 1, "the cooperative loads of P end before the barrier");
 
-    // P of a tile.  128-bit loads: requested a tile ahead, straight into the layout of the products.  Cooperative
-    // loads: requested TWO tiles ahead (tile kt + 2 during tile kt), stored during the tile after that into the
-    // buffer that tile kt's values have left (every wave has read them before the barrier that ended tile kt), read
-    // from LDS with the operands of the group that needs them.
-    f32x4 p_next[KB], pr[KB];
+    f32x4 p_next[KB];
     load_v(0);
     load_kq(0);
-    if constexpr (PCOOP) {
-        static_for<0, NPC>([&](auto jc) { load_pc(jc, 0); });
-        static_for<0, NPC>([&](auto jc) { store_pc(jc, 0); });
-        static_for<0, NPC>([&](auto jc) { load_pc(jc, min(1, nkt - 1)); });
-    } else {
-        load_p(p_next, 0);
-    }
+    load_p(p_next, 0);
     store_v(0);
     store_kq(0);
     __syncthreads();
@@ -390,11 +350,6 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
 #pragma unroll
             for (int kb = 0; kb < KB; kb++)
                 vf[par][kb] = *reinterpret_cast<const f32x4*>(lv + (16 * kb + r16) * kStride + 16 * i + 4 * g);
-            if constexpr (PCOOP && i == NA - 1) {
-                const float* lp = &lds_p[buf * (kAbRows * kPStride) + (16 * qg + r16) * kPStride + 16 * KB * kgp + 4 * g];
-#pragma unroll
-                for (int kb = 0; kb < KB; kb++) pr[kb] = *reinterpret_cast<const f32x4*>(lp + 16 * kb);
-            }
         } else {
             constexpr int kb = (i - NA) / 4, e = (i - NA) % 4;
             const float* lk = &lds[buf][1][16 * KB * kgp * kStride] + (16 * kb + 4 * g + e) * kStride + r16;
@@ -432,11 +387,9 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
         const int buf = kt & 1;
         const int nxt = min(kt + 1, nkt - 1);      // the surplus loads and stores of the last tile are never used
         const int key0 = kt * kKeys + 16 * KB * kgp;    // first key of this wave's part of the tile
-        const int nxt2 = min(kt + 2, nkt - 1);
-        if constexpr (!PCOOP) {
+        f32x4 pr[KB];
 #pragma unroll
-            for (int kb = 0; kb < KB; kb++) pr[kb] = p_next[kb];
-        }
+        for (int kb = 0; kb < KB; kb++) pr[kb] = p_next[kb];
         f32x4 part[KB][NCHAIN];
 #pragma unroll
         for (int kb = 0; kb < KB; kb++)
@@ -454,20 +407,10 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
                 if (kt + 1 < nkt) stage(std::integral_constant<int, 0>{}, buf ^ 1);
             }
             // -- this group's share of the next tile's traffic
-            if constexpr (PCOOP) {
-                // the values of P that arrived for the next tile go to LDS, their registers take the tile after it
-                static_for<0, kPcPerGroup>([&](auto lc) {
-                    constexpr int j = i * kPcPerGroup + decltype(lc)::value;
-                    if constexpr (j < NPC) {
-                        store_pc(std::integral_constant<int, j>{}, buf ^ 1);
-                        load_pc(std::integral_constant<int, j>{}, nxt2);
-                    }
-                });
-            }
             static_for<0, kLoadsPerGroup>([&](auto lc) {
                 constexpr int j = i * kLoadsPerGroup + decltype(lc)::value;
                 if constexpr (j < NLOAD) load_one(std::integral_constant<int, j>{}, nxt);
-                else if constexpr (j == NLOAD && !PCOOP) load_p(p_next, nxt);
+                else if constexpr (j == NLOAD) load_p(p_next, nxt);
             });
             if constexpr (i >= kFirstStoreGroup && i < NG - 1) {
                 static_for<0, kStoresPerGroup>([&](auto sc) {
@@ -563,11 +506,10 @@ bool attention_backward_applies(const float* gq, const float* gk, const float* g
            aligned16(q) && aligned16(k) && aligned16(v) && (reinterpret_cast<uintptr_t>(pp) & 3u) == 0;
 }
 
-// KBC: the key blocks per wave of the variant with cooperative loads of P, whose second LDS array must fit as well
-template <int DB, int KB, int KBC = KB>
+template <int DB, int KB>
 static void launch_rows(const AttnBwdParams& p, bool pvec, dim3 grid, hipStream_t stream) {
     if (pvec) attention_backward_rows_kernel<DB, KB, true><<<grid, dim3(kAbThreads), 0, stream>>>(p);
-    else attention_backward_rows_kernel<DB, KBC, false><<<grid, dim3(kAbThreads), 0, stream>>>(p);
+    else attention_backward_rows_kernel<DB, KB, false><<<grid, dim3(kAbThreads), 0, stream>>>(p);
 }
 
 int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const float* m, const float* pp,
@@ -588,7 +530,7 @@ int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const 
     case 2: launch_rows<2, 2>(p, pvec, grid, stream); break;
     case 3: launch_rows<3, 2>(p, pvec, grid, stream); break;
     case 4: launch_rows<4, 2>(p, pvec, grid, stream); break;
-    case 5: launch_rows<5, 2, 1>(p, pvec, grid, stream); break;
+    case 5: launch_rows<5, 2>(p, pvec, grid, stream); break;
     case 6: launch_rows<6, 1>(p, pvec, grid, stream); break;
     case 7: launch_rows<7, 1>(p, pvec, grid, stream); break;
     default: launch_rows<8, 1>(p, pvec, grid, stream); break;
