@@ -100,6 +100,12 @@ int launch_attention_probs(float* o, float* pp, const float* q, const float* k, 
                            int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
                            hipStream_t stream);
 
+// attention_value_grad.hip: gV = P^T.gY per (batch entry, head) without LDS passes of the operands; 0 = geometry not
+// served, else the heads a workgroup owns (1 or 4)
+int attention_value_grad_heads(const float* gv, const float* gy, const float* pp, int64_t ntimes, int64_t nvec,
+                               int64_t nhead, int64_t npiece);
+int launch_attention_value_grad(float* gv, const float* gy, const float* pp, int64_t nbat, int64_t ntimes, int64_t nvec,
+                                int64_t nhead, int64_t npiece, hipStream_t stream);
 // attention_backward.hip: gQ and gK of the attention block from gM, P (and M) without storing gP or gS
 bool attention_backward_applies(const float* gq, const float* gk, const float* gm, const float* m, const float* pp,
                                 const float* q, const float* k, const float* v, int64_t ntimes, int64_t nvec,

@@ -620,6 +620,8 @@ int kai_mix_values_backward_value(int device, float* pgV, const float* pgy, cons
     KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
     if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
     KAI_REQUIRE_PTR(pgV); KAI_REQUIRE_PTR(pgy); KAI_REQUIRE_PTR(pp);
+    if (attention_value_grad_heads(pgV, pgy, pp, ntimes, nvec, nhead, npiece))
+        return launch_attention_value_grad(pgV, pgy, pp, nbat, ntimes, nvec, nhead, npiece, current_stream());
     // per (b,h): gV[k,p] = sum_q P[b,q,k,h] * gY[b,q,h,p] : rows of the product are k, reduction over q
     GemmDesc d;
     d.A = pp; d.B = pgy; d.C = pgV;
@@ -911,7 +913,8 @@ int kai_gemm_force_plan(const char* text) { return set_forced_gemm_plan(text); }
 int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, char* out,
                        int buflen) {
     KAI_REQUIRE(out != nullptr && buflen > 0, KAI_ERR_INVALID_POINTER, "null output buffer");
-    KAI_REQUIRE(which >= 0 && which <= 2, KAI_ERR_INVALID_ARGUMENT, "which must be 0 (forward), 1 (forward, training) or 2 (backward)");
+    KAI_REQUIRE(which >= 0 && which <= 3, KAI_ERR_INVALID_ARGUMENT,
+                "which must be 0 (forward), 1 (forward, training), 2 (backward) or 3 (value gradient)");
     KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
     // 16-byte aligned operands are assumed: a pointer value that satisfies every alignment test
     const float* a = reinterpret_cast<const float*>(uintptr_t(256));
@@ -922,6 +925,10 @@ int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, in
         text = attention_probs_four_heads(a, ntimes, nhead, npiece) ? "fused, four heads per workgroup" : "fused";
     else if (which == 2 && attention_backward_applies(a, a, a, a, a, a, a, a, ntimes, nvec, nhead, npiece))
         text = "fused rows + value gradient";
+    else if (which == 3) {
+        const int hv = attention_value_grad_heads(a, a, a, ntimes, nvec, nhead, npiece);
+        text = hv == 1 ? "streamed, one head per workgroup" : hv == 4 ? "streamed, four heads per workgroup" : "tiled";
+    }
     snprintf(out, (size_t)buflen, "%s", text.c_str());
     return KAI_OK;
 }

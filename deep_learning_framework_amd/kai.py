@@ -434,10 +434,10 @@ class VMath:
     @staticmethod
     def attention_plan(which, nbat, ntimes, nvec, nhead, npiece):
         """How an attention entry point would run this geometry (host arithmetic only): which = "forward",
-        "forward_train" or "backward"."""
+        "forward_train", "backward" or "value_gradient"."""
         buf = ctypes.create_string_buffer(128)
-        _ck(load().kai_attention_plan({"forward": 0, "forward_train": 1, "backward": 2}[which], nbat, ntimes, nvec, nhead,
-                                      npiece, buf, 128))
+        code = {"forward": 0, "forward_train": 1, "backward": 2, "value_gradient": 3}[which]
+        _ck(load().kai_attention_plan(code, nbat, ntimes, nvec, nhead, npiece, buf, 128))
         return buf.value.decode()
 
     @staticmethod

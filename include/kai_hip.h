@@ -344,7 +344,9 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
 /* No counterpart in the reference.  Writes into `out` how the attention entry points would run this geometry with
  * 16-byte aligned operands, as text: which = 0 kai_attention_forward ("fused" or "separate"), 1
  * kai_attention_forward_train ("fused", "fused, four heads per workgroup" or "separate"), 2 kai_attention_backward
- * ("fused rows + value gradient" or "separate").  Host arithmetic only, nothing is launched and no GPU is needed.
+ * ("fused rows + value gradient" or "separate"), 3 kai_mix_values_backward_value, also the value gradient inside
+ * kai_attention_backward ("streamed, one head per workgroup", "streamed, four heads per workgroup" or "tiled").
+ * Host arithmetic only, nothing is launched and no GPU is needed.
  * For maintainers and tests. */
 int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, char* out,
                        int buflen);

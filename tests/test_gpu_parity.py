@@ -853,6 +853,39 @@ def test_attention_backward_one_call_when_the_heads_do_not_fill_the_vector():
     assert (gq.to_numpy(q.shape)[:, :, nhead * npiece:] == 0).all()
 
 
+# the value gradient on the kernel that streams P straight into the matrix cores' operand layout: every head size with
+# one head per workgroup, every head size up to 64 with four, lengths that leave the last block of keys and the last
+# step of four rows partly empty, a vector wider than the heads (columns beyond them stay untouched)
+@pytest.mark.parametrize("nbat,ntimes,nhead,npiece,extra", [
+    (2, 128, 1, 16, 0), (1, 200, 1, 32, 0), (2, 64, 1, 48, 0), (32, 512, 1, 64, 0), (1, 132, 1, 80, 0), (1, 260, 1, 96, 0),
+    (1, 96, 1, 112, 0), (2, 320, 1, 128, 0), (1, 100, 1, 64, 64),
+    (1, 77, 4, 16, 0), (2, 130, 8, 32, 0), (1, 97, 12, 48, 0), (4, 512, 8, 64, 0), (2, 384, 12, 64, 0), (1, 50, 4, 64, 32),
+    (1, 1030, 4, 32, 0)])
+def test_value_gradient_streamed(nbat, ntimes, nhead, npiece, extra):
+    nvec = nhead * npiece + extra
+    want = "streamed, %s per workgroup" % ("one head" if nhead == 1 else "four heads")
+    assert VMath.attention_plan("value_gradient", nbat, ntimes, nvec, nhead, npiece) == want
+    rng = np.random.default_rng(nbat * 1000 + ntimes + nhead + npiece)
+    p = rng.random((nbat, ntimes, ntimes, nhead), dtype=np.float32)
+    p /= p.sum(axis=2, keepdims=True)
+    gy = rng.standard_normal((nbat, ntimes, nhead * npiece)).astype(np.float32)
+    start = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    gv = dev(start)
+    VMath.mix_values_backward_value(0, gv, dev(gy), dev(p), nbat, ntimes, nvec, nhead, npiece)
+    got = gv.to_numpy((nbat, ntimes, nvec))
+    if nbat * ntimes * ntimes * nhead * npiece <= 1 << 28:
+        ref = ko.mix_values_backward_value(gy, p, nhead)
+        check(got[:, :, :nhead * npiece], ref, what="value gradient")
+    else:   # the large cases: the oracle on the first and the last batch entry
+        for b in (0, nbat - 1):
+            ref = ko.mix_values_backward_value(gy[b:b + 1], p[b:b + 1], nhead)
+            check(got[b:b + 1, :, :nhead * npiece], ref, what="value gradient, batch entry %d" % b)
+        f64 = np.matmul(p.astype(np.float64).transpose(0, 3, 2, 1),
+                        gy.reshape(nbat, ntimes, nhead, npiece).astype(np.float64).transpose(0, 2, 1, 3))   # [b, h, k, d]
+        assert rel_fro(got[:, :, :nhead * npiece], f64.transpose(0, 2, 1, 3).reshape(nbat, ntimes, -1)) <= REL_FRO_TOL
+    np.testing.assert_array_equal(got[:, :, nhead * npiece:], start[:, :, nhead * npiece:])
+
+
 # one case per kernel variant: rows in registers (1 head; 2..128 heads, short and long axis), rows through
 # LDS (long axis, odd lengths), one thread per head (more than 128 heads)
 SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8), (3, 20, 128), (2, 9, 129),
