@@ -317,7 +317,8 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
             L.kai_mult_on_heads_backward(0, P(gq), P(gp), P(k), I(nbat), I(T), I(nvec), I(nhead), I(D))
 
         row(tag + "backward: the five calls back to back", five_calls, flops=4 * fl)
-        row(tag + "backward: gQ, gK, gV in one call, two launches (kai_attention_backward)",
+        row(tag + "backward: gQ, gK, gV in one call (kai_attention_backward: %s)"
+            % kai.VMath.attention_plan("backward", nbat, T, nvec, nhead, D),
             lambda: L.kai_attention_backward(0, P(gq), P(gk), P(gv), P(go), P(pbuf), P(mo), P(q), P(k), P(v), I(nbat), I(T),
                                              I(nvec), I(nhead), I(D), P(coef), 0),
             flops=4 * fl)

@@ -25,6 +25,7 @@
 
 #include <type_traits>
 
+#include "attention_value_grad.h"
 #include "elementwise.h"
 
 namespace kai {
@@ -81,8 +82,14 @@ struct AttnBwdParams {
 
 // DB = head size / 16; KB = blocks of 16 keys per wave and tile (a tile holds 32 * KB keys); PVEC: one head and
 // rows of P that allow 128-bit loads.
+template <int DB, int KB>
+constexpr int rows_lds_floats() {
+    return 2 * 3 * (16 * KB * kAbKGroups) * (16 * DB + 4);
+}
+
+// Workgroup `bid` of `nblocks`; smem: rows_lds_floats<DB, KB>() floats, 16-byte aligned.
 template <int DB, int KB, bool PVEC>
-__global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(const AttnBwdParams p) {
+__device__ __forceinline__ void attention_backward_rows_body(const AttnBwdParams& p, const int bid, const int nblocks, float* smem) {
     constexpr int D = 16 * DB;
     constexpr int kKeys = 16 * KB * kAbKGroups;
     constexpr int kStride = D + 4;           // tiles [keys][D] lie in LDS as in memory
@@ -93,7 +100,8 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     constexpr bool kPartial = kTileChunks % kAbThreads != 0;
     constexpr int NP = PVEC ? KB : 4 * KB;   // loads of P per lane and tile
     // [buffer][operand V, K, Q][tile]
-    __shared__ __attribute__((aligned(16))) float lds[2][3][kTile];
+    static_assert(6 * kTile == rows_lds_floats<DB, KB>(), "the size the callers reserve");
+    float (*lds)[3][kTile] = reinterpret_cast<float (*)[3][kTile]>(smem);
     static_assert(8 * DB * 64 * kAbQGroups + 64 * kAbQGroups <= 6 * kTile, "the merge buffer must fit the tiles");
 
     const int tid = threadIdx.x;
@@ -106,7 +114,7 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     const int T = p.ntimes;
     const int H = p.nhead;
     int b, h, ttile;
-    attention_block_of(blockIdx.x, gridDim.x, (T + kAbRows - 1) / kAbRows, H, b, h, ttile);
+    attention_block_of(bid, nblocks, (T + kAbRows - 1) / kAbRows, H, b, h, ttile);
     const int t0 = ttile * kAbRows;
     const int64_t base = (int64_t)b * p.batch_stride + (int64_t)h * p.npiece;
     const float coef = p.coef ? *p.coef : 0.f;
@@ -493,6 +501,29 @@ __global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(con
     }
 }
 
+template <int DB, int KB, bool PVEC>
+__global__ void __launch_bounds__(kAbThreads) attention_backward_rows_kernel(const AttnBwdParams p) {
+    __shared__ __attribute__((aligned(16))) float smem[rows_lds_floats<DB, KB>()];
+    attention_backward_rows_body<DB, KB, PVEC>(p, blockIdx.x, gridDim.x, smem);
+}
+
+// The whole backward middle in one launch: the first `nrows` workgroups are those of the rows kernel, the others
+// compute the value gradient (attention_value_grad.h; one head per workgroup where P allows 128-bit loads along the
+// keys, else four).  The two kinds share nothing; one launch saves the second launch's start-up, and the value
+// gradient's workgroups start as the first rows workgroups leave their compute units.
+template <int DB, int KB, bool PVEC>
+__global__ void __launch_bounds__(kAbThreads) attention_backward_all_kernel(const AttnBwdParams p, const vgrad::ValueGradParams v,
+                                                                            const int nrows) {
+    constexpr int HV = PVEC ? 1 : 4;
+    constexpr int kFloats = rows_lds_floats<DB, KB>() > vgrad::value_grad_lds_floats<DB, HV>() ? rows_lds_floats<DB, KB>()
+                                                                                             : vgrad::value_grad_lds_floats<DB, HV>();
+    static_assert(vgrad::kVgThreads == kAbThreads, "one block size for both kinds of workgroup");
+    __shared__ __attribute__((aligned(16))) float smem[kFloats];
+    const int bid = blockIdx.x;
+    if (bid < nrows) attention_backward_rows_body<DB, KB, PVEC>(p, bid, nrows, smem);
+    else vgrad::attention_value_grad_body<DB, HV>(v, bid - nrows, (int)gridDim.x - nrows, smem);
+}
+
 }  // namespace
 
 bool attention_backward_applies(const float* gq, const float* gk, const float* gm, const float* m, const float* pp,
@@ -506,13 +537,36 @@ bool attention_backward_applies(const float* gq, const float* gk, const float* g
            aligned16(q) && aligned16(k) && aligned16(v) && (reinterpret_cast<uintptr_t>(pp) & 3u) == 0;
 }
 
-template <int DB, int KB>
-static void launch_rows(const AttnBwdParams& p, bool pvec, dim3 grid, hipStream_t stream) {
-    if (pvec) attention_backward_rows_kernel<DB, KB, true><<<grid, dim3(kAbThreads), 0, stream>>>(p);
-    else attention_backward_rows_kernel<DB, KB, false><<<grid, dim3(kAbThreads), 0, stream>>>(p);
+// gv null: the rows kernel alone; else the one-launch kernel, whose value gradient workgroups follow the rows workgroups
+template <int DB, int KB, bool MERGE_NOVEC = (DB <= 4)>
+static void launch_rows(const AttnBwdParams& p, const vgrad::ValueGradParams* v, int64_t vblocks, bool pvec, dim3 grid,
+                        hipStream_t stream) {
+    const dim3 block(kAbThreads);
+    if (v == nullptr) {
+        if (pvec) attention_backward_rows_kernel<DB, KB, true><<<grid, block, 0, stream>>>(p);
+        else attention_backward_rows_kernel<DB, KB, false><<<grid, block, 0, stream>>>(p);
+        return;
+    }
+    const dim3 all(grid.x + (unsigned)vblocks);
+    if (pvec) attention_backward_all_kernel<DB, KB, true><<<all, block, 0, stream>>>(p, *v, (int)grid.x);
+    else if constexpr (MERGE_NOVEC) attention_backward_all_kernel<DB, KB, false><<<all, block, 0, stream>>>(p, *v, (int)grid.x);
 }
 
-int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const float* m, const float* pp,
+// Whether kai_attention_backward runs this geometry as ONE launch: the rows kernel applies (the caller has checked)
+// and the value gradient's kernel takes the geometry with the heads per workgroup that go with the rows kernel's
+// way of loading P (one head with 128-bit loads along the keys, four heads otherwise).
+bool attention_backward_one_launch(const float* gv, const float* gm, const float* pp, int64_t nbat, int64_t ntimes,
+                                   int64_t nvec, int64_t nhead, int64_t npiece) {
+    const int hv = attention_value_grad_heads(gv, gm, pp, ntimes, nvec, nhead, npiece);
+    const bool pvec = nhead == 1 && ntimes % 4 == 0 && aligned16(pp);
+    if (!(pvec ? hv == 1 : hv == 4)) return false;
+    const int64_t ttiles = (ntimes + kAbRows - 1) / kAbRows;
+    return ttiles * nbat * nhead + value_grad_blocks(hv, nbat, ntimes, nhead) <= kMaxDim;
+}
+
+// gv null: gQ and gK only (the caller computes the value gradient); else all three in one launch, which
+// attention_backward_one_launch must have allowed
+int launch_attention_backward_rows(float* gq, float* gk, float* gv, const float* gm, const float* m, const float* pp,
                                    const float* q, const float* k, const float* v, int64_t nbat, int64_t ntimes,
                                    int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
                                    hipStream_t stream) {
@@ -525,17 +579,26 @@ int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const 
     if (ttiles * nbat * nhead > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "attention backward: grid too large");
     const dim3 grid((unsigned)(ttiles * nbat * nhead));
     const bool pvec = nhead == 1 && ntimes % 4 == 0 && aligned16(pp);
-    switch (npiece / 16) {
-    case 1: launch_rows<1, 2>(p, pvec, grid, stream); break;
-    case 2: launch_rows<2, 2>(p, pvec, grid, stream); break;
-    case 3: launch_rows<3, 2>(p, pvec, grid, stream); break;
-    case 4: launch_rows<4, 2>(p, pvec, grid, stream); break;
-    case 5: launch_rows<5, 2>(p, pvec, grid, stream); break;
-    case 6: launch_rows<6, 1>(p, pvec, grid, stream); break;
-    case 7: launch_rows<7, 1>(p, pvec, grid, stream); break;
-    default: launch_rows<8, 1>(p, pvec, grid, stream); break;
+    vgrad::ValueGradParams vp{};
+    int64_t vblocks = 0;
+    if (gv != nullptr) {
+        if (!attention_backward_one_launch(gv, gm, pp, nbat, ntimes, nvec, nhead, npiece))
+            return fail(KAI_ERR_INVALID_ARGUMENT, "attention backward: the value gradient does not fit the one-launch kernel");
+        vp = value_grad_params(gv, gm, pp, ntimes, nvec, nhead, npiece);
+        vblocks = value_grad_blocks(pvec ? 1 : 4, nbat, ntimes, nhead);
     }
-    return check_launch("attention_backward_rows_kernel");
+    const vgrad::ValueGradParams* vptr = gv != nullptr ? &vp : nullptr;
+    switch (npiece / 16) {
+    case 1: launch_rows<1, 2>(p, vptr, vblocks, pvec, grid, stream); break;
+    case 2: launch_rows<2, 2>(p, vptr, vblocks, pvec, grid, stream); break;
+    case 3: launch_rows<3, 2>(p, vptr, vblocks, pvec, grid, stream); break;
+    case 4: launch_rows<4, 2>(p, vptr, vblocks, pvec, grid, stream); break;
+    case 5: launch_rows<5, 2>(p, vptr, vblocks, pvec, grid, stream); break;
+    case 6: launch_rows<6, 1>(p, vptr, vblocks, pvec, grid, stream); break;
+    case 7: launch_rows<7, 1>(p, vptr, vblocks, pvec, grid, stream); break;
+    default: launch_rows<8, 1>(p, vptr, vblocks, pvec, grid, stream); break;
+    }
+    return check_launch(gv != nullptr ? "attention_backward_all_kernel" : "attention_backward_rows_kernel");
 }
 
 }  // namespace kai

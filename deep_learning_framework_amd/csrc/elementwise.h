@@ -110,7 +110,10 @@ int launch_attention_value_grad(float* gv, const float* gy, const float* pp, int
 bool attention_backward_applies(const float* gq, const float* gk, const float* gm, const float* m, const float* pp,
                                 const float* q, const float* k, const float* v, int64_t ntimes, int64_t nvec,
                                 int64_t nhead, int64_t npiece);
-int launch_attention_backward_rows(float* gq, float* gk, const float* gm, const float* m, const float* pp,
+bool attention_backward_one_launch(const float* gv, const float* gm, const float* pp, int64_t nbat, int64_t ntimes,
+                                   int64_t nvec, int64_t nhead, int64_t npiece);
+// gv null: gQ and gK only; else gV in the same launch (where attention_backward_one_launch says so)
+int launch_attention_backward_rows(float* gq, float* gk, float* gv, const float* gm, const float* m, const float* pp,
                                    const float* q, const float* k, const float* v, int64_t nbat, int64_t ntimes,
                                    int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
                                    hipStream_t stream);

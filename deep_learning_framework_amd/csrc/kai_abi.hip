@@ -924,7 +924,8 @@ int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, in
     else if (which == 1 && attention_probs_applies(a, a, a, a, a, ntimes, nvec, nhead, npiece))
         text = attention_probs_four_heads(a, ntimes, nhead, npiece) ? "fused, four heads per workgroup" : "fused";
     else if (which == 2 && attention_backward_applies(a, a, a, a, a, a, a, a, ntimes, nvec, nhead, npiece))
-        text = "fused rows + value gradient";
+        text = attention_backward_one_launch(a, a, a, nbat, ntimes, nvec, nhead, npiece) ? "fused rows and value gradient in one launch"
+                                                                                        : "fused rows + value gradient";
     else if (which == 3) {
         const int hv = attention_value_grad_heads(a, a, a, ntimes, nvec, nhead, npiece);
         text = hv == 1 ? "streamed, one head per workgroup" : hv == 4 ? "streamed, four heads per workgroup" : "tiled";
@@ -959,11 +960,15 @@ int kai_attention_backward(int device, float* pgQ, float* pgK, float* pgV, const
     if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
     KAI_REQUIRE_PTR(pgQ); KAI_REQUIRE_PTR(pgK); KAI_REQUIRE_PTR(pgV); KAI_REQUIRE_PTR(pgm); KAI_REQUIRE_PTR(pp);
     KAI_REQUIRE_PTR(pQ); KAI_REQUIRE_PTR(pK); KAI_REQUIRE_PTR(pV);
-    // the value gradient is a reduction over the rows: its own launch either way
+    // The value gradient is a reduction over the rows, workgroups of its own: behind the rows workgroups in the
+    // same launch where its streaming kernel takes the geometry, else a launch of its own.
+    if (attention_backward_applies(pgQ, pgK, pgm, pm, pp, pQ, pK, pV, ntimes, nvec, nhead, npiece)) {
+        const bool one = attention_backward_one_launch(pgV, pgm, pp, nbat, ntimes, nvec, nhead, npiece);
+        if (!one) KAI_TRY(kai_mix_values_backward_value(device, pgV, pgm, pp, nbat, ntimes, nvec, nhead, npiece));
+        return launch_attention_backward_rows(pgQ, pgK, one ? pgV : nullptr, pgm, pm, pp, pQ, pK, pV, nbat, ntimes, nvec,
+                                              nhead, npiece, hCoef, masked != 0, current_stream());
+    }
     KAI_TRY(kai_mix_values_backward_value(device, pgV, pgm, pp, nbat, ntimes, nvec, nhead, npiece));
-    if (attention_backward_applies(pgQ, pgK, pgm, pm, pp, pQ, pK, pV, ntimes, nvec, nhead, npiece))
-        return launch_attention_backward_rows(pgQ, pgK, pgm, pm, pp, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece,
-                                              hCoef, masked != 0, current_stream());
     // any other shape: the reference's calls one by one, the gradient of the probabilities in the library's scratch
     const int64_t pbytes = nbat * ntimes * ntimes * nhead * (int64_t)sizeof(float);
     float* pgp = nullptr;

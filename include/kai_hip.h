@@ -344,8 +344,9 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
 /* No counterpart in the reference.  Writes into `out` how the attention entry points would run this geometry with
  * 16-byte aligned operands, as text: which = 0 kai_attention_forward ("fused" or "separate"), 1
  * kai_attention_forward_train ("fused", "fused, four heads per workgroup" or "separate"), 2 kai_attention_backward
- * ("fused rows + value gradient" or "separate"), 3 kai_mix_values_backward_value, also the value gradient inside
- * kai_attention_backward ("streamed, one head per workgroup", "streamed, four heads per workgroup" or "tiled").
+ * ("fused rows and value gradient in one launch", "fused rows + value gradient" (two launches) or "separate"), 3
+ * kai_mix_values_backward_value, also the value gradient inside kai_attention_backward ("streamed, one head per
+ * workgroup", "streamed, four heads per workgroup" or "tiled").
  * Host arithmetic only, nothing is launched and no GPU is needed.
  * For maintainers and tests. */
 int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, char* out,
@@ -360,7 +361,7 @@ int kai_attention_forward_train(int device, float* py, float* pp, const float* p
                                 int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece,
                                 const float* hCoef, int masked);
 
-/* The backward middle of the same block in two launches: the calls of VTensor::multihead_attention_backprop between
+/* The backward middle of the same block in one or two launches: the calls of VTensor::multihead_attention_backprop between
  * the output projection and the input projections (vtensor.cpp:3145-3154),
  *   mix_values_backward_prop, mix_values_backward_value, softmax_direct_on_axis_backward,
  *   [set_mh_attention_mask(backward) when masked != 0], mult_on_heads_backward (key gradient from pQ),
@@ -371,7 +372,9 @@ int kai_attention_forward_train(int device, float* py, float* pp, const float* p
  * mixed output of the forward pass (the engine keeps it, vtensor.cpp:3050), or null -- with it the softmax
  * derivative's row sum is one dot product (sum_k P*gP = sum_d gM*M), without it a first pass over the keys forms
  * it.  Outputs: pgQ, pgK, pgV, each [nbat, ntimes, nvec].  Head sizes that are multiples of 16 up to 128 with
- * nhead * npiece == nvec and 16-byte aligned operands run fused (the value gradient in its own launch); any other
+ * nhead * npiece == nvec and 16-byte aligned operands run fused -- the value gradient as further workgroups of the
+ * same launch with one head and a length in whole fours, or head counts in whole fours with head sizes up to 64
+ * (lengths from 32 on), otherwise in a launch of its own; any other
  * shape runs the six calls with the gradient of the probabilities in the library's scratch memory.  Results equal
  * the separate calls up to the order of the sums. */
 int kai_attention_backward(int device, float* pgQ, float* pgK, float* pgV, const float* pgm, const float* pp,

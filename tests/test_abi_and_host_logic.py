@@ -317,14 +317,19 @@ def test_attention_plans():
     assert plan("forward", 4, 512, 512, 8, 64) == "fused"
     assert plan("forward_train", 32, 512, 64, 1, 64) == "fused"
     assert plan("forward_train", 4, 512, 512, 8, 64) == "fused, four heads per workgroup"
-    assert plan("backward", 32, 512, 64, 1, 64) == "fused rows + value gradient"
-    assert plan("backward", 4, 512, 512, 8, 64) == "fused rows + value gradient"
+    assert plan("backward", 32, 512, 64, 1, 64) == "fused rows and value gradient in one launch"
+    assert plan("backward", 4, 512, 512, 8, 64) == "fused rows and value gradient in one launch"
+    assert plan("value_gradient", 32, 512, 64, 1, 64) == "streamed, one head per workgroup"
+    assert plan("value_gradient", 4, 512, 512, 8, 64) == "streamed, four heads per workgroup"
     # head sizes 96 and 128, twelve heads of 64, lengths that are no multiple of 32, six heads
     for nbat, ntimes, nhead, npiece in ((2, 384, 12, 64), (1, 500, 16, 96), (2, 1024, 8, 128), (3, 200, 6, 32)):
         nvec = nhead * npiece
         assert plan("forward", nbat, ntimes, nvec, nhead, npiece) == "fused"
         assert plan("forward_train", nbat, ntimes, nvec, nhead, npiece).startswith("fused")
-        assert plan("backward", nbat, ntimes, nvec, nhead, npiece) == "fused rows + value gradient"
+        # one launch where the value gradient's kernel takes the geometry too (head counts in whole fours with head
+        # sizes up to 64, or one head), else the rows kernel and the tiled value gradient
+        assert plan("backward", nbat, ntimes, nvec, nhead, npiece) == (
+            "fused rows and value gradient in one launch" if nhead % 4 == 0 and npiece <= 64 else "fused rows + value gradient")
     # what the one-launch kernels leave to the separate ones: head sizes that are no multiple of 16 or beyond 128,
     # heads that do not fill the vector, the training forward beyond 1024 keys
     assert plan("forward", 2, 100, 48, 2, 24) == "separate"
