@@ -145,7 +145,7 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // columns for one workgroup per compute unit, a matrix of at most 192 MB): W streams once in one launch
     // (4096 x 4096 from HBM: 17 rows 21.2 -> 15.0 us, 32 rows 21.3 -> 17.9, on a row of 32 x 128 tiles with eight
     // parts of K and their second launch before)
-    if (!plan.skinny && d.M > kSkinnyMaxRows && d.M <= 2 * kSkinnyMaxRows && d.nbatch == 1 && d.a_ks == 1 && d.b_ks == 1 &&
+    if (!plan.skinny && d.M > kSkinnyMaxRows && d.M <= 4 * kSkinnyMaxRows && d.nbatch == 1 && d.a_ks == 1 && d.b_ks == 1 &&
         d.c_cs == 1 && !d.has_alpha && d.rowsum == nullptr) {
         SkinnyParams sp{};
         sp.W = d.B; sp.X = d.A; sp.ldw = d.b_rs; sp.ldx = d.a_rs; sp.N = d.N; sp.M = (int)d.M; sp.K = (int)d.K;

@@ -1,4 +1,4 @@
-// Skinny products (at most 16 rows; 17..32 on the streaming kernel where skinny_stream32_applies): parameters and
+// Skinny products (at most 16 rows; 17..64 on the streaming kernel where skinny_stream32_applies): parameters and
 // launcher, see gemv_skinny.hip.
 #pragma once
 
@@ -46,7 +46,7 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream);
 
 // skinny_stream.hip: aligned operands, K split over workgroups (uses the library's scratch memory)
 bool skinny_stream_applies(const SkinnyParams& p);
-bool skinny_stream32_applies(const SkinnyParams& p);   // 17..32 rows
+bool skinny_stream32_applies(const SkinnyParams& p);   // 17..32 rows, and 33..64 where workgroups of 32 / 48 rows of W apply
 bool skinny_stream8_applies(const SkinnyParams& p);    // workgroups of 8 rows of W
 int launch_skinny_stream8(const SkinnyParams& p, hipStream_t stream);
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream);

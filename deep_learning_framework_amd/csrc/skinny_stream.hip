@@ -76,7 +76,8 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 //
 // XB: blocks of 16 rows of X.  2 (17..32 rows; whole tiles and written-out slices only, XL = 3 or 4): a tile of W meets
 // two tiles of X and a wave keeps two accumulators -- W still streams once, where a tiled product of 17..32 rows
-// cuts K over workgroups and sums the parts in a second launch.
+// cuts K over workgroups and sums the parts in a second launch.  3 and 4 (33..64 rows, XL = 5..8) with workgroups of
+// 32 or 48 rows of W only: 6 to 12 accumulators per wave, and the matrix cores set the time.
 //
 // WR: rows of W per workgroup, 16, or 8 (whole tiles only) where workgroups of 16 rows would not cover the compute
 // units: the second half of the W tile then stays zero and only eight columns of the result are stored.  32 and 48
@@ -93,8 +94,12 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     constexpr int WB = WR <= 16 ? 1 : WR / 16;      // blocks of 16 rows of W
     constexpr int kWTileRows = 16 * WB;
     __shared__ __attribute__((aligned(16))) float lds_w[kSsWaves][kWTileRows * kSsTileStride];
-    static_assert(XB == 1 || (XB == 2 && WHOLE && SLICES && XL > kSsLoadsPerTile && XL <= 2 * kSsLoadsPerTile),
-                  "two blocks of X rows exist for whole tiles in written-out slices");
+    static_assert(XB == 1 || (XB >= 2 && XB <= 4 && WHOLE && SLICES && XL > kSsLoadsPerTile * (XB - 1) && XL <= kSsLoadsPerTile * XB),
+                  "several blocks of X rows exist for whole tiles in written-out slices");
+    static_assert(XB <= 2 || WR >= 32, "three and four blocks of X rows: with two or three blocks of W rows only");
+    // tiles of a wave in registers (written-out slices): with three and four blocks of X rows a tile is 10 to 14 loads
+    // per lane, and two tiles are what the registers hold
+    constexpr int kRing = XB >= 3 ? 2 : kSsRing;
     static_assert(WR == 16 || (WR == 8 && WHOLE && XB == 1 && kSsRowsPerLoad == 8) ||
                       ((WR == 32 || WR == 48) && WHOLE && SLICES && XL > 0),
                   "eight rows of W: one load per tile; 32 and 48: whole tiles in written-out slices");
@@ -237,8 +242,8 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         }
     };
     if constexpr (SLICES) {
-        // wave w owns the slices of 512 steps number w, w + 8, ...; per slice a ring of kSsRing tiles, the loads of
-        // tile t + kSsRing issued as soon as tile t has left its registers
+        // wave w owns the slices of 512 steps number w, w + 8, ...; per slice a ring of kRing tiles, the loads of
+        // tile t + kRing issued as soon as tile t has left its registers
         constexpr int kSlice = 512, kTiles = kSlice / kSsTileK;
         // Rows of 32 KiB and more that are a power of two apart: with every wave walking its slice from the slice's
         // first tile the requests of a moment crowd onto few memory channels; wave w starts 2 w tiles into its slice
@@ -246,21 +251,21 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         // lengths unchanged).  At 4096 steps the plain order is the faster one (12.1 against 12.4 us).
         const int stag = p.K >= 8192 ? 2 * wave : 0;
         for (int k0 = wave * kSlice; k0 < p.K; k0 += kSsWaves * kSlice) {
-            f32x4 w[kSsRing][kWRegs], x[kSsRing][kXLoads];
-            ss_static_for<0, kSsRing>([&](auto tc) {
+            f32x4 w[kRing][kWRegs], x[kRing][kXLoads];
+            ss_static_for<0, kRing>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
                 load_w(w[t], k0 + ((t + stag) & (kTiles - 1)) * kSsTileK);
                 load_x(x[t], k0 + ((t + stag) & (kTiles - 1)) * kSsTileK);
             });
             ss_static_for<0, kTiles>([&](auto tc) {
                 constexpr int t = decltype(tc)::value;
-                constexpr int slot = t % kSsRing;
+                constexpr int slot = t % kRing;
                 __builtin_amdgcn_sched_barrier(0);
                 consume(w[slot], x[slot], k0 + ((t + stag) & (kTiles - 1)) * kSsTileK);
                 __builtin_amdgcn_sched_barrier(0);
-                if constexpr (t + kSsRing < kTiles) {
-                    load_w(w[slot], k0 + ((t + kSsRing + stag) & (kTiles - 1)) * kSsTileK);
-                    load_x(x[slot], k0 + ((t + kSsRing + stag) & (kTiles - 1)) * kSsTileK);
+                if constexpr (t + kRing < kTiles) {
+                    load_w(w[slot], k0 + ((t + kRing + stag) & (kTiles - 1)) * kSsTileK);
+                    load_x(x[slot], k0 + ((t + kRing + stag) & (kTiles - 1)) * kSsTileK);
                 }
             });
         }
@@ -305,32 +310,37 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     }
 
     // acc[a][b][v] = D[m = 16 * b + 4 * g + v][n = n0 + 16 * a + r]; the tiles are free now: wave w parks its
-    // results in its W tile, a 16 x 16 block per (a, b)
-    static_assert(256 * XB * WB <= kWTileRows * kSsTileStride, "a wave's results fit its W tile");
-    __syncthreads();
+    // results in its W tile, a 16 x 16 block per (a, b), kXbPass blocks of X rows at a time
+    constexpr int kParkFloats = kWTileRows * kSsTileStride;
+    constexpr int kXbPass = 256 * XB * WB <= kParkFloats ? XB : (XB % 2 == 0 && 512 * WB <= kParkFloats) ? 2 : 1;
+    static_assert(256 * kXbPass * WB <= kWTileRows * kSsTileStride && XB % kXbPass == 0, "a pass of a wave's results fits its W tile");
 #pragma unroll
-    for (int a = 0; a < WB; a++)
+    for (int b0 = 0; b0 < XB; b0 += kXbPass) {
+        __syncthreads();
 #pragma unroll
-        for (int b = 0; b < XB; b++)
+        for (int a = 0; a < WB; a++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) tw[((a * XB + b) * 16 + 4 * g + v) * 16 + r] = acc[a][b][v];
-    __syncthreads();
+            for (int b = 0; b < kXbPass; b++)
 #pragma unroll
-    for (int i0 = 0; i0 < 256 * XB * WB; i0 += kSsThreads) {
-        const int e = i0 + tid;
-        const int blk = e >> 8, a = blk / XB, b = blk % XB;
-        const int m = 16 * b + ((e >> 4) & 15), j = e & 15;
-        const int64_t n = n0 + 16 * a + j;
-        if (e < 256 * XB * WB && m < p.M && n < p.N && j < WR) {
-            float v = 0.f;
+                for (int v = 0; v < 4; v++) tw[((a * kXbPass + b) * 16 + 4 * g + v) * 16 + r] = acc[a][b0 + b][v];
+        __syncthreads();
 #pragma unroll
-            for (int i = 0; i < kSsWaves; i++) v += lds_w[i][e];
-            const float leaky = p.leaky ? *p.leaky : 0.f;
-            const int64_t idx = (int64_t)m * p.ldy + n;
-            if (p.accflag) v += p.Y[idx];
-            if (p.bias) v += p.bias[n];
-            if (p.Y2) p.Y2[idx] = v;
-            p.Y[idx] = apply_act(v, p.act, leaky);
+        for (int i0 = 0; i0 < 256 * kXbPass * WB; i0 += kSsThreads) {
+            const int e = i0 + tid;
+            const int blk = e >> 8, a = blk / kXbPass, b = b0 + blk % kXbPass;
+            const int m = 16 * b + ((e >> 4) & 15), j = e & 15;
+            const int64_t n = n0 + 16 * a + j;
+            if (e < 256 * kXbPass * WB && m < p.M && n < p.N && j < WR) {
+                float v = 0.f;
+#pragma unroll
+                for (int i = 0; i < kSsWaves; i++) v += lds_w[i][e];
+                const float leaky = p.leaky ? *p.leaky : 0.f;
+                const int64_t idx = (int64_t)m * p.ldy + n;
+                if (p.accflag) v += p.Y[idx];
+                if (p.bias) v += p.bias[n];
+                if (p.Y2) p.Y2[idx] = v;
+                p.Y[idx] = apply_act(v, p.act, leaky);
+            }
         }
     }
 }
@@ -345,11 +355,17 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
 // 44.0 -> 52.2 / 51.3 -> 63.5.
 // Rows longer than 4096 steps are taken only up to 96 MB: a weight matrix that a serving loop multiplies again and
 // again stays in the last-level cache, and there 4096 x 8192 lost 8..11 % (the warm figures above).
-bool skinny_stream32_applies(const SkinnyParams& p) {
-    return p.M > kSkinnyMaxRows && p.M <= 2 * kSkinnyMaxRows && p.K % (kSsWaves * 512) == 0 && p.N % 16 == 0 &&
+// 33..64 rows (three and four blocks of X rows) run here only where workgroups of 32 or 48 rows of W apply: with
+// 16 rows of W a workgroup would load four times as many bytes of X as of W.
+static bool stream_many_rows_base(const SkinnyParams& p) {
+    return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && p.K % (kSsWaves * 512) == 0 && p.N % 16 == 0 &&
            p.N >= 16 * (int64_t)compute_units() && p.N * (int64_t)p.K * 4 <= (192ll << 20) &&
            (p.K <= 4096 || p.N * (int64_t)p.K * 4 <= (96ll << 20)) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
            (15 * p.ldw + p.K) * 4 < (1ll << 31) && ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
+}
+
+bool skinny_stream32_applies(const SkinnyParams& p) {
+    return stream_many_rows_base(p) && (p.M <= 2 * kSkinnyMaxRows || skinny_stream_wide_rows(p) != 0);
 }
 
 bool skinny_stream_applies(const SkinnyParams& p) {
@@ -388,7 +404,11 @@ int launch_wide(const SkinnyParams& p, const SkinnyTail& t, hipStream_t stream) 
     if (p.M <= 8) skinny_stream_kernel<true, true, 1, 1, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     else if (p.M <= 16) skinny_stream_kernel<true, true, 2, 1, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     else if (p.M <= 24) skinny_stream_kernel<true, true, 3, 2, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
-    else skinny_stream_kernel<true, true, 4, 2, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (p.M <= 32) skinny_stream_kernel<true, true, 4, 2, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (p.M <= 40) skinny_stream_kernel<true, true, 5, 3, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (p.M <= 48) skinny_stream_kernel<true, true, 6, 3, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else if (p.M <= 56) skinny_stream_kernel<true, true, 7, 4, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+    else skinny_stream_kernel<true, true, 8, 4, WR><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
     return check_launch("skinny_stream_kernel");
 }
 }  // namespace
@@ -404,11 +424,15 @@ void set_skinny_stream_rows_override(int rows) { g_stream_rows_override = rows; 
 // 16 rows 90.2 -> 84.8; 8192 (256 of 32) 16 / 24 / 32 rows 23.9 / 28.5 / 32.0 -> 28.2 / 28.9 / 29.8; 7168 (224 of 32)
 // 23.8 / 27.7 / 30.7 -> 25.1 / 26.5 / 27.8; 6144 (192 of 32) 22.9 / 26.5 / 29.9 -> 22.5 / 24.8 / 26.1; 16384 (342 of 48,
 // 512 of 32) 16 rows 45.6 -> 51.4 / 51.8.  Hence: 48 rows from 9 rows of X on where the workgroups fill their rounds
-// over the compute units to 85 %; 32 rows from 17 rows of X on where the workgroups are one round, at least three
-// quarters full.
+// over the compute units to 85 % (17 rows and more: one round, four fifths full: 10240 columns, 214 workgroups,
+// 33 / 48 rows 50.6 / 51.9 on the tiled kernel -> 43.6 / 45.5); 32 rows from 17 rows of X on where the workgroups
+// are one round, at least three quarters full.
+// 33..64 rows run on these workgroups only, tiled kernel -> here: 11008 columns 33 / 48 / 64 rows 67.7 / 63.5 / 65.3 ->
+// 46.8 / 46.0 / 57.2; 8192 61.3 / 62.6 / 61.7 -> 33.1 / 35.9 / 45.2; 6144 61.5 / 61.3 / 61.4 -> 30.9 / 32.1 / 40.5 (a ring
+// of three tiles with three blocks of X rows: 46.0 -> 48.8 at 11008 x 48 rows, no gain elsewhere).
 int skinny_stream_wide_rows(const SkinnyParams& p) {
-    if (g_stream_rows_override == 16) return 0;
-    const bool base = p.M > kSkinnyMaxRows ? skinny_stream32_applies(p) : (p.M >= 2 && skinny_stream_applies(p));
+    if (g_stream_rows_override == 16 && p.M <= 2 * kSkinnyMaxRows) return 0;
+    const bool base = p.M > kSkinnyMaxRows ? stream_many_rows_base(p) : (p.M >= 2 && skinny_stream_applies(p));
     if (!base || p.K % (kSsWaves * 512) != 0 || p.N % 16 != 0 || (47 * p.ldw + p.K) * 4 >= (1ll << 31) ||
         ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 >= 0x7FFFFFF0ll)
         return 0;
@@ -416,7 +440,7 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
     if (p.M <= 8) return 0;
     const int64_t cus = compute_units();
     const int64_t groups48 = (p.N + 47) / 48, rounds48 = (groups48 + cus - 1) / cus;
-    if (groups48 * 100 >= 85 * rounds48 * cus && (rounds48 == 1 || p.M <= kSkinnyMaxRows)) return 48;
+    if (p.M <= kSkinnyMaxRows ? groups48 * 100 >= 85 * rounds48 * cus : (rounds48 == 1 && groups48 * 100 >= 80 * cus)) return 48;
     const int64_t groups32 = (p.N + 31) / 32;
     if (p.M > kSkinnyMaxRows && groups32 <= cus && groups32 * 4 >= 3 * cus) return 32;
     return 0;
@@ -435,7 +459,8 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     const bool slices = p.K % (kSsWaves * 512) == 0;
     const dim3 grid((unsigned)blocks), block(kSsThreads);
     if (p.M > kSkinnyMaxRows) {
-        if (!skinny_stream32_applies(p)) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
+        if (!skinny_stream32_applies(p) || p.M > 2 * kSkinnyMaxRows)
+            return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
         if (p.M <= 24) skinny_stream_kernel<true, true, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         else skinny_stream_kernel<true, true, 4, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         return check_launch("skinny_stream_kernel");

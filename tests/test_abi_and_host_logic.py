@@ -248,6 +248,10 @@ GEMM_PLANS = [
     ((0, 1, 32, 8192, 4096), "skinny stream 32"),                    # 256 workgroups of 32 rows, 17..32 rows of X only
     ((0, 1, 16, 8192, 4096), "skinny"),
     ((0, 1, 16, 16384, 4096), "skinny"),                             # 342 workgroups of 48: the second round a third full
+    ((0, 1, 48, 8192, 4096), "skinny stream 32"),                    # 33..64 rows stream only on the wide workgroups
+    ((0, 1, 64, 11008, 4096), "skinny stream 48"),
+    ((0, 1, 33, 10240, 4096), "skinny stream 48"),                   # 214 workgroups: one round, four fifths full
+    ((0, 1, 65, 11008, 4096), "mfma flat ragged pipelined split 8"),
     ((0, 0, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
     ((0, 1, 96, 4096, 4096), "mfma flat ragged pipelined split 8"),  # 65..96 rows: three row tiles of 32, not two of 64

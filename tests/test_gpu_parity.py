@@ -403,7 +403,9 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    (8, 4096, 2048), (16, 8192, 1024), (3, 4096, 1544), (2, 4096, 2048), (9, 12288, 1032),
                                    # workgroups of 48 and 32 rows of W where they fill the compute units (the last one
                                    # of 11008 and of 7184 owns 16 rows)
-                                   (32, 4096, 11008), (16, 4096, 11008), (9, 4096, 12288), (24, 4096, 7184), (17, 4096, 6144)])
+                                   (32, 4096, 11008), (16, 4096, 11008), (9, 4096, 12288), (24, 4096, 7184), (17, 4096, 6144),
+                                   # 33..64 rows: three and four blocks of X rows
+                                   (48, 4096, 8192), (64, 4096, 11008), (33, 4096, 6160)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n >= 6144:
         want = "skinny stream %d" % (48 if n >= 11008 else 32)
@@ -437,7 +439,7 @@ def test_skinny_stream_with_wide_workgroups_forced(rows):
     dwp, dbias = dev(wp), dev(bias)
     try:
         VMath.gemm_force_plan("stream %d" % rows)
-        for m in (2, 8, 9, 16, 17, 24, 25, 32):
+        for m in (2, 8, 9, 16, 17, 24, 25, 32, 33, 40, 47, 48, 49, 56, 64):
             assert VMath.gemm_plan(0, 1, m, n, k, k + padx, k + padw, n) == "skinny stream %d" % rows
             x = rng.standard_normal((m, k)).astype(np.float32)
             xp = np.full((m, k + padx), np.nan, np.float32); xp[:, :k] = x
