@@ -363,6 +363,16 @@ def test_gemm_plan_override_for_audits():
         with pytest.raises(kai.KaiError) as e:
             V.gemm_force_plan("bogus")
         assert e.value.code == 510
+        # "stream N": the rows of W per workgroup of the skinny streaming kernel, where that kernel runs anyway
+        V.gemm_force_plan("stream 32")
+        assert V.gemm_plan(0, 1, 16, 11008, 4096) == "skinny stream 32"
+        assert V.gemm_plan(0, 1, 144, 4096, 4096) == auto                    # forces no tile
+        V.gemm_force_plan("stream 16")
+        assert V.gemm_plan(0, 1, 32, 11008, 4096) == "skinny"
+        assert V.gemm_plan(0, 1, 48, 11008, 4096) == "skinny stream 48"     # 33..64 rows exist on the wide workgroups only
+        with pytest.raises(kai.KaiError):
+            V.gemm_force_plan("stream 24")
     finally:
         V.gemm_force_plan(None)
     assert V.gemm_plan(0, 1, 144, 4096, 4096) == auto
+    assert V.gemm_plan(0, 1, 16, 11008, 4096) == "skinny stream 48"
