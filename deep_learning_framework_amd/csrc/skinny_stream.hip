@@ -427,9 +427,15 @@ void set_skinny_stream_rows_override(int rows) { g_stream_rows_override = rows; 
 // over the compute units to 85 % (17 rows and more: one round, four fifths full: 10240 columns, 214 workgroups,
 // 33 / 48 rows 50.6 / 51.9 on the tiled kernel -> 43.6 / 45.5); 32 rows from 17 rows of X on where the workgroups
 // are one round, at least three quarters full.
-// 33..64 rows run on these workgroups only, tiled kernel -> here: 11008 columns 33 / 48 / 64 rows 67.7 / 63.5 / 65.3 ->
-// 46.8 / 46.0 / 57.2; 8192 61.3 / 62.6 / 61.7 -> 33.1 / 35.9 / 45.2; 6144 61.5 / 61.3 / 61.4 -> 30.9 / 32.1 / 40.5 (a ring
-// of three tiles with three blocks of X rows: 46.0 -> 48.8 at 11008 x 48 rows, no gain elsewhere).
+// 17..24 rows on 32-row workgroups only while these are at most nine tenths of the compute units (8192 columns, 256
+// workgroups, 17 / 24 rows: 25.4 / 28.9 with 16-row workgroups, 29.5 / 30.4 with these; 6144 columns 26.0 / 27.0 -> 24.5 / 25.3).
+// 33..64 rows run on these workgroups only; fastest tiled plan (tile and part count forced) -> here, W from HBM |
+// W in the last-level cache: 11008 columns 33 / 48 / 64 rows 58.5 / 60.1 / 63.1 -> 43.1 / 45.1 / 55.7 | 53.3 / 53.8 / 54.9 ->
+// 41.7 / 42.6 / 55.5; 12288 58.5 / 60.7 / 63.9 -> 44.7 / 46.2 / 58.7; 10240 33 / 48 rows 50.7 / 50.8 -> 42.5 / 44.4; 8192
+// (32-row workgroups) 39.9 / 40.3 -> 34.9 / 35.3 | 37.8 / 38.3 -> 31.9 / 34.7; 6144 33.7 / 35.3 -> 30.2 / 32.7.  With four
+// blocks of X rows (49..64 rows) the 32-row workgroups lose to the tiles (8192 columns 43.5 against 41.7 | 43.3 against
+// 39.4; 6144 39.6 against 37.3 | 38.7 against 33.3), so those rows stream on 48-row workgroups only.  (A ring of three
+// tiles with three blocks of X rows: 46.0 -> 48.8 at 11008 x 48 rows, no gain elsewhere.)
 int skinny_stream_wide_rows(const SkinnyParams& p) {
     if (g_stream_rows_override == 16 && p.M <= 2 * kSkinnyMaxRows) return 0;
     const bool base = p.M > kSkinnyMaxRows ? stream_many_rows_base(p) : (p.M >= 2 && skinny_stream_applies(p));
@@ -439,10 +445,14 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
     if (g_stream_rows_override == 32 || g_stream_rows_override == 48) return g_stream_rows_override;
     if (p.M <= 8) return 0;
     const int64_t cus = compute_units();
+    const bool many = p.M > 3 * kSkinnyMaxRows;      // 49..64 rows: four blocks of X rows
     const int64_t groups48 = (p.N + 47) / 48, rounds48 = (groups48 + cus - 1) / cus;
-    if (p.M <= kSkinnyMaxRows ? groups48 * 100 >= 85 * rounds48 * cus : (rounds48 == 1 && groups48 * 100 >= 80 * cus)) return 48;
+    if (p.M <= kSkinnyMaxRows ? groups48 * 100 >= 85 * rounds48 * cus
+                              : (rounds48 == 1 && groups48 * 100 >= (many ? 85 : 80) * cus))
+        return 48;
     const int64_t groups32 = (p.N + 31) / 32;
-    if (p.M > kSkinnyMaxRows && groups32 <= cus && groups32 * 4 >= 3 * cus) return 32;
+    if (p.M > kSkinnyMaxRows && !many && groups32 <= cus && groups32 * 4 >= 3 * cus && (p.M > 24 || groups32 * 10 <= 9 * cus))
+        return 32;
     return 0;
 }
 
