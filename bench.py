@@ -380,7 +380,8 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
         flops=2.0 * m * n * k, cpu=lambda: ko.matmul(wc, xc))
     # batches of a per-shard size against a wide weight matrix (kai_matmul, the matrix warm in the caches)
     for m, n, k in ((32, 4096, 4096), (64, 4096, 4096), (96, 4096, 4096), (144, 4096, 4096), (256, 2048, 2048),
-                    (16, 11008, 4096), (32, 11008, 4096), (96, 4096, 11008), (144, 5120, 4096), (200, 6656, 4096)):
+                    (16, 11008, 4096), (32, 11008, 4096), (48, 11008, 4096), (48, 8192, 4096), (96, 4096, 11008), (144, 5120, 4096),
+                    (200, 6656, 4096)):
         x = torch.randn((m, k), device=dev, generator=g)
         w = torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05
         y = torch.empty((m, n), device=dev)
