@@ -347,20 +347,28 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
 
 }  // namespace
 
-// 17..32 rows: whole tiles, written-out slices, workgroups that cover the compute units, a matrix of at most 192 MB.
-// Measured against a row of 32 x 128 tiles with K in parts, us per call at 17 / 32 rows, the matrix streamed from
-// HBM (rotating buffers) | still in the last-level cache: 4096 x 4096 21.2 -> 15.0 / 21.3 -> 17.9 | 16.7 -> 14.4 /
-// 20.2 -> 17.2; 11008 x 4096 45.4 -> 38.3 / 49.7 -> 45.8 | 39.0 -> 36.1 / 47.3 -> 44.2; 4096 x 8192 37.4 -> 28.9 /
-// 38.7 -> 34.0 | 25.8 -> 27.9 / 29.6 -> 33.0; 8192 x 8192 (256 MB, left out) 64.8 -> 54.5 / 67.5 -> 64.9 |
-// 44.0 -> 52.2 / 51.3 -> 63.5.
-// Rows longer than 4096 steps are taken only up to 96 MB: a weight matrix that a serving loop multiplies again and
-// again stays in the last-level cache, and there 4096 x 8192 lost 8..11 % (the warm figures above).
+// 17..32 rows: whole tiles, written-out slices, workgroups that cover the compute units.
+// Measured against a row of 32 x 128 tiles with K in parts, us per call at 17 / 32 rows with 16-row workgroups, the
+// matrix streamed from HBM (rotating buffers) | still in the last-level cache: 4096 x 4096 21.2 -> 15.0 / 21.3 -> 17.9 |
+// 16.7 -> 14.4 / 20.2 -> 17.2; 11008 x 4096 45.4 -> 38.3 / 49.7 -> 45.8 | 39.0 -> 36.1 / 47.3 -> 44.2; 4096 x 8192
+// 37.4 -> 28.9 / 38.7 -> 34.0 | 25.8 -> 27.9 / 29.6 -> 33.0.
+// Which matrices 17 and more rows stream.  Up to 192 MB a matrix may still lie in the 256 MB last-level cache when a
+// serving loop multiplies it again and again, and there the tiled kernels win for rows longer than 4096 steps
+// (4096 x 8192, 128 MB, 17 / 32 rows, us per call from HBM | from the cache: tiles 37.7 / 38.9 | 26.2 / 31.2, this
+// kernel 30.9 / 35.2 | 30.0 / 34.3), so such matrices stream only up to 96 MB.  Beyond 192 MB a matrix comes from
+// HBM on every call and streams whatever its shape (8192 x 8192 at 24 / 32 / 48 rows: tiles 64.9 / 66.9 / 78.8, this
+// kernel 53.8 / 55.4 / 66.7; 11008 x 8192: 87.3 / 96.3 / 105.9 against 68.4 / 72.1 / 87.3; 28672 x 4096 at 32 / 48 rows
+// 110.4 / 135.8 against 98.7 / 126.6).
+static bool stream_size_rule(int64_t n, int64_t k) {
+    const int64_t bytes = n * k * 4;
+    return bytes > (192ll << 20) || k <= 4096 || bytes <= (96ll << 20);
+}
+
 // 33..64 rows (three and four blocks of X rows) run here only where workgroups of 32 or 48 rows of W apply: with
 // 16 rows of W a workgroup would load four times as many bytes of X as of W.
 static bool stream_many_rows_base(const SkinnyParams& p) {
     return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && p.K % (kSsWaves * 512) == 0 && p.N % 16 == 0 &&
-           p.N >= 16 * (int64_t)compute_units() && p.N * (int64_t)p.K * 4 <= (192ll << 20) &&
-           (p.K <= 4096 || p.N * (int64_t)p.K * 4 <= (96ll << 20)) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
+           p.N >= 16 * (int64_t)compute_units() && stream_size_rule(p.N, p.K) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
            (15 * p.ldw + p.K) * 4 < (1ll << 31) && ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
 }
 
@@ -429,6 +437,11 @@ void set_skinny_stream_rows_override(int rows) { g_stream_rows_override = rows; 
 // are one round, at least three quarters full.
 // 17..24 rows on 32-row workgroups only while these are at most nine tenths of the compute units (8192 columns, 256
 // workgroups, 17 / 24 rows: 25.4 / 28.9 with 16-row workgroups, 29.5 / 30.4 with these; 6144 columns 26.0 / 27.0 -> 24.5 / 25.3).
+// Rows of 8192 steps (us, W from HBM, 16-row -> 32-row workgroups): 8192 columns 16 / 24 / 32 rows 55.1 / 59.5 / 66.3 ->
+// 50.4 / 53.8 / 55.4; 6144 columns 45.4 / 53.8 / 59.6 -> 38.6 / 46.6 / 49.6 (hence 32-row workgroups from 9 rows on there);
+// several rounds of 32-row workgroups at K = 4096: 14336 columns (448) 24 / 32 rows 54.2 / 58.9 -> 50.4 / 52.4, 16384
+// (512) 57.5 / 63.0 -> 53.9 / 54.6, 28672 (896) 96.4 / 109.5 -> 95.0 / 98.7, while 48-row workgroups in a partly filled
+// second or third round lose (16384: 65.7 / 69.4; 28672: 102.0 / 104.5).
 // 33..64 rows run on these workgroups only; fastest tiled plan (tile and part count forced) -> here, W from HBM |
 // W in the last-level cache: 11008 columns 33 / 48 / 64 rows 58.5 / 60.1 / 63.1 -> 43.1 / 45.1 / 55.7 | 53.3 / 53.8 / 54.9 ->
 // 41.7 / 42.6 / 55.5; 12288 58.5 / 60.7 / 63.9 -> 44.7 / 46.2 / 58.7; 10240 33 / 48 rows 50.7 / 50.8 -> 42.5 / 44.4; 8192
@@ -450,9 +463,15 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
     if (p.M <= kSkinnyMaxRows ? groups48 * 100 >= 85 * rounds48 * cus
                               : (rounds48 == 1 && groups48 * 100 >= (many ? 85 : 80) * cus))
         return 48;
-    const int64_t groups32 = (p.N + 31) / 32;
-    if (p.M > kSkinnyMaxRows && !many && groups32 <= cus && groups32 * 4 >= 3 * cus && (p.M > 24 || groups32 * 10 <= 9 * cus))
-        return 32;
+    const int64_t groups32 = (p.N + 31) / 32, rounds32 = (groups32 + cus - 1) / cus;
+    if (many || groups32 * 4 < 3 * cus) return 0;
+    // 9..16 rows: only with rows of 8192 steps and more, one round
+    if (p.M <= kSkinnyMaxRows) return p.K >= 8192 && rounds32 == 1 ? 32 : 0;
+    // 17..48 rows: one round, or several that are filled to 85 %; 17..24 rows with rows of up to 4096 steps only
+    // while the workgroups number at most nine tenths of the compute units
+    if (rounds32 > 1 && groups32 * 100 < 85 * rounds32 * cus) return 0;
+    if (p.M <= 24 && p.K <= 4096 && rounds32 == 1 && groups32 * 10 > 9 * cus) return 0;
+    return 32;
     return 0;
 }
 

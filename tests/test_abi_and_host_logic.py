@@ -252,6 +252,11 @@ GEMM_PLANS = [
     ((0, 1, 64, 11008, 4096), "skinny stream 48"),
     ((0, 1, 33, 10240, 4096), "skinny stream 48"),                   # 214 workgroups: one round, four fifths full
     ((0, 1, 65, 11008, 4096), "mfma flat ragged pipelined split 8"),
+    ((0, 1, 24, 8192, 8192), "skinny stream 32"),                    # 256 MB: comes from HBM on every call, streams
+    ((0, 1, 24, 4096, 8192), "mfma flat ragged pipelined staged 2 split 8"),   # 128 MB with long rows may stay cached: tiles
+    ((0, 1, 12, 8192, 8192), "skinny stream 32"),                    # rows of 8192 steps: 32-row workgroups from 9 rows on
+    ((0, 1, 32, 16384, 4096), "skinny stream 32"),                   # two full rounds of 32-row workgroups
+    ((0, 1, 48, 28672, 4096), "skinny stream 32"),
     ((0, 0, 32, 8192, 8192), "mfma flat whole split 4"),
     ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
     ((0, 1, 96, 4096, 4096), "mfma flat ragged pipelined split 8"),  # 65..96 rows: three row tiles of 32, not two of 64

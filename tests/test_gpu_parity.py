@@ -405,10 +405,12 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # of 11008 and of 7184 owns 16 rows)
                                    (32, 4096, 11008), (16, 4096, 11008), (9, 4096, 12288), (24, 4096, 7184), (17, 4096, 6144),
                                    # 33..64 rows: three and four blocks of X rows
-                                   (48, 4096, 8192), (64, 4096, 11008), (33, 4096, 6160)])
+                                   (48, 4096, 8192), (64, 4096, 11008), (33, 4096, 6160),
+                                   # rows of 8192 steps against a 256 MB matrix, and two rounds of 32-row workgroups
+                                   (12, 8192, 8192), (40, 8192, 8192), (25, 4096, 16384)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n >= 6144:
-        want = "skinny stream %d" % (48 if n >= 11008 else 32)
+        want = "skinny stream %d" % (48 if n in (11008, 12288) else 32)
         assert VMath.gemm_plan(0, 1, m, n, k) == want
     rng = np.random.default_rng(m + k + n)
     w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
