@@ -542,6 +542,76 @@ def plan_audit(torch, kai, stream, dev, out_path):
     print(json.dumps({"plan_audit": summary, "written_to": out_path}))
 
 
+def stream_audit(torch, kai, stream, dev, out_path):
+    """The same audit for the rules of the skinny streaming kernel (csrc/skinny_stream.hip: which row counts and
+    matrices stream, and on workgroups of how many rows of W): 9..64 rows against wide weight matrices stored [N, K],
+    the matrix streamed from HBM (rotating buffers beyond the last-level cache), the chosen plan against workgroups of
+    16 / 32 / 48 rows of W and against the tiled kernels with 1..8 parts of the reduction."""
+    import ctypes
+    L = kai.load()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    I = ctypes.c_int64
+    g = torch.Generator(device=dev)
+    g.manual_seed(6)
+    mats = ((4096, 4096), (6144, 4096), (8192, 4096), (10240, 4096), (11008, 4096), (12288, 4096), (14336, 4096),
+            (16384, 4096), (4096, 8192), (8192, 8192), (11008, 8192))
+    row_counts = (12, 16, 24, 32, 48, 64)
+    cands = ["stream 16", "stream 32", "stream 48"] + ["%s split %d" % (t, sp) for t in ("flat", "small", "wide") for sp in (1, 2, 3, 4, 6, 8)]
+    rows = []
+    for n, k in mats:
+        nb = max(2, (640 << 20) // (n * k * 4))
+        ws = [torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05 for _ in range(nb)]
+        for m in row_counts:
+            x = torch.randn((m, k), device=dev, generator=g)
+            y = torch.empty((m, n), device=dev)
+
+            def time_us(iters=30):
+                for i in range(max(nb, 4)):
+                    L.kai_matmul(0, P(y), P(ws[i % nb]), P(x), I(n), I(m), I(k), 0)
+                torch.cuda.synchronize()
+                reps = []
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    for i in range(iters):
+                        if L.kai_matmul(0, P(y), P(ws[i % nb]), P(x), I(n), I(m), I(k), 0) != 0:
+                            raise RuntimeError(L.kai_last_error().decode())
+                    e1.record(stream)
+                    torch.cuda.synchronize()
+                    reps.append(e0.elapsed_time(e1) * 1e3 / iters)
+                return sorted(reps)[1]
+
+            kai.VMath.gemm_force_plan(None)
+            chosen = kai.VMath.gemm_plan(0, 1, m, n, k)
+            seen = {chosen: time_us()}
+            want = (x.double() @ ws[29 % nb].double().T)
+            for cand in cands:
+                kai.VMath.gemm_force_plan(cand)
+                text = kai.VMath.gemm_plan(0, 1, m, n, k)
+                if text in seen:
+                    continue
+                seen[text] = time_us()
+                err = float(torch.linalg.norm(y.double() - want) / torch.linalg.norm(want))
+                if not err <= 1e-5:
+                    raise RuntimeError("forced plan %r gives another result for %dx%dx%d: %.2e" % (text, m, n, k, err))
+            kai.VMath.gemm_force_plan(None)
+            seen[chosen] = min(seen[chosen], time_us())
+            best = min(seen, key=seen.get)
+            rows.append({"M": m, "N": n, "K": k, "chosen": chosen, "chosen_us": round(seen[chosen], 2), "best": best,
+                         "best_us": round(seen[best], 2), "ratio": round(seen[chosen] / seen[best], 3), "candidates": len(seen)})
+        del ws
+    geo = float(np.exp(np.mean([np.log(r["ratio"]) for r in rows])))
+    summary = {"cases": len(rows), "worst_ratio": max(r["ratio"] for r in rows), "geomean_ratio": round(geo, 4),
+               "over_1_08": sum(r["ratio"] > 1.08 for r in rows), "over_1_03": sum(r["ratio"] > 1.03 for r in rows)}
+    lines = ["| M x N x K | chosen plan | us | fastest alternative | us | chosen / fastest |", "|---|---|---|---|---|---|"]
+    for r in rows:
+        lines.append("| %d x %d x %d | %s | %.2f | %s | %.2f | %.3f |" % (r["M"], r["N"], r["K"], r["chosen"], r["chosen_us"],
+                                                                        r["best"], r["best_us"], r["ratio"]))
+    with open(out_path, "w") as f:
+        f.write(json.dumps(summary) + "\n\n" + "\n".join(lines) + "\n")
+    print(json.dumps({"stream_audit": summary, "written_to": out_path}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -552,6 +622,9 @@ def main():
     ap.add_argument("--plan-audit", metavar="FILE", default=None,
                     help="instead of the benchmark: time the dispatcher's choice against every forced alternative on "
                          "shapes around its thresholds and write the table to FILE")
+    ap.add_argument("--stream-audit", metavar="FILE", default=None,
+                    help="instead of the benchmark: the same audit for the skinny streaming kernel's rules (9..64 rows "
+                         "against wide weight matrices streamed from HBM), table written to FILE")
     ap.add_argument("--only", action="append", default=None, metavar="TEXT",
                     help="measure only the rows of the table whose name contains TEXT (may be given several times)")
     ap.add_argument("--row-warmup-ms", type=float, default=40.0,
@@ -578,6 +651,9 @@ def main():
 
     if args.plan_audit:
         plan_audit(torch, kai, stream, dev, args.plan_audit)
+        return
+    if args.stream_audit:
+        stream_audit(torch, kai, stream, dev, args.stream_audit)
         return
 
     n = 8192

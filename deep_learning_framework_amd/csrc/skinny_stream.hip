@@ -432,9 +432,9 @@ void set_skinny_stream_rows_override(int rows) { g_stream_rows_override = rows; 
 // 16 rows 90.2 -> 84.8; 8192 (256 of 32) 16 / 24 / 32 rows 23.9 / 28.5 / 32.0 -> 28.2 / 28.9 / 29.8; 7168 (224 of 32)
 // 23.8 / 27.7 / 30.7 -> 25.1 / 26.5 / 27.8; 6144 (192 of 32) 22.9 / 26.5 / 29.9 -> 22.5 / 24.8 / 26.1; 16384 (342 of 48,
 // 512 of 32) 16 rows 45.6 -> 51.4 / 51.8.  Hence: 48 rows from 9 rows of X on where the workgroups fill their rounds
-// over the compute units to 85 % (17 rows and more: one round, four fifths full: 10240 columns, 214 workgroups,
-// 33 / 48 rows 50.6 / 51.9 on the tiled kernel -> 43.6 / 45.5); 32 rows from 17 rows of X on where the workgroups
-// are one round, at least three quarters full.
+// over the compute units to 85 %, or are one round that is four fifths full (10240 columns, 214 workgroups: 12 / 16
+// rows 31.1 / 33.0 -> 27.8 / 28.4, 33 / 48 rows 50.6 / 51.9 on the tiled kernel -> 43.6 / 45.5), from 17 rows on in one
+// round only; 32 rows from 17 rows of X on where the workgroups are one round, at least three quarters full.
 // 17..24 rows on 32-row workgroups only while these are at most nine tenths of the compute units (8192 columns, 256
 // workgroups, 17 / 24 rows: 25.4 / 28.9 with 16-row workgroups, 29.5 / 30.4 with these; 6144 columns 26.0 / 27.0 -> 24.5 / 25.3).
 // Rows of 8192 steps (us, W from HBM, 16-row -> 32-row workgroups): 8192 columns 16 / 24 / 32 rows 55.1 / 59.5 / 66.3 ->
@@ -460,8 +460,7 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
     const int64_t cus = compute_units();
     const bool many = p.M > 3 * kSkinnyMaxRows;      // 49..64 rows: four blocks of X rows
     const int64_t groups48 = (p.N + 47) / 48, rounds48 = (groups48 + cus - 1) / cus;
-    if (p.M <= kSkinnyMaxRows ? groups48 * 100 >= 85 * rounds48 * cus
-                              : (rounds48 == 1 && groups48 * 100 >= (many ? 85 : 80) * cus))
+    if (rounds48 == 1 ? groups48 * 100 >= (many ? 85 : 80) * cus : (p.M <= kSkinnyMaxRows && groups48 * 100 >= 85 * rounds48 * cus))
         return 48;
     const int64_t groups32 = (p.N + 31) / 32, rounds32 = (groups32 + cus - 1) / cus;
     if (many || groups32 * 4 < 3 * cus) return 0;
