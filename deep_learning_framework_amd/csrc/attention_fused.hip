@@ -162,86 +162,150 @@ __global__ void __launch_bounds__(kFaThreads) attention_fused_kernel(const Fused
 #pragma unroll
     for (int db = 0; db < DB; db++) acc_o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // The schedule of a tile is written out (as in attention_backward.hip): its products are dealt with in NG groups
+    // -- DB groups of 8 (S^T, one 16-wide slice of the head dimension each), then 8 groups of DB (O^T, one key column
+    // of one block each) -- with fences between them.  The LDS reads of group i + 1 are issued before the products of
+    // group i (operands double buffered by group parity), the global loads of the next tile are dealt out over the
+    // first groups and its LDS stores over the last, and the barrier sits before the last group, whose products
+    // cover the first reads of the next tile.  A half tile past the end or above the diagonal is not skipped: its
+    // scores are masked to -inf and add nothing.
+    constexpr int NA = DB, NC = 8, NG = NA + NC;
+    constexpr int NLOAD = 2 * NCH;    // K chunks, then V chunks
+    constexpr int kLoadsPerGroup = (NLOAD + (NG - 3) - 1) / (NG - 3);
+    constexpr int kStoresPerGroup = 2;
+    constexpr int kStoreGroups = (NLOAD + kStoresPerGroup - 1) / kStoresPerGroup;
+    constexpr int kFirstStoreGroup = NG - 1 - kStoreGroups;     // the last store is in group NG - 2
+    static_assert(kFirstStoreGroup >= 1 && kLoadsPerGroup * (kFirstStoreGroup) >= 1, "too many chunks for this schedule");
+    auto load_one = [&](auto jc, int kt) {
+        constexpr int jj = decltype(jc)::value;
+        constexpr int i = jj % NCH;
+        const int c = tid + i * kFaThreads;
+        if (!kPartial || c < kTileChunks) {
+            if constexpr (jj / NCH == 0) rk[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, choff[i], kt * tile_bytes, 0));
+            else rv[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_v, choff[i], kt * tile_bytes, 0));
+        }
+    };
+    auto store_one = [&](auto jc, int buf) {
+        constexpr int jj = decltype(jc)::value;
+        constexpr int i = jj % NCH;
+        const int c = tid + i * kFaThreads;
+        if (!kPartial || c < kTileChunks) {
+            const int off = (c / kChunksPerKey) * kKStride + (c % kChunksPerKey) * 4;
+            if constexpr (jj / NCH == 0) *reinterpret_cast<f32x4*>(&lds_k[buf][off]) = rk[i];
+            else *reinterpret_cast<f32x4*>(&lds_v[buf][off]) = rv[i];
+        }
+    };
+    static_assert(kKStride == kVStride, "one chunk offset for both tiles");
+    // operand registers of the groups, double buffered by group parity
+    f32x4 kf[2][2];
+    float vf[2][DB];
+    auto stage = [&](auto ic, int buf) {
+        constexpr int i = decltype(ic)::value;
+        constexpr int par = i & 1;
+        if constexpr (i < NA) {
+            const float* lk = lds_k[buf] + 32 * kgp * kKStride;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+                kf[par][kb] = *reinterpret_cast<const f32x4*>(lk + (16 * kb + r16) * kKStride + 16 * i + 4 * g);
+        } else {
+            // V^T[d = 16*db + r16][key = 16*kb + 4*g + e]: 32-bit reads down a column of the tile (consecutive
+            // lanes, consecutive d: no bank conflict); a transposed tile would allow 128-bit reads but costs
+            // element-wise LDS stores with 8-way conflicts on the way in.
+            constexpr int kb = (i - NA) / 4, e = (i - NA) % 4;
+            const float* vp = lds_v[buf] + 32 * kgp * kVStride + (16 * kb + 4 * g + e) * kVStride + r16;
+#pragma unroll
+            for (int db = 0; db < DB; db++) vf[par][db] = vp[16 * db];
+        }
+    };
+
     load_tile(0);
     store_tile(0, 0);
     __syncthreads();
+    stage(std::integral_constant<int, 0>{}, 0);
 
     for (int kt = 0; kt < nkt; kt++) {
         const int buf = kt & 1;
-        load_tile(min(kt + 1, nkt - 1));   // in flight during the work below; the surplus load is never stored
+        const int nxt = min(kt + 1, nkt - 1);       // the surplus loads and stores of the last tile are never used
         const int key0 = kt * kFaKeys + 32 * kgp;   // first key of this wave's half
-        // a half tile past the end, or entirely above the diagonal of the workgroup's last query, adds nothing
-        if (key0 < T && !(p.masked && key0 > q_last)) {
-            const float* lk = lds_k[buf] + 32 * kgp * kKStride;
-            const float* lv = lds_v[buf] + 32 * kgp * kVStride;
-            // S^T: 2 blocks of 16 keys x 16 queries
-            f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
-            // the two key blocks alternate, so that no MFMA waits for the one before it
-#pragma unroll
-            for (int s = 0; s < DB; s++) {
-                f32x4 kf[2];
-#pragma unroll
-                for (int kb = 0; kb < 2; kb++)
-                    kf[kb] = *reinterpret_cast<const f32x4*>(lk + (16 * kb + r16) * kKStride + 16 * s + 4 * g);
+        // S^T: 2 blocks of 16 keys x 16 queries; the two key blocks alternate, so that no MFMA waits for the one before it
+        f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+        static_for<0, NG>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            constexpr int par = i & 1;
+            // -- the next group's operands
+            if constexpr (i + 1 < NG) {
+                stage(std::integral_constant<int, i + 1>{}, buf);
+            } else {
+                __syncthreads();     // the next tile is in LDS, and every wave has read this one
+                if (kt + 1 < nkt) stage(std::integral_constant<int, 0>{}, buf ^ 1);
+            }
+            // -- this group's share of the next tile's traffic
+            static_for<0, kLoadsPerGroup>([&](auto lc) {
+                constexpr int jj = i * kLoadsPerGroup + decltype(lc)::value;
+                if constexpr (jj < NLOAD) load_one(std::integral_constant<int, jj>{}, nxt);
+            });
+            if constexpr (i >= kFirstStoreGroup && i < NG - 1) {
+                static_for<0, kStoresPerGroup>([&](auto sc_) {
+                    constexpr int jj = (i - kFirstStoreGroup) * kStoresPerGroup + decltype(sc_)::value;
+                    if constexpr (jj < NLOAD) store_one(std::integral_constant<int, jj>{}, buf ^ 1);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // -- this group's products
+            if constexpr (i < NA) {
 #pragma unroll
                 for (int e = 0; e < 4; e++)
 #pragma unroll
                     for (int kb = 0; kb < 2; kb++)
-                        sc[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[kb][e], qf[s][e], sc[kb], 0, 0, 0);
-            }
-            // sc[kb][v] = score of (query q, key key0 + 16*kb + 4*g + v) in the base-2 domain (Q was scaled by
-            // c2 = coef * log2(e) when it was loaded): exp(coef * s - m) = 2^(c2 * s - m2), one v_exp_f32 per element
-            const bool edge_tile = key0 + 32 > T || (p.masked && key0 + 31 > q0 + 16 * qg);   // wave-uniform
-            // fp32 MFMAs and vector ALU instructions take turns on a SIMD (measured: their times add up), so the
-            // 16 compares and selects of the mask are kept off the tiles that do not need them by a real branch
-            if (edge_tile) {   // keys past the end or above the diagonal of some query of this wave
+                        sc[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[par][kb][e], qf[i][e], sc[kb], 0, 0, 0);
+                if constexpr (i == NA - 1) {
+                    // sc[kb][v] = score of (query q, key key0 + 16*kb + 4*g + v) in the base-2 domain (Q was scaled by
+                    // c2 = coef * log2(e) when it was loaded): exp(coef * s - m) = 2^(c2 * s - m2), one v_exp_f32 per element
+                    const bool edge_tile = key0 + 32 > T || (p.masked && key0 + 31 > q0 + 16 * qg);   // wave-uniform
+                    // fp32 MFMAs and vector ALU instructions take turns on a SIMD (measured: their times add up), so the
+                    // 16 compares and selects of the mask are kept off the tiles that do not need them by a real branch
+                    if (edge_tile) {   // keys past the end or above the diagonal of some query of this wave
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                        for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                    for (int v = 0; v < 4; v++) {
-                        const int key = key0 + 16 * kb + 4 * g + v;
-                        if (key >= T || (p.masked && key > q)) sc[kb][v] = -INFINITY;
+                            for (int v = 0; v < 4; v++) {
+                                const int key = key0 + 16 * kb + 4 * g + v;
+                                if (key >= T || (p.masked && key > q)) sc[kb][v] = -INFINITY;
+                            }
                     }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            float m_tile = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
-                                 fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
-            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16));
-            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32));
-            const float m_new = fmaxf(m_run, m_tile);
-            const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // nothing unmasked for this query so far
-            const float rescale = __builtin_amdgcn_exp2f(m_run - m_safe);   // 2^-inf = 0 on the first tile
-            float l_tile = 0.f;
+                    float m_tile = fmaxf(fmaxf(fmaxf(sc[0][0], sc[0][1]), fmaxf(sc[0][2], sc[0][3])),
+                                         fmaxf(fmaxf(sc[1][0], sc[1][1]), fmaxf(sc[1][2], sc[1][3])));
+                    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 16));
+                    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32));
+                    const float m_new = fmaxf(m_run, m_tile);
+                    const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // nothing unmasked for this query so far
+                    const float rescale = __builtin_amdgcn_exp2f(m_run - m_safe);   // 2^-inf = 0 on the first tile
+                    float l_tile = 0.f;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+                    for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    sc[kb][v] = __builtin_amdgcn_exp2f(sc[kb][v] - m_safe);
-                    l_tile += sc[kb][v];
+                        for (int v = 0; v < 4; v++) {
+                            sc[kb][v] = __builtin_amdgcn_exp2f(sc[kb][v] - m_safe);
+                            l_tile += sc[kb][v];
+                        }
+                    l_run = l_run * rescale + l_tile;
+                    m_run = m_new;
+                    // O^T[d, q] = O^T * rescale + sum_key V[key, d] * P[q, key]
+                    // the running maximum rarely moves after the first tiles: skip the 4*DB multiplies when no lane needs them
+                    if (__builtin_amdgcn_ballot_w64(rescale != 1.0f) != 0) {
+#pragma unroll
+                        for (int db = 0; db < DB; db++) acc_o[db] *= rescale;
+                    }
                 }
-            l_run = l_run * rescale + l_tile;
-            m_run = m_new;
-            // O^T[d, q] = O^T * rescale + sum_key V[key, d] * P[q, key]
-            // the running maximum rarely moves after the first tiles: skip the 4*DB multiplies when no lane needs them
-            if (__builtin_amdgcn_ballot_w64(rescale != 1.0f) != 0) {
+            } else {
+                // the DB output blocks alternate
+                constexpr int kb = (i - NA) / 4, e = (i - NA) % 4;
 #pragma unroll
-                for (int db = 0; db < DB; db++) acc_o[db] *= rescale;
+                for (int db = 0; db < DB; db++)
+                    acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[par][db], sc[kb][e], acc_o[db], 0, 0, 0);
             }
-            // V^T[d = 16*db + r16][key = 16*kb + 4*g + e]: 32-bit reads down a column of the tile (consecutive
-            // lanes, consecutive d: no bank conflict); a transposed tile would allow 128-bit reads but costs
-            // element-wise LDS stores with 8-way conflicts on the way in.  The DB output blocks alternate.
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const float* vp = lv + (16 * kb + 4 * g + e) * kVStride + r16;
-#pragma unroll
-                    for (int db = 0; db < DB; db++)
-                        acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(vp[16 * db], sc[kb][e], acc_o[db], 0, 0, 0);
-                }
-        }
-        if (kt + 1 < nkt) store_tile(kt + 1, buf ^ 1);
-        __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+        });
     }
 
     // merge the two key halves: the second set of waves hands (m, l, O) over through LDS
