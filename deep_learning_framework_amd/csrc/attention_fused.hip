@@ -587,7 +587,7 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
             for (int kb = 0; kb < 2; kb++) {
                 const int key = key0 + 16 * kb + 4 * g;
                 if (PVEC) {
-                    if (key < T) *reinterpret_cast<f32x4*>(Pq + key) = pr[kb];
+                    if (key < T) __builtin_nontemporal_store(pr[kb], reinterpret_cast<f32x4*>(Pq + key));
                 } else {
 #pragma unroll
                     for (int v = 0; v < 4; v++)
@@ -613,7 +613,7 @@ __global__ void __launch_bounds__(kFaThreads) attention_probs_kernel(const Probs
             const float* src = &lds_p[qq * kPStride + kk];
             const f32x4 w = {src[0], src[kPPlane], src[2 * kPPlane], src[3 * kPPlane]};
             if (q0 + qq < T && key < T)
-                *reinterpret_cast<f32x4*>(pp.P + (int64_t)b * pp.p_batch_stride + (((int64_t)(q0 + qq) * T + key) * H + h0)) = w;
+                __builtin_nontemporal_store(w, reinterpret_cast<f32x4*>(pp.P + (int64_t)b * pp.p_batch_stride + (((int64_t)(q0 + qq) * T + key) * H + h0)));
         }
     };
     stage_v(I0{}, 0, 0);
