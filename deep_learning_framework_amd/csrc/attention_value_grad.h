@@ -18,6 +18,13 @@
 // 32 bits per lane.  A wave keeps the whole block of the output (64 keys x D, or 16 keys x 4 heads x D) in
 // 4 x D / 16 accumulators and walks over every eighth step of four rows, its loads a few steps ahead; the eight
 // waves' sums meet in LDS at the end, in a fixed order, and leave as 128-bit stores.
+//
+// TR (four heads only): the same with the roles of P's two middle indices exchanged,
+//   Y[b, t, h, :] = sum_k P[b, t, k, h] * B[b, k, h, :]
+// which is VMath::mix_values (vmath.cu:6977-7025, B = V) and VMath::mult_on_heads_backward (vmath.cu:6783-6829, P = the
+// gradient of the scores, B = Q or K): the lane's row of P is the output row t = m, the step runs over the keys.
+// The four heads of a (t, k) pair are still one 128-bit word, so the loads are the same.  Here a key past the end
+// would read the next row's value into a row that IS stored, so those operand values are set to zero.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -43,8 +50,8 @@ constexpr int kVgThreads = 64 * kVgWaves;
 
 struct ValueGradParams {
     const float* P;      // [nbat, ntimes, ntimes, nhead]
-    const float* gY;     // [nbat, ntimes, nhead, npiece]
-    float* gV;           // [nbat, ntimes, nvec], head h at column h * npiece
+    const float* gY;     // the other operand: rows of gy_rs floats, head h at column h * npiece
+    float* gV;           // the output: rows of gv_rs floats, head h at column h * npiece
     int64_t p_batch_stride;
     int64_t gy_rs, gv_rs;
     int ntimes, nhead, npiece;
@@ -57,7 +64,7 @@ constexpr int value_grad_lds_floats() {
 }
 
 // bid of `total` workgroups; lds: value_grad_lds_floats<DB, HV>() floats, 16-byte aligned
-template <int DB, int HV>
+template <int DB, int HV, bool TR = false>
 __device__ __forceinline__ void attention_value_grad_body(const ValueGradParams& p, const int bid, const int total, float* lds) {
     constexpr int D = 16 * DB;
     constexpr int kVgDepth = 4;                   // steps of a wave whose loads are in flight
@@ -68,6 +75,7 @@ __device__ __forceinline__ void attention_value_grad_body(const ValueGradParams&
     constexpr int kRegion = kKeys * kRowStride;   // floats; also holds a wave's 16 * DB registers x 64 lanes
     static_assert(kRegion >= 16 * DB * 64, "a region holds a wave's accumulators");
     static_assert(4 * kRegion == value_grad_lds_floats<DB, HV>(), "the size the callers reserve");
+    static_assert(!TR || HV == 4, "the exchanged roles exist for four heads per workgroup");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -105,10 +113,12 @@ __device__ __forceinline__ void attention_value_grad_body(const ValueGradParams&
     const __amdgpu_buffer_rsrc_t rsrc_y = __builtin_amdgcn_make_buffer_rsrc(
         uniform_ptr(p.gY + (int64_t)b * T * p.gy_rs + (int64_t)h0 * D), 0, extent_y, 0x00020000);
     // byte offsets of this lane at row g of step `wave`; a step later for this wave is 32 rows further on
+    // (TR: key0 is the block's first output row t, the lane's row of P is t, the step runs over the keys)
     const int key_l = key0 + (HV == 1 ? 4 * r16 : r16);
-    int poff = (int)((((int64_t)(4 * wave + g) * T + key_l) * H) * 4);
-    int yoff = (int)(((int64_t)(4 * wave + g) * p.gy_rs + (YV ? 4 * r16 : r16)) * 4);
-    const int pstep = (int)((int64_t)4 * kVgWaves * T * H * 4);
+    int red = 4 * wave + g;      // this lane's index along the reduction in the current step
+    int poff = TR ? (int)((((int64_t)min(key_l, T) * T + red) * H) * 4) : (int)((((int64_t)red * T + key_l) * H) * 4);
+    int yoff = (int)(((int64_t)red * p.gy_rs + (YV ? 4 * r16 : r16)) * 4);
+    const int pstep = TR ? 4 * kVgWaves * H * 4 : (int)((int64_t)4 * kVgWaves * T * H * 4);
     const int ystep = (int)((int64_t)4 * kVgWaves * p.gy_rs * 4);
 
     f32x4 acc[4][DB];
@@ -121,7 +131,10 @@ __device__ __forceinline__ void attention_value_grad_body(const ValueGradParams&
     float gb[kVgDepth][HV][DB];
     auto load_step = [&](auto sc) {
         constexpr int s = decltype(sc)::value;
-        pa[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, poff, 0, 0));
+        // (TR: a key past the end is steered behind the end of the resource, where the load returns zero)
+        const int po = (!TR || red < T) ? poff : 0x7FFFFFF0;
+        pa[s] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_p, po, 0, 0));
+        if constexpr (TR) red += 4 * kVgWaves;
 #pragma unroll
         for (int i = 0; i < HV; i++) {
             if constexpr (YV) {

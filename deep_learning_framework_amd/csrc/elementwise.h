@@ -106,6 +106,12 @@ int attention_value_grad_heads(const float* gv, const float* gy, const float* pp
                                int64_t nhead, int64_t npiece);
 int launch_attention_value_grad(float* gv, const float* gy, const float* pp, int64_t nbat, int64_t ntimes, int64_t nvec,
                                 int64_t nhead, int64_t npiece, hipStream_t stream);
+// the same kernel with the roles of P's middle indices exchanged: Y[b,t,h,:] = sum_k P[b,t,k,h] * B[b,k,h,:] (mix_values,
+// mult_on_heads_backward) for head counts in whole fours and head sizes up to 64
+bool attention_heads_mix_applies(const float* out, int64_t out_rs, const float* pp, const float* other, int64_t other_rs,
+                                 int64_t ntimes, int64_t nhead, int64_t npiece);
+int launch_attention_heads_mix(float* out, int64_t out_rs, const float* pp, const float* other, int64_t other_rs, int64_t nbat,
+                               int64_t ntimes, int64_t nhead, int64_t npiece, hipStream_t stream);
 // attention_backward.hip: gQ and gK of the attention block from gM, P (and M) without storing gP or gS
 bool attention_backward_applies(const float* gq, const float* gk, const float* gm, const float* m, const float* pp,
                                 const float* q, const float* k, const float* v, int64_t ntimes, int64_t nvec,

@@ -535,6 +535,8 @@ int kai_mult_on_heads_backward(int device, float* pgQKV, const float* pgp, const
     KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
     if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
     KAI_REQUIRE_PTR(pgQKV); KAI_REQUIRE_PTR(pgp); KAI_REQUIRE_PTR(pQKV);
+    if (attention_heads_mix_applies(pgQKV, nvec, pgp, pQKV, nvec, ntimes, nhead, npiece))
+        return launch_attention_heads_mix(pgQKV, nvec, pgp, pQKV, nvec, nbat, ntimes, nhead, npiece, current_stream());
     // per (b,h): G[t,p] = sum_k gp[b,t,k,h] * KQ[b,k,h*npiece+p]
     GemmDesc d;
     d.A = pgp; d.B = pQKV; d.C = pgQKV;
@@ -580,6 +582,8 @@ int kai_mix_values(int device, float* py, const float* pp, const float* pV, int6
     KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
     if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) return KAI_OK;
     KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pp); KAI_REQUIRE_PTR(pV);
+    if (attention_heads_mix_applies(py, nhead * npiece, pp, pV, nvec, ntimes, nhead, npiece))
+        return launch_attention_heads_mix(py, nhead * npiece, pp, pV, nvec, nbat, ntimes, nhead, npiece, current_stream());
     // per (b,h): Y[q,p] = sum_k P[b,q,k,h] * V[b,k,h*npiece+p]; Y is [nbat, ntimes, nhead, npiece]
     GemmDesc d;
     d.A = pp; d.B = pV; d.C = py;
@@ -913,8 +917,8 @@ int kai_gemm_force_plan(const char* text) { return set_forced_gemm_plan(text); }
 int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, char* out,
                        int buflen) {
     KAI_REQUIRE(out != nullptr && buflen > 0, KAI_ERR_INVALID_POINTER, "null output buffer");
-    KAI_REQUIRE(which >= 0 && which <= 3, KAI_ERR_INVALID_ARGUMENT,
-                "which must be 0 (forward), 1 (forward, training), 2 (backward) or 3 (value gradient)");
+    KAI_REQUIRE(which >= 0 && which <= 4, KAI_ERR_INVALID_ARGUMENT,
+                "which must be 0 (forward), 1 (forward, training), 2 (backward), 3 (value gradient) or 4 (mix_values)");
     KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
     // 16-byte aligned operands are assumed: a pointer value that satisfies every alignment test
     const float* a = reinterpret_cast<const float*>(uintptr_t(256));
@@ -929,6 +933,9 @@ int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, in
     else if (which == 3) {
         const int hv = attention_value_grad_heads(a, a, a, ntimes, nvec, nhead, npiece);
         text = hv == 1 ? "streamed, one head per workgroup" : hv == 4 ? "streamed, four heads per workgroup" : "tiled";
+    } else if (which == 4) {
+        text = attention_heads_mix_applies(a, nhead * npiece, a, a, nvec, ntimes, nhead, npiece) ? "streamed, four heads per workgroup"
+                                                                                               : "tiled";
     }
     snprintf(out, (size_t)buflen, "%s", text.c_str());
     return KAI_OK;

@@ -434,9 +434,9 @@ class VMath:
     @staticmethod
     def attention_plan(which, nbat, ntimes, nvec, nhead, npiece):
         """How an attention entry point would run this geometry (host arithmetic only): which = "forward",
-        "forward_train", "backward" or "value_gradient"."""
+        "forward_train", "backward", "value_gradient" or "mix_values" (also mult_on_heads_backward)."""
         buf = ctypes.create_string_buffer(128)
-        code = {"forward": 0, "forward_train": 1, "backward": 2, "value_gradient": 3}[which]
+        code = {"forward": 0, "forward_train": 1, "backward": 2, "value_gradient": 3, "mix_values": 4}[which]
         _ck(load().kai_attention_plan(code, nbat, ntimes, nvec, nhead, npiece, buf, 128))
         return buf.value.decode()
 

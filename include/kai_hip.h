@@ -346,7 +346,8 @@ int kai_attention_forward(int device, float* py, const float* pQ, const float* p
  * kai_attention_forward_train ("fused", "fused, four heads per workgroup" or "separate"), 2 kai_attention_backward
  * ("fused rows and value gradient in one launch", "fused rows + value gradient" (two launches) or "separate"), 3
  * kai_mix_values_backward_value, also the value gradient inside kai_attention_backward ("streamed, one head per
- * workgroup", "streamed, four heads per workgroup" or "tiled").
+ * workgroup", "streamed, four heads per workgroup" or "tiled"), 4 kai_mix_values and kai_mult_on_heads_backward
+ * ("streamed, four heads per workgroup" or "tiled").
  * Host arithmetic only, nothing is launched and no GPU is needed.
  * For maintainers and tests. */
 int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, char* out,

@@ -330,6 +330,9 @@ def test_attention_plans():
     assert plan("backward", 4, 512, 512, 8, 64) == "fused rows and value gradient in one launch"
     assert plan("value_gradient", 32, 512, 64, 1, 64) == "streamed, one head per workgroup"
     assert plan("value_gradient", 4, 512, 512, 8, 64) == "streamed, four heads per workgroup"
+    assert plan("mix_values", 4, 512, 512, 8, 64) == "streamed, four heads per workgroup"
+    assert plan("mix_values", 32, 512, 64, 1, 64) == "tiled"            # one head: the reduction index is the contiguous one
+    assert plan("mix_values", 2, 384, 1536, 12, 128) == "tiled"        # head sizes beyond 64
     # head sizes 96 and 128, twelve heads of 64, lengths that are no multiple of 32, six heads
     for nbat, ntimes, nhead, npiece in ((2, 384, 12, 64), (1, 500, 16, 96), (2, 1024, 8, 128), (3, 200, 6, 32)):
         nvec = nhead * npiece

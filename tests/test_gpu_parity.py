@@ -894,6 +894,44 @@ def test_value_gradient_streamed(nbat, ntimes, nhead, npiece, extra):
     np.testing.assert_array_equal(got[:, :, nhead * npiece:], start[:, :, nhead * npiece:])
 
 
+# mix_values and mult_on_heads_backward on the same kernel with the roles of P's middle indices exchanged (head counts
+# in whole fours, head sizes up to 64): lengths that leave the last block of rows and the last step of four keys partly
+# empty (a key past the end must not bring the next row's values in), a vector wider than the heads
+@pytest.mark.parametrize("nbat,ntimes,nhead,npiece,extra", [
+    (1, 77, 4, 16, 0), (2, 130, 8, 32, 0), (1, 97, 12, 48, 0), (4, 512, 8, 64, 0), (2, 384, 12, 64, 0), (1, 50, 4, 64, 32),
+    (1, 1030, 4, 32, 0), (3, 33, 16, 16, 0)])
+def test_heads_products_streamed(nbat, ntimes, nhead, npiece, extra):
+    nvec = nhead * npiece + extra
+    assert VMath.attention_plan("mix_values", nbat, ntimes, nvec, nhead, npiece) == "streamed, four heads per workgroup"
+    rng = np.random.default_rng(nbat * 1000 + ntimes + nhead + npiece)
+    # no zeros, and large values right behind every row's end, so that a read past the row shows
+    p = rng.standard_normal((nbat, ntimes, ntimes, nhead)).astype(np.float32) * 0.1 + 1.0
+    p[:, :, 0, :] += 100.0
+    v = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    used = slice(0, nhead * npiece)
+    vc = np.ascontiguousarray(v[:, :, used])
+    small = nbat * ntimes * ntimes * nhead * npiece <= 1 << 28
+    batches = range(nbat) if small else (0, nbat - 1)
+    # mix_values: Y [nbat, ntimes, nhead, npiece]
+    y = DB(nbat * ntimes * nhead * npiece * 4)
+    VMath.mix_values(0, y, dev(p), dev(v), nbat, ntimes, nvec, nhead, npiece)
+    got = y.to_numpy((nbat, ntimes, nhead * npiece))
+    for b in batches:
+        check(got[b:b + 1], ko.mix_values(p[b:b + 1], vc[b:b + 1], nhead), what="mix_values, batch entry %d" % b)
+    # mult_on_heads_backward: G [nbat, ntimes, nvec], columns beyond the heads untouched
+    start = rng.standard_normal((nbat, ntimes, nvec)).astype(np.float32)
+    gq = dev(start)
+    VMath.mult_on_heads_backward(0, gq, dev(p), dev(v), nbat, ntimes, nvec, nhead, npiece)
+    got = gq.to_numpy((nbat, ntimes, nvec))
+    for b in batches:
+        check(got[b:b + 1, :, used], ko.mult_on_heads_backward(p[b:b + 1], vc[b:b + 1], nhead),
+              what="mult_on_heads_backward, batch entry %d" % b)
+    np.testing.assert_array_equal(got[:, :, nhead * npiece:], start[:, :, nhead * npiece:])
+    f64 = np.matmul(p.astype(np.float64).transpose(0, 3, 1, 2),
+                    vc.reshape(nbat, ntimes, nhead, npiece).astype(np.float64).transpose(0, 2, 1, 3))   # [b, h, t, d]
+    assert rel_fro(got[:, :, used], f64.transpose(0, 2, 1, 3).reshape(nbat, ntimes, -1)) <= REL_FRO_TOL
+
+
 # one case per kernel variant: rows in registers (1 head; 2..128 heads, short and long axis), rows through
 # LDS (long axis, odd lengths), one thread per head (more than 128 heads)
 SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 512, 8), (3, 20, 128), (2, 9, 129),
