@@ -539,17 +539,25 @@ bool attention_backward_applies(const float* gq, const float* gk, const float* g
 
 // gv null: the rows kernel alone; else the one-launch kernel, whose value gradient workgroups follow the rows workgroups
 template <int DB, int KB, bool MERGE_NOVEC = (DB <= 4)>
-static void launch_rows(const AttnBwdParams& p, const vgrad::ValueGradParams* v, int64_t vblocks, bool pvec, dim3 grid,
-                        hipStream_t stream) {
+static int launch_rows(const AttnBwdParams& p, const vgrad::ValueGradParams* v, int64_t vblocks, bool pvec, dim3 grid,
+                       hipStream_t stream) {
     const dim3 block(kAbThreads);
     if (v == nullptr) {
         if (pvec) attention_backward_rows_kernel<DB, KB, true><<<grid, block, 0, stream>>>(p);
         else attention_backward_rows_kernel<DB, KB, false><<<grid, block, 0, stream>>>(p);
-        return;
+        return KAI_OK;
     }
     const dim3 all(grid.x + (unsigned)vblocks);
-    if (pvec) attention_backward_all_kernel<DB, KB, true><<<all, block, 0, stream>>>(p, *v, (int)grid.x);
-    else if constexpr (MERGE_NOVEC) attention_backward_all_kernel<DB, KB, false><<<all, block, 0, stream>>>(p, *v, (int)grid.x);
+    if (pvec) {
+        attention_backward_all_kernel<DB, KB, true><<<all, block, 0, stream>>>(p, *v, (int)grid.x);
+        return KAI_OK;
+    }
+    if constexpr (MERGE_NOVEC) {
+        attention_backward_all_kernel<DB, KB, false><<<all, block, 0, stream>>>(p, *v, (int)grid.x);
+        return KAI_OK;
+    }
+    // four heads per workgroup exist for head sizes up to 64 only; attention_backward_one_launch never sends others here
+    return fail(KAI_ERR_INVALID_ARGUMENT, "attention backward: no one-launch kernel for this head size with several heads");
 }
 
 // Whether kai_attention_backward runs this geometry as ONE launch: the rows kernel applies (the caller has checked)
@@ -589,14 +597,14 @@ int launch_attention_backward_rows(float* gq, float* gk, float* gv, const float*
     }
     const vgrad::ValueGradParams* vptr = gv != nullptr ? &vp : nullptr;
     switch (npiece / 16) {
-    case 1: launch_rows<1, 2>(p, vptr, vblocks, pvec, grid, stream); break;
-    case 2: launch_rows<2, 2>(p, vptr, vblocks, pvec, grid, stream); break;
-    case 3: launch_rows<3, 2>(p, vptr, vblocks, pvec, grid, stream); break;
-    case 4: launch_rows<4, 2>(p, vptr, vblocks, pvec, grid, stream); break;
-    case 5: launch_rows<5, 2>(p, vptr, vblocks, pvec, grid, stream); break;
-    case 6: launch_rows<6, 1>(p, vptr, vblocks, pvec, grid, stream); break;
-    case 7: launch_rows<7, 1>(p, vptr, vblocks, pvec, grid, stream); break;
-    default: launch_rows<8, 1>(p, vptr, vblocks, pvec, grid, stream); break;
+    case 1: KAI_TRY((launch_rows<1, 2>(p, vptr, vblocks, pvec, grid, stream))); break;
+    case 2: KAI_TRY((launch_rows<2, 2>(p, vptr, vblocks, pvec, grid, stream))); break;
+    case 3: KAI_TRY((launch_rows<3, 2>(p, vptr, vblocks, pvec, grid, stream))); break;
+    case 4: KAI_TRY((launch_rows<4, 2>(p, vptr, vblocks, pvec, grid, stream))); break;
+    case 5: KAI_TRY((launch_rows<5, 2>(p, vptr, vblocks, pvec, grid, stream))); break;
+    case 6: KAI_TRY((launch_rows<6, 1>(p, vptr, vblocks, pvec, grid, stream))); break;
+    case 7: KAI_TRY((launch_rows<7, 1>(p, vptr, vblocks, pvec, grid, stream))); break;
+    default: KAI_TRY((launch_rows<8, 1>(p, vptr, vblocks, pvec, grid, stream))); break;
     }
     return check_launch(gv != nullptr ? "attention_backward_all_kernel" : "attention_backward_rows_kernel");
 }
