@@ -12,6 +12,7 @@
 //               rows the vector ALU would need 8 LDS bytes of X per byte of W and become LDS-bound.
 //               It is also the plan for unaligned or ragged skinny operands (scalar loads).
 #include "gemv_skinny.h"
+#include <stdlib.h>
 
 #include "act_funcs.h"
 
@@ -579,13 +580,25 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
     if (vec && p.K >= 256) {
         if (p.M == 1) return launch_gemv_rows(p, stream);
         if (skinny_stream8_applies(p)) return launch_skinny_stream8(p, stream);
-        // 3 and 4 rows: the streaming kernel once its workgroups (16 rows of W each) cover the chip (measured at
-        // 4096 x 4096: 12.6 against 16.0 us, 11008 x 4096: 30 against 40; at 2048 x 8192, 128 workgroups:
-        // 19.8 against 15.3); 2 rows: the streaming kernel where its slices are written out (K a multiple of 4096:
-        // 12.3 against 12.45 us at 4096 x 4096, 29.0 against 30.5 at 11008 x 4096), the slice kernel otherwise
-        // (4096 x 11008: 30.7 against 33.3)
-        if ((p.M >= 3 || p.K % 4096 == 0) && p.N >= 16 * (int64_t)compute_units() && skinny_stream_applies(p))
-            return launch_skinny_stream(p, stream);
+        // 2..4 rows: the streaming kernel (16 rows of W per workgroup) or the slice kernels (8 rows per workgroup,
+        // a second round of workgroups beyond 8 rows per compute unit).  Measured, us per call with W from HBM,
+        // slice kernel -> streaming kernel:
+        //   * N >= 16 per compute unit: 3 and 4 rows 4096 x 4096 16.0 -> 12.6, 11008 x 4096 40 -> 30; 2 rows where
+        //     the streaming kernel's slices are written out (K a multiple of 4096) 12.45 -> 12.3, 30.5 -> 29.0, else
+        //     the slice kernel (4096 x 11008: 30.7 against 33.3);
+        //   * more than 8 and fewer than 16 per compute unit, 3 and 4 rows: 3072 x 4096 12.4 -> 10.0, 2304 x 4096
+        //     11.3 -> 9.2, 3072 x 5120 18.2 -> 13.2, 3072 x 8192 21.3 -> 19.2, 3840 x 12288 35.5 -> 30.8, 2304 x 1024
+        //     6.0 -> 5.3 (every K from 1024 to 12288 by 10..38 %), except the rolled loop over long rows
+        //     (K > 8192 that is not a multiple of 4096: 3072 x 11008 27.2 -> 29.3, from 13 per compute unit on
+        //     31.6 -> 30.4); 2 rows with K = 4096 / 8192 by 2..5 %;
+        //   * 8 per compute unit and fewer: the slice kernels (2048 x 8192, 128 workgroups: 15.3 against 19.8;
+        //     2048 x 3072 8.4 against 8.8) unless K <= 2048 (2048 x 2048 6.9 -> 6.4, 2048 x 1024 5.8 -> 5.3).
+        const int64_t cus = compute_units();
+        bool streamed = p.N >= 16 * cus && (p.M >= 3 || p.K % 4096 == 0);
+        if (!streamed && p.N > 8 * cus)
+            streamed = p.M >= 3 ? !(p.K > 8192 && p.K % 4096 != 0 && p.N < 13 * cus) : (p.K % 4096 == 0 && p.K <= 8192);
+        if (!streamed && p.M >= 3 && p.N == 8 * cus && p.K <= 2048) streamed = true;
+        if (streamed && skinny_stream_applies(p)) return launch_skinny_stream(p, stream);
         if (p.M == 2) return launch_slice<2>(p, stream);
         if (p.M <= 4) return launch_slice<4>(p, stream);
     }

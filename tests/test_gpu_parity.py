@@ -407,7 +407,11 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # 33..64 rows: three and four blocks of X rows
                                    (48, 4096, 8192), (64, 4096, 11008), (33, 4096, 6160),
                                    # rows of 8192 steps against a 256 MB matrix, and two rounds of 32-row workgroups
-                                   (12, 8192, 8192), (40, 8192, 8192), (25, 4096, 16384)])
+                                   (12, 8192, 8192), (40, 8192, 8192), (25, 4096, 16384),
+                                   # 2..4 rows against 9..15 rows of W per compute unit: the streaming kernel, except
+                                   # the rolled loop over long rows (the slice kernel keeps 3072 x 11008)
+                                   (3, 4096, 2304), (4, 5120, 3072), (4, 12288, 3840), (2, 8192, 2560), (3, 2048, 2048),
+                                   (4, 1024, 2320), (4, 11008, 3072), (3, 11008, 3328), (2, 12288, 3072)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n >= 6144:
         want = "skinny stream %d" % (48 if n in (11008, 12288) else 32)
