@@ -578,7 +578,20 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
     }
     const bool vec = p.K % 4 == 0 && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X);
     if (vec && p.K >= 256) {
-        if (p.M == 1) return launch_gemv_rows(p, stream);
+        if (p.M == 1) {
+            // The batch-1 kernel walks K in chunks of 4096 with all of a chunk's loads in flight; a chunk that K does
+            // not fill is loaded all the same (clamped), so it is the kernel for K in whole chunks only.  Other K:
+            // the slice kernel with one row of X (slices of 1024), us per call with W from HBM, 5120 x 2048
+            // 14.8 -> 8.7, 8192 x 2048 17.4 -> 11.8, 5120 x 3072 18.2 -> 11.3, 4096 x 11008 31.7 -> 29.3, 1024 x 11008
+            // 14.2 -> 9.9, 11008 x 5120 37.3 -> 33.1 (K = 1024 .. 11008: 7..69 %); rows shorter than a slice, and
+            // K = 1024 up to 8 rows of W per compute unit, through the streaming kernel (2048 x 512 5.5 -> 4.1,
+            // 1024 x 1024 5.4 -> 4.5).  K in whole chunks: 4096 x 4096 11.3 against 11.7 / 12.2, 5120 x 4096 14.4
+            // against 17.0 / 17.5.
+            if (p.K % 4096 == 0) return launch_gemv_rows(p, stream);
+            if ((p.K < kSliceK || (p.K == kSliceK && p.N <= 8 * (int64_t)compute_units())) && skinny_stream_applies(p))
+                return launch_skinny_stream(p, stream);
+            return launch_slice<1>(p, stream);
+        }
         if (skinny_stream8_applies(p)) return launch_skinny_stream8(p, stream);
         // 2..4 rows: the streaming kernel (16 rows of W per workgroup) or the slice kernels (8 rows per workgroup,
         // a second round of workgroups beyond 8 rows per compute unit).  Measured, us per call with W from HBM,

@@ -411,7 +411,11 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # 2..4 rows against 9..15 rows of W per compute unit: the streaming kernel, except
                                    # the rolled loop over long rows (the slice kernel keeps 3072 x 11008)
                                    (3, 4096, 2304), (4, 5120, 3072), (4, 12288, 3840), (2, 8192, 2560), (3, 2048, 2048),
-                                   (4, 1024, 2320), (4, 11008, 3072), (3, 11008, 3328), (2, 12288, 3072)])
+                                   (4, 1024, 2320), (4, 11008, 3072), (3, 11008, 3328), (2, 12288, 3072),
+                                   # one row with K not in whole chunks of 4096: the slice kernel, short rows the
+                                   # streaming kernel
+                                   (1, 2048, 5120), (1, 11008, 4096), (1, 512, 2048), (1, 1024, 1024), (1, 1024, 4100),
+                                   (1, 3072, 1031), (1, 260, 300), (1, 5124, 4096)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n >= 6144:
         want = "skinny stream %d" % (48 if n in (11008, 12288) else 32)
