@@ -12,7 +12,6 @@
 //               rows the vector ALU would need 8 LDS bytes of X per byte of W and become LDS-bound.
 //               It is also the plan for unaligned or ragged skinny operands (scalar loads).
 #include "gemv_skinny.h"
-#include <stdlib.h>
 
 #include "act_funcs.h"
 

@@ -71,10 +71,11 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // of a slice is written out (16 tiles, every wait counted exactly by the compiler): 12.2 us at M = 4 against
 // 12.9 us for the rolled loop that other lengths use.
 //
-// XL (with SLICES): 1 = at most 8 rows of X (one load per tile), 2 = more (two); 0 = decided per tile from M.  With
-// the number of X loads a compile-time constant and every tile inside K, the written-out slice has no branch left.
+// XL (whole tiles): 1 = at most 8 rows of X (one load per tile), 2 = more (two); 0 = decided per tile from M.  With
+// the number of X loads a compile-time constant and every tile inside K, the written-out slice has no branch left,
+// and the rolled loop only its own.
 //
-// XB: blocks of 16 rows of X.  2 (17..32 rows; whole tiles and written-out slices only, XL = 3 or 4): a tile of W meets
+// XB: blocks of 16 rows of X.  2 (17..32 rows; whole tiles only, XL = 3 or 4): a tile of W meets
 // two tiles of X and a wave keeps two accumulators -- W still streams once, where a tiled product of 17..32 rows
 // cuts K over workgroups and sums the parts in a second launch.  3 and 4 (33..64 rows, XL = 5..8) with workgroups of
 // 32 or 48 rows of W only: 6 to 12 accumulators per wave, and the matrix cores set the time.
@@ -94,8 +95,9 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     constexpr int WB = WR <= 16 ? 1 : WR / 16;      // blocks of 16 rows of W
     constexpr int kWTileRows = 16 * WB;
     __shared__ __attribute__((aligned(16))) float lds_w[kSsWaves][kWTileRows * kSsTileStride];
-    static_assert(XB == 1 || (XB >= 2 && XB <= 4 && WHOLE && SLICES && XL > kSsLoadsPerTile * (XB - 1) && XL <= kSsLoadsPerTile * XB),
-                  "several blocks of X rows exist for whole tiles in written-out slices");
+    static_assert(XB == 1 || (XB >= 2 && XB <= 4 && WHOLE && (SLICES || XB == 2) && XL > kSsLoadsPerTile * (XB - 1) && XL <= kSsLoadsPerTile * XB),
+                  "several blocks of X rows exist for whole tiles (three and four: in written-out slices)");
+    static_assert(XL == 0 || WHOLE, "a compile-time number of X loads: whole tiles");
     static_assert(XB <= 2 || WR >= 32, "three and four blocks of X rows: with two or three blocks of W rows only");
     // tiles of a wave in registers (written-out slices): with three and four blocks of X rows a tile is 10 to 14 loads
     // per lane, and two tiles are what the registers hold
@@ -194,7 +196,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         }
     };
     auto consume = [&](const f32x4(&w)[kWRegs], const f32x4(&x)[kXLoads], int kt) {
-        if ((SLICES && XL) || kt < p.K) {   // uniform
+        if ((WHOLE && XL) || kt < p.K) {   // uniform (whole tiles with a fixed number of X loads: the callers pass tiles inside K only)
 #pragma unroll
             for (int j = 0; j < kWLoads; j++) {
                 const int row = kSsRowsPerLoad * j + lrow;
@@ -367,8 +369,25 @@ static bool stream_size_rule(int64_t n, int64_t k) {
 // 33..64 rows (three and four blocks of X rows) run here only where workgroups of 32 or 48 rows of W apply: with
 // 16 rows of W a workgroup would load four times as many bytes of X as of W.
 static bool stream_many_rows_base(const SkinnyParams& p) {
-    return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && p.K % (kSsWaves * 512) == 0 && p.N % 16 == 0 &&
-           p.N >= 16 * (int64_t)compute_units() && stream_size_rule(p.N, p.K) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
+    // Which K and N, by the row count.  Rows in written-out slices (K a multiple of 4096): from 16 rows of W per
+    // compute unit on, K = 4096 from 9 on (17 / 24 / 32 rows, us with W from HBM | from the last-level cache, fastest
+    // tiled plan -> here: 3072 x 4096 20.1 / 20.3 / 19.5 -> 13.8 / 15.1 / 16.7 | 15.5 / 15.8 / 18.4 -> 13.4 / 14.5 / 16.0;
+    // 2304 x 4096 19.2 / 19.6 / 18.4 -> 13.5 / 14.7 / 16.4 | 15.2 / 15.5 / 18.2 -> 13.1 / 14.1 / 15.8; at 8192 steps
+    // 3072 columns 23.5 -> 25.0 from the cache; 2048 columns and fewer: no gain at any K).  Other K in whole tiles,
+    // 17..32 rows only, through the rolled loop: 1024..2048 steps from 9 rows of W per compute unit on (4096 x 2048
+    // 14.7 / 14.8 / 15.1 -> 9.9 / 10.3 / 11.5 | 11.7 / 12.1 / 14.3 -> 9.3 / 9.8 / 10.6; 3072 x 1024 10.9 / 12.2 / 13.8 ->
+    // 6.9 / 7.3 / 7.8; 8192 x 2048 20.9 / 21.2 / 21.5 -> 16.6 / 17.9 / 19.5 | 15.9 / 16.2 / 19.5 -> 15.6 / 16.6 / 18.1),
+    // up to 4096 steps for 12..16 rows of W per compute unit (4096 x 3072 18.7 / 18.8 / 18.7 -> 14.5 / 15.7 / 17.6 |
+    // 14.6 / 14.8 / 17.5 -> 13.7 / 14.8 / 16.5; 5120 x 3072 and wider lose, 21.4 -> 24.1, and so does 2304 x 3072 from
+    // the cache); longer rows (5120, 6144, 11008 steps) gain with W from HBM but lose 8..30 % from the cache.
+    const int64_t cus = compute_units();
+    bool k_ok;
+    if (p.K % (kSsWaves * 512) == 0) k_ok = p.N >= (p.K == kSsWaves * 512 && p.M <= 2 * kSkinnyMaxRows ? 9 : 16) * cus;
+    else if (p.M > 2 * kSkinnyMaxRows || p.K % kSsTileK != 0) k_ok = false;
+    else if (p.K >= 1024 && p.K <= 2048) k_ok = p.N >= 9 * cus;
+    else k_ok = p.K > 2048 && p.K < 4096 && p.N >= 12 * cus && p.N <= 16 * cus;
+    return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && k_ok && p.N % 16 == 0 &&
+           stream_size_rule(p.N, p.K) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
            (15 * p.ldw + p.K) * 4 < (1ll << 31) && ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
 }
 
@@ -489,8 +508,16 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     if (p.M > kSkinnyMaxRows) {
         if (!skinny_stream32_applies(p) || p.M > 2 * kSkinnyMaxRows)
             return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
-        if (p.M <= 24) skinny_stream_kernel<true, true, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        if (!slices && p.M <= 24) skinny_stream_kernel<true, false, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        else if (!slices) skinny_stream_kernel<true, false, 4, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        else if (p.M <= 24) skinny_stream_kernel<true, true, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         else skinny_stream_kernel<true, true, 4, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        return check_launch("skinny_stream_kernel");
+    }
+    // (the rolled loop with one load of X per tile as a compile-time fact: 4096 x 2048 at 4 rows 8.1 -> 7.6 us, 3072 x
+    // 3072 10.0 -> 9.6, 1..3 % elsewhere; with two, 9..16 rows, -2..+2 %: those keep the count read from M)
+    if (whole && !slices && p.M <= 8) {
+        skinny_stream_kernel<true, false, 1><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         return check_launch("skinny_stream_kernel");
     }
     if (whole && slices && p.M <= 8) skinny_stream_kernel<true, true, 1><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);

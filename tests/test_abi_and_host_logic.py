@@ -261,6 +261,10 @@ GEMM_PLANS = [
     ((0, 1, 48, 4096, 4096), "mfma small ragged pipelined staged 4 split 4"),   # 33..64 rows: one row of 64-row tiles with edges, 4 parts of K, one workgroup per unit
     ((0, 1, 96, 4096, 4096), "mfma flat ragged pipelined split 8"),  # 65..96 rows: three row tiles of 32, not two of 64
     ((0, 1, 32, 4096, 4096), "skinny"),                              # 17..32 rows, K a multiple of 4096: W streams once
+    ((0, 1, 24, 4096, 2048), "skinny"),                              # ... or K of 1024..2048 in whole tiles (the rolled loop), from 9 rows of W per compute unit
+    ((0, 1, 17, 2304, 1024), "skinny"),
+    ((0, 1, 32, 3072, 4096), "skinny"),                              # K = 4096 likewise from 9 rows of W per compute unit
+    ((0, 1, 17, 4096, 3072), "skinny"),                              # 2048 < K < 4096: 12..16 rows of W per compute unit only
     ((0, 1, 32, 4096, 11008), "mfma flat whole split 8"),            # one row of whole 32 x 128 tiles: the simple schedule
     ((0, 0, 32, 4096, 4096), "mfma flat whole split 8"),             # ... and a [K, N] weight matrix
     # 129..160 rows: five row tiles of 32 where their workgroups fill the compute units' rounds

@@ -415,11 +415,17 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # one row with K not in whole chunks of 4096: the slice kernel, short rows the
                                    # streaming kernel
                                    (1, 2048, 5120), (1, 11008, 4096), (1, 512, 2048), (1, 1024, 1024), (1, 1024, 4100),
-                                   (1, 3072, 1031), (1, 260, 300), (1, 5124, 4096)])
+                                   (1, 3072, 1031), (1, 260, 300), (1, 5124, 4096),
+                                   # 17..32 rows through the rolled loop (K in whole tiles, not in whole slices), and
+                                   # K = 4096 against 9..15 rows of W per compute unit
+                                   (17, 2048, 4096), (32, 1024, 3072), (24, 3072, 4096), (25, 4096, 3072), (17, 4096, 2304),
+                                   (32, 2048, 11008), (20, 1056, 2320), (8, 2080, 4096), (5, 11008, 4096)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
-    if n >= 6144:
+    if n >= 6144 and k % 4096 == 0:
         want = "skinny stream %d" % (48 if n in (11008, 12288) else 32)
         assert VMath.gemm_plan(0, 1, m, n, k) == want
+    elif m > 16 and k % 4096 != 0:
+        assert VMath.gemm_plan(0, 1, m, n, k) == "skinny"      # 16-row workgroups, rolled loop
     rng = np.random.default_rng(m + k + n)
     w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
     x = rng.standard_normal((m, k)).astype(np.float32)
