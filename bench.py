@@ -448,7 +448,7 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
     return rows
 
 
-def plan_audit(torch, kai, stream, dev, out_path):
+def plan_audit(torch, kai, stream, dev, out_path, shapes_text=None):
     """Times the dispatcher's choice against every alternative it could have made (forced through
     kai_gemm_force_plan) on shapes that sit on both sides of the thresholds coded in csrc/gemm_dispatch.hip, in the
     three operand forms of the dense layer, and writes a table: chosen plan, its time, the fastest alternative, the
@@ -468,6 +468,8 @@ def plan_audit(torch, kai, stream, dev, out_path):
             shapes.append((m,) + nk)
     shapes += [(64, 512, 784), (256, 1024, 1024), (1000, 333, 777), (512, 2048, 2048), (1024, 1024, 1024),
                (32, 4096, 4096), (33, 4096, 4096), (96, 4096, 11008), (200, 6656, 4096), (144, 5120, 4096)]
+    if shapes_text:   # "M,N,K;M,N,K;...": the caller's own shapes instead of the built-in list
+        shapes = [tuple(int(v) for v in item.split(",")) for item in shapes_text.split(";") if item.strip()]
     tiles = ("medium", "wide", "small", "flat")
     splits = (1, 2, 3, 4, 6, 8, 12, 16)
     forms = (("NT", 0, 1), ("NN", 0, 0), ("TN", 1, 0))
@@ -622,6 +624,8 @@ def main():
     ap.add_argument("--plan-audit", metavar="FILE", default=None,
                     help="instead of the benchmark: time the dispatcher's choice against every forced alternative on "
                          "shapes around its thresholds and write the table to FILE")
+    ap.add_argument("--plan-audit-shapes", metavar="M,N,K;...", default=None,
+                    help="with --plan-audit: audit these shapes instead of the built-in list")
     ap.add_argument("--stream-audit", metavar="FILE", default=None,
                     help="instead of the benchmark: the same audit for the skinny streaming kernel's rules (9..64 rows "
                          "against wide weight matrices streamed from HBM), table written to FILE")
@@ -650,7 +654,7 @@ def main():
     dev = torch.device("cuda:0")
 
     if args.plan_audit:
-        plan_audit(torch, kai, stream, dev, args.plan_audit)
+        plan_audit(torch, kai, stream, dev, args.plan_audit, args.plan_audit_shapes)
         return
     if args.stream_audit:
         stream_audit(torch, kai, stream, dev, args.stream_audit)

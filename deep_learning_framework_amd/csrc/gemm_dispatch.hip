@@ -184,7 +184,13 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // 17..32 rows against at least 256 columns: a 64-row tile would spend half of its MFMAs on padding, and these
     // products are bound by the stream of the other operand (32 x 4096 x 4096: 30.6 -> 21.5 us).  65..96 rows
     // likewise: three row tiles of 32 instead of two of 64 (96 x 4096 x 4096: 55 -> 43 us; 144 rows: 67 against 73)
-    if (plan.tile == kTileSmall && (d.M <= 32 || (d.M > 64 && d.M <= 96)) && d.N >= 256) plan.tile = kTileFlat;
+    // One row of them needs enough column tiles: while the 64 x 64 tile's column tiles with the most parts of K (16)
+    // still find a compute unit each (1024 columns at 256 units), that tile is the faster one although half of its
+    // MFMAs multiply padding -- the flat row has half as many workgroups (17 x 1024 x 11008: 23.4 -> 20.0 us with the
+    // matrix in the last-level cache, 31 -> 21 from HBM; 32 x 256 x 8192 17.0 -> 14.7; 32 x 1024 x 4096 13.0 -> 12.1);
+    // beyond that it has to take fewer parts and the flat row wins (17 x 1280 x 8192: 15.8 against 21.5).
+    const bool flat_row_fills = d.M > 32 || ((d.N + 63) / 64) * kSplitMax > cus || d.K < kSplitFromK;
+    if (plan.tile == kTileSmall && (d.M <= 32 || (d.M > 64 && d.M <= 96)) && d.N >= 256 && flat_row_fills) plan.tile = kTileFlat;
 
     // Small products: one launch of the wave-split kernel where it is expected to finish before the tiled
     // kernel (plus, for long K, its second launch) could: measured, it wins wherever its estimate stays below
@@ -331,7 +337,8 @@ GemmPlan plan_gemm(const GemmDesc& d) {
         // unit, as split = units / tiles says, measured best or within 8 % of it at 4096 ... 16384 columns and steps
         // (32 x 8192 x 8192: 94 us with the model's 8 parts, 68 with 4); the model below is for the products that
         // the matrix cores bound
-        const bool one_flat_row = plan.tile == kTileFlat && d.M <= 32;
+        // (the same for the 64 x 64 tile where it stands in for that row because the row's column tiles are too few)
+        const bool one_flat_row = d.M <= 32 && (plan.tile == kTileFlat || (plan.tile == kTileSmall && d.N >= 256));
         if ((plan.tile == kTileSmall || plan.tile == kTileFlat) && d.K >= 1024 && !one_flat_row)
             split = small_tile_split(tiles, d.K, cus);
         while (split > 1 && split * d.M * d.N * (int64_t)sizeof(float) > scratch_cap) split /= 2;

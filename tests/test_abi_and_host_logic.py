@@ -267,6 +267,9 @@ GEMM_PLANS = [
     ((0, 1, 17, 4096, 3072), "skinny"),                              # 2048 < K < 4096: 12..16 rows of W per compute unit only
     ((0, 1, 32, 4096, 11008), "mfma flat whole split 8"),            # one row of whole 32 x 128 tiles: the simple schedule
     ((0, 0, 32, 4096, 4096), "mfma flat whole split 8"),             # ... and a [K, N] weight matrix
+    ((0, 1, 17, 1024, 11008), "mfma small ragged pipelined staged 4 split 16"),   # up to 1024 columns one row of 32 x 128 tiles cannot fill the compute units: 64 x 64 tiles, 16 parts
+    ((0, 0, 32, 1024, 8192), "mfma small ragged pipelined staged 4 split 16"),
+    ((0, 1, 17, 1280, 8192), "mfma flat ragged pipelined split 16"),              # beyond: the flat row
     # 129..160 rows: five row tiles of 32 where their workgroups fill the compute units' rounds
     ((0, 1, 144, 4096, 4096), "mfma flat ragged pipelined staged 2 split 3"),     # 480 workgroups
     ((0, 0, 160, 4096, 4096), "mfma flat ragged pipelined staged 2 split 3"),
