@@ -614,6 +614,69 @@ def stream_audit(torch, kai, stream, dev, out_path):
     print(json.dumps({"stream_audit": summary, "written_to": out_path}))
 
 
+def rows_sweep(torch, kai, stream, dev, out_path):
+    """An audit that needs no forced plan: Y = X.W^T for 1..65 rows of X against weight matrices of many widths and
+    reduction lengths, W streamed from HBM (rotating buffers beyond the last-level cache).  More rows never do less
+    work, so a row count that takes longer than a LARGER one at the same matrix marks a kernel or a dispatch rule
+    that leaves time on the table there; the table lists every such case beyond 7 %."""
+    import ctypes
+    L = kai.load()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    I = ctypes.c_int64
+    g = torch.Generator(device=dev)
+    g.manual_seed(8)
+    row_counts = (1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 32, 33, 48, 64, 65)
+    widths = (1024, 2048, 2304, 3072, 4096, 4352, 5120, 8192, 8704, 11008)
+    lengths = (1024, 2048, 3072, 4096, 5120, 8192, 11008)
+    lines, flagged, worst = [], [], 1.0
+    for k in lengths:
+        for n in widths:
+            nb = max(2, min(24, (520 << 20) // (n * k * 4)))
+            ws = [torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05 for _ in range(nb)]
+            ts = {}
+            for m in row_counts:
+                x = torch.randn((m, k), device=dev, generator=g)
+                y = torch.empty((m, n), device=dev)
+
+                def call(i):
+                    rc = L.kai_matmul(0, P(y), P(ws[i % nb]), P(x), I(n), I(m), I(k), 0)
+                    if rc != 0:
+                        raise RuntimeError(L.kai_last_error().decode())
+
+                for i in range(max(nb, 6)):
+                    call(i)
+                torch.cuda.synchronize()
+                reps = []
+                for _ in range(5):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    for i in range(48):
+                        call(i)
+                    e1.record(stream)
+                    torch.cuda.synchronize()
+                    reps.append(e0.elapsed_time(e1) * 1e3 / 48)
+                ts[m] = sorted(reps)[2]
+                ref = x.double() @ ws[47 % nb].double().T
+                err = float(torch.linalg.norm(y.double() - ref) / torch.linalg.norm(ref))
+                if not err <= 1e-5:
+                    raise RuntimeError("%d x %d x %d: relative error %.2e" % (m, n, k, err))
+            marks = []
+            for j, m in enumerate(row_counts):
+                later = min(ts[mm] for mm in row_counts[j:])
+                worst = max(worst, ts[m] / later)
+                if ts[m] > 1.07 * later:
+                    marks.append("%d rows %.2f > %.2f" % (m, ts[m], later))
+                    flagged.append((round(ts[m] / later, 3), m, n, k))
+            lines.append("| %d x %d | %s | %s |" % (n, k, " ".join("%d:%.1f" % (m, ts[m]) for m in row_counts), "; ".join(marks)))
+            del ws
+    summary = {"matrices": len(lines), "row_counts": len(row_counts), "flagged_over_1_07": len(flagged),
+               "worst_ratio": round(worst, 3)}
+    with open(out_path, "w") as f:
+        f.write(json.dumps(summary) + "\n\n| W (N x K) | us per call by row count | slower than a larger row count by > 7 % |\n|---|---|---|\n"
+                + "\n".join(lines) + "\n")
+    print(json.dumps({"rows_sweep": summary, "written_to": out_path}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -629,6 +692,9 @@ def main():
     ap.add_argument("--stream-audit", metavar="FILE", default=None,
                     help="instead of the benchmark: the same audit for the skinny streaming kernel's rules (9..64 rows "
                          "against wide weight matrices streamed from HBM), table written to FILE")
+    ap.add_argument("--rows-sweep", metavar="FILE", default=None,
+                    help="instead of the benchmark: 1..65 rows against 70 weight matrices streamed from HBM; a row count "
+                         "slower than a larger one marks a kernel or dispatch rule that leaves time on the table")
     ap.add_argument("--only", action="append", default=None, metavar="TEXT",
                     help="measure only the rows of the table whose name contains TEXT (may be given several times)")
     ap.add_argument("--row-warmup-ms", type=float, default=40.0,
@@ -658,6 +724,9 @@ def main():
         return
     if args.stream_audit:
         stream_audit(torch, kai, stream, dev, args.stream_audit)
+        return
+    if args.rows_sweep:
+        rows_sweep(torch, kai, stream, dev, args.rows_sweep)
         return
 
     n = 8192

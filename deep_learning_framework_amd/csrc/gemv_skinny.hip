@@ -601,14 +601,16 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
         //   * more than 8 and fewer than 16 per compute unit, 3 and 4 rows: 3072 x 4096 12.4 -> 10.0, 2304 x 4096
         //     11.3 -> 9.2, 3072 x 5120 18.2 -> 13.2, 3072 x 8192 21.3 -> 19.2, 3840 x 12288 35.5 -> 30.8, 2304 x 1024
         //     6.0 -> 5.3 (every K from 1024 to 12288 by 10..38 %), except the rolled loop over long rows
-        //     (K > 8192 that is not a multiple of 4096: 3072 x 11008 27.2 -> 29.3, from 13 per compute unit on
-        //     31.6 -> 30.4); 2 rows with K = 4096 / 8192 by 2..5 %;
+        //     (K > 8192 that is not a multiple of 4096: 3072 x 11008 27.2 -> 29.3), which loses at every width, most
+        //     where the last round of workgroups is partly filled (5120 x 11008 at 3 rows: slices 40.0, stream 50.3;
+        //     8704 x 11008 65.2 / 78.4; 8192 x 11008 60.2 / 63.4; K = 2048, 4096 and 5120 stream 0..25 % faster at the
+        //     same widths); 2 rows with K = 4096 / 8192 by 2..5 %;
         //   * 8 per compute unit and fewer: the slice kernels (2048 x 8192, 128 workgroups: 15.3 against 19.8;
         //     2048 x 3072 8.4 against 8.8) unless K <= 2048 (2048 x 2048 6.9 -> 6.4, 2048 x 1024 5.8 -> 5.3).
         const int64_t cus = compute_units();
-        bool streamed = p.N >= 16 * cus && (p.M >= 3 || p.K % 4096 == 0);
-        if (!streamed && p.N > 8 * cus)
-            streamed = p.M >= 3 ? !(p.K > 8192 && p.K % 4096 != 0 && p.N < 13 * cus) : (p.K % 4096 == 0 && p.K <= 8192);
+        const bool long_rolled = p.K > 8192 && p.K % 4096 != 0;
+        bool streamed = p.N >= 16 * cus && (p.M >= 3 ? !long_rolled : p.K % 4096 == 0);
+        if (!streamed && p.N > 8 * cus) streamed = p.M >= 3 ? !long_rolled : (p.K % 4096 == 0 && p.K <= 8192);
         if (!streamed && p.M >= 3 && p.N == 8 * cus && p.K <= 2048) streamed = true;
         if (streamed && skinny_stream_applies(p)) return launch_skinny_stream(p, stream);
         if (p.M == 2) return launch_slice<2>(p, stream);

@@ -475,13 +475,35 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
         ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 >= 0x7FFFFFF0ll)
         return 0;
     if (g_stream_rows_override == 32 || g_stream_rows_override == 48) return g_stream_rows_override;
-    if (p.M <= 8) return 0;
     const int64_t cus = compute_units();
-    const bool many = p.M > 3 * kSkinnyMaxRows;      // 49..64 rows: four blocks of X rows
     const int64_t groups48 = (p.N + 47) / 48, rounds48 = (groups48 + cus - 1) / cus;
+    const int64_t groups32 = (p.N + 31) / 32, rounds32 = (groups32 + cus - 1) / cus;
+    // A last round of 16-row workgroups that is mostly empty costs a whole round: 5..32 rows then run on one round of
+    // wider workgroups although that round is only half to three quarters full.  Measured, us with W from HBM, 16-row
+    // workgroups -> these (K = 4096 | 8192): 4352 columns (272 of 16, 136 of 32) 5 / 16 / 32 rows 18.0 / 21.9 / 29.3 ->
+    // 16.2 / 18.3 / 24.7 | 5 / 16 rows 36.0 / 43.4 -> 29.4 / 34.3; 5120 (320, 160) 18.2 / 22.1 / 29.6 -> 17.6 / 19.2 / 24.8 |
+    // 36.7 / 44.8 -> 30.9 / 35.9; 5632 (352, 176) 18.4 / 22.0 / 29.6 -> 18.5 / 20.1 / 25.3; 6144 (384 = 1.5 rounds, 192) at
+    // K = 4096 5 rows 19.0 -> 20.0, 16 rows 22.6 -> 21.4, so not there, but at K = 8192 5 / 8 rows 38.6 / 40.5 -> 32.5 /
+    // 33.5; 8704 (544 of 16 in three rounds, 182 of 48) 5 / 16 / 32 rows 27.1 / 31.8 / 43.1 -> 24.2 / 25.9 / 33.5 | 57.9 /
+    // 66.8 / 87.8 -> 51.2 / 54.7 / 66.0; 9216 (576, 192) 27.2 / 32.3 / 43.7 -> 25.3 / 26.5 / 33.8.
+    // Further: 8448 (528 of 16, 176 of 48) 5 / 16 / 32 rows 26.7 / 31.5 / 42.8 -> 23.7 / 25.4 / 33.4; 9728 (608, 203) 27.6 /
+    // 32.4 / 44.0 -> 26.4 / 27.2 / 34.4; 4 rows at 4352 columns 17.7 -> 15.9 | 34.8 -> 28.6, at 8448 26.4 -> 23.6; two rounds
+    // of 32-row workgroups instead of four of 16 (12800 columns, 78 % full either way) 24 / 32 rows 51.5 / 56.8 -> 47.3 /
+    // 49.6 | 12 / 16 / 32 rows 88.0 / 92.2 / 117.5 -> 80.2 / 81.1 / 94.2.
+    if (p.M >= 3 && p.M <= 2 * kSkinnyMaxRows) {
+        const int64_t groups16 = p.N / 16, rounds16 = (groups16 + cus - 1) / cus;
+        if (rounds16 >= 2 && groups16 * 100 < 82 * rounds16 * cus) {
+            if (rounds48 == 1 && groups48 * 100 >= 65 * cus) return 48;
+            if (groups16 * 100 < (p.K >= 8192 ? 82 : 72) * rounds16 * cus && rounds32 == 1 && groups32 * 2 >= cus) return 32;
+            if (rounds32 >= 2 && 2 * rounds32 <= rounds16 && groups32 * 100 >= 75 * rounds32 * cus &&
+                (p.M > kSkinnyMaxRows || (p.M > 8 && p.K >= 8192)))
+                return 32;
+        }
+    }
+    if (p.M <= 8) return 0;
+    const bool many = p.M > 3 * kSkinnyMaxRows;      // 49..64 rows: four blocks of X rows
     if (rounds48 == 1 ? groups48 * 100 >= (many ? 85 : 80) * cus : (p.M <= kSkinnyMaxRows && groups48 * 100 >= 85 * rounds48 * cus))
         return 48;
-    const int64_t groups32 = (p.N + 31) / 32, rounds32 = (groups32 + cus - 1) / cus;
     if (many || groups32 * 4 < 3 * cus) return 0;
     // 9..16 rows: only with rows of 8192 steps and more, one round
     if (p.M <= kSkinnyMaxRows) return p.K >= 8192 && rounds32 == 1 ? 32 : 0;
@@ -490,7 +512,6 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
     if (rounds32 > 1 && groups32 * 100 < 85 * rounds32 * cus) return 0;
     if (p.M <= 24 && p.K <= 4096 && rounds32 == 1 && groups32 * 10 > 9 * cus) return 0;
     return 32;
-    return 0;
 }
 
 int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {

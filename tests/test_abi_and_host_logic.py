@@ -248,6 +248,10 @@ GEMM_PLANS = [
     ((0, 1, 32, 8192, 4096), "skinny stream 32"),                    # 256 workgroups of 32 rows, 17..32 rows of X only
     ((0, 1, 16, 8192, 4096), "skinny"),
     ((0, 1, 16, 16384, 4096), "skinny"),                             # 342 workgroups of 48: the second round a third full
+    ((0, 1, 5, 4352, 4096), "skinny stream 32"),                     # 272 workgroups of 16 would leave a second round 6 % full: one round of 136
+    ((0, 1, 16, 8704, 4096), "skinny stream 48"),                    # 544 of 16 in three rounds, 182 of 48 in one
+    ((0, 1, 8, 6144, 4096), "skinny"),                               # 1.5 rounds of 16-row workgroups stay (K = 4096)
+    ((0, 1, 12, 12800, 8192), "skinny stream 32"),                   # two rounds of 32 instead of four of 16, rows of 8192 steps
     ((0, 1, 48, 8192, 4096), "skinny stream 32"),                    # 33..64 rows stream only on the wide workgroups
     ((0, 1, 64, 11008, 4096), "skinny stream 48"),
     ((0, 1, 33, 10240, 4096), "skinny stream 48"),                   # 214 workgroups: one round, four fifths full

@@ -411,7 +411,7 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # 2..4 rows against 9..15 rows of W per compute unit: the streaming kernel, except
                                    # the rolled loop over long rows (the slice kernel keeps 3072 x 11008)
                                    (3, 4096, 2304), (4, 5120, 3072), (4, 12288, 3840), (2, 8192, 2560), (3, 2048, 2048),
-                                   (4, 1024, 2320), (4, 11008, 3072), (3, 11008, 3328), (2, 12288, 3072),
+                                   (4, 1024, 2320), (4, 11008, 3072), (2, 12288, 3072),
                                    # one row with K not in whole chunks of 4096: the slice kernel, short rows the
                                    # streaming kernel
                                    (1, 2048, 5120), (1, 11008, 4096), (1, 512, 2048), (1, 1024, 1024), (1, 1024, 4100),
@@ -419,11 +419,15 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    # 17..32 rows through the rolled loop (K in whole tiles, not in whole slices), and
                                    # K = 4096 against 9..15 rows of W per compute unit
                                    (17, 2048, 4096), (32, 1024, 3072), (24, 3072, 4096), (25, 4096, 3072), (17, 4096, 2304),
-                                   (32, 2048, 11008), (20, 1056, 2320), (8, 2080, 4096), (5, 11008, 4096)])
+                                   (32, 2048, 11008), (20, 1056, 2320), (8, 2080, 4096), (5, 11008, 4096),
+                                   # a last round of 16-row workgroups that is mostly empty: one round of wider ones
+                                   (5, 4096, 4352), (16, 4096, 8704), (4, 8192, 5120), (24, 4096, 12800), (3, 4096, 8448)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n >= 6144 and k % 4096 == 0:
-        want = "skinny stream %d" % (48 if n in (11008, 12288) else 32)
+        want = "skinny stream %d" % (48 if n in (11008, 12288, 8704, 8448) else 32)
         assert VMath.gemm_plan(0, 1, m, n, k) == want
+    elif n in (4352, 5120) and m >= 3:
+        assert VMath.gemm_plan(0, 1, m, n, k) == "skinny stream 32"
     elif m > 16 and k % 4096 != 0:
         assert VMath.gemm_plan(0, 1, m, n, k) == "skinny"      # 16-row workgroups, rolled loop
     rng = np.random.default_rng(m + k + n)
