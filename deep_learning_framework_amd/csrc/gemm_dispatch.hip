@@ -141,6 +141,11 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // skinny: y = x . w^T with both operands K-contiguous, a contiguous output row, no scaling
     plan.skinny = d.M <= kSkinnyMaxRows && d.nbatch == 1 && d.a_ks == 1 && d.b_ks == 1 && d.c_cs == 1 &&
                   !d.has_alpha && d.K > 0 && d.N >= 256;
+    // 5..16 rows against few and long rows that the streaming kernel walks in its rolled loop (K > 8192, not a multiple
+    // of 4096; up to four rows of W per compute unit): its 64 workgroups stream 11008 steps each, and the 64 x 64 tiles
+    // with 16 parts of K are faster (1024 x 11008 with W from HBM, 5 / 8 / 12 / 16 rows: 21.9 / 24.0 / 27.6 / 30.1 us ->
+    // 20.5 .. 21.0; 256 x 13824 at 5 rows 24.5 -> 19.5; rows of 8192 steps: 13.0 / 14.6 / 15.9 against 17)
+    if (plan.skinny && d.M >= 5 && d.N <= 4 * compute_units() && d.K > 8192 && d.K % 4096 != 0) plan.skinny = false;
     // 17..32 rows where the streaming kernel's two-block variant applies (whole tiles, K a multiple of 4096, enough
     // columns for one workgroup per compute unit, a matrix of at most 192 MB): W streams once in one launch
     // (4096 x 4096 from HBM: 17 rows 21.2 -> 15.0 us, 32 rows 21.3 -> 17.9, on a row of 32 x 128 tiles with eight

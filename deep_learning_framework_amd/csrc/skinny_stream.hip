@@ -490,7 +490,7 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
     // 32.4 / 44.0 -> 26.4 / 27.2 / 34.4; 4 rows at 4352 columns 17.7 -> 15.9 | 34.8 -> 28.6, at 8448 26.4 -> 23.6; two rounds
     // of 32-row workgroups instead of four of 16 (12800 columns, 78 % full either way) 24 / 32 rows 51.5 / 56.8 -> 47.3 /
     // 49.6 | 12 / 16 / 32 rows 88.0 / 92.2 / 117.5 -> 80.2 / 81.1 / 94.2.
-    if (p.M >= 3 && p.M <= 2 * kSkinnyMaxRows) {
+    if (p.M <= 2 * kSkinnyMaxRows) {
         const int64_t groups16 = p.N / 16, rounds16 = (groups16 + cus - 1) / cus;
         if (rounds16 >= 2 && groups16 * 100 < 82 * rounds16 * cus) {
             if (rounds48 == 1 && groups48 * 100 >= 65 * cus) return 48;

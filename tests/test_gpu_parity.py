@@ -421,12 +421,13 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    (17, 2048, 4096), (32, 1024, 3072), (24, 3072, 4096), (25, 4096, 3072), (17, 4096, 2304),
                                    (32, 2048, 11008), (20, 1056, 2320), (8, 2080, 4096), (5, 11008, 4096),
                                    # a last round of 16-row workgroups that is mostly empty: one round of wider ones
-                                   (5, 4096, 4352), (16, 4096, 8704), (4, 8192, 5120), (24, 4096, 12800), (3, 4096, 8448)])
+                                   (5, 4096, 4352), (16, 4096, 8704), (4, 8192, 5120), (24, 4096, 12800), (3, 4096, 8448),
+                                   (2, 4096, 4352), (12, 11008, 1024), (5, 13824, 256)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n >= 6144 and k % 4096 == 0:
         want = "skinny stream %d" % (48 if n in (11008, 12288, 8704, 8448) else 32)
         assert VMath.gemm_plan(0, 1, m, n, k) == want
-    elif n in (4352, 5120) and m >= 3:
+    elif n in (4352, 5120) and m >= 2 and k % 4096 == 0:
         assert VMath.gemm_plan(0, 1, m, n, k) == "skinny stream 32"
     elif m > 16 and k % 4096 != 0:
         assert VMath.gemm_plan(0, 1, m, n, k) == "skinny"      # 16-row workgroups, rolled loop
