@@ -71,7 +71,12 @@ double wavesplit_estimate(const GemmDesc& d, int T) {
     if (T == 16) {
         if (d.K > 2048) return -1.0;
         const double per_step = (d.a_ks == 1 && d.b_ks == 1) ? 3.2e-3 : 2.5e-3;
-        return std::max(3.9, 2.9 + per_step * K) + more_rounds * 3.2e-3 * K;
+        // one row of blocks against a matrix whose rows run along the output index: a block reads 64 bytes of each
+        // row, and beyond one workgroup per compute unit the rounds cost more than twice the fit (16 x 8192 x 1024:
+        // 13.9 us, 16 x 11008 x 1024: 19.9; 32 x 32 blocks 9.8, the tiles 15.8)
+        // (the fit holds up to 768 steps, up to 512 from two full rounds on: 16 x 8192 x 768 9.7 against 7.7 us)
+        const double per_round = (d.M <= 16 && d.b_ks != 1 && (d.K > 768 || (d.K > 512 && wgs >= 2 * cus))) ? 7.5e-3 : 3.2e-3;
+        return std::max(3.9, 2.9 + per_step * K) + more_rounds * per_round * K;
     }
     if (d.K > 1024) return -1.0;
     return std::max(3.9, 2.7 + 6.4e-3 * K) + 1.0e-3 * (double)std::min(wgs, cus) + more_rounds * (0.2 + 8.0e-3 * K);

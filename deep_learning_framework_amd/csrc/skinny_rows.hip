@@ -128,10 +128,20 @@ skinny_rows_kernel(const float* __restrict__ A, const float* __restrict__ B, con
 
 // a K-contiguous, b contiguous along its output index with whole groups of four columns, at most 16 rows, a
 // contiguous output row, and enough of b for the stream to matter
+// Which products: up to 8 rows, and 9..16 rows (where the vector FMAs of this kernel begin to show) only in the
+// window in which a sweep of 1..65 rows over 5 reduction lengths x 7 widths, the matrix streamed from HBM, found it
+// faster than the tiled kernels at 17 rows: widths of 3072..5120 with up to 2048 steps, about 4096 columns with up
+// to 8192 steps, and short reductions up to 4096 columns (us at 9 rows against the tiles at 17: 2048 x 4096 13.6 /
+// 14.5, 8192 x 4096 31.4 / 33.1, 1024 x 4096 8.7 / 12.4; outside the window 4096 x 1024 18.7 / 13.7, 8192 x 1024 28.5 /
+// 17.1, 11008 x 2048 38.4 / 27.1, 4096 x 8192 43.9 / 30.0, 11008 x 11008 105.5 / 94.2).  Reductions of up to 1024 steps
+// against more than 4096 columns go to the tiles at every row count (1024 x 5120: 14.0 .. 16.2 against 10.4).
 bool skinny_rows_applies(const GemmDesc& d) {
-    return d.nbatch == 1 && d.M >= 1 && d.M <= 16 && d.a_ks == 1 && d.b_rs == 1 && d.b_ks >= d.N && d.c_cs == 1 &&
-           d.N % 4 == 0 && d.N >= 1024 && d.K >= 256 && d.K * d.N >= (1ll << 21) && d.rowsum == nullptr &&
-           d.k_part == 0;
+    if (!(d.nbatch == 1 && d.M >= 1 && d.M <= 16 && d.a_ks == 1 && d.b_rs == 1 && d.b_ks >= d.N && d.c_cs == 1 &&
+          d.N % 4 == 0 && d.N >= 1024 && d.K >= 256 && d.K * d.N >= (1ll << 21) && d.rowsum == nullptr && d.k_part == 0))
+        return false;
+    if (d.K <= 1024 && d.N > 4096) return false;
+    if (d.M <= 8) return true;
+    return d.N <= 5120 && ((d.K <= 1024 && d.N <= 4096) || (d.N >= 3072 && d.K <= 2048) || (d.N >= 3584 && d.N <= 4608 && d.K <= 8192));
 }
 
 int launch_skinny_rows(const GemmDesc& d, hipStream_t stream) {

@@ -235,7 +235,9 @@ GEMM_PLANS = [
     ((0, 1, 4, 4096, 4096), "skinny"),
     ((0, 1, 16, 4096, 4096), "skinny"),
     ((0, 0, 4, 4096, 4096), "skinny rows"),                          # backward_x at a small batch: b stored [K, N]
-    ((0, 0, 16, 11008, 4096), "skinny rows"),
+    ((0, 0, 8, 11008, 4096), "skinny rows"),
+    ((0, 0, 16, 4096, 4096), "skinny rows"),                         # 9..16 rows: only in the window where it beats the tiles
+    ((0, 0, 16, 11008, 4096), "mfma flat ragged pipelined staged 2 split 2"),
     ((0, 0, 17, 4096, 4096), "mfma flat ragged pipelined split 8"),
     ((0, 1, 16, 1024, 1024), "wavesplit 16"),                        # 5..16 rows against a small weight matrix
     ((0, 1, 4, 1024, 1024), "skinny"),                               # up to 4 rows always stream
