@@ -60,7 +60,8 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // What the first loads need comes as scalars (14 dwords): this file is compiled with kernel-argument preload, so
 // a wave finds them in SGPRs at its start instead of fetching the argument buffer first.
 //
-// WHOLE: N is a multiple of 16 and K of 32 (every tile of W lies inside the matrix).  The tiles then come through
+// WHOLE: K is a multiple of 32 (every tile of W lies inside its rows; N need not be a multiple of the workgroup's rows:
+// the rows past N lie behind the end of the last workgroup's resource and read as zero).  The tiles then come through
 // buffer loads: a resource over this workgroup's 16 rows of W and one over the M rows of X, a constant byte
 // offset per lane and a scalar offset per tile.  Nothing is clamped or masked (a row of X past M lies behind the
 // end of its resource and reads as zero), so a tile costs no vector instruction besides its LDS accesses and
@@ -143,7 +144,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
         return reinterpret_cast<float*>(((uint64_t)hi << 32) | lo);
     };
-    const int w_rows = WR > 16 ? (int)min((int64_t)WR, p.N - n0) : WR;   // rows of W this workgroup has (uniform)
+    const int w_rows = WR >= 16 ? (int)min((int64_t)WR, p.N - n0) : WR;   // rows of W this workgroup has (uniform; the last workgroup may have fewer)
     const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
         uniform_ptr(p.W + n0 * p.ldw), 0, (int)(((int64_t)(w_rows - 1) * p.ldw + p.K) * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
@@ -153,7 +154,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     for (int j = 0; j < kWRegs; j++) {
         // a row past the workgroup's last must land behind the end of the resource whatever ldw is
         const int row = kSsRowsPerLoad * j + lrow;
-        woff[j] = WR > 16 && row >= w_rows ? 0x7FFFFFF0 : (int)(((int64_t)row * p.ldw + lk) * 4);
+        woff[j] = WR >= 16 && row >= w_rows ? 0x7FFFFFF0 : (int)(((int64_t)row * p.ldw + lk) * 4);
     }
 #pragma unroll
     for (int j = 0; j < kXLoads; j++) {
@@ -386,7 +387,7 @@ static bool stream_many_rows_base(const SkinnyParams& p) {
     else if (p.M > 2 * kSkinnyMaxRows || p.K % kSsTileK != 0) k_ok = false;
     else if (p.K >= 1024 && p.K <= 2048) k_ok = p.N >= 9 * cus;
     else k_ok = p.K > 2048 && p.K < 4096 && p.N >= 12 * cus && p.N <= 16 * cus;
-    return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && k_ok && p.N % 16 == 0 &&
+    return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && k_ok &&
            stream_size_rule(p.N, p.K) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&
            (15 * p.ldw + p.K) * 4 < (1ll << 31) && ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
 }
@@ -471,7 +472,7 @@ void set_skinny_stream_rows_override(int rows) { g_stream_rows_override = rows; 
 int skinny_stream_wide_rows(const SkinnyParams& p) {
     if (g_stream_rows_override == 16 && p.M <= 2 * kSkinnyMaxRows) return 0;
     const bool base = p.M > kSkinnyMaxRows ? stream_many_rows_base(p) : (p.M >= 2 && skinny_stream_applies(p));
-    if (!base || p.K % (kSsWaves * 512) != 0 || p.N % 16 != 0 || (47 * p.ldw + p.K) * 4 >= (1ll << 31) ||
+    if (!base || p.K % (kSsWaves * 512) != 0 || (47 * p.ldw + p.K) * 4 >= (1ll << 31) ||
         ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 >= 0x7FFFFFF0ll)
         return 0;
     if (g_stream_rows_override == 32 || g_stream_rows_override == 48) return g_stream_rows_override;
@@ -491,7 +492,7 @@ int skinny_stream_wide_rows(const SkinnyParams& p) {
     // of 32-row workgroups instead of four of 16 (12800 columns, 78 % full either way) 24 / 32 rows 51.5 / 56.8 -> 47.3 /
     // 49.6 | 12 / 16 / 32 rows 88.0 / 92.2 / 117.5 -> 80.2 / 81.1 / 94.2.
     if (p.M <= 2 * kSkinnyMaxRows) {
-        const int64_t groups16 = p.N / 16, rounds16 = (groups16 + cus - 1) / cus;
+        const int64_t groups16 = (p.N + 15) / 16, rounds16 = (groups16 + cus - 1) / cus;
         if (rounds16 >= 2 && groups16 * 100 < 82 * rounds16 * cus) {
             if (rounds48 == 1 && groups48 * 100 >= 65 * cus) return 48;
             if (groups16 * 100 < (p.K >= 8192 ? 82 : 72) * rounds16 * cus && rounds32 == 1 && groups32 * 2 >= cus) return 32;
@@ -522,7 +523,7 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     if (wide == 48) return launch_wide<48>(p, t, stream);
     if (wide == 32) return launch_wide<32>(p, t, stream);
     // whole tiles, and byte offsets inside a workgroup's 16 rows of W and inside X that fit 31 bits
-    const bool whole = p.N % 16 == 0 && p.K % kSsTileK == 0 && (15 * p.ldw + p.K) * 4 < (1ll << 31) &&
+    const bool whole = p.K % kSsTileK == 0 && (15 * p.ldw + p.K) * 4 < (1ll << 31) &&
                        ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
     const bool slices = p.K % (kSsWaves * 512) == 0;
     const dim3 grid((unsigned)blocks), block(kSsThreads);

@@ -422,9 +422,14 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    (32, 2048, 11008), (20, 1056, 2320), (8, 2080, 4096), (5, 11008, 4096),
                                    # a last round of 16-row workgroups that is mostly empty: one round of wider ones
                                    (5, 4096, 4352), (16, 4096, 8704), (4, 8192, 5120), (24, 4096, 12800), (3, 4096, 8448),
-                                   (2, 4096, 4352), (12, 11008, 1024), (5, 13824, 256)])
+                                   (2, 4096, 4352), (12, 11008, 1024), (5, 13824, 256),
+                                   # widths that are not a multiple of the workgroup's rows of W: whole tiles all the same
+                                   (8, 4096, 4100), (16, 2048, 5003), (24, 4096, 4100), (32, 4096, 11001), (3, 4096, 4099),
+                                   (12, 4096, 8707), (5, 1024, 4353)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
-    if n >= 6144 and k % 4096 == 0:
+    if n % 16 != 0:
+        pass
+    elif n >= 6144 and k % 4096 == 0:
         want = "skinny stream %d" % (48 if n in (11008, 12288, 8704, 8448) else 32)
         assert VMath.gemm_plan(0, 1, m, n, k) == want
     elif n in (4352, 5120) and m >= 2 and k % 4096 == 0:
