@@ -151,6 +151,14 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // with 16 parts of K are faster (1024 x 11008 with W from HBM, 5 / 8 / 12 / 16 rows: 21.9 / 24.0 / 27.6 / 30.1 us ->
     // 20.5 .. 21.0; 256 x 13824 at 5 rows 24.5 -> 19.5; rows of 8192 steps: 13.0 / 14.6 / 15.9 against 17)
     if (plan.skinny && d.M >= 5 && d.N <= 4 * compute_units() && d.K > 8192 && d.K % 4096 != 0) plan.skinny = false;
+    // 5..16 rows against long rows of W that do not start on 128-byte lines (the streaming kernel's 128-byte pieces
+    // straddle two lines each): the tiles from 8192 steps on (4100 x 11012 at 8 / 16 rows 62.2 / 78.4 us against 46.4 at
+    // 17 rows; 4100 x 8200 45.6 / 55.1 against 33.7; at 5004 steps and fewer the streaming kernel holds up to 12 rows)
+    // (8..16 rows from 5000 steps on: 8200 x 5004 at 8 / 16 rows 52.8 / 64.3 against 46.5; 13..16 rows from 4096 steps
+    // on: 5000 x 4100 at 16 rows 38.3 against 32.2)
+    if (plan.skinny && d.M >= 5 && d.b_rs % 32 != 0 &&
+        (d.K >= 8192 || (d.M >= 8 && d.K > 4608) || (d.M >= 13 && d.K >= 4096)))
+        plan.skinny = false;
     // 17..32 rows where the streaming kernel's two-block variant applies (whole tiles, K a multiple of 4096, enough
     // columns for one workgroup per compute unit, a matrix of at most 192 MB): W streams once in one launch
     // (4096 x 4096 from HBM: 17 rows 21.2 -> 15.0 us, 32 rows 21.3 -> 17.9, on a row of 32 x 128 tiles with eight

@@ -612,6 +612,10 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
         bool streamed = p.N >= 16 * cus && (p.M >= 3 ? !long_rolled : p.K % 4096 == 0);
         if (!streamed && p.N > 8 * cus) streamed = p.M >= 3 ? !long_rolled : (p.K % 4096 == 0 && p.K <= 8192);
         if (!streamed && p.M >= 3 && p.N == 8 * cus && p.K <= 2048) streamed = true;
+        // rows of W that do not start on a 128-byte line: each of the streaming kernel's 128-byte pieces of a row
+        // straddles two lines, the slice kernel's 1 KiB runs one in eight (4100 x 4100 at 4 rows: 21.8 us streamed,
+        // 14.3 at 2 rows in slices)
+        if (p.ldw % 32 != 0) streamed = false;
         if (streamed && skinny_stream_applies(p)) return launch_skinny_stream(p, stream);
         if (p.M == 2) return launch_slice<2>(p, stream);
         if (p.M <= 4) return launch_slice<4>(p, stream);

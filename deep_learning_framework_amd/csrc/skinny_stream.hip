@@ -72,6 +72,8 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // of a slice is written out (16 tiles, every wait counted exactly by the compiler): 12.2 us at M = 4 against
 // 12.9 us for the rolled loop that other lengths use.
 //
+// KT (rolled loop, whole-tile loads): K is a multiple of 4 but not of 32; the last tile's lanes past K load zeros.
+//
 // XL (whole tiles): 1 = at most 8 rows of X (one load per tile), 2 = more (two); 0 = decided per tile from M.  With
 // the number of X loads a compile-time constant and every tile inside K, the written-out slice has no branch left,
 // and the rolled loop only its own.
@@ -88,7 +90,7 @@ __device__ __forceinline__ f32x4 keep_if(f32x4 v, bool keep) {
 // bytes as those of W (twice as many with two blocks of X rows) and the compute unit's load path, not HBM, sets
 // the time; with two or three blocks of W rows a tile of X meets two or three tiles of W.  The last workgroup may
 // own fewer blocks (N a multiple of 16): the rows behind N lie behind the end of its resource and read as zero.
-template <bool WHOLE, bool SLICES, int XL = 0, int XB = 1, int WR = 16>
+template <bool WHOLE, bool SLICES, int XL = 0, int XB = 1, int WR = 16, bool KT = false>
 __global__ void __launch_bounds__(kSsThreads)
 skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, const int64_t ldw, const int64_t ldx,
                      const int64_t N, const int M, const int K, float* __restrict__ Y, const SkinnyTail t) {
@@ -99,6 +101,7 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     static_assert(XB == 1 || (XB >= 2 && XB <= 4 && WHOLE && (SLICES || XB == 2) && XL > kSsLoadsPerTile * (XB - 1) && XL <= kSsLoadsPerTile * XB),
                   "several blocks of X rows exist for whole tiles (three and four: in written-out slices)");
     static_assert(XL == 0 || WHOLE, "a compile-time number of X loads: whole tiles");
+    static_assert(!KT || (WHOLE && !SLICES && XL > 0 && WR == 16), "a last tile that K does not fill: the rolled loop over whole-tile loads");
     static_assert(XB <= 2 || WR >= 32, "three and four blocks of X rows: with two or three blocks of W rows only");
     // tiles of a wave in registers (written-out slices): with three and four blocks of X rows a tile is 10 to 14 loads
     // per lane, and two tiles are what the registers hold
@@ -166,10 +169,13 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
         if constexpr (WHOLE) {
             // a tile past the end of K (a wave's last slice may be short) re-reads the last whole tile instead of
             // counting on the range check for the scalar part of the address; it is never consumed
-            const int kc = min(kt, p.K - kSsTileK) * 4;
+            // KT: the tile is addressed as it lies, and a lane whose four steps are past K (K is a multiple of 4) is
+            // steered behind the end of the resource: zeros, in W and in X alike
+            const int kc = KT ? kt * 4 : min(kt, p.K - kSsTileK) * 4;
+            const bool past = KT && kt + lk >= p.K;
 #pragma unroll
             for (int j = 0; j < kWLoads; j++)   // aux 2: non-temporal, as the general variant's loads
-                dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff[j], kc, 2));
+                dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, past ? 0x7FFFFFF0 : woff[j], kc, 2));
             return;
         }
 #pragma unroll
@@ -181,11 +187,12 @@ skinny_stream_kernel(const float* __restrict__ W, const float* __restrict__ X, c
     };
     auto load_x = [&](f32x4(&dst)[kXLoads], int kt) {
         if constexpr (WHOLE) {
-            const int kc = min(kt, p.K - kSsTileK) * 4;
+            const int kc = KT ? kt * 4 : min(kt, p.K - kSsTileK) * 4;
+            const bool past = KT && kt + lk >= p.K;
 #pragma unroll
             for (int j = 0; j < kXLoads; j++)
                 if (XL ? j < XL : kSsRowsPerLoad * j < p.M)   // uniform
-                    dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, xoff[j], kc, 0));
+                    dst[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, past ? 0x7FFFFFF0 : xoff[j], kc, 0));
             return;
         }
 #pragma unroll
@@ -384,7 +391,7 @@ static bool stream_many_rows_base(const SkinnyParams& p) {
     const int64_t cus = compute_units();
     bool k_ok;
     if (p.K % (kSsWaves * 512) == 0) k_ok = p.N >= (p.K == kSsWaves * 512 && p.M <= 2 * kSkinnyMaxRows ? 9 : 16) * cus;
-    else if (p.M > 2 * kSkinnyMaxRows || p.K % kSsTileK != 0) k_ok = false;
+    else if (p.M > 2 * kSkinnyMaxRows || p.K % 4 != 0) k_ok = false;
     else if (p.K >= 1024 && p.K <= 2048) k_ok = p.N >= 9 * cus;
     else k_ok = p.K > 2048 && p.K < 4096 && p.N >= 12 * cus && p.N <= 16 * cus;
     return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && k_ok &&
@@ -526,11 +533,16 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     const bool whole = p.K % kSsTileK == 0 && (15 * p.ldw + p.K) * 4 < (1ll << 31) &&
                        ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
     const bool slices = p.K % (kSsWaves * 512) == 0;
+    // whole-tile loads with a last tile that K does not fill
+    const bool ktail = !whole && p.K % 4 == 0 && p.K > kSsTileK && (15 * p.ldw + p.K) * 4 < (1ll << 31) &&
+                       ((int64_t)(p.M - 1) * p.ldx + p.K) * 4 < 0x7FFFFFF0ll;
     const dim3 grid((unsigned)blocks), block(kSsThreads);
     if (p.M > kSkinnyMaxRows) {
         if (!skinny_stream32_applies(p) || p.M > 2 * kSkinnyMaxRows)
             return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: more than 16 rows");
-        if (!slices && p.M <= 24) skinny_stream_kernel<true, false, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        if (ktail && p.M <= 24) skinny_stream_kernel<true, false, 3, 2, 16, true><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        else if (ktail) skinny_stream_kernel<true, false, 4, 2, 16, true><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        else if (!slices && p.M <= 24) skinny_stream_kernel<true, false, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         else if (!slices) skinny_stream_kernel<true, false, 4, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         else if (p.M <= 24) skinny_stream_kernel<true, true, 3, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         else skinny_stream_kernel<true, true, 4, 2><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
@@ -540,6 +552,11 @@ int launch_skinny_stream(const SkinnyParams& p, hipStream_t stream) {
     // 3072 10.0 -> 9.6, 1..3 % elsewhere; with two, 9..16 rows, -2..+2 %: those keep the count read from M)
     if (whole && !slices && p.M <= 8) {
         skinny_stream_kernel<true, false, 1><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        return check_launch("skinny_stream_kernel");
+    }
+    if (ktail) {
+        if (p.M <= 8) skinny_stream_kernel<true, false, 1, 1, 16, true><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
+        else skinny_stream_kernel<true, false, 2, 1, 16, true><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);
         return check_launch("skinny_stream_kernel");
     }
     if (whole && slices && p.M <= 8) skinny_stream_kernel<true, true, 1><<<grid, block, 0, stream>>>(p.W, p.X, p.ldw, p.ldx, p.N, p.M, p.K, p.Y, t);

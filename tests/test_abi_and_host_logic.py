@@ -278,6 +278,8 @@ GEMM_PLANS = [
     ((0, 1, 17, 1280, 8192), "mfma flat ragged pipelined split 16"),              # beyond: the flat row
     ((0, 1, 12, 1024, 11008), "mfma small ragged pipelined staged 4 split 16"),   # 5..16 rows, few long rows outside whole slices: not the streaming kernel's rolled loop
     ((0, 1, 12, 1024, 8192), "skinny"),
+    ((0, 1, 8, 4100, 11012), "mfma flat ragged pipelined staged 2 split 7"),      # long rows of W off the 128-byte lines: tiles from 5 rows on
+    ((0, 1, 8, 4100, 4100), "skinny"),
     ((0, 1, 2, 4352, 4096), "skinny stream 32"),                                  # the wide workgroups from 2 rows on
     # 129..160 rows: five row tiles of 32 where their workgroups fill the compute units' rounds
     ((0, 1, 144, 4096, 4096), "mfma flat ragged pipelined staged 2 split 3"),     # 480 workgroups

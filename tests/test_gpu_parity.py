@@ -425,7 +425,10 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    (2, 4096, 4352), (12, 11008, 1024), (5, 13824, 256),
                                    # widths that are not a multiple of the workgroup's rows of W: whole tiles all the same
                                    (8, 4096, 4100), (16, 2048, 5003), (24, 4096, 4100), (32, 4096, 11001), (3, 4096, 4099),
-                                   (12, 4096, 8707), (5, 1024, 4353)])
+                                   (12, 4096, 8707), (5, 1024, 4353),
+                                   # K a multiple of 4 but not of 32: whole-tile loads, the last tile's lanes past K read zeros
+                                   (8, 4100, 4096), (16, 5004, 4100), (24, 2052, 4096), (32, 1028, 3000), (3, 4100, 4352),
+                                   (12, 1060, 4099), (5, 68, 4096)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n % 16 != 0:
         pass
@@ -434,7 +437,7 @@ def test_skinny_shapes_bias_act_acc(m, k, n):
         assert VMath.gemm_plan(0, 1, m, n, k) == want
     elif n in (4352, 5120) and m >= 2 and k % 4096 == 0:
         assert VMath.gemm_plan(0, 1, m, n, k) == "skinny stream 32"
-    elif m > 16 and k % 4096 != 0:
+    elif m > 16 and k % 4096 != 0 and k % 32 == 0:
         assert VMath.gemm_plan(0, 1, m, n, k) == "skinny"      # 16-row workgroups, rolled loop
     rng = np.random.default_rng(m + k + n)
     w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
