@@ -159,6 +159,11 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     if (plan.skinny && d.M >= 5 && d.b_rs % 32 != 0 &&
         (d.K >= 8192 || (d.M >= 8 && d.K > 4608) || (d.M >= 13 && d.K >= 4096)))
         plan.skinny = false;
+    // 5..16 rows against many short rows (50257 x 768: 43 / 55 us at 8 / 16 rows on the streaming kernel, whose 3142
+    // workgroups of 48 KB are all prologue and epilogue; 29 us on the tiles at 17 rows)
+    // (9..16 rows up to 1536 steps: 16 x 50257 x 1280 60.2 against 45.2, 16 x 20000 x 1536 32.5 against 24.7, matrices
+    // of up to 257 MB multiplied again and again; at 2048 steps the streaming kernel wins from 400 MB on and loses 20 % at 262)
+    if (plan.skinny && d.N >= 64 * compute_units() && ((d.M >= 5 && d.K <= 1024) || (d.M >= 9 && d.K <= 1536))) plan.skinny = false;
     // 17..32 rows where the streaming kernel's two-block variant applies (whole tiles, K a multiple of 4096, enough
     // columns for one workgroup per compute unit, a matrix of at most 192 MB): W streams once in one launch
     // (4096 x 4096 from HBM: 17 rows 21.2 -> 15.0 us, 32 rows 21.3 -> 17.9, on a row of 32 x 128 tiles with eight

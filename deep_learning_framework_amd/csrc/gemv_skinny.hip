@@ -584,10 +584,12 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
             // 14.8 -> 8.7, 8192 x 2048 17.4 -> 11.8, 5120 x 3072 18.2 -> 11.3, 4096 x 11008 31.7 -> 29.3, 1024 x 11008
             // 14.2 -> 9.9, 11008 x 5120 37.3 -> 33.1 (K = 1024 .. 11008: 7..69 %); rows shorter than a slice, and
             // K = 1024 up to 8 rows of W per compute unit, through the streaming kernel (2048 x 512 5.5 -> 4.1,
-            // 1024 x 1024 5.4 -> 4.5).  K in whole chunks: 4096 x 4096 11.3 against 11.7 / 12.2, 5120 x 4096 14.4
+            // 1024 x 1024 5.4 -> 4.5; matrices of up to 24 MB only: 50257 x 768 takes 35 us there and 24 in slices).
+            // K in whole chunks: 4096 x 4096 11.3 against 11.7 / 12.2, 5120 x 4096 14.4
             // against 17.0 / 17.5.
             if (p.K % 4096 == 0) return launch_gemv_rows(p, stream);
-            if ((p.K < kSliceK || (p.K == kSliceK && p.N <= 8 * (int64_t)compute_units())) && skinny_stream_applies(p))
+            if ((p.K < kSliceK || (p.K == kSliceK && p.N <= 8 * (int64_t)compute_units())) && p.N * p.K <= (6ll << 20) &&
+                skinny_stream_applies(p))
                 return launch_skinny_stream(p, stream);
             return launch_slice<1>(p, stream);
         }
@@ -616,6 +618,9 @@ int launch_skinny_nt(const SkinnyParams& p, hipStream_t stream) {
         // straddles two lines, the slice kernel's 1 KiB runs one in eight (4100 x 4100 at 4 rows: 21.8 us streamed,
         // 14.3 at 2 rows in slices)
         if (p.ldw % 32 != 0) streamed = false;
+        // many short rows (a vocabulary of 50257 against 768 steps): 3142 workgroups of 48 KB each are all prologue
+        // and epilogue, 38 us at 4 rows against 24 at 2 rows in slices
+        if (p.K <= 1024 && p.N >= 64 * cus) streamed = false;
         if (streamed && skinny_stream_applies(p)) return launch_skinny_stream(p, stream);
         if (p.M == 2) return launch_slice<2>(p, stream);
         if (p.M <= 4) return launch_slice<4>(p, stream);

@@ -392,7 +392,7 @@ static bool stream_many_rows_base(const SkinnyParams& p) {
     bool k_ok;
     if (p.K % (kSsWaves * 512) == 0) k_ok = p.N >= (p.K == kSsWaves * 512 && p.M <= 2 * kSkinnyMaxRows ? 9 : 16) * cus;
     else if (p.M > 2 * kSkinnyMaxRows || p.K % 4 != 0) k_ok = false;
-    else if (p.K >= 1024 && p.K <= 2048) k_ok = p.N >= 9 * cus;
+    else if (p.K >= 1024 && p.K <= 2048) k_ok = p.N >= 9 * cus && p.N <= 48 * cus;   // (measured up to 11008 columns; 32000 x 1024 at 17 rows: 36 us here, 22 on the tiles)
     else k_ok = p.K > 2048 && p.K < 4096 && p.N >= 12 * cus && p.N <= 16 * cus;
     return p.M > kSkinnyMaxRows && p.M <= 4 * kSkinnyMaxRows && k_ok &&
            stream_size_rule(p.N, p.K) && p.ldw % 4 == 0 && p.ldx % 4 == 0 && aligned16(p.W) && aligned16(p.X) &&

@@ -428,7 +428,9 @@ def test_engine_calls_with_acc_and_unaligned_subbuffers():
                                    (12, 4096, 8707), (5, 1024, 4353),
                                    # K a multiple of 4 but not of 32: whole-tile loads, the last tile's lanes past K read zeros
                                    (8, 4100, 4096), (16, 5004, 4100), (24, 2052, 4096), (32, 1028, 3000), (3, 4100, 4352),
-                                   (12, 1060, 4099), (5, 68, 4096)])
+                                   (12, 1060, 4099), (5, 68, 4096),
+                                   # many short rows (a vocabulary against a narrow model): slices up to 4 rows, tiles beyond
+                                   (1, 768, 30522), (4, 768, 30522), (8, 768, 30522), (16, 1280, 20000)])
 def test_skinny_shapes_bias_act_acc(m, k, n):
     if n % 16 != 0:
         pass
@@ -461,7 +463,7 @@ def test_skinny_stream_with_wide_workgroups_forced(rows):
     # or two blocks of X rows), on a matrix whose last workgroup owns fewer blocks, with padded rows, bias,
     # activation and acc; the override is the audit hook, the dispatcher's own rule is asserted elsewhere
     rng = np.random.default_rng(rows)
-    n, k, padw, padx = 4112, 4096, 4, 8
+    n, k, padw, padx = 4112, 4096, 32, 8    # (rows of W on 128-byte lines: off them 13 and more rows run on the tiles)
     w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
     wp = np.full((n, k + padw), np.nan, np.float32); wp[:, :k] = w
     bias = rng.standard_normal(n).astype(np.float32)
