@@ -457,6 +457,30 @@ def test_skinny_shapes_bias_act_acc(m, k, n):
     check(ya.to_numpy((m, n)), ko.matmul(w, x, acc_into=y0), what="skinny acc")
 
 
+@pytest.mark.parametrize("seed", list(range(1, 13)))
+def test_few_rows_random_shapes(seed):
+    """1..33 rows against weight matrices of random width, length and row padding (multiples of 4, on and off the
+    streaming kernels' tile grid and the 128-byte lines), with and without accumulation: whatever kernel the
+    dispatcher's rules pick must give the oracle's product."""
+    rng = np.random.default_rng(1000 + seed)
+    for _ in range(10):
+        m = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 13, 16, 17, 24, 33]))
+        k = int(rng.choice([68, 768, 1028, 2048, 2052, 4096, 4100, 5004])) if rng.integers(0, 2) else 4 * int(rng.integers(16, 1500))
+        n = int(rng.choice([256, 1000, 2304, 4099, 4352, 5120])) if rng.integers(0, 2) else int(rng.integers(256, 6000))
+        n = min(n, max(256, int(6e6 // k)))
+        padw = int(rng.choice([0, 4, 32]))
+        w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+        wp = np.full((n, k + padw), np.nan, np.float32); wp[:, :k] = w
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        y0 = rng.standard_normal((m, n)).astype(np.float32)
+        acc = int(rng.integers(0, 2))
+        dwp, dx, dy = dev(wp), dev(x), dev(y0)
+        plan = VMath.gemm_plan(0, 1, m, n, k, k, k + padw, n)
+        VMath.gemm_f32(0, 0, 1, m, n, k, dx, k, dwp, k + padw, dy, n, None, 0, None, acc)
+        check(dy.to_numpy((m, n)), ko.matmul(w, x, acc_into=y0 if acc else None),
+              what="%d x %d x %d, rows of W %d floats apart, acc %d (%s)" % (m, n, k, k + padw, acc, plan))
+
+
 @pytest.mark.parametrize("rows", [32, 48])
 def test_skinny_stream_with_wide_workgroups_forced(rows):
     # every variant of the streaming kernel with 32 / 48 rows of W per workgroup (one or two loads of X per tile, one
