@@ -458,6 +458,11 @@ int set_forced_gemm_plan(const char* text) {
 
 bool gemm_fuses_rowsum(const GemmDesc& d) {
     if (!valid_dims(d) || d.M == 0 || d.N == 0 || d.K == 0 || d.nbatch != 1) return false;
+    // The row sums ride along where the product is short: they save a launch of 3 us.  A long product pays for them
+    // in every tile of its first tile column and loses more than that (gw of 11008 x 4096 at a batch of 1024: 1445 us
+    // with the sums riding along against 1289 with colsum_kernel on its own; 4096 x 1024 at 512: 92.2 against 85.2;
+    // at a batch of 64: 29.1 against 29.6).
+    if (d.K >= 64 && d.M * d.N * d.K > (1ll << 28)) return false;
     const GemmPlan plan = plan_gemm(d);
     return !plan.skinny && !plan.wavesplit_edge && !skinny_rows_applies(plan.dn) && !plan.a_kc && !plan.b_kc && plan.tile != kTileLarge &&
            plan.tile != kTileFlat && plan.tile != kTileWide && plan.split == 1;
