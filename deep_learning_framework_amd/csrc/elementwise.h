@@ -96,6 +96,8 @@ int launch_attention_fused(float* o, const float* q, const float* k, const float
 bool attention_probs_applies(const float* q, const float* k, const float* v, const float* o, const float* pp,
                              int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece);
 bool attention_probs_four_heads(const float* pp, int64_t ntimes, int64_t nhead, int64_t npiece);
+// whether the one-launch training forward is expected to beat the three separate calls for this geometry
+bool attention_probs_pays(const float* pp, int64_t nbat, int64_t ntimes, int64_t nhead, int64_t npiece);
 int launch_attention_probs(float* o, float* pp, const float* q, const float* k, const float* v, int64_t nbat,
                            int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece, const float* hcoef, int masked,
                            hipStream_t stream);

@@ -925,7 +925,8 @@ int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, in
     std::string text = "separate";
     if (nbat == 0 || ntimes == 0 || nhead == 0 || npiece == 0) text = "nothing";
     else if (which == 0 && attention_fused_applies(a, a, a, a, ntimes, nvec, nhead, npiece)) text = "fused";
-    else if (which == 1 && attention_probs_applies(a, a, a, a, a, ntimes, nvec, nhead, npiece))
+    else if (which == 1 && attention_probs_applies(a, a, a, a, a, ntimes, nvec, nhead, npiece) &&
+             attention_probs_pays(a, nbat, ntimes, nhead, npiece))
         text = attention_probs_four_heads(a, ntimes, nhead, npiece) ? "fused, four heads per workgroup" : "fused";
     else if (which == 2 && attention_backward_applies(a, a, a, a, a, a, a, a, ntimes, nvec, nhead, npiece))
         text = attention_backward_one_launch(a, a, a, nbat, ntimes, nvec, nhead, npiece) ? "fused rows and value gradient in one launch"
@@ -948,7 +949,8 @@ int kai_attention_forward_train(int device, float* py, float* pp, const float* p
     KAI_TRY(check_heads(__func__, nbat, ntimes, nvec, nhead, npiece));
     if (nbat == 0 || ntimes == 0 || nhead == 0) return KAI_OK;
     KAI_REQUIRE_PTR(py); KAI_REQUIRE_PTR(pp); KAI_REQUIRE_PTR(pQ); KAI_REQUIRE_PTR(pK); KAI_REQUIRE_PTR(pV);
-    if (npiece > 0 && attention_probs_applies(pQ, pK, pV, py, pp, ntimes, nvec, nhead, npiece))
+    if (npiece > 0 && attention_probs_applies(pQ, pK, pV, py, pp, ntimes, nvec, nhead, npiece) &&
+        attention_probs_pays(pp, nbat, ntimes, nhead, npiece))
         return launch_attention_probs(py, pp, pQ, pK, pV, nbat, ntimes, nvec, nhead, npiece, hCoef, masked != 0,
                                       current_stream());
     // any other shape: the reference's calls one by one

@@ -357,7 +357,9 @@ int kai_attention_plan(int which, int64_t nbat, int64_t ntimes, int64_t nvec, in
  * calls leave them (masked keys exactly 0), for the backward pass (VTensor::mh_attention keeps them,
  * vtensor.cpp:3005, 3048).  One launch for head sizes that are multiples of 16 up to 128 with nhead * npiece == nvec, 16-byte aligned
  * operands and ntimes <= 1024 (a wave keeps the scores of its queries in registers between the maximum and the
- * stores); any other shape runs the four separate kernels.  Equal to the separate calls up to rounding. */
+ * stores); any other shape runs the four separate kernels, and so do geometries with more than 512 keys, one head
+ * per workgroup and workgroups for at most half of the compute units, where those kernels are the faster ones
+ * (kai_attention_plan tells).  Equal to the separate calls up to rounding. */
 int kai_attention_forward_train(int device, float* py, float* pp, const float* pQ, const float* pK, const float* pV,
                                 int64_t nbat, int64_t ntimes, int64_t nvec, int64_t nhead, int64_t npiece,
                                 const float* hCoef, int masked);

@@ -366,6 +366,10 @@ def test_attention_plans():
     assert plan("forward", 1, 64, 256, 1, 256) == "separate"
     assert plan("forward", 2, 70, 80, 2, 32) == "separate"
     assert plan("forward_train", 1, 1100, 64, 1, 64) == "separate"
+    # more than 512 keys, one head per workgroup, workgroups for at most half of the compute units: the separate calls
+    assert plan("forward_train", 1, 1024, 1024, 8, 128) == "separate"
+    assert plan("forward_train", 8, 1000, 128, 1, 128) == "separate"
+    assert plan("forward_train", 8, 1000, 64, 1, 64) == "fused"
     assert plan("forward", 1, 1100, 64, 1, 64) == "fused"
     assert plan("backward", 1, 64, 24, 1, 24) == "separate"
     assert plan("backward", 0, 64, 64, 1, 64) == "nothing"

@@ -1035,13 +1035,19 @@ def test_attention_forward_fused(nbat, ntimes, nhead, npiece, masked):
                                                       (2, 257, 1, 64), (1, 640, 4, 64), (3, 33, 5, 16),
                                                       (2, 384, 12, 64), (1, 500, 16, 96), (1, 1024, 8, 128),
                                                       (3, 200, 6, 32), (1, 300, 4, 48), (1, 100, 1, 128), (1, 512, 2, 128),
-                                                      (1, 700, 2, 96), (1, 600, 1, 128)])
+                                                      (1, 700, 2, 96), (1, 600, 1, 128),
+                                                      (4, 640, 4, 64), (2, 1024, 8, 128), (16, 600, 1, 128)])
 def test_attention_forward_train(nbat, ntimes, nhead, npiece):
     nvec = nhead * npiece
     plan = VMath.attention_plan("forward_train", nbat, ntimes, nvec, nhead, npiece)
-    if npiece % 16 != 0 or ntimes > 1024:
+    four = nhead % 4 == 0 and npiece <= 64 and not (npiece == 64 and ntimes > 512)
+    # more than 512 keys, one head per workgroup and workgroups for at most half of the compute units: the three
+    # separate calls are the faster ones for 1 / 4 / 8 heads of 96 / 64 / 64 and more
+    few = ntimes > 512 and not four and nbat * nhead * ((ntimes + 63) // 64) <= 128 and (
+        (nhead == 1 and npiece >= 96) or (nhead in (4, 8) and npiece >= 64))
+    if npiece % 16 != 0 or ntimes > 1024 or few:
         assert plan == "separate"
-    elif nhead % 4 == 0 and npiece <= 64 and not (npiece == 64 and ntimes > 512):
+    elif four:
         assert plan == "fused, four heads per workgroup"
     else:
         assert plan == "fused"
