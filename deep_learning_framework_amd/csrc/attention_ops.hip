@@ -507,7 +507,7 @@ static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, in
         const int64_t len = nvec * ncol;
         const int64_t quarter = ncol / 4;
         const bool heads4 = ncol % 4 == 0 && (quarter & (quarter - 1)) == 0 && aligned16(io) &&
-                            (pp == nullptr || aligned16(pp)) && len <= 4 * kTB * 8;
+                            (pp == nullptr || aligned16(pp)) && len <= 4 * kTB * 16;
         // forward, many rows that each fit a wave's registers: one wave per row, no barrier (at least four waves
         // per compute unit; fewer rows keep the workgroup-per-row kernel, which puts more threads on each).  The
         // backward pass holds two rows per wave and measured slower this way (17.4 -> 19.6 us): it stays.
@@ -521,12 +521,19 @@ static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, in
             const dim3 g((unsigned)nrow);
             if (len <= 4 * kTB * 2) softmax_axis_heads4_kernel<BACKWARD, 2><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
             else if (len <= 4 * kTB * 4) softmax_axis_heads4_kernel<BACKWARD, 4><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
-            else softmax_axis_heads4_kernel<BACKWARD, 8><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
+            else if (len <= 4 * kTB * 8) softmax_axis_heads4_kernel<BACKWARD, 8><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
+            // (16 heads x 1000 keys: 71.9 us with the three passes over memory)
+            else softmax_axis_heads4_kernel<BACKWARD, 16><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
         } else if (len <= (int64_t)tb * 16)
             softmax_axis_block_reg_kernel<BACKWARD, 16><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol,
                                                                                                  tb, hcoef);
         else if (len <= (int64_t)tb * 32)
             softmax_axis_block_reg_kernel<BACKWARD, 32><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol,
+                                                                                                 tb, hcoef);
+        // (12 heads x 1000 keys: 56.0 us with the three passes over memory, 26.3 here; the backward pass would hold two
+        // rows, 256 registers: 85 us against 40 with the three passes)
+        else if (!BACKWARD && len <= (int64_t)tb * 64)
+            softmax_axis_block_reg_kernel<BACKWARD, 64><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol,
                                                                                                  tb, hcoef);
         else
             softmax_axis_block_kernel<BACKWARD><<<dim3((unsigned)nrow), kTB, 0, stream>>>(io, pp, nvec, (int)ncol, tb,

@@ -663,7 +663,10 @@ def test_softmax_activation_rows():
                                                       # 32s: the kernels that take four heads per workgroup
                                                       (2, 64, 4, 32), (1, 96, 8, 64), (3, 32, 12, 32), (4, 128, 4, 96),
                                                       # whole 128-query tiles of four heads, one workgroup per compute unit
-                                                      (4, 512, 4, 64)])
+                                                      (4, 512, 4, 64),
+                                                      # rows of the scores longer than 8192 floats: the deepest
+                                                      # register-resident softmax variants (12 and 16 heads)
+                                                      (1, 1000, 12, 16), (1, 900, 16, 16)])
 def test_attention_ops_small(nbat, ntimes, nhead, npiece):
     nvec = nhead * npiece
     rng = np.random.default_rng(nbat * 100 + ntimes * 10 + nhead)
