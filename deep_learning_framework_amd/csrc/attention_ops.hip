@@ -483,6 +483,75 @@ __global__ void __launch_bounds__(kTB) softmax_axis_thread_kernel(float* __restr
     }
 }
 
+// Any head count up to 32, a whole outer row per wave, E elements per lane: the first A = H * (64 / H) lanes of a wave
+// walk the row A floats at a time, so a lane's elements all belong to head lane % H and consecutive lanes read
+// consecutive floats; the 64 / H lanes of a head meet by reading each other's partial result (one ds_bpermute per
+// member): no LDS, no barrier.  For the head counts the four-heads layout does not take (2, 3, 6, 12, ...) and rows
+// short enough for a wave's registers the workgroup-per-row kernels above spend their time in two block-wide folds:
+// [64, 128, 128, 12] forward 33.5 us there, [64, 128, 128, 2] 79.7.
+template <bool BACKWARD, int E>
+__global__ void __launch_bounds__(kTB) softmax_axis_wave_heads_kernel(float* __restrict__ io,
+                                                                      const float* __restrict__ pp, int64_t nrow,
+                                                                      int64_t nvec, int ncol,
+                                                                      const float* __restrict__ hcoef) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (kTB / 64) + (threadIdx.x >> 6);
+    if (row >= nrow) return;   // whole waves leave; there is no barrier below
+    const int members = 64 / ncol;           // lanes per head
+    const int active = members * ncol;       // lanes that hold elements
+    const int len = (int)(nvec * ncol);
+    const int head = lane % ncol;
+    const bool on = lane < active;
+    float* __restrict__ r = io + row * (int64_t)len;
+    // every lane ends up with the result of its head (lanes past `active` hold the neutral element and are never read)
+    auto fold = [&](float mine, bool is_max) -> float {
+        float a = is_max ? -FLT_MAX : 0.f;
+        for (int j = 0; j < members; j++) {
+            const float o = __shfl(mine, head + ncol * j);
+            a = is_max ? fmaxf(a, o) : a + o;
+        }
+        return a;
+    };
+    float v[E], q[E];
+#pragma unroll
+    for (int i = 0; i < E; i++) {
+        const int idx = lane + active * i;
+        v[i] = r[min(idx, len - 1)];
+        if (BACKWARD) q[i] = pp[row * (int64_t)len + min(idx, len - 1)];
+    }
+#pragma unroll
+    for (int i = 0; i < E; i++) {
+        const bool in = on && lane + active * i < len;
+        v[i] = in ? v[i] : (BACKWARD ? 0.f : -INFINITY);
+        if (BACKWARD) q[i] = in ? q[i] : 0.f;
+    }
+    if (!BACKWARD) {
+        float mx = -FLT_MAX;
+#pragma unroll
+        for (int i = 0; i < E; i++) mx = fmaxf(mx, v[i]);
+        mx = fold(mx, true);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < E; i++) {
+            v[i] = exp_nonpositive(v[i] - mx);   // padding holds -inf: exp gives 0
+            sum += v[i];
+        }
+        const float inv = 1.0f / fold(sum, false);
+#pragma unroll
+        for (int i = 0; i < E; i++)
+            if (on && lane + active * i < len) r[lane + active * i] = v[i] * inv;
+    } else {
+        const float coef = hcoef ? *hcoef : 0.f;
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < E; i++) dot += q[i] * v[i];
+        dot = fold(dot, false);
+#pragma unroll
+        for (int i = 0; i < E; i++)
+            if (on && lane + active * i < len) r[lane + active * i] = coef * q[i] * (v[i] - dot);
+    }
+}
+
 template <bool BACKWARD>
 static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, int64_t nvec, int64_t ncol,
                                     const float* hcoef, hipStream_t stream) {
@@ -517,6 +586,17 @@ static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, in
             if (len <= 4 * 64 * 4) softmax_axis_heads4_wave_kernel<BACKWARD, 4><<<g, kTB, 0, stream>>>(io, pp, nrow, nvec, nc, hcoef);
             else if (len <= 4 * 64 * 8) softmax_axis_heads4_wave_kernel<BACKWARD, 8><<<g, kTB, 0, stream>>>(io, pp, nrow, nvec, nc, hcoef);
             else softmax_axis_heads4_wave_kernel<BACKWARD, 16><<<g, kTB, 0, stream>>>(io, pp, nrow, nvec, nc, hcoef);
+        } else if (!heads4 && ncol <= 32 && nrow >= 4 * (int64_t)compute_units() &&
+                   len <= (int64_t)(64 / ncol) * ncol * (BACKWARD ? 16 : 32)) {
+            // many rows that each fit a wave's registers, any head count: [64, 128, 128, 12] forward 33.5 -> 17.3 us, 6 heads
+            // 39.5 -> 9.0, 2 heads 79.7 -> 10.2 (backward 37.8 -> 6.9), [256, 64, 64, 12] 53.7 -> 16.4
+            const dim3 g((unsigned)((nrow + kTB / 64 - 1) / (kTB / 64)));
+            const int nc = (int)ncol;
+            const int64_t per_lane = (len + (64 / ncol) * ncol - 1) / ((64 / ncol) * ncol);
+            if (per_lane <= 4) softmax_axis_wave_heads_kernel<BACKWARD, 4><<<g, kTB, 0, stream>>>(io, pp, nrow, nvec, nc, hcoef);
+            else if (per_lane <= 8) softmax_axis_wave_heads_kernel<BACKWARD, 8><<<g, kTB, 0, stream>>>(io, pp, nrow, nvec, nc, hcoef);
+            else if (per_lane <= 16) softmax_axis_wave_heads_kernel<BACKWARD, 16><<<g, kTB, 0, stream>>>(io, pp, nrow, nvec, nc, hcoef);
+            else softmax_axis_wave_heads_kernel<BACKWARD, 32><<<g, kTB, 0, stream>>>(io, pp, nrow, nvec, nc, hcoef);
         } else if (heads4) {
             const dim3 g((unsigned)nrow);
             if (len <= 4 * kTB * 2) softmax_axis_heads4_kernel<BACKWARD, 2><<<g, kTB, 0, stream>>>(io, pp, nvec, (int)ncol, hcoef);
