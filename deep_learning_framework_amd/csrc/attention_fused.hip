@@ -775,12 +775,13 @@ bool attention_probs_four_heads(const float* pp, int64_t ntimes, int64_t nhead, 
 // one or two) the launch neither fills the compute units nor hides its latencies: the three separate calls, whose
 // kernels spread the same work over more workgroups, are faster there.  Measured at 1000 keys, one launch | three
 // calls, us: 8 x 1 head of 128 100.0 | 61.7, of 96 61.3 | 57.1 (of 64: 45.0 | 52.6, stays); 2 x 4 heads of 64 82.0 | 60.9,
-// 1 x 8 heads of 64 83.1 | 53.8, of 96 97.5 | 85.3, of 128 110.0 | 88.9; 12 heads and head counts outside whole fours
-// stay (1 x 12 heads of 64: 91.9 | 132.8).
+// 1 x 8 heads of 64 83.1 | 53.8, of 96 97.5 | 85.3, of 128 110.0 | 88.9; 4 x 2 heads of 128 98.1 | 73.7, 1 x 6 heads of 128
+// 105.2 | 80.9; with workgroups for more than half of the compute units the one launch stays (1 x 12 heads of 64:
+// 91.7 | 102.7, 3 x 3 heads of 128: 102.6 | 115.4).
 bool attention_probs_pays(const float* pp, int64_t nbat, int64_t ntimes, int64_t nhead, int64_t npiece) {
     if (ntimes <= 512 || probs_four_heads(pp, nhead, npiece, ntimes)) return true;
     if (nbat * nhead * ((ntimes + kFaQ - 1) / kFaQ) > compute_units() / 2) return true;
-    return !((nhead == 1 && npiece >= 96) || ((nhead == 4 || nhead == 8) && npiece >= 64));
+    return !((nhead == 1 && npiece >= 96) || (nhead >= 2 && npiece >= 64));
 }
 
 int launch_attention_probs(float* o, float* pp, const float* q, const float* k, const float* v, int64_t nbat,

@@ -1045,9 +1045,9 @@ def test_attention_forward_train(nbat, ntimes, nhead, npiece):
     plan = VMath.attention_plan("forward_train", nbat, ntimes, nvec, nhead, npiece)
     four = nhead % 4 == 0 and npiece <= 64 and not (npiece == 64 and ntimes > 512)
     # more than 512 keys, one head per workgroup and workgroups for at most half of the compute units: the three
-    # separate calls are the faster ones for 1 / 4 / 8 heads of 96 / 64 / 64 and more
+    # separate calls are the faster ones for one head of 96 and more, several heads of 64 and more
     few = ntimes > 512 and not four and nbat * nhead * ((ntimes + 63) // 64) <= 128 and (
-        (nhead == 1 and npiece >= 96) or (nhead in (4, 8) and npiece >= 64))
+        (nhead == 1 and npiece >= 96) or (nhead >= 2 and npiece >= 64))
     if npiece % 16 != 0 or ntimes > 1024 or few:
         assert plan == "separate"
     elif four:
