@@ -387,6 +387,37 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
         y = torch.empty((m, n), device=dev)
         row("batch of %d rows: Y = X.W^T, W %d x %d (%s)" % (m, n, k, kai.VMath.gemm_plan(0, 1, m, n, k)),
             lambda: L.kai_matmul(0, P(y), P(w), P(x), I(n), I(m), I(k), 0), flops=2.0 * m * n * k)
+    # shapes off the configurations' grid that the sweep over row counts (--rows-sweep) brought rules for: W from HBM
+    # (rotating buffers beyond the last-level cache)
+    for m, n, k in ((1, 4096, 11008), (4, 3072, 4096), (16, 4352, 4096), (24, 4096, 2048), (1, 50257, 768)):
+        nb = max(2, min(24, (520 << 20) // (n * k * 4)))
+        ws2 = [torch.rand((n, k), device=dev, generator=g) * 0.1 - 0.05 for _ in range(nb)]
+        x = torch.randn((m, k), device=dev, generator=g)
+        y = torch.empty((m, n), device=dev)
+        cnt = [0]
+
+        def call_cold(ws2=ws2, x=x, y=y, m=m, n=n, k=k, nb=nb, cnt=cnt):
+            cnt[0] += 1
+            L.kai_matmul(0, P(y), P(ws2[cnt[0] % nb]), P(x), I(n), I(m), I(k), 0)
+
+        row("%d row%s: Y = X.W^T, W %d x %d from HBM (%s)" % (m, "" if m == 1 else "s", n, k, kai.VMath.gemm_plan(0, 1, m, n, k)),
+            call_cold, iters=48, flops=2.0 * m * n * k, nbytes=4.0 * (k * n + m * k + m * n))
+        del ws2
+    # the score softmax for a head count outside the four-heads layout, short sequences (one row of the scores per wave)
+    sp = torch.randn((64, 128, 128, 12), device=dev, generator=g)
+    row("softmax_direct_on_axis [64,128,128,12] (in place)", lambda: L.kai_softmax_direct_on_axis(0, P(sp), I(64 * 128), I(128), I(12)),
+        nbytes=2.0 * sp.numel() * 4)
+    del sp
+    # a dense layer's whole backward at a training batch (the bias gradient on a kernel of its own from here on)
+    yv_, nd2_, xv_ = 4096, 512, 1024
+    gy_ = torch.randn((nd2_, yv_), device=dev, generator=g) * 0.01
+    x_ = torch.randn((nd2_, xv_), device=dev, generator=g)
+    w_ = torch.rand((yv_, xv_), device=dev, generator=g) * 0.1 - 0.05
+    pre_ = torch.randn((nd2_, yv_), device=dev, generator=g)
+    gx_, gw_, gb_ = torch.empty((nd2_, xv_), device=dev), torch.empty((yv_, xv_), device=dev), torch.empty((yv_,), device=dev)
+    row("dense backward with ReLU, 512 x (1024 -> 4096): dX, dW, db in one call (kai_dense_backward)",
+        lambda: L.kai_dense_backward(0, P(gx_), P(gw_), P(gb_), None, P(gy_), P(w_), P(x_), P(pre_), I(yv_), I(nd2_), I(xv_), 1, None, 0),
+        iters=20, flops=4.0 * yv_ * nd2_ * xv_)
     # one LSTM layer forward as the engine's loop issues it (vtensor.cpp:2455-2492): 32 steps of 64 x 256 -> 4 x 256
     nt_, nd_, ni_, nr_ = 32, 64, 256, 256
     xs = torch.randn((nt_, nd_, ni_), device=dev, generator=g)
