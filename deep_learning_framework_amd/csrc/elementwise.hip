@@ -207,8 +207,118 @@ __global__ void __launch_bounds__(kEwThreads) softmax_rows_kernel(float* __restr
     }
 }
 
+// The same with the row in a wave's registers (ncol <= 64 * E): one read of x, one expf per element, the three
+// loops of the kernel above become one load, one store; up to 4096 columns (E = 64).
+template <bool BACKWARD, int E>
+__global__ void __launch_bounds__(kEwThreads) softmax_rows_reg_kernel(float* __restrict__ out,
+                                                                      const float* __restrict__ gy,
+                                                                      const float* __restrict__ x, int64_t nrow,
+                                                                      int64_t ncol) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
+    if (row >= nrow) return;
+    const float* __restrict__ xr = x + row * ncol;
+    float v[E], gr[E];
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int i = 0; i < E; i++) {
+        const int64_t c = lane + 64 * i;
+        v[i] = c < ncol ? xr[c] : -INFINITY;
+        if (BACKWARD) gr[i] = c < ncol ? gy[row * ncol + c] : 0.f;
+        mx = fmaxf(mx, v[i]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < E; i++) {
+        v[i] = lane + 64 * i < ncol ? expf(v[i] - mx) : 0.f;
+        sum += v[i];
+    }
+    sum = wave_add(sum);
+    if (!BACKWARD) {
+#pragma unroll
+        for (int i = 0; i < E; i++)
+            if (lane + 64 * i < ncol) out[row * ncol + lane + 64 * i] = v[i] / sum;
+    } else {
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < E; i++) {
+            v[i] = v[i] / sum;
+            dot += v[i] * gr[i];
+        }
+        dot = wave_add(dot);
+#pragma unroll
+        for (int i = 0; i < E; i++)
+            if (lane + 64 * i < ncol) out[row * ncol + lane + 64 * i] = v[i] * gr[i] - v[i] * dot;
+    }
+}
+
+// Long rows, or few of them: a workgroup of 1024 threads per row, the three passes of the first kernel with
+// block-wide reductions (a row of 50257 floats is 200 KB: it comes from L2 on the second and third pass).  One wave
+// per row left [64, 50257] on 64 waves: 368 us.
+constexpr int kSmxThreads = 1024;
+template <bool BACKWARD>
+__global__ void __launch_bounds__(kSmxThreads) softmax_rows_block_kernel(float* __restrict__ out,
+                                                                         const float* __restrict__ gy,
+                                                                         const float* __restrict__ x, int64_t ncol) {
+    __shared__ float red[3][kSmxThreads / 64];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int64_t row = blockIdx.x;
+    const float* __restrict__ xr = x + row * ncol;
+    auto block_fold = [&](float mine, bool is_max, int which) -> float {
+        mine = is_max ? wave_max(mine) : wave_add(mine);
+        if (lane == 0) red[which][wave] = mine;
+        __syncthreads();
+        float a = red[which][0];
+        for (int w = 1; w < kSmxThreads / 64; w++) a = is_max ? fmaxf(a, red[which][w]) : a + red[which][w];
+        return a;
+    };
+    float mx = -FLT_MAX;
+    for (int64_t c = t; c < ncol; c += kSmxThreads) mx = fmaxf(mx, xr[c]);
+    mx = block_fold(mx, true, 0);
+    float sum = 0.f;
+    for (int64_t c = t; c < ncol; c += kSmxThreads) sum += expf(xr[c] - mx);
+    sum = block_fold(sum, false, 1);
+    if (!BACKWARD) {
+        for (int64_t c = t; c < ncol; c += kSmxThreads) out[row * ncol + c] = expf(xr[c] - mx) / sum;
+    } else {
+        const float* __restrict__ gr = gy + row * ncol;
+        float dot = 0.f;
+        for (int64_t c = t; c < ncol; c += kSmxThreads) dot += (expf(xr[c] - mx) / sum) * gr[c];
+        dot = block_fold(dot, false, 2);
+        for (int64_t c = t; c < ncol; c += kSmxThreads) {
+            const float yi = expf(xr[c] - mx) / sum;
+            out[row * ncol + c] = yi * gr[c] - yi * dot;
+        }
+    }
+}
+
+// which of the three: rows of up to 4096 columns in registers, one wave each; longer rows, and rows of 1024 columns
+// and more when there are fewer rows than waves that the compute units hold, a workgroup each; else the first kernel
+template <bool BACKWARD>
+static int launch_softmax_rows_impl(float* out, const float* gy, const float* x, int64_t nrow, int64_t ncol,
+                                    hipStream_t stream) {
+    const int64_t blocks = (nrow + kEwThreads / 64 - 1) / (kEwThreads / 64);
+    if (blocks > kMaxDim || nrow > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "activate(softmax): too many rows");
+    const bool few_rows = nrow < 8 * (int64_t)compute_units();
+    if (ncol > 4096 || (few_rows && ncol >= 1024)) {
+        softmax_rows_block_kernel<BACKWARD><<<dim3((unsigned)nrow), kSmxThreads, 0, stream>>>(out, gy, x, ncol);
+        return check_launch("softmax_rows_block_kernel");
+    }
+    const dim3 g((unsigned)blocks);
+    if (ncol <= 64) softmax_rows_reg_kernel<BACKWARD, 1><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    else if (ncol <= 128) softmax_rows_reg_kernel<BACKWARD, 2><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    else if (ncol <= 256) softmax_rows_reg_kernel<BACKWARD, 4><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    else if (ncol <= 512) softmax_rows_reg_kernel<BACKWARD, 8><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    else if (ncol <= 1024) softmax_rows_reg_kernel<BACKWARD, 16><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    else if (ncol <= 2048) softmax_rows_reg_kernel<BACKWARD, 32><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    else softmax_rows_reg_kernel<BACKWARD, 64><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    return check_launch("softmax_rows_reg_kernel");
+}
+
 int launch_softmax_rows(float* y, const float* x, int64_t nrow, int64_t ncol, hipStream_t stream) {
     if (nrow <= 0 || ncol <= 0) return KAI_OK;
+    if (y != x) return launch_softmax_rows_impl<false>(y, nullptr, x, nrow, ncol, stream);
     const int64_t blocks = (nrow + kEwThreads / 64 - 1) / (kEwThreads / 64);
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "activate(softmax): too many rows");
     softmax_rows_kernel<false><<<dim3((unsigned)blocks), kEwThreads, 0, stream>>>(y, nullptr, x, nrow, ncol);
@@ -218,6 +328,7 @@ int launch_softmax_rows(float* y, const float* x, int64_t nrow, int64_t ncol, hi
 int launch_softmax_rows_backward(float* gx, const float* gy, const float* x, int64_t nrow, int64_t ncol,
                                  hipStream_t stream) {
     if (nrow <= 0 || ncol <= 0) return KAI_OK;
+    if (gx != x && gx != gy) return launch_softmax_rows_impl<true>(gx, gy, x, nrow, ncol, stream);
     const int64_t blocks = (nrow + kEwThreads / 64 - 1) / (kEwThreads / 64);
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "activate_backward(softmax): too many rows");
     softmax_rows_kernel<true><<<dim3((unsigned)blocks), kEwThreads, 0, stream>>>(gx, gy, x, nrow, ncol);

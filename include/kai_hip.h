@@ -325,7 +325,8 @@ int kai_subtract_param_grad(int device, float* pp, const float* pg, int64_t nrow
 int kai_apply_decay(int device, float* pd, const float* pp, const float* pg, int64_t nrow, const float* hL1Decay,
                     const float* hL2Decay);
 /* VMath::eval_adam_delta, vmath.cu:449-490 (vmath.h:31).  One Adam step: ps, pt (moments) and pn (step
- * count, a float tensor) are updated in place, pa receives sterm / (sqrt(tterm) + epsilon). */
+ * count, a float tensor) are updated in place, pa receives sterm / (sqrt(tterm) + epsilon).  All five tensors
+ * hold nrow elements, pn included: the reference keeps one step count per parameter element (pn[n] += 1). */
 int kai_eval_adam_delta(int device, float* pa, const float* pg, float* ps, float* pt, float* pn, int64_t nrow,
                         const float* hRo1, const float* hRo2, const float* hEpsilon);
 

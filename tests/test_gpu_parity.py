@@ -636,19 +636,34 @@ def test_relu_special_values_and_null_leaky_alpha():
     np.testing.assert_array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)])
 
 
-def test_softmax_activation_rows():
-    rng = np.random.default_rng(5)
-    x = (4 * rng.standard_normal((50, 77))).astype(np.float32)
+# rows in a wave's registers (up to 4096 columns, every register depth), a workgroup per row (longer rows, and few
+# rows of 1024 columns and more), one element, in place (the three-pass kernel)
+@pytest.mark.parametrize("nrow,ncol", [(50, 77), (3000, 10), (300, 64), (300, 65), (500, 130), (300, 300), (300, 600),
+                                       (2100, 1000), (2100, 2048), (40, 1500), (300, 2049), (2100, 3000), (2060, 4096), (64, 4097), (7, 50257), (5, 1)])
+def test_softmax_activation_rows(nrow, ncol):
+    rng = np.random.default_rng(5 + nrow + ncol)
+    x = (4 * rng.standard_normal((nrow, ncol))).astype(np.float32)
     gy = rng.standard_normal(x.shape).astype(np.float32)
     dx, dgy = dev(x), dev(gy)
     y, gx = DB(x.nbytes), DB(x.nbytes)
-    VMath.activate(0, y, dx, 50, 77, kai.ACT["softmax"], None)
-    ref = ko.activate(x, "softmax")
+    VMath.activate(0, y, dx, nrow, ncol, kai.ACT["softmax"], None)
+    if ncol <= 4096 and nrow * ncol <= 1000000:
+        ref = ko.activate(x, "softmax")
+    else:
+        # the large cases against the exact value (the oracle's row loop would take minutes, and it agrees with the
+        # exact value to 1e-6 at these lengths, as the smaller cases show); beyond 4096 columns the exact value is the
+        # better check anyway: the reference adds the 50257 exponentials of a row one after the other in float, which
+        # alone is worth 7e-5 of the sum, while the kernel's tree of partial sums is closer to the exact value
+        e = np.exp(x.astype(np.float64) - x.max(axis=1, keepdims=True))
+        ref = e / e.sum(axis=1, keepdims=True)
     check(y.to_numpy(x.shape), ref, what="softmax activation")
-    VMath.activate_backward(0, gx, dgy, dx, 50, 77, kai.ACT["softmax"], None)
-    p = ref.astype(np.float64)
+    VMath.activate_backward(0, gx, dgy, dx, nrow, ncol, kai.ACT["softmax"], None)
+    p = np.asarray(ref, np.float64)
     ref_g = p * (gy - (p * gy).sum(axis=1, keepdims=True))
     check(gx.to_numpy(x.shape), ref_g, what="softmax activation backward")
+    if nrow * ncol < 100000:
+        VMath.activate(0, dx, dx, nrow, ncol, kai.ACT["softmax"], None)     # in place
+        check(dx.to_numpy(x.shape), ref, what="softmax activation in place")
 
 
 # ---- attention ops at small sizes, masks, backward --------------------------------------------------------------------
