@@ -6,7 +6,10 @@
 namespace kai {
 
 int launch_add_bias(float* y, const float* a, const float* b, int64_t nrow, int64_t ncol, hipStream_t stream);
-int launch_colsum(float* gb, const float* gy, int64_t nrow, int64_t ncol, int acc, hipStream_t stream);
+// parts: the number colsum_row_parts() gives; with two and more, parts_buf holds parts * ncol floats of scratch
+int colsum_row_parts(int64_t nrow, int64_t ncol);
+int launch_colsum(float* gb, const float* gy, int64_t nrow, int64_t ncol, int acc, hipStream_t stream,
+                  float* parts_buf = nullptr, int parts = 1);
 int launch_activate(float* y, const float* x, int64_t total, int act, const float* hleaky, hipStream_t stream);
 int launch_activate_backward(float* gx, const float* gy, const float* x, int64_t total, int act, const float* hleaky,
                              hipStream_t stream);

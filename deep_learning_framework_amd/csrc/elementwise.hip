@@ -67,15 +67,20 @@ constexpr int kColsumCols = 32;
 constexpr int kColsumRows = 32;
 
 __global__ void __launch_bounds__(kColsumCols* kColsumRows)
-    colsum_kernel(float* __restrict__ gb, const float* __restrict__ gy, int64_t nrow, int64_t ncol, int acc) {
+    colsum_kernel(float* __restrict__ gb, const float* __restrict__ gy, int64_t nrow_all, int64_t ncol, int acc,
+                  int64_t rows_per_part) {
     __shared__ float part[kColsumRows][kColsumCols + 1];
     const int tx = threadIdx.x % kColsumCols;
     const int ty = threadIdx.x / kColsumCols;
     const int64_t c = (int64_t)blockIdx.x * kColsumCols + tx;
+    // blockIdx.y: a run of rows_per_part rows whose sums go to row blockIdx.y of gb (one run: gb itself)
+    const int64_t r_first = (int64_t)blockIdx.y * rows_per_part;
+    const int64_t nrow = min(nrow_all, r_first + rows_per_part);
+    gb += (int64_t)blockIdx.y * ncol;
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     if (c < ncol) {
         const float* __restrict__ p = gy + c;
-        int64_t r = ty;
+        int64_t r = r_first + ty;
         for (; r + 3 * kColsumRows < nrow; r += 4 * kColsumRows) {
             s0 += p[r * ncol];
             s1 += p[(r + kColsumRows) * ncol];
@@ -95,11 +100,35 @@ __global__ void __launch_bounds__(kColsumCols* kColsumRows)
     }
 }
 
-int launch_colsum(float* gb, const float* gy, int64_t nrow, int64_t ncol, int acc, hipStream_t stream) {
+// Few columns and many rows (the bias gradient of a narrow output layer over a long batch): one workgroup per 32
+// columns walks all the rows alone, [100000, 12] took 249 us.  The rows are then cut into runs, one workgroup per run
+// and column block, and a second launch adds the runs' sums.
+int colsum_row_parts(int64_t nrow, int64_t ncol) {
+    const int64_t blocks = (ncol + kColsumCols - 1) / kColsumCols;
+    const int64_t cus = compute_units();
+    if (blocks * 2 > cus || nrow < 6144) return 1;   // shorter: the second launch costs what the runs save
+    int64_t parts = 4 * cus / blocks;
+    if (parts > nrow / 256) parts = nrow / 256;
+    if (parts > 512) parts = 512;
+    return parts < 2 ? 1 : (int)parts;
+}
+
+int launch_colsum(float* gb, const float* gy, int64_t nrow, int64_t ncol, int acc, hipStream_t stream, float* parts_buf,
+                  int parts) {
     if (ncol <= 0) return KAI_OK;
     const int64_t blocks = (ncol + kColsumCols - 1) / kColsumCols;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "add_bias_backward_b: too many columns");
-    colsum_kernel<<<dim3((unsigned)blocks), dim3(kColsumCols * kColsumRows), 0, stream>>>(gb, gy, nrow, ncol, acc);
+    if (parts < 2 || parts_buf == nullptr) {
+        colsum_kernel<<<dim3((unsigned)blocks), dim3(kColsumCols * kColsumRows), 0, stream>>>(gb, gy, nrow, ncol, acc, nrow);
+        return check_launch("colsum_kernel");
+    }
+    const int64_t rows_per_part = ((nrow + parts - 1) / parts + kColsumRows - 1) / kColsumRows * kColsumRows;
+    const int nparts = (int)((nrow + rows_per_part - 1) / rows_per_part);
+    colsum_kernel<<<dim3((unsigned)blocks, (unsigned)nparts), dim3(kColsumCols * kColsumRows), 0, stream>>>(
+        parts_buf, gy, nrow, ncol, 0, rows_per_part);
+    KAI_TRY(check_launch("colsum_kernel"));
+    // the runs' sums are a matrix of nparts rows: the same kernel adds them up, in its fixed order
+    colsum_kernel<<<dim3((unsigned)blocks), dim3(kColsumCols * kColsumRows), 0, stream>>>(gb, parts_buf, nparts, ncol, acc, nparts);
     return check_launch("colsum_kernel");
 }
 

@@ -461,7 +461,10 @@ int kai_add_bias_backward_b(int device, float* pgb, const float* pgy, int64_t nr
     if (ncol == 0) return KAI_OK;
     KAI_REQUIRE_PTR(pgb);
     if (nrow > 0) KAI_REQUIRE_PTR(pgy);
-    return launch_colsum(pgb, pgy, nrow, ncol, acc != 0, current_stream());
+    const int parts = colsum_row_parts(nrow, ncol);
+    float* parts_buf = nullptr;
+    if (parts >= 2) KAI_TRY(workspace(parts * ncol * (int64_t)sizeof(float), &parts_buf));
+    return launch_colsum(pgb, pgy, nrow, ncol, acc != 0, current_stream(), parts_buf, parts);
 }
 
 int kai_activate(int device, float* py, const float* px, int64_t nrow, int64_t ncol, int actFunc,

@@ -562,7 +562,9 @@ def test_empty_and_degenerate_sizes():
 
 # ---- bias, activations ----------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("nrow,ncol", [(1, 1), (7, 13), (256, 1024), (33, 4), (1000, 333), (5000, 64)])
+@pytest.mark.parametrize("nrow,ncol", [(1, 1), (7, 13), (256, 1024), (33, 4), (1000, 333), (5000, 64),
+                                       # few columns under many rows: the rows are cut into runs, two launches
+                                       (100000, 12), (32768, 10), (6144, 1), (20001, 100), (8193, 2000)])
 def test_add_bias_and_column_sum(nrow, ncol):
     rng = np.random.default_rng(nrow * 31 + ncol)
     a = rng.standard_normal((nrow, ncol)).astype(np.float32)
