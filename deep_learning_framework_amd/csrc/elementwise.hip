@@ -603,9 +603,60 @@ __global__ void __launch_bounds__(kEwThreads)
     }
 }
 
+// Four elements per thread.  The two powers are most of the arithmetic of a step; the four step counts of a thread
+// are equal wherever a tensor has been updated as a whole, and then one pair of powers serves all four (the same
+// function on the same arguments: the same bits).
+__global__ void __launch_bounds__(kEwThreads)
+    adam_delta_vec_kernel(float4* __restrict__ a, const float4* __restrict__ g, float4* __restrict__ s,
+                          float4* __restrict__ t, float4* __restrict__ nstep, int64_t n4,
+                          const float* __restrict__ hro1, const float* __restrict__ hro2,
+                          const float* __restrict__ heps) {
+    const float ro1 = hro1 ? *hro1 : 0.f;
+    const float ro2 = hro2 ? *hro2 : 0.f;
+    const float eps = heps ? *heps : 0.f;
+    const int64_t stride = (int64_t)gridDim.x * kEwThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < n4; i += stride) {
+        const float4 gv = g[i], nv = nstep[i], sv = s[i], tv = t[i];
+        const float gi[4] = {gv.x, gv.y, gv.z, gv.w};
+        const float so[4] = {sv.x, sv.y, sv.z, sv.w};
+        const float to[4] = {tv.x, tv.y, tv.z, tv.w};
+        const float ns[4] = {nv.x + 1.f, nv.y + 1.f, nv.z + 1.f, nv.w + 1.f};
+        float p1[4], p2[4];
+        if (ns[0] == ns[1] && ns[0] == ns[2] && ns[0] == ns[3]) {
+            p1[0] = p1[1] = p1[2] = p1[3] = powf(ro1, ns[0]);
+            p2[0] = p2[1] = p2[2] = p2[3] = powf(ro2, ns[0]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                p1[j] = powf(ro1, ns[j]);
+                p2[j] = powf(ro2, ns[j]);
+            }
+        }
+        float si[4], ti[4], ai[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            si[j] = ro1 * so[j] + (1.f - ro1) * gi[j];
+            ti[j] = ro2 * to[j] + (1.f - ro2) * gi[j] * gi[j];
+            const float sterm = si[j] / (1.f - p1[j]);
+            const float tterm = ti[j] / (1.f - p2[j]);
+            ai[j] = sterm / (sqrtf(tterm) + eps);
+        }
+        s[i] = make_float4(si[0], si[1], si[2], si[3]);
+        t[i] = make_float4(ti[0], ti[1], ti[2], ti[3]);
+        a[i] = make_float4(ai[0], ai[1], ai[2], ai[3]);
+        nstep[i] = make_float4(ns[0], ns[1], ns[2], ns[3]);
+    }
+}
+
 int launch_eval_adam_delta(float* a, const float* g, float* s, float* t, float* nstep, int64_t n, const float* hro1,
                            const float* hro2, const float* heps, hipStream_t stream) {
     if (n <= 0) return KAI_OK;
+    if (n % 4 == 0 && aligned16(a) && aligned16(g) && aligned16(s) && aligned16(t) && aligned16(nstep)) {
+        adam_delta_vec_kernel<<<blocks_for(n / 4), kEwThreads, 0, stream>>>(
+            reinterpret_cast<float4*>(a), reinterpret_cast<const float4*>(g), reinterpret_cast<float4*>(s),
+            reinterpret_cast<float4*>(t), reinterpret_cast<float4*>(nstep), n / 4, hro1, hro2, heps);
+        return check_launch("adam_delta_vec_kernel");
+    }
     adam_delta_kernel<<<blocks_for(n), kEwThreads, 0, stream>>>(a, g, s, t, nstep, n, hro1, hro2, heps);
     return check_launch("adam_delta_kernel");
 }

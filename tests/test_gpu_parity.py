@@ -1700,6 +1700,15 @@ def test_parameter_update_ops(n):
         np.testing.assert_array_equal(ds.to_numpy((n,)), s)        # the moments use only +, * (rounded as in the oracle)
         np.testing.assert_array_equal(dt.to_numpy((n,)), t)
         np.testing.assert_allclose(da.to_numpy((n,)), a, rtol=2e-6, atol=1e-7)   # powf and sqrtf of two libraries
+    # step counts that differ from element to element (parts of a tensor updated at different times)
+    cnt = (np.arange(n) % 3 + (np.arange(n) // 8) % 2 * 5).astype(np.float32)
+    dn = dev(cnt)
+    gs = rng.standard_normal(n).astype(np.float32)
+    VMath.eval_adam_delta(0, da, dev(gs), ds, dt, dn, n, h1, h2, he)
+    a, s, t, cnt = ko.eval_adam_delta(gs, s, t, cnt, 0.9, 0.999, 1e-8)
+    np.testing.assert_array_equal(dn.to_numpy((n,)), cnt)
+    np.testing.assert_array_equal(ds.to_numpy((n,)), s)
+    np.testing.assert_allclose(da.to_numpy((n,)), a, rtol=2e-6, atol=1e-7)
 
 
 # ---- memory helpers and errors ----------------------------------------------------------------------------------------
