@@ -282,6 +282,47 @@ __global__ void __launch_bounds__(kEwThreads) softmax_rows_reg_kernel(float* __r
     }
 }
 
+// Short rows (ncol <= G = 2 ... 32): 64 / G rows per wave, the folds stay inside a row's G lanes.  A wave per row
+// leaves 52 of 64 lanes idle on the 12 classes of an output layer ([100000, 12] 16 us).
+template <bool BACKWARD, int G>
+__global__ void __launch_bounds__(kEwThreads) softmax_rows_short_kernel(float* __restrict__ out,
+                                                                        const float* __restrict__ gy,
+                                                                        const float* __restrict__ x, int64_t nrow,
+                                                                        int64_t ncol) {
+    const int lane = threadIdx.x & 63, col = lane % G;
+    const int64_t wave = (int64_t)blockIdx.x * (kEwThreads / 64) + (threadIdx.x >> 6);
+    const int64_t row = wave * (64 / G) + lane / G;
+    const bool live = row < nrow && col < ncol;      // no early exit: every lane takes part in the shuffles
+    const int64_t at = live ? row * ncol + col : 0;
+    const float v = live ? x[at] : -INFINITY;
+    float mx = fmaxf(v, -FLT_MAX);
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    const float e = live ? expf(v - mx) : 0.f;
+    float sum = e;
+#pragma unroll
+    for (int off = G / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (!BACKWARD) {
+        if (live) out[at] = e / sum;
+    } else {
+        const float yi = live ? e / sum : 0.f;
+        const float g = live ? gy[at] : 0.f;
+        float dot = yi * g;
+#pragma unroll
+        for (int off = G / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+        if (live) out[at] = yi * g - yi * dot;
+    }
+}
+
+template <bool BACKWARD, int G>
+static int launch_softmax_rows_short(float* out, const float* gy, const float* x, int64_t nrow, int64_t ncol,
+                                     hipStream_t stream) {
+    const int64_t rows_per_block = (kEwThreads / 64) * (64 / G);
+    const int64_t blocks = (nrow + rows_per_block - 1) / rows_per_block;
+    softmax_rows_short_kernel<BACKWARD, G><<<dim3((unsigned)blocks), kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
+    return check_launch("softmax_rows_short_kernel");
+}
+
 // Long rows, or few of them: a workgroup of 1024 threads per row, the three passes of the first kernel with
 // block-wide reductions (a row of 50257 floats is 200 KB: it comes from L2 on the second and third pass).  One wave
 // per row left [64, 50257] on 64 waves: 368 us.
@@ -396,6 +437,11 @@ static int launch_softmax_rows_impl(float* out, const float* gy, const float* x,
         softmax_rows_block_kernel<BACKWARD><<<dim3((unsigned)nrow), kSmxThreads, 0, stream>>>(out, gy, x, ncol);
         return check_launch("softmax_rows_block_kernel");
     }
+    if (ncol <= 2) return launch_softmax_rows_short<BACKWARD, 2>(out, gy, x, nrow, ncol, stream);
+    if (ncol <= 4) return launch_softmax_rows_short<BACKWARD, 4>(out, gy, x, nrow, ncol, stream);
+    if (ncol <= 8) return launch_softmax_rows_short<BACKWARD, 8>(out, gy, x, nrow, ncol, stream);
+    if (ncol <= 16) return launch_softmax_rows_short<BACKWARD, 16>(out, gy, x, nrow, ncol, stream);
+    if (ncol <= 32) return launch_softmax_rows_short<BACKWARD, 32>(out, gy, x, nrow, ncol, stream);
     const dim3 g((unsigned)blocks);
     if (ncol <= 64) softmax_rows_reg_kernel<BACKWARD, 1><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);
     else if (ncol <= 128) softmax_rows_reg_kernel<BACKWARD, 2><<<g, kEwThreads, 0, stream>>>(out, gy, x, nrow, ncol);

@@ -638,12 +638,14 @@ def test_relu_special_values_and_null_leaky_alpha():
     np.testing.assert_array_equal(got[~np.isnan(ref)], ref[~np.isnan(ref)])
 
 
-# rows in a wave's registers (up to 4096 columns, every register depth), a workgroup per row (longer rows, and few
+# several short rows per wave, rows in a wave's registers (up to 4096 columns, every register depth), a workgroup per row (longer rows, and few
 # rows of 1024 columns and more), one element, in place (the three-pass kernel)
 @pytest.mark.parametrize("nrow,ncol", [(50, 77), (3000, 10), (300, 64), (300, 65), (500, 130), (300, 300), (300, 600),
                                        (2100, 1000), (2100, 2048), (40, 1500), (300, 2049), (2100, 3000), (2060, 4096), (64, 4097), (7, 50257), (5, 1),
                                        # a workgroup's registers: every depth, and the first length beyond them
-                                       (40, 4096), (33, 8192), (20, 8193), (20, 12289), (16, 16384), (9, 16385)])
+                                       (40, 4096), (33, 8192), (20, 8193), (20, 12289), (16, 16384), (9, 16385),
+                                       # several short rows per wave
+                                       (100001, 12), (1001, 2), (1001, 3), (999, 5), (777, 17), (501, 32), (501, 33)])
 def test_softmax_activation_rows(nrow, ncol):
     rng = np.random.default_rng(5 + nrow + ncol)
     x = (4 * rng.standard_normal((nrow, ncol))).astype(np.float32)
