@@ -501,7 +501,7 @@ def plan_audit(torch, kai, stream, dev, out_path, shapes_text=None):
                (32, 4096, 4096), (33, 4096, 4096), (96, 4096, 11008), (200, 6656, 4096), (144, 5120, 4096)]
     if shapes_text:   # "M,N,K;M,N,K;...": the caller's own shapes instead of the built-in list
         shapes = [tuple(int(v) for v in item.split(",")) for item in shapes_text.split(";") if item.strip()]
-    tiles = ("medium", "wide", "small", "flat")
+    tiles = ("large", "medium", "wide", "small", "flat")
     splits = (1, 2, 3, 4, 6, 8, 12, 16)
     forms = (("NT", 0, 1), ("NN", 0, 0), ("TN", 1, 0))
 
