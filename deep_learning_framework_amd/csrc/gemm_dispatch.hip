@@ -132,7 +132,10 @@ double tiled_cost(int tile, bool both_kc, bool whole, int64_t M, int64_t N, int6
         // (the surcharge for edge tiles applies to the forms with an operand that is not K-contiguous only: the
         // sweeps this was fitted to were run with exactly this expression, and with both operands K-contiguous the
         // edge variant's range-checked loads measured like the whole-tile ones)
-        const double c = both_kc ? 0.48 : (per_cu == 1 ? 0.57 : per_cu == 2 ? 0.54 : 0.52) * (whole ? 1.0 : 1.05);
+        // (16 rounds and more of edge-checked tiles with both operands K-contiguous measured 0.52 .. 0.57: 5000^3 2020 us
+        // where the 64 x 128 tile takes 1889, 7000 x 3000 x 3000 1057 against 990, 5000 x 5000 x 1000 445 against 418)
+        const double c = both_kc ? (!whole && per_cu >= 16 ? 0.52 : 0.48)
+                                 : (per_cu == 1 ? 0.57 : per_cu == 2 ? 0.54 : 0.52) * (whole ? 1.0 : 1.05);
         t = (double)per_cu * steps * c;
     }
     // the pipelined kernels run the steps after the last whole tile of 32 as a tile of their own, loaded, masked
@@ -194,7 +197,14 @@ GemmPlan plan_gemm(const GemmDesc& d) {
     // fixed buffer (the allocation-free entry point) may be smaller, and the part count is then chosen to fit it
     const int64_t scratch_cap = d.scratch ? std::min(kSplitScratchMax, d.scratch_bytes) : kSplitScratchMax;
     const int64_t t256 = tiles_of(d.M, d.N, d.nbatch, 256), t128 = tiles_of(d.M, d.N, d.nbatch, 128);
-    if (short_side > 128 && t256 >= (3 * cus) / 4 && 4 * ((t256 + cus - 1) / cus) <= (t128 + cus - 1) / cus)
+    // A single round of them must also be well filled, padding counted: 196 .. 210 tiles on 256 units lost 8 .. 15 % to
+    // the smaller tiles (3584^3 796 us against 693 on 64 x 64 tiles, 3600 x 3400 x 4096 912 against 814, 3200 x 4000 x
+    // 2500 564 against 522: M N / (65536 units) = 0.73 .. 0.77), 3840 x 3700 x 2048 1 .. 6 % at 0.85; from 0.88 on
+    // (3840^3, 3712 x 3968 x 3000, 4000^2) the large tile is the fastest.  Two rounds and more only get here with
+    // fills of 0.875 and more.
+    const int64_t rounds256 = (t256 + cus - 1) / cus;
+    const bool fills256 = rounds256 > 1 || d.nbatch > 1 || 100 * d.M * d.N >= 86 * 65536 * cus;
+    if (short_side > 128 && t256 >= (3 * cus) / 4 && 4 * rounds256 <= (t128 + cus - 1) / cus && fills256)
         plan.tile = kTileLarge;
     else if (short_side > 64 && t128 >= cus / 2) {
         // The same count between the 128- and the 64-wide tile, which runs at about 0.88 of the medium tile's

@@ -226,7 +226,12 @@ GEMM_PLANS = [
     ((0, 0, 8192, 8192, 8192), "mfma large whole pipelined staged 2 split 1"),  # the headline product
     ((0, 1, 8192, 8192, 8192), "mfma large whole pipelined staged 2 split 1"),
     ((0, 0, 8191, 8191, 8191), "mfma large ragged pipelined staged 2 split 1"),  # odd sizes keep the pipelined loop
-    ((0, 1, 4100, 4100, 4100), "mfma small ragged pipelined split 1"),   # edges in every dimension: 4225 small tiles (17 rounds) rather than 1089 medium ones (2 + 2 + 1)
+    ((0, 1, 4100, 4100, 4100), "mfma wide ragged pipelined split 1"),   # edges in every dimension: 2145 tiles of 64 x 128 (9 rounds) rather than 1089 medium ones (2 + 2 + 1) or 17 rounds of edge-checked small ones
+    ((0, 1, 3584, 3584, 3584), "mfma small whole pipelined split 1"),   # 196 large tiles would leave a quarter of the units idle for the whole product
+    ((0, 0, 3584, 3584, 3584), "mfma small whole split 1"),
+    ((0, 1, 3840, 3840, 3840), "mfma large whole pipelined staged 2 split 1"),   # 225 of them fill the round well enough
+    ((0, 1, 3840, 3700, 2048), "mfma small ragged pipelined split 1"),   # 225 again, but a fifteenth of a tile column is padding
+    ((0, 1, 5000, 5000, 5000), "mfma wide ragged pipelined split 1"),
     ((0, 1, 4096, 4096, 4096), "mfma large whole pipelined staged 2 split 1"),   # exactly one round of large tiles
     ((0, 1, 3072, 4096, 4096), "mfma medium whole pipelined split 1"),  # 192 large tiles leave a quarter of the chip idle
     ((0, 1, 2048, 2048, 2048), "mfma medium whole pipelined staged 2 split 1"),
