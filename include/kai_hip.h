@@ -78,7 +78,7 @@ int kai_device_synchronize(void);
  * No counterpart in the reference, which only uses the legacy default stream. */
 int kai_set_stream(void* hip_stream);
 /* Releases the scratch memory the library allocated for itself (partial sums of reductions cut into parts,
- * row norms of kai_cosinesim, the probabilities of a kai_attention_forward call that runs as separate
+ * of the column sums of long narrow matrices, row norms of kai_cosinesim, the probabilities of a kai_attention_forward call that runs as separate
  * kernels; one buffer per device, created on first need).  Waits for the device first.  The library stays
  * usable: the buffer is created again on demand.  No counterpart in the reference, whose kernels need no
  * scratch. */
@@ -155,7 +155,8 @@ int64_t kai_matmul_noalloc_scratch_bytes(void);
 
 /* VMath::add_bias, vmath.cu:875-897.  y[r,c] = a[r,c] + b[c]; py may equal pa */
 int kai_add_bias(int device, float* py, const float* pa, const float* pb, int64_t nrow, int64_t ncol);
-/* VMath::add_bias_backward_b, vmath.cu:901-932.  gb[c] (=|+=) sum_r gy[r,c] */
+/* VMath::add_bias_backward_b, vmath.cu:901-932.  gb[c] (=|+=) sum_r gy[r,c].  With 6144 rows and more over few
+ * columns the rows are summed in runs whose sums pass through the library scratch (at most 8 MiB). */
 int kai_add_bias_backward_b(int device, float* pgb, const float* pgy, int64_t nrow, int64_t ncol, int acc);
 
 /* VMath::activate, vmath.cu:3097-3243; py may equal px (except for softmax).  The softmax case
