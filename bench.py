@@ -471,6 +471,15 @@ def per_config_table(torch, kai, stream, dev, with_cpu, warm_ms=40.0, only=None)
     row("transpose [4,512,8,64] -> [4,8,512,64]",
         lambda: L.kai_transpose(0, P(y), P(x), P(info), I(4), I(x.numel())),
         nbytes=8.0 * x.numel(), cpu=lambda: ko.transpose(xc, axes))
+    # the innermost axis changes (keys to the last axis): tiles through LDS inside the general entry point
+    x = torch.randn((16, 512, 12, 64), device=dev, generator=g)
+    y = torch.empty_like(x)
+    info = torch.tensor([[0, 12 * 64 * 512, 512 * 12 * 64], [2, 64 * 512, 12 * 64], [3, 512, 64], [1, 1, 1]],
+                        dtype=torch.int32, device=dev)
+    xc = x.cpu().numpy()
+    row("transpose [16,512,12,64] -> [16,12,64,512]",
+        lambda: L.kai_transpose(0, P(y), P(x), P(info), I(4), I(x.numel())),
+        nbytes=8.0 * x.numel(), cpu=lambda: ko.transpose(xc, (0, 2, 3, 1)))
     x = torch.randn((4096, 4096), device=dev, generator=g)
     y = torch.empty_like(x)
     xc = x.cpu().numpy()

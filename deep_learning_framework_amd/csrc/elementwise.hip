@@ -566,6 +566,83 @@ __device__ __forceinline__ void transpose_axes_body(float* __restrict__ out, con
     }
 }
 
+// The innermost output axis is NOT the innermost source axis (a matrix transposed through the general entry point,
+// channels first <-> channels last, [B, T, H, D] -> [B, H, D, T]): element by element one side is a gather or scatter
+// with a stride of whole rows (4096 x 4096: 67 us, 2.0 TB/s; [64, 512, 12, 64] -> [64, 12, 64, 512] backward 301 us).
+// Here a workgroup moves tiles of TI positions of the innermost output axis (source step s_i) x TJ positions of the
+// innermost source axis (output axis mj, output step y_j) through LDS, so that it reads runs along one and writes
+// runs along the other; TI x TJ = 1024, the side of a short axis (3 channels) shrinks to 4 / 8 / 16 and the other
+// grows.  The remaining axes are counted through per tile.
+constexpr int kTrTileFloats = 1024 + 256;
+// (tensors below 2^31 elements: everything counts in 32 bits; the table stays in LDS -- osz = positions per output
+// axis -- and is read once per tile, so that this path adds no registers to the kernel it shares with the loops above)
+template <bool BACKWARD>
+__device__ __forceinline__ void transpose_axes_tiled(float* __restrict__ out, const float* __restrict__ in,
+                                                     const int64_t* yblk, const int64_t* xblk, const int* osz,
+                                                     int axis_size, int mj, float* tile) {
+    auto uniform = [](int64_t v) -> int { return __builtin_amdgcn_readfirstlane((int)v); };
+    const int last = axis_size - 1;
+    mj = __builtin_amdgcn_readfirstlane(mj);
+    const int len_i = uniform(osz[last]), len_j = uniform(osz[mj]);
+    const int s_i = uniform(xblk[last]), y_j = uniform(yblk[mj]);
+    int log_ti = len_i <= 4 ? 2 : len_i <= 8 ? 3 : len_i <= 16 ? 4 : 5;
+    if (len_j <= 16 && len_i > 16) log_ti = len_j <= 4 ? 8 : len_j <= 8 ? 7 : 6;
+    const int log_tj = 10 - log_ti;
+    const int ti_size = 1 << log_ti, tj_size = 1 << log_tj, pitch = tj_size + 1;
+    const int tiles_i = (len_i + ti_size - 1) >> log_ti, tiles_j = (len_j + tj_size - 1) >> log_tj;
+    int outer = 1;
+    for (int m = 0; m < last; m++)
+        if (m != mj) outer *= uniform(osz[m]);
+    const int tiles = outer * tiles_i * tiles_j;   // at most n / 4: a tile side is 4 at least
+    const int tid = threadIdx.x;
+    for (int t = blockIdx.x; t < tiles; t += gridDim.x) {
+        const int ti = t % tiles_i, rest = t / tiles_i;
+        const int tj = rest % tiles_j;
+        int o = rest / tiles_j, ybase = 0, xbase = 0;
+        for (int m = last - 1; m >= 0; m--) {
+            if (m != mj) {
+                const int sz = uniform(osz[m]);
+                const int c = o % sz;
+                o /= sz;
+                ybase += c * uniform(yblk[m]);
+                xbase += c * uniform(xblk[m]);
+            }
+        }
+        const int i0 = ti << log_ti, j0 = tj << log_tj;
+        const int ni = min(ti_size, len_i - i0), nj = min(tj_size, len_j - j0);
+        const float* __restrict__ src_x = in + (xbase + i0 * s_i + j0);      // forward: in is the source tensor
+        float* __restrict__ dst_y = out + (ybase + j0 * y_j + i0);
+        const float* __restrict__ src_y = in + (ybase + j0 * y_j + i0);      // backward: in is laid out like the output
+        float* __restrict__ dst_x = out + (xbase + i0 * s_i + j0);
+        // runs along j (the source's rows)
+        auto along_j = [&](auto body) {
+#pragma unroll
+            for (int idx = tid; idx < 1024; idx += kEwThreads) {
+                const int ii = idx >> log_tj, jj = idx & (tj_size - 1);
+                if (ii < ni && jj < nj) body(ii, jj);
+            }
+        };
+        // runs along i (the output's rows)
+        auto along_i = [&](auto body) {
+#pragma unroll
+            for (int idx = tid; idx < 1024; idx += kEwThreads) {
+                const int jj = idx >> log_ti, ii = idx & (ti_size - 1);
+                if (ii < ni && jj < nj) body(ii, jj);
+            }
+        };
+        if (!BACKWARD) {
+            along_j([&](int ii, int jj) { tile[ii * pitch + jj] = src_x[ii * s_i + jj]; });
+            __syncthreads();
+            along_i([&](int ii, int jj) { __builtin_nontemporal_store(tile[ii * pitch + jj], dst_y + (jj * y_j + ii)); });
+        } else {
+            along_i([&](int ii, int jj) { tile[ii * pitch + jj] = src_y[jj * y_j + ii]; });
+            __syncthreads();
+            along_j([&](int ii, int jj) { __builtin_nontemporal_store(tile[ii * pitch + jj], dst_x + (ii * s_i + jj)); });
+        }
+        __syncthreads();   // the tile is free for the next one
+    }
+}
+
 // The table lives in device memory (the engine builds it there), so the kernel itself looks whether the innermost
 // output axis is the innermost source axis (the head split / merge [B, T, H, D] <-> [B, H, T, D] of the attention
 // layers and every permutation of outer axes): then whole 128-bit words move, the innermost 4 * k floats being
@@ -575,19 +652,50 @@ __global__ void __launch_bounds__(kEwThreads) transpose_axes_kernel(float* __res
                                                                     const float* __restrict__ in,
                                                                     const int* __restrict__ pn, int axis_size,
                                                                     int64_t n, int aligned16) {
-    // the table is tiny and the same for every thread
+    // the table is tiny and the same for every thread; thread m reads the row of output axis m and leaves what the
+    // choice among the loops needs as bits, so that no thread walks the table again:
+    //   bit 1: the axis allows 128-bit moves (steps in whole fours; the last axis: innermost on both sides)
+    //   bit 2: the axis allows the tiles (only the last one can forbid them: it must be innermost in the output only)
+    //   bit 0, with m in the bits above: the axis walks the source's innermost axis and has more than one position
     __shared__ int64_t yblk[kTrMaxAxes], xblk[kTrMaxAxes];
-    if (threadIdx.x < axis_size) {
-        yblk[threadIdx.x] = pn[threadIdx.x * 3 + 1];
-        xblk[threadIdx.x] = pn[pn[threadIdx.x * 3] * 3 + 2];
+    __shared__ int osz[kTrMaxAxes];   // positions per output axis (where the tensor counts in 32 bits)
+    __shared__ __attribute__((aligned(16))) int flags[kTrMaxAxes];
+    const bool small = n < (1ll << 31);
+    const int last = axis_size - 1;
+    if (threadIdx.x < kTrMaxAxes) {
+        const int m = threadIdx.x;
+        int f = 2 | 4;
+        if (m < axis_size) {
+            const int64_t yb = pn[m * 3 + 1], xb = pn[pn[m * 3] * 3 + 2];
+            const int64_t span = m == 0 ? n : pn[(m - 1) * 3 + 1];   // output elements per step of the axis before
+            yblk[m] = yb;
+            xblk[m] = xb;
+            osz[m] = small ? (int)((uint32_t)span / (uint32_t)max((int)yb, 1)) : 0;
+            if (m == last) f = (yb == 1 && xb == 1 ? 2 : 0) | (yb == 1 && xb > 1 && span > 1 ? 4 : 0);
+            else f = (xb % 4 == 0 && yb % 4 == 0 ? 2 : 0) | 4;
+            if (xb == 1 && span >= 2 * yb) f |= 1 | (m << 4);
+        }
+        flags[m] = f;
     }
     __syncthreads();
-    const int last = axis_size - 1;
+    const int4 fa = *reinterpret_cast<const int4*>(&flags[0]), fb = *reinterpret_cast<const int4*>(&flags[4]);
+    const int fl[kTrMaxAxes] = {fa.x, fa.y, fa.z, fa.w, fb.x, fb.y, fb.z, fb.w};
+    int all = 6, mj = -1;
+#pragma unroll
+    for (int m = 0; m < kTrMaxAxes; m++) {
+        all &= fl[m];
+        mj = max(mj, (fl[m] & 1) ? (fl[m] >> 4) : -1);
+    }
     // length of the innermost output axis = output elements per step of the axis before it
     const int64_t inner = last > 0 ? yblk[last - 1] : n;
-    bool vec = aligned16 && yblk[last] == 1 && xblk[last] == 1 && inner % 4 == 0 && n % 4 == 0;
-    for (int m = 0; m < last; m++) vec = vec && xblk[m] % 4 == 0 && yblk[m] % 4 == 0;
-    const bool small = n < (1ll << 31);
+    const bool vec = aligned16 && (all & 2) && inner % 4 == 0 && n % 4 == 0;
+    // the tiles: the source's innermost axis is not the output's (tensors of 2^31 elements and more stay with the
+    // element-wise loop: the tiles count in 32 bits)
+    if (small && mj >= 0 && mj != last && (all & 4)) {
+        __shared__ float tile[kTrTileFloats];
+        transpose_axes_tiled<BACKWARD>(out, in, yblk, xblk, osz, axis_size, mj, tile);
+        return;
+    }
     if (vec) {
         if (small) transpose_axes_body<int32_t, BACKWARD, true>(out, in, yblk, xblk, axis_size, n);
         else transpose_axes_body<int64_t, BACKWARD, true>(out, in, yblk, xblk, axis_size, n);

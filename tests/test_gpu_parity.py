@@ -1648,7 +1648,13 @@ def test_rnn_layer_loop(cell, ntimes, ndat, ninp, nrec, forward, bias):
 # ---- transposes ---------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("shape,axes", [((5,), (0,)), ((33, 70), (1, 0)), ((2, 3, 4), (2, 0, 1)), ((4, 512, 8, 64), (0, 2, 1, 3)),
-                                        ((3, 1, 5, 2), (3, 2, 1, 0)), ((2, 2, 2, 2, 3, 2, 2, 5), (7, 0, 6, 1, 5, 2, 4, 3))])
+                                        ((3, 1, 5, 2), (3, 2, 1, 0)), ((2, 2, 2, 2, 3, 2, 2, 5), (7, 0, 6, 1, 5, 2, 4, 3)),
+                                        # the innermost axis changes: tiles through LDS, every tile shape, edges, axes of one
+                                        ((1000, 777), (1, 0)), ((257, 1025), (1, 0)), ((8, 3, 50, 60), (0, 2, 3, 1)),
+                                        ((8, 50, 60, 3), (0, 3, 1, 2)), ((4, 70, 5, 33), (0, 2, 3, 1)), ((3, 40, 7, 9, 2), (4, 0, 3, 1, 2)),
+                                        ((2, 1, 100, 37), (3, 1, 0, 2)), ((37, 1), (1, 0)), ((1, 37), (1, 0)), ((6, 300, 10), (2, 0, 1)),
+                                        ((5, 2000, 2), (2, 1, 0)), ((2, 9, 1200), (2, 0, 1)), ((2, 1200, 13), (2, 1, 0)),
+                                        ((4, 64, 12, 16), (0, 2, 3, 1)), ((3, 5, 1, 1), (3, 1, 0, 2)), ((40, 6, 1), (1, 2, 0))])
 def test_transpose_axes(shape, axes):
     rng = np.random.default_rng(len(shape))
     x = rng.standard_normal(shape).astype(np.float32)
