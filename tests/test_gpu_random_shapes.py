@@ -242,3 +242,29 @@ def test_skinny_whole_tile_shapes_random():
         what = "case %d: %dx%dx%d pad %d/%d acc=%s bias=%s %s" % (it, m, n, k, padw, padx, acc, use_bias, act)
         assert np.isfinite(got).all(), what
         assert rel_fro(got, ref) <= REL_FRO_TOL, "%s: %.3e" % (what, rel_fro(got, ref))
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_transpose_random_permutations(seed):
+    """Random shapes of 1 to 6 axes (axes of one position among them, short and long innermost axes on either side)
+    under random permutations: every path of the general transpose kernel (128-bit words, tiles through LDS, element
+    by element), forward and backward, bit for bit against the oracle."""
+    kai, DB, VMath = _kai()
+    rng = np.random.default_rng(seed)
+    for it in range(60):
+        rank = int(rng.integers(1, 7))
+        shape = [int(rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 31, 32, 33, 64, 100, 257])) for _ in range(rank)]
+        while int(np.prod(shape)) > 3_000_000:
+            shape[int(np.argmax(shape))] = max(1, max(shape) // 2)
+        axes = [int(a) for a in rng.permutation(rank)]
+        x = rng.standard_normal(shape).astype(np.float32)
+        info = DB.from_numpy(ko.transpose_axinfo(tuple(shape), tuple(axes)))
+        what = "case %d: %s under %s" % (it, shape, axes)
+        y = DB(x.size * 4)
+        VMath.transpose(0, y, DB.from_numpy(x), info, rank, x.size)
+        yshape = [shape[a] for a in axes]
+        assert np.array_equal(y.to_numpy(yshape), ko.transpose(x, axes)), what
+        gy = rng.standard_normal(yshape).astype(np.float32)
+        gx = DB(x.size * 4)
+        VMath.transpose_backward(0, gx, DB.from_numpy(gy), info, rank, x.size)
+        assert np.array_equal(gx.to_numpy(shape), ko.transpose_backward(gy, tuple(shape), tuple(axes))), what + " (backward)"
