@@ -66,6 +66,10 @@ int launch_gru_process_from(float* r, const float* h_prev, const float* ai, cons
 // the nrow1 + nrow2 rows go to norms, then y[i,j] /= norms[i] * norms[nrow1 + j] + 1e-20
 int launch_cosine_norms_and_scale(float* y, float* norms, const float* x1, const float* x2, int64_t nrow1,
                                   int64_t nrow2, int64_t ncol, hipStream_t stream);
+// up to four rows of x1 against 512 and more of x2: both in one pass over x2
+bool cosine_few_rows_applies(const float* x1, const float* x2, int64_t nrow1, int64_t nrow2, int64_t ncol);
+int launch_cosine_few_rows(float* y, const float* x1, const float* x2, int64_t nrow1, int64_t nrow2, int64_t ncol,
+                           hipStream_t stream);
 
 // Final pass of a split-K product: C(m,n) (=|+=) act(alpha * sum_s part[s][m][n] + bias[n]), the
 // pre-activation value also to C2 when given.  `part` holds nsplit dense [M,N] matrices.

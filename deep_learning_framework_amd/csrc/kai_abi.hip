@@ -724,6 +724,8 @@ int kai_cosinesim(int device, float* py, const float* px1, const float* px2, int
     KAI_REQUIRE_PTR(py);
     if (ncol == 0) return launch_fill_float(py, nrow1 * nrow2, 0.0f, current_stream());   // 0 / 1e-20
     KAI_REQUIRE_PTR(px1); KAI_REQUIRE_PTR(px2);
+    if (cosine_few_rows_applies(px1, px2, nrow1, nrow2, ncol))
+        return launch_cosine_few_rows(py, px1, px2, nrow1, nrow2, ncol, current_stream());
     // the products are y = x1 . x2^T, the same NT product as matmul with x2 in the weight's place
     KAI_TRY(kai_matmul(device, py, px2, px1, nrow2, nrow1, ncol, 0));
     // the product may have used the scratch for its own partial sums; in stream order it is free again here

@@ -1482,7 +1482,10 @@ def test_matmul_with_a_two_gib_tile_span():
 
 # ---- cosinesim ----------------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("nrow1,nrow2,ncol", [(1, 1, 1), (6, 4, 33), (64, 512, 784), (300, 70, 1000), (2048, 2048, 64), (5, 4100, 128)])
+@pytest.mark.parametrize("nrow1,nrow2,ncol", [(1, 1, 1), (6, 4, 33), (64, 512, 784), (300, 70, 1000), (2048, 2048, 64), (5, 4100, 128),
+                                              # up to four rows against many: one pass over the many (and just outside its conditions)
+                                              (1, 100000, 256), (4, 5001, 2048), (3, 513, 4), (2, 1000, 36), (1, 600, 8192),
+                                              (4, 515, 100), (1, 600, 8196), (2, 700, 30), (4, 511, 64)])
 def test_cosinesim(nrow1, nrow2, ncol):
     rng = np.random.default_rng(nrow1 + ncol)
     a = rng.standard_normal((nrow1, ncol)).astype(np.float32)
