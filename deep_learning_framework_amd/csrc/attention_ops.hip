@@ -20,6 +20,7 @@
 namespace kai {
 
 constexpr int kTB = 256;
+typedef float f32x4s __attribute__((ext_vector_type(4)));
 
 // Wave-wide reductions through the DPP data path (result in every lane); see gemv_skinny.hip for
 // the sequence.  For the maximum, lanes that a row-masked broadcast step does not write keep their
@@ -47,23 +48,36 @@ __device__ __forceinline__ float wsum(float v) {
 
 // ---- mask -------------------------------------------------------------------------------------
 
-__global__ void __launch_bounds__(kTB) attention_mask_kernel(float* __restrict__ pp, int64_t total, int64_t ntimes,
-                                                             int64_t nhead, int forward) {
-    const int64_t stride = (int64_t)gridDim.x * kTB;
+// The masked elements of a query's row are one contiguous run: keys q + 1 .. T - 1 of every head.  A wave per row
+// fills it, 128-bit words between its unaligned ends (one thread per element of the WHOLE tensor with two 64-bit
+// divisions each took 20 us for 32 x 512 x 512, of which half is written).
+__global__ void __launch_bounds__(kTB) attention_mask_kernel(float* __restrict__ pp, int64_t nrows, int64_t ntimes,
+                                                             int64_t nhead, int forward, int aligned) {
     const float fillv = forward ? -INFINITY : 0.f;
-    for (int64_t n = (int64_t)blockIdx.x * kTB + threadIdx.x; n < total; n += stride) {
-        const int64_t nq = n / (ntimes * nhead) % ntimes;
-        const int64_t nk = n / nhead % ntimes;
-        if (nq < nk) pp[n] = fillv;
+    const int lane = threadIdx.x & 63;
+    const int64_t nwaves = (int64_t)gridDim.x * (kTB / 64);
+    for (int64_t row = (int64_t)blockIdx.x * (kTB / 64) + (threadIdx.x >> 6); row < nrows; row += nwaves) {
+        const int64_t q = row % ntimes;
+        const int64_t start = (row * ntimes + q + 1) * nhead, end = (row + 1) * ntimes * nhead;
+        if (!aligned) {
+            for (int64_t i = start + lane; i < end; i += 64) pp[i] = fillv;
+            continue;
+        }
+        const int64_t first = min(end, (start + 3) & ~(int64_t)3), last = max(first, end & ~(int64_t)3);
+        if (start + lane < first) pp[start + lane] = fillv;
+        const f32x4s w = {fillv, fillv, fillv, fillv};
+        for (int64_t i = first + 4 * lane; i < last; i += 256) *reinterpret_cast<f32x4s*>(pp + i) = w;
+        if (last + lane < end) pp[last + lane] = fillv;
     }
 }
 
 int launch_attention_mask(float* pp, int64_t ndat, int64_t ntimes, int64_t nhead, int forward, hipStream_t stream) {
-    const int64_t total = ndat * ntimes * ntimes * nhead;
-    if (total <= 0) return KAI_OK;
-    int64_t blocks = (total + kTB - 1) / kTB;
+    const int64_t nrows = ndat * ntimes;
+    if (nrows <= 0 || ntimes * nhead <= 0) return KAI_OK;
+    int64_t blocks = (nrows + kTB / 64 - 1) / (kTB / 64);
     if (blocks > 256 * 32) blocks = 256 * 32;
-    attention_mask_kernel<<<dim3((unsigned)blocks), kTB, 0, stream>>>(pp, total, ntimes, nhead, forward);
+    const int aligned = (reinterpret_cast<uintptr_t>(pp) & 15u) == 0;
+    attention_mask_kernel<<<dim3((unsigned)blocks), kTB, 0, stream>>>(pp, nrows, ntimes, nhead, forward, aligned);
     return check_launch("attention_mask_kernel");
 }
 
@@ -143,7 +157,6 @@ __global__ void __launch_bounds__(kTB) softmax_axis_block_kernel(float* __restri
 
 // ncol == 1, row length a multiple of 4 and at most 64*4*NV4: the whole row lives in registers
 // (NV4 float4 per lane), so HBM sees exactly one 128-bit read and one 128-bit write per element.
-typedef float f32x4s __attribute__((ext_vector_type(4)));
 
 // v where keep, else `other` in every element.  Bitwise on purpose: with a select the compiler moves
 // the load that produced v under the condition, and a conditional load is waited for before the next

@@ -1480,6 +1480,24 @@ def test_matmul_with_a_two_gib_tile_span():
     np.testing.assert_array_equal(got[40], ko.matmul_rows(w, x, [40])[0])
 
 
+@pytest.mark.parametrize("nbat,ntimes,nhead", [(1, 1, 1), (2, 2, 1), (3, 7, 3), (2, 33, 5), (1, 130, 4), (2, 64, 12), (1, 257, 1), (4, 100, 2)])
+def test_attention_mask_exact(nbat, ntimes, nhead):
+    """The masked run of every row filled, nothing else touched: both fill values, a buffer that starts on a 16-byte
+    line and one that does not, a guard behind the tensor."""
+    rng = np.random.default_rng(nbat + ntimes + nhead)
+    shape = (nbat, ntimes, ntimes, nhead)
+    n = int(np.prod(shape))
+    for shift in (0, 1, 3):
+        for forward in (True, False):
+            buf = rng.standard_normal(shift + n + 8).astype(np.float32)
+            d = dev(buf)
+            VMath.set_mh_attention_mask(0, d.offset(4 * shift), nbat, ntimes, nhead, forward)
+            got = d.to_numpy((shift + n + 8,))
+            want = buf.copy()
+            want[shift:shift + n] = ko.set_mh_attention_mask(buf[shift:shift + n].reshape(shape), forward).reshape(-1)
+            np.testing.assert_array_equal(got, want)
+
+
 # ---- cosinesim ----------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("nrow1,nrow2,ncol", [(1, 1, 1), (6, 4, 33), (64, 512, 784), (300, 70, 1000), (2048, 2048, 64), (5, 4100, 128),
