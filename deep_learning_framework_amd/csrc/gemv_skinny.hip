@@ -469,8 +469,16 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int kMmWaves = 8;
 constexpr int kMmUnroll = 16;  // steps of 16 k (1 KiB of W and of X each) per chunk
 
-template <bool VEC>
+// LOADS: 1 = 128-bit loads of operands whose rows start on 16-byte lines (K, ldw, ldx multiples of 4); 2 = 128-bit
+// BUFFER loads, which need 4-byte alignment only, for every other operand (K = 4095, rows of 769 floats: element by
+// element these took 26.5 us for 4096 x 4095 where 4096 x 4096 takes 12); what such a load reads past the end of a
+// row is masked like before, past the end of the matrix the buffer returns zeros; 0 = element by element (rows too
+// long for a buffer's 32-bit offsets).
+// CHUNK: steps of 16 k whose loads a wave issues together (0: 16 with 128-bit loads, 8 element by element); a wave's
+// share of a short row is a few steps, and a chunk is loaded whole (50257 x 769: 7 steps per wave).
+template <int LOADS, int CHUNK = 0>
 __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const SkinnyParams p) {
+    constexpr bool VEC = LOADS != 0;
     __shared__ float part[kMmWaves][256];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -492,9 +500,21 @@ __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const Skinny
     // Loads are raw: the address is clamped into the row, so that no branch sits between the loads
     // of a chunk and all of them are in flight together.  What lies beyond the row, the slice or the
     // matrix is zeroed when the value is consumed (bitwise, so that the load stays unconditional).
-    auto load4 = [&](const float* base, int k) -> f32x4v {
+    // (the buffers start at the workgroup's first row of W and at X; offsets fit 32 bits, the host has checked)
+    const int64_t w_bytes = ((p.N - 1 - min(n0, p.N - 1)) * p.ldw + p.K) * 4, x_bytes = ((int64_t)(p.M - 1) * p.ldx + p.K) * 4;
+    const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(p.W + n0 * p.ldw), 0, (int)min(w_bytes, (int64_t)0x7FFFFFFF), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(p.X), 0, (int)min(x_bytes, (int64_t)0x7FFFFFFF), 0x00020000);
+    const int w_row_off = (int)(r * p.ldw) * 4, x_row_off = (int)(r * p.ldx) * 4;
+    auto load4 = [&](auto of_w, int k) -> f32x4v {
+        constexpr bool kOfW = decltype(of_w)::value;
+        const float* base = kOfW ? wp : xp;
         f32x4v v;
-        if (VEC) {
+        if (LOADS == 2) {
+            v = __builtin_bit_cast(f32x4v, __builtin_amdgcn_raw_buffer_load_b128(kOfW ? rsrc_w : rsrc_x,
+                                                                                  (kOfW ? w_row_off : x_row_off) + k * 4, 0, 0));
+        } else if (VEC) {
             // K % 4 == 0: the float4 at k is entirely inside or outside
             v = *reinterpret_cast<const f32x4v*>(base + min(k, p.K - 4));
         } else {
@@ -518,13 +538,13 @@ __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const Skinny
     // flight per wave), then its MFMAs; the second wave of the SIMD computes meanwhile
     // (element-wise loads, 128 of them per chunk of 16 steps with an address each, do not fit the registers:
     // chunks of 8 steps there)
-    constexpr int UN = VEC ? kMmUnroll : kMmUnroll / 2;
+    constexpr int UN = CHUNK ? CHUNK : VEC ? kMmUnroll : kMmUnroll / 2;   // (VEC: both kinds of 128-bit loads)
     for (int base = s_begin; base < s_end; base += UN) {
         f32x4v w[UN], x[UN];
 #pragma unroll
-        for (int u = 0; u < UN; u++) w[u] = load4(wp, (base + u) * 16 + 4 * g);
+        for (int u = 0; u < UN; u++) w[u] = load4(std::true_type{}, (base + u) * 16 + 4 * g);
 #pragma unroll
-        for (int u = 0; u < UN; u++) x[u] = load4(xp, (base + u) * 16 + 4 * g);
+        for (int u = 0; u < UN; u++) x[u] = load4(std::false_type{}, (base + u) * 16 + 4 * g);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < UN; u++) {
@@ -562,10 +582,18 @@ __global__ void __launch_bounds__(64 * kMmWaves) skinny_mfma_kernel(const Skinny
 static int launch_skinny_mfma(const SkinnyParams& p, bool vec, hipStream_t stream) {
     const int64_t blocks = (p.N + 15) / 16;
     if (blocks > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "skinny matmul: too many output columns");
+    // 16 rows of W (and of X) and the chunks loaded past a row's end within a buffer's 31-bit offsets
+    const bool buffers = (16 * p.ldw + p.K + 1024) * 4 < (1ll << 31) && (16 * p.ldx + p.K + 1024) * 4 < (1ll << 31);
     if (vec)
-        skinny_mfma_kernel<true><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
+        skinny_mfma_kernel<1><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
+    else if (buffers && p.K <= 4 * 16 * kMmWaves)
+        skinny_mfma_kernel<2, 4><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
+    else if (buffers && p.K <= 8 * 16 * kMmWaves)
+        skinny_mfma_kernel<2, 8><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
+    else if (buffers)
+        skinny_mfma_kernel<2><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
     else
-        skinny_mfma_kernel<false><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
+        skinny_mfma_kernel<0><<<dim3((unsigned)blocks), dim3(64 * kMmWaves), 0, stream>>>(p);
     return check_launch("skinny_mfma_kernel");
 }
 

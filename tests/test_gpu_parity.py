@@ -457,6 +457,32 @@ def test_skinny_shapes_bias_act_acc(m, k, n):
     check(ya.to_numpy((m, n)), ko.matmul(w, x, acc_into=y0), what="skinny acc")
 
 
+@pytest.mark.parametrize("m,k,n,padw,padx", [(1, 4095, 4096, 0, 0), (1, 4097, 1000, 0, 0), (4, 4098, 300, 0, 0), (16, 4095, 1030, 0, 0),
+                                            (8, 1001, 513, 0, 0), (3, 769, 5000, 0, 0), (16, 37, 256, 0, 0), (5, 4096, 700, 3, 0),
+                                            (5, 4096, 700, 0, 1), (2, 999, 999, 5, 7), (13, 130, 2000, 1, 2), (1, 5, 256, 0, 0)])
+def test_few_rows_rows_off_16_byte_lines(m, k, n, padw, padx):
+    """Rows of W or X that do not start on 16-byte lines (K or a leading dimension not a multiple of 4): 128-bit buffer
+    loads at 4-byte alignment.  The last rows end with the buffers, NaN lies between the rows."""
+    rng = np.random.default_rng(m * 7 + k + n)
+    w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    wp = np.full(n * (k + padw) - padw, np.nan, np.float32)       # the last row is not padded: the buffer ends with it
+    xp = np.full(m * (k + padx) - padx, np.nan, np.float32)
+    for r in range(n):
+        wp[r * (k + padw): r * (k + padw) + k] = w[r]
+    for r in range(m):
+        xp[r * (k + padx): r * (k + padx) + k] = x[r]
+    b = rng.standard_normal(n).astype(np.float32)
+    y0 = rng.standard_normal((m, n)).astype(np.float32)
+    for acc in (0, 1):
+        dy = dev(y0)
+        VMath.gemm_f32(0, 0, 1, m, n, k, dev(xp), k + padx, dev(wp), k + padw, dy, n, dev(b), kai.ACT["tanh"], None, acc)
+        ref = ko.activate(ko.add_bias(ko.matmul(w, x, acc_into=y0 if acc else None), b), "tanh")
+        got = dy.to_numpy((m, n))
+        assert np.isfinite(got).all()
+        check(got, ref, what="rows off 16-byte lines, acc=%d, plan %s" % (acc, VMath.gemm_plan(0, 1, m, n, k, k + padx, k + padw, n)))
+
+
 @pytest.mark.parametrize("seed", list(range(1, 13)))
 def test_few_rows_random_shapes(seed):
     """1..33 rows against weight matrices of random width, length and row padding (multiples of 4, on and off the
