@@ -179,7 +179,24 @@ __device__ __forceinline__ f32x4s keep_or(f32x4s v, bool keep, float other) {
 // of these kernels' run time.  -inf gives 0, results below the normal range are flushed to 0.
 __device__ __forceinline__ float exp_nonpositive(float d) { return __builtin_amdgcn_exp2f(d * 1.44269504088896341f); }
 
-template <bool BACKWARD, int NV4>
+// the same element by element (a word that straddles the end of its row)
+__device__ __forceinline__ f32x4s keep_each_or(f32x4s v, int k, int nvec, float other) {
+    f32x4s r;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int m = k + j < nvec ? -1 : 0;
+        const float e = v[j];
+        r[j] = __int_as_float((__float_as_int(e) & m) | (__float_as_int(other) & ~m));
+    }
+    return r;
+}
+
+// UNAL: rows of any length at any 4-byte alignment (511 keys).  The 128-bit loads are buffer loads, which need no
+// more than that; the word that straddles the end of a row brings the next row's first elements (zeros behind the
+// last row: the buffer ends with the tensor), masked element by element, and is stored element by element, the
+// words before it as 128-bit buffer stores.  (Three passes of 32-bit accesses before: 32 x 511 x 511 20.8 us where
+// 512 keys take 8.3.)
+template <bool BACKWARD, int NV4, bool UNAL = false>
 __global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __restrict__ io,
                                                                     const float* __restrict__ pp, int64_t nrow,
                                                                     int nvec, const float* __restrict__ hcoef) {
@@ -187,12 +204,26 @@ __global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __res
     const int64_t wave = (int64_t)blockIdx.x * (kTB / 64) + (threadIdx.x >> 6);
     const int64_t nwaves = (int64_t)gridDim.x * (kTB / 64);
     const float coef = (BACKWARD && hcoef) ? *hcoef : 0.f;
+    auto row_resource = [&](const float* base, int64_t row) -> __amdgpu_buffer_rsrc_t {
+        const uint64_t a = reinterpret_cast<uint64_t>(base + row * nvec);
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+        const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+        const int64_t bytes = (nrow - row) * nvec * 4;
+        const int ext = __builtin_amdgcn_readfirstlane((int)(bytes < 0x7FFFFFFF ? bytes : 0x7FFFFFFF));
+        return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<float*>(((uint64_t)hi << 32) | lo), 0, ext, 0x00020000);
+    };
     for (int64_t row = wave; row < nrow; row += nwaves) {
         float* __restrict__ r = io + row * nvec;
         f32x4s v[NV4];
+        __amdgpu_buffer_rsrc_t rs_io;
+        if (UNAL) rs_io = row_resource(io, row);
 #pragma unroll
         for (int i = 0; i < NV4; i++) {
             const int k = 4 * lane + 256 * i;   // loads are unconditional (clamped), padding is masked below
+            if (UNAL) {
+                v[i] = __builtin_bit_cast(f32x4s, __builtin_amdgcn_raw_buffer_load_b128(rs_io, k * 4, 0, 0));
+                continue;
+            }
             // forward: rows that come straight from HBM gain 7 % from the non-temporal hint (14.5 -> 13.5 us for
             // 16384 rows of 512), rows still in the last-level cache lose nothing; backward it costs 1 us there
             const f32x4s* src = reinterpret_cast<const f32x4s*>(r + min(k, nvec - 4));
@@ -201,14 +232,31 @@ __global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __res
         f32x4s q[NV4];   // backward only
         if (BACKWARD) {
             const float* __restrict__ pr = pp + row * nvec;
+            __amdgpu_buffer_rsrc_t rs_p;
+            if (UNAL) rs_p = row_resource(pp, row);
 #pragma unroll
             for (int i = 0; i < NV4; i++) {
                 const int k = 4 * lane + 256 * i;
-                q[i] = *reinterpret_cast<const f32x4s*>(pr + min(k, nvec - 4));
+                if (UNAL) q[i] = __builtin_bit_cast(f32x4s, __builtin_amdgcn_raw_buffer_load_b128(rs_p, k * 4, 0, 0));
+                else q[i] = *reinterpret_cast<const f32x4s*>(pr + min(k, nvec - 4));
             }
         }
+        // a word of the row: 128 bits at once, or element by element where it straddles the row's end
+        auto store_word = [&](int k, f32x4s w) {
+            if (!UNAL) {
+                if (k < nvec) *reinterpret_cast<f32x4s*>(r + k) = w;
+            } else if (k + 4 <= nvec) {
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int, w), rs_io, k * 4, 0, 0);
+            } else {
 #pragma unroll
-        for (int i = 0; i < NV4; i++) v[i] = keep_or(v[i], 4 * lane + 256 * i < nvec, BACKWARD ? 0.f : -INFINITY);
+                for (int j = 0; j < 3; j++)
+                    if (k + j < nvec) r[k + j] = w[j];
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < NV4; i++)
+            v[i] = UNAL ? keep_each_or(v[i], 4 * lane + 256 * i, nvec, BACKWARD ? 0.f : -INFINITY)
+                        : keep_or(v[i], 4 * lane + 256 * i < nvec, BACKWARD ? 0.f : -INFINITY);
         if (!BACKWARD) {
             float mx = -FLT_MAX;
 #pragma unroll
@@ -224,23 +272,17 @@ __global__ void __launch_bounds__(kTB) softmax_axis_wave_reg_kernel(float* __res
                 }
             const float inv = 1.0f / wsum(sum);
 #pragma unroll
-            for (int i = 0; i < NV4; i++) {
-                const int k = 4 * lane + 256 * i;
-                if (k < nvec) *reinterpret_cast<f32x4s*>(r + k) = v[i] * inv;
-            }
+            for (int i = 0; i < NV4; i++) store_word(4 * lane + 256 * i, v[i] * inv);
         } else {
             float dot = 0.f;
 #pragma unroll
             for (int i = 0; i < NV4; i++) {
-                q[i] = keep_or(q[i], 4 * lane + 256 * i < nvec, 0.f);
+                q[i] = UNAL ? keep_each_or(q[i], 4 * lane + 256 * i, nvec, 0.f) : keep_or(q[i], 4 * lane + 256 * i < nvec, 0.f);
                 dot += q[i][0] * v[i][0] + q[i][1] * v[i][1] + q[i][2] * v[i][2] + q[i][3] * v[i][3];
             }
             dot = wsum(dot);
 #pragma unroll
-            for (int i = 0; i < NV4; i++) {
-                const int k = 4 * lane + 256 * i;
-                if (k < nvec) *reinterpret_cast<f32x4s*>(r + k) = coef * q[i] * (v[i] - dot);
-            }
+            for (int i = 0; i < NV4; i++) store_word(4 * lane + 256 * i, coef * q[i] * (v[i] - dot));
         }
     }
 }
@@ -580,6 +622,14 @@ static int launch_softmax_axis_impl(float* io, const float* pp, int64_t nrow, in
             else if (nvec <= 512) softmax_axis_wave_reg_kernel<BACKWARD, 2><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
             else if (nvec <= 1024) softmax_axis_wave_reg_kernel<BACKWARD, 4><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
             else softmax_axis_wave_reg_kernel<BACKWARD, 8><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+        } else if (nvec >= 64 && nvec <= 2048) {
+            // rows off 16-byte lines: the same kernels through buffer accesses
+            const unsigned g = (unsigned)(blocks < 256 * 8 ? blocks : 256 * 8);
+            const int nv = (int)nvec;
+            if (nvec <= 256) softmax_axis_wave_reg_kernel<BACKWARD, 1, true><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+            else if (nvec <= 512) softmax_axis_wave_reg_kernel<BACKWARD, 2, true><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+            else if (nvec <= 1024) softmax_axis_wave_reg_kernel<BACKWARD, 4, true><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
+            else softmax_axis_wave_reg_kernel<BACKWARD, 8, true><<<g, kTB, 0, stream>>>(io, pp, nrow, nv, hcoef);
         } else {
             softmax_axis_wave_kernel<BACKWARD><<<dim3((unsigned)blocks), kTB, 0, stream>>>(io, pp, nrow, nvec, hcoef);
         }

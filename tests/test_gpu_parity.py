@@ -1041,7 +1041,10 @@ SOFTMAX_AXIS_SHAPES = [(5, 1, 1), (3, 1000, 1), (4, 3000, 1), (7, 33, 3), (2, 51
                        (2, 5, 300), (300, 512, 1), (3, 2048, 1), (2, 2052, 1), (2, 700, 8), (1, 2000, 8),
                        (2, 1030, 2), (40, 64, 16),
                        # many rows with 4, 8, 16 or 128 heads: a whole head-interleaved row per wave
-                       (1100, 33, 8), (2048, 512, 8), (1030, 100, 4), (1200, 30, 128), (1024, 1024, 4), (1500, 7, 16)]
+                       (1100, 33, 8), (2048, 512, 8), (1030, 100, 4), (1200, 30, 128), (1024, 1024, 4), (1500, 7, 16),
+                       # one head, rows off 16-byte lines: every register depth of the buffer-access variant and its bounds
+                       (37, 65, 1), (1031, 77, 1), (300, 255, 1), (300, 257, 1), (1200, 511, 1), (50, 513, 1), (20, 1001, 1),
+                       (9, 2047, 1), (9, 2049, 1), (33, 63, 1), (5, 66, 1)]
 
 
 # fused forward attention against the oracle's four separate steps: both cfg4 mappings, ragged lengths, the three
@@ -1155,15 +1158,45 @@ def test_softmax_axis_layouts(nrow, nvec, ncol):
 @pytest.mark.parametrize("nbat,ntimes,nhead", [(3, 512, 1), (1, 512, 8), (2, 700, 8), (1, 2000, 4), (1, 300, 130), (3, 400, 4), (9, 130, 16),
                                                (2, 2052, 1)])
 def test_softmax_axis_backward_layouts(nbat, ntimes, nhead):
+    _softmax_axis_backward_case(nbat, ntimes, nhead, 0)
+
+
+@pytest.mark.parametrize("nbat,ntimes,shift", [(3, 511, 0), (2, 257, 0), (40, 65, 0), (1, 1001, 0), (1, 2047, 0), (2, 77, 0),
+                                               (3, 512, 1), (2, 128, 3)])
+def test_softmax_axis_one_head_rows_off_16_byte_lines(nbat, ntimes, shift):
+    """One head with an odd number of keys, or a tensor that does not start on a 16-byte line: forward in place and
+    backward, the words behind the tensor untouched."""
+    rng = np.random.default_rng(nbat + ntimes + shift)
+    n = nbat * ntimes * ntimes
+    buf = np.full(shift + n + 8, 7.0, np.float32)
+    logits = (4 * rng.standard_normal(n)).astype(np.float32)
+    buf[shift:shift + n] = logits
+    d = dev(buf)
+    VMath.softmax_direct_on_axis(0, d.offset(4 * shift), nbat * ntimes, ntimes, 1)
+    got = d.to_numpy((shift + n + 8,))
+    assert (got[:shift] == 7.0).all() and (got[shift + n:] == 7.0).all()
+    check(got[shift:shift + n].reshape(nbat * ntimes, ntimes),
+          ko.softmax_direct_on_axis(logits.reshape(nbat * ntimes, ntimes, 1), nbat * ntimes, ntimes, 1).reshape(nbat * ntimes, ntimes),
+          what="softmax axis, one head, shift %d" % shift)
+    _softmax_axis_backward_case(nbat, ntimes, 1, shift)
+
+
+def _softmax_axis_backward_case(nbat, ntimes, nhead, shift):
     rng = np.random.default_rng(nbat + ntimes + nhead)
     shape = (nbat, ntimes, ntimes, nhead)
     logits = (3 * rng.standard_normal(shape)).astype(np.float32)
     probs = ko.softmax_direct_on_axis(logits, nbat * ntimes, ntimes, nhead).reshape(shape)
     gp = rng.standard_normal(shape).astype(np.float32)
     coef = 0.125
-    dgp, dp, hcoef = dev(gp), dev(probs), kai.hyper(coef)
-    VMath.softmax_direct_on_axis_backward(0, dgp, dp, nbat, ntimes, nhead, hcoef)
-    check(dgp.to_numpy(shape), ko.softmax_direct_on_axis_backward(gp, probs, coef), what="softmax axis backward")
+    n = gp.size
+    gbuf, pbuf = np.full(shift + n + 8, 7.0, np.float32), np.full(shift + n + 8, np.nan, np.float32)
+    gbuf[shift:shift + n] = gp.reshape(-1)
+    pbuf[shift:shift + n] = probs.reshape(-1)
+    dgp, dp, hcoef = dev(gbuf), dev(pbuf), kai.hyper(coef)
+    VMath.softmax_direct_on_axis_backward(0, dgp.offset(4 * shift), dp.offset(4 * shift), nbat, ntimes, nhead, hcoef)
+    got = dgp.to_numpy((shift + n + 8,))
+    assert (got[:shift] == 7.0).all() and (got[shift + n:] == 7.0).all()
+    check(got[shift:shift + n].reshape(shape), ko.softmax_direct_on_axis_backward(gp, probs, coef), what="softmax axis backward")
 
 
 def test_split_k_scratch_survives_shutdown_and_growth():
