@@ -79,6 +79,7 @@ struct GemmParams {
     int64_t a_bs0, a_bs1, b_bs0, b_bs1, c_bs0, c_bs1;
     int bdiv;
     int a_vec, b_vec, c_vec;  // 16-byte aligned 128-bit access along the contiguous index is legal
+    int c_buf;                // short-reduction kernel: rows of C off 16-byte lines take 128-bit buffer stores
     int a_cont, b_cont;       // the operand has a unit stride (then buffer loads may fetch 128 bits at 4-byte alignment)
     int edge_buf;             // general kernels: a tile of either operand spans less than 2 GiB (buffer loads)
     int act;

@@ -111,6 +111,15 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
     // the two scalars of the epilogue are fetched before any store is in flight
     float alpha = p.has_alpha ? (p.alpha ? *p.alpha : 0.f) : 1.f;
     float leaky = p.leaky ? *p.leaky : 0.f;
+    // this batch entry's C as a buffer (used where p.c_buf says so; the host has checked that it spans less than 2 GiB)
+    // (the halves as unsigned 32-bit values before they are joined: readfirstlane returns a signed int, and a low
+    // half with its top bit set would otherwise fill the high half with ones)
+    const uint64_t c_addr = reinterpret_cast<uint64_t>(p.C + c_off);
+    const uint32_t c_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)c_addr);
+    const uint32_t c_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(c_addr >> 32));
+    const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<float*>(((uint64_t)c_hi << 32) | c_lo), 0,
+        p.c_buf ? (int)((((int64_t)p.M - 1) * p.c_rs + p.N) * 4) : 0, 0x00020000);
 
     constexpr int NCHA = kSkBM * kSkK / 4 / kSkThreads;
     constexpr int NCHB = kSkBN * kSkK / 4 / kSkThreads;
@@ -206,6 +215,11 @@ __global__ void __launch_bounds__(kSkThreads) shortk_nt_kernel(const GemmParams 
                             // streaming: whole 512-byte rows that this kernel never reads again; otherwise the
                             // dirty lines pile up in L2 and are written back after the last wave has ended
                             if (col < p.N) __builtin_nontemporal_store(o, reinterpret_cast<f32x4*>(out));
+                        } else if (p.c_buf && col + 4 <= p.N) {
+                            // rows of C off 16-byte lines (511 keys): a buffer store needs 4-byte alignment only
+                            __builtin_amdgcn_raw_buffer_store_b128(
+                                __builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int, o),
+                                rsrc_c, (int)(((int64_t)row * p.c_rs + col) * 4), 0, 0);
                         } else {
 #pragma unroll
                             for (int j = 0; j < 4; j++)
@@ -428,6 +442,7 @@ int launch_gemm_shortk_nt(GemmParams p, int64_t nbatch, hipStream_t stream) {
     if (p.accflag || p.bias || p.C2 || p.act != kActNone)
         return fail(KAI_ERR_INVALID_ARGUMENT, "gemm: the short-reduction kernel has no accumulate / bias / activation epilogue");
     const bool whole = p.M % kSkBM == 0 && p.N % kSkBN == 0 && p.K == kSkK && p.a_vec && p.b_vec && p.c_vec;
+    p.c_buf = !p.c_vec && ((int64_t)p.M * p.c_rs + 4) * 4 < (1ll << 31);
     if (whole) {
         shortk_nt_kernel<8, true><<<grid, dim3(kSkThreads), 0, stream>>>(p);
     } else if (p.K <= 32) {
