@@ -1043,6 +1043,8 @@ int launch_gru_process_backward(float* gr, float* gai, float* gar, const float* 
 // y[i,j] = <a_i, b_j> / (|a_i| |b_j| + 1e-20).  The products come from the GEMM; row_norm_kernel writes
 // |row| for the rows of both operands (a wave per row), cosine_scale_kernel divides.
 
+// VEC: ncol a multiple of 4 and both operands on 16-byte lines: 128-bit loads
+template <bool VEC>
 __global__ void __launch_bounds__(256) row_norm_kernel(float* __restrict__ out, const float* __restrict__ x1,
                                                        int64_t nrow1, const float* __restrict__ x2, int64_t nrow2,
                                                        int64_t ncol) {
@@ -1051,7 +1053,15 @@ __global__ void __launch_bounds__(256) row_norm_kernel(float* __restrict__ out, 
     if (row >= nrow1 + nrow2) return;
     const float* xr = row < nrow1 ? x1 + row * ncol : x2 + (row - nrow1) * ncol;
     float s = 0.f;
-    for (int64_t c = lane; c < ncol; c += 64) s += xr[c] * xr[c];
+    if (VEC) {
+        const f32x4* __restrict__ x4 = reinterpret_cast<const f32x4*>(xr);
+        for (int64_t c = lane; c < ncol / 4; c += 64) {
+            const f32x4 v = x4[c];
+            s += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+        }
+    } else {
+        for (int64_t c = lane; c < ncol; c += 64) s += xr[c] * xr[c];
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
     if (lane == 0) out[row] = sqrtf(s);
@@ -1072,7 +1082,10 @@ int launch_cosine_norms_and_scale(float* y, float* norms, const float* x1, const
     const int64_t rows = nrow1 + nrow2;
     if (rows <= 0 || nrow1 * nrow2 <= 0) return KAI_OK;
     if ((rows + 3) / 4 > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "cosinesim: too many rows");
-    row_norm_kernel<<<dim3((unsigned)((rows + 3) / 4)), 256, 0, stream>>>(norms, x1, nrow1, x2, nrow2, ncol);
+    if (ncol % 4 == 0 && aligned16(x1) && aligned16(x2))
+        row_norm_kernel<true><<<dim3((unsigned)((rows + 3) / 4)), 256, 0, stream>>>(norms, x1, nrow1, x2, nrow2, ncol);
+    else
+        row_norm_kernel<false><<<dim3((unsigned)((rows + 3) / 4)), 256, 0, stream>>>(norms, x1, nrow1, x2, nrow2, ncol);
     KAI_TRY(check_launch("row_norm_kernel"));
     cosine_scale_kernel<<<blocks_for(nrow1 * nrow2), kEwThreads, 0, stream>>>(y, norms, nrow1, nrow2);
     return check_launch("cosine_scale_kernel");
