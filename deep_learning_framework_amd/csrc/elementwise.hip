@@ -425,12 +425,20 @@ static int launch_softmax_rows_impl(float* out, const float* gy, const float* x,
     const int64_t blocks = (nrow + kEwThreads / 64 - 1) / (kEwThreads / 64);
     if (blocks > kMaxDim || nrow > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "activate(softmax): too many rows");
     const bool few_rows = nrow < 8 * (int64_t)compute_units();
-    if ((ncol > 4096 || (few_rows && ncol >= 1024)) && ncol <= 16 * kSmxThreads) {
+    // (a vocabulary of 50257 columns: 50 registers per thread forward; the derivative holds two rows and stays within
+    // a thread's 128 registers up to 32 per row)
+    constexpr int kRegCols = (BACKWARD ? 32 : 64) * kSmxThreads;
+    if ((ncol > 4096 || (few_rows && ncol >= 1024)) && ncol <= kRegCols) {
         const dim3 g((unsigned)nrow);
         if (ncol <= 4096) softmax_rows_block_reg_kernel<BACKWARD, 4><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
         else if (ncol <= 8192) softmax_rows_block_reg_kernel<BACKWARD, 8><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
         else if (ncol <= 12288) softmax_rows_block_reg_kernel<BACKWARD, 12><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
-        else softmax_rows_block_reg_kernel<BACKWARD, 16><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
+        else if (ncol <= 16384) softmax_rows_block_reg_kernel<BACKWARD, 16><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
+        else if (ncol <= 32768) softmax_rows_block_reg_kernel<BACKWARD, 32><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
+        else if constexpr (!BACKWARD) {
+            if (ncol <= 53248) softmax_rows_block_reg_kernel<BACKWARD, 52><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
+            else softmax_rows_block_reg_kernel<BACKWARD, 64><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
+        }
         return check_launch("softmax_rows_block_reg_kernel");
     }
     if (ncol > 4096 || (few_rows && ncol >= 1024)) {

@@ -669,7 +669,7 @@ def test_relu_special_values_and_null_leaky_alpha():
 @pytest.mark.parametrize("nrow,ncol", [(50, 77), (3000, 10), (300, 64), (300, 65), (500, 130), (300, 300), (300, 600),
                                        (2100, 1000), (2100, 2048), (40, 1500), (300, 2049), (2100, 3000), (2060, 4096), (64, 4097), (7, 50257), (5, 1),
                                        # a workgroup's registers: every depth, and the first length beyond them
-                                       (40, 4096), (33, 8192), (20, 8193), (20, 12289), (16, 16384), (9, 16385),
+                                       (40, 4096), (33, 8192), (20, 8193), (20, 12289), (16, 16384), (9, 16385), (5, 20000), (4, 32769), (3, 60000), (2, 70000),
                                        # several short rows per wave
                                        (100001, 12), (1001, 2), (1001, 3), (999, 5), (777, 17), (501, 32), (501, 33)])
 def test_softmax_activation_rows(nrow, ncol):
