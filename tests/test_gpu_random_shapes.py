@@ -268,3 +268,40 @@ def test_transpose_random_permutations(seed):
         gx = DB(x.size * 4)
         VMath.transpose_backward(0, gx, DB.from_numpy(gy), info, rank, x.size)
         assert np.array_equal(gx.to_numpy(shape), ko.transpose_backward(gy, tuple(shape), tuple(axes))), what + " (backward)"
+
+
+@pytest.mark.parametrize("seed", [51, 52, 53])
+def test_few_rows_odd_lengths_random(seed):
+    """1..16 rows against matrices whose reduction length and leading dimensions are NOT multiples of 4 (rows off
+    16-byte lines: 128-bit buffer loads in chunks of 4, 8 or 16 steps), NaN between the rows, the buffers ending with
+    their last rows; bias, activation and accumulation at random."""
+    kai, DB, VMath = _kai()
+    rng = np.random.default_rng(seed)
+    for it in range(24):
+        m = int(rng.integers(1, 17))
+        k = int(rng.choice([5, 37, 63, 65, 130, 511, 513, 769, 1001, 1027, 2049, 4095, 4097, 6001]))
+        n = int(rng.choice([256, 257, 300, 1000, 1030, 2500, 4099]))
+        n = min(n, max(256, int(4e6 // k)))
+        padw, padx = int(rng.choice([0, 1, 2, 3, 5])), int(rng.choice([0, 1, 3]))
+        w = rng.uniform(-0.05, 0.05, (n, k)).astype(np.float32)
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        wp = np.full(n * (k + padw) - padw, np.nan, np.float32)
+        xp = np.full(m * (k + padx) - padx, np.nan, np.float32)
+        for r in range(n):
+            wp[r * (k + padw): r * (k + padw) + k] = w[r]
+        for r in range(m):
+            xp[r * (k + padx): r * (k + padx) + k] = x[r]
+        bias = rng.standard_normal(n).astype(np.float32)
+        y0 = rng.standard_normal((m, n)).astype(np.float32)
+        acc, use_bias, act = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), str(rng.choice(["none", "relu", "tanh"]))
+        y = DB.from_numpy(y0)
+        VMath.gemm_f32(0, 0, 1, m, n, k, DB.from_numpy(xp), k + padx, DB.from_numpy(wp), k + padw, y, n,
+                       DB.from_numpy(bias) if use_bias else None, kai.ACT[act], None, acc)
+        ref = ko.matmul(w, x, acc_into=y0 if acc else None)
+        if use_bias:
+            ref = ko.add_bias(ref, bias)
+        ref = ko.activate(ref, act)
+        got = y.to_numpy((m, n))
+        what = "case %d: %dx%dx%d pad %d/%d acc=%s bias=%s %s" % (it, m, n, k, padw, padx, acc, use_bias, act)
+        assert np.isfinite(got).all(), what
+        assert rel_fro(got, ref) <= REL_FRO_TOL, "%s: %.3e" % (what, rel_fro(got, ref))
