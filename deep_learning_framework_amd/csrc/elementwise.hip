@@ -365,7 +365,10 @@ __global__ void __launch_bounds__(kSmxThreads) softmax_rows_block_kernel(float* 
 
 // A workgroup per row with the row in its registers (ncol <= 1024 * E, up to 16384 columns): one read of x and one
 // expf per element where the kernel above has three and two ([8192, 8192] 215 us there).
-template <bool BACKWARD, int E>
+// KEEP_G (the derivative only): the incoming gradient waits in registers next to the row; without it the gradient is
+// read a second time for the last pass (from L2: a row of 65536 floats is 256 KB), which leaves room for rows twice
+// as long.
+template <bool BACKWARD, int E, bool KEEP_G = true>
 __global__ void __launch_bounds__(kSmxThreads) softmax_rows_block_reg_kernel(float* __restrict__ out,
                                                                              const float* __restrict__ gy,
                                                                              const float* __restrict__ x, int64_t ncol) {
@@ -381,13 +384,13 @@ __global__ void __launch_bounds__(kSmxThreads) softmax_rows_block_reg_kernel(flo
         for (int w = 1; w < kSmxThreads / 64; w++) a = is_max ? fmaxf(a, red[which][w]) : a + red[which][w];
         return a;
     };
-    float v[E], gr[E];
+    float v[E], gr[KEEP_G ? E : 1];
     float mx = -FLT_MAX;
 #pragma unroll
     for (int i = 0; i < E; i++) {
         const int64_t c = t + kSmxThreads * i;
         v[i] = c < ncol ? xr[c] : -INFINITY;
-        if (BACKWARD) gr[i] = c < ncol ? gy[row * ncol + c] : 0.f;
+        if (BACKWARD && KEEP_G) gr[i] = c < ncol ? gy[row * ncol + c] : 0.f;
         mx = fmaxf(mx, v[i]);
     }
     mx = block_fold(mx, true, 0);
@@ -407,12 +410,16 @@ __global__ void __launch_bounds__(kSmxThreads) softmax_rows_block_reg_kernel(flo
 #pragma unroll
         for (int i = 0; i < E; i++) {
             v[i] = v[i] / sum;
-            dot += v[i] * gr[i];
+            if (KEEP_G) dot += v[i] * gr[i];
+            else if (t + kSmxThreads * i < ncol) dot += v[i] * gy[row * ncol + t + kSmxThreads * i];
         }
         dot = block_fold(dot, false, 2);
 #pragma unroll
         for (int i = 0; i < E; i++)
-            if (t + kSmxThreads * i < ncol) out[row * ncol + t + kSmxThreads * i] = v[i] * gr[i] - v[i] * dot;
+            if (t + kSmxThreads * i < ncol) {
+                const float g = KEEP_G ? gr[i] : gy[row * ncol + t + kSmxThreads * i];
+                out[row * ncol + t + kSmxThreads * i] = v[i] * g - v[i] * dot;
+            }
     }
 }
 
@@ -426,8 +433,8 @@ static int launch_softmax_rows_impl(float* out, const float* gy, const float* x,
     if (blocks > kMaxDim || nrow > kMaxDim) return fail(KAI_ERR_INVALID_ARGUMENT, "activate(softmax): too many rows");
     const bool few_rows = nrow < 8 * (int64_t)compute_units();
     // (a vocabulary of 50257 columns: 50 registers per thread forward; the derivative holds two rows and stays within
-    // a thread's 128 registers up to 32 per row)
-    constexpr int kRegCols = (BACKWARD ? 32 : 64) * kSmxThreads;
+    // a thread's 128 registers up to 32 per row: beyond, it keeps the row and reads the gradient twice)
+    constexpr int kRegCols = 64 * kSmxThreads;
     if ((ncol > 4096 || (few_rows && ncol >= 1024)) && ncol <= kRegCols) {
         const dim3 g((unsigned)nrow);
         if (ncol <= 4096) softmax_rows_block_reg_kernel<BACKWARD, 4><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
@@ -435,10 +442,8 @@ static int launch_softmax_rows_impl(float* out, const float* gy, const float* x,
         else if (ncol <= 12288) softmax_rows_block_reg_kernel<BACKWARD, 12><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
         else if (ncol <= 16384) softmax_rows_block_reg_kernel<BACKWARD, 16><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
         else if (ncol <= 32768) softmax_rows_block_reg_kernel<BACKWARD, 32><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
-        else if constexpr (!BACKWARD) {
-            if (ncol <= 53248) softmax_rows_block_reg_kernel<BACKWARD, 52><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
-            else softmax_rows_block_reg_kernel<BACKWARD, 64><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
-        }
+        else if (ncol <= 53248) softmax_rows_block_reg_kernel<BACKWARD, 52, !BACKWARD><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
+        else softmax_rows_block_reg_kernel<BACKWARD, 64, !BACKWARD><<<g, kSmxThreads, 0, stream>>>(out, gy, x, ncol);
         return check_launch("softmax_rows_block_reg_kernel");
     }
     if (ncol > 4096 || (few_rows && ncol >= 1024)) {
