@@ -461,9 +461,14 @@ int kai_add_bias_backward_b(int device, float* pgb, const float* pgy, int64_t nr
     if (ncol == 0) return KAI_OK;
     KAI_REQUIRE_PTR(pgb);
     if (nrow > 0) KAI_REQUIRE_PTR(pgy);
-    const int parts = colsum_row_parts(nrow, ncol);
+    int parts = colsum_row_parts(nrow, ncol);
     float* parts_buf = nullptr;
-    if (parts >= 2) KAI_TRY(workspace(parts * ncol * (int64_t)sizeof(float), &parts_buf));
+    // no scratch to be had (the stream is being captured and the buffer would have to grow, or the allocation
+    // failed): the single launch needs none
+    if (parts >= 2 && workspace(parts * ncol * (int64_t)sizeof(float), &parts_buf) != KAI_OK) {
+        parts = 1;
+        parts_buf = nullptr;
+    }
     return launch_colsum(pgb, pgy, nrow, ncol, acc != 0, current_stream(), parts_buf, parts);
 }
 

@@ -156,7 +156,8 @@ int64_t kai_matmul_noalloc_scratch_bytes(void);
 /* VMath::add_bias, vmath.cu:875-897.  y[r,c] = a[r,c] + b[c]; py may equal pa */
 int kai_add_bias(int device, float* py, const float* pa, const float* pb, int64_t nrow, int64_t ncol);
 /* VMath::add_bias_backward_b, vmath.cu:901-932.  gb[c] (=|+=) sum_r gy[r,c].  With 6144 rows and more over few
- * columns the rows are summed in runs whose sums pass through the library scratch (at most 128 KiB). */
+ * columns the rows are summed in runs whose sums pass through the library scratch (at most 128 KiB); where that would have to grow during a stream
+ * capture the call takes its single launch instead, which needs none. */
 int kai_add_bias_backward_b(int device, float* pgb, const float* pgy, int64_t nrow, int64_t ncol, int acc);
 
 /* VMath::activate, vmath.cu:3097-3243; py may equal px (except for softmax).  The softmax case

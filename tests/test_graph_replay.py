@@ -105,6 +105,32 @@ def _body():
                     assert torch.equal(a, ref_a), "replay for seed %d differs from the eager calls" % seed
     finally:
         kai.set_stream(None)
+    # A column sum over many rows of a narrow matrix cuts the rows into runs whose sums pass through the library
+    # scratch; recorded on a stream that has no scratch yet (nothing may be allocated during a capture) it must take
+    # its single launch instead of failing, and the replays must give the column sums.
+    tall, sums = t(20000, 12), t(12)
+    stream2 = torch.cuda.Stream()
+    try:
+        kai.set_stream(stream2.cuda_stream)
+        with torch.cuda.stream(stream2):
+            tall.normal_(generator=gen)
+            stream2.synchronize()
+            graph2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph2, stream=stream2):
+                VMath.add_bias_backward_b(0, P(sums), P(tall), 20000, 12, False)
+            for seed in (21, 22):
+                gen.manual_seed(seed)
+                tall.normal_(generator=gen)
+                sums.fill_(float("nan"))
+                graph2.replay()
+                stream2.synchronize()
+                ref = tall.double().sum(0)
+                assert float((sums.double() - ref).norm() / ref.norm()) <= REL_FRO_TOL
+            VMath.add_bias_backward_b(0, P(sums), P(tall), 20000, 12, False)   # eager: the runs, through the scratch
+            stream2.synchronize()
+            assert float((sums.double() - ref).norm() / ref.norm()) <= REL_FRO_TOL
+    finally:
+        kai.set_stream(None)
     print("graph replays equal eager")
 
 
